@@ -1,0 +1,107 @@
+// Entry points of decode attention: argument checks and the choice between the
+// MFMA kernel (head_dim 128, 4 query heads per KV head, block_size 64) and the
+// shape-agnostic kernel.
+#include "fdattn_common.h"
+
+namespace fdattn {
+size_t generic_workspace_bytes(int batch, int hq, int d);
+int decode_generic_launch(const void* q, const void* key_cache, const void* value_cache,
+                          const float* k_scale, const float* v_scale, const int32_t* block_tables,
+                          const int32_t* seq_lens_decoder, const int32_t* seq_lens_this_time,
+                          const int32_t* kept_blocks, const int32_t* kept_counts, int max_kept,
+                          void* out, void* workspace, size_t workspace_bytes, int batch, int hq,
+                          int hkv, int d, int bs, int max_blocks, int num_blocks, int quant,
+                          float sm_scale, hipStream_t s);
+size_t c8_workspace_bytes(int batch, int hkv);
+bool c8_supported(int hq, int hkv, int d, int bs, int quant);
+int decode_c8_launch(const void* q, const void* key_cache, const void* value_cache,
+                     const float* k_scale, const float* v_scale, const int32_t* block_tables,
+                     const int32_t* seq_lens_decoder, const int32_t* seq_lens_this_time,
+                     const int32_t* kept_blocks, const int32_t* kept_counts, int max_kept,
+                     void* out, void* workspace, size_t workspace_bytes, int batch, int hq,
+                     int hkv, int d, int bs, int max_blocks, int num_blocks, int quant,
+                     float sm_scale, hipStream_t s);
+
+static int check_decode_args(const char* fn, const void* q, const void* kc, const void* vc, const float* ks,
+                             const float* vs, const int32_t* bt, const int32_t* dec, const void* out,
+                             const void* ws, int batch, int hq, int hkv, int d, int bs, int max_blocks,
+                             int num_blocks, int quant) {
+  if (!q || !kc || !vc || !ks || !vs || !bt || !dec || !out || !ws)
+    return fail(FDATTN_ERR_NULL, "%s: a required pointer is NULL", fn);
+  if (batch <= 0 || hq <= 0 || hkv <= 0 || hq % hkv != 0 || d <= 0 || bs <= 0 || max_blocks <= 0 ||
+      num_blocks <= 0)
+    return fail(FDATTN_ERR_SHAPE, "%s: bad shape batch=%d hq=%d hkv=%d head_dim=%d block_size=%d max_blocks=%d "
+                "num_blocks=%d", fn, batch, hq, hkv, d, bs, max_blocks, num_blocks);
+  if (quant != FDATTN_CACHE_INT8 && quant != FDATTN_CACHE_FP8_E4M3)
+    return fail(FDATTN_ERR_QUANT, "%s: unknown cache_quant_type %d", fn, quant);
+  return 0;
+}
+
+}  // namespace fdattn
+
+using namespace fdattn;
+
+extern "C" size_t fdattn_decode_workspace_bytes(int batch, int hq, int hkv, int head_dim) {
+  if (batch <= 0 || hq <= 0 || hkv <= 0 || head_dim <= 0) return 256;
+  size_t a = generic_workspace_bytes(batch, hq, head_dim);
+  size_t b = c8_workspace_bytes(batch, hkv);
+  size_t n = a > b ? a : b;
+  return (n + 255) & ~(size_t)255;
+}
+
+extern "C" int fdattn_decode_attention(
+    const void* q, const void* key_cache, const void* value_cache, const float* cache_k_scale,
+    const float* cache_v_scale, const int32_t* block_tables, const int32_t* seq_lens_decoder,
+    const int32_t* seq_lens_this_time, void* out, void* workspace, size_t workspace_bytes, int batch,
+    int hq, int hkv, int head_dim, int block_size, int max_blocks_per_seq, int num_blocks,
+    int cache_quant_type, float softmax_scale, void* stream) {
+  int rc = check_decode_args("fdattn_decode_attention", q, key_cache, value_cache, cache_k_scale,
+                             cache_v_scale, block_tables, seq_lens_decoder, out, workspace, batch, hq, hkv,
+                             head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type);
+  if (rc) return rc;
+  auto fn = c8_supported(hq, hkv, head_dim, block_size, cache_quant_type) ? decode_c8_launch : decode_generic_launch;
+  return fn(q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables, seq_lens_decoder,
+            seq_lens_this_time, nullptr, nullptr, 0, out, workspace, workspace_bytes, batch, hq, hkv,
+            head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type, softmax_scale,
+            (hipStream_t)stream);
+}
+
+extern "C" int fdattn_decode_attention_generic(
+    const void* q, const void* key_cache, const void* value_cache, const float* cache_k_scale,
+    const float* cache_v_scale, const int32_t* block_tables, const int32_t* seq_lens_decoder,
+    const int32_t* seq_lens_this_time, const int32_t* kept_blocks, const int32_t* kept_counts, int max_kept,
+    void* out, void* workspace, size_t workspace_bytes, int batch,
+    int hq, int hkv, int head_dim, int block_size, int max_blocks_per_seq, int num_blocks,
+    int cache_quant_type, float softmax_scale, void* stream) {
+  int rc = check_decode_args("fdattn_decode_attention_generic", q, key_cache, value_cache, cache_k_scale,
+                             cache_v_scale, block_tables, seq_lens_decoder, out, workspace, batch, hq, hkv,
+                             head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type);
+  if (rc) return rc;
+  if ((kept_blocks == nullptr) != (kept_counts == nullptr))
+    return fail(FDATTN_ERR_NULL, "fdattn_decode_attention_generic: kept_blocks and kept_counts go together");
+  return decode_generic_launch(q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
+                               seq_lens_decoder, seq_lens_this_time, kept_blocks, kept_counts, max_kept, out,
+                               workspace, workspace_bytes, batch, hq, hkv, head_dim, block_size,
+                               max_blocks_per_seq, num_blocks, cache_quant_type, softmax_scale,
+                               (hipStream_t)stream);
+}
+
+extern "C" int fdattn_decode_attention_sparse(
+    const void* q, const void* key_cache, const void* value_cache, const float* cache_k_scale,
+    const float* cache_v_scale, const int32_t* block_tables, const int32_t* seq_lens_decoder,
+    const int32_t* seq_lens_this_time, const int32_t* kept_blocks, const int32_t* kept_counts, int max_kept,
+    void* out, void* workspace, size_t workspace_bytes, int batch, int hq, int hkv, int head_dim,
+    int block_size, int max_blocks_per_seq, int num_blocks, int cache_quant_type, float softmax_scale,
+    void* stream) {
+  int rc = check_decode_args("fdattn_decode_attention_sparse", q, key_cache, value_cache, cache_k_scale,
+                             cache_v_scale, block_tables, seq_lens_decoder, out, workspace, batch, hq, hkv,
+                             head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type);
+  if (rc) return rc;
+  if (!kept_blocks || !kept_counts || max_kept <= 0)
+    return fail(FDATTN_ERR_NULL, "fdattn_decode_attention_sparse: kept_blocks / kept_counts / max_kept missing");
+  auto fn = c8_supported(hq, hkv, head_dim, block_size, cache_quant_type) ? decode_c8_launch : decode_generic_launch;
+  return fn(q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables, seq_lens_decoder,
+            seq_lens_this_time, kept_blocks, kept_counts, max_kept, out, workspace, workspace_bytes, batch,
+            hq, hkv, head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type, softmax_scale,
+            (hipStream_t)stream);
+}

@@ -1,0 +1,326 @@
+"""Python op surface of the paged-KV attention path.
+
+Argument names follow FastDeploy's attention operator surface (qkv, key_cache,
+value_cache, cache_k_scale, cache_v_scale, block_tables, seq_lens_encoder,
+seq_lens_decoder, seq_lens_this_time).  Tensors cross into the library as
+(address, shape, dtype) triples, the same contract as the reference's
+FDTensor.from_external_data (fastdeploy/pybind/fd_tensor.cc:248-286); work is
+enqueued on torch's current stream and nothing synchronises, as the reference's
+custom operators do on their input's stream
+(fastdeploy/runtime/backends/paddle/ops/voxelize_op.cu:287-351).  Bad arguments
+raise ValueError where the reference's operators PD_THROW
+(fastdeploy/runtime/backends/paddle/ops/voxelize_op.cc:172).
+"""
+import math
+
+import torch
+
+from . import _lib
+
+CACHE_INT8 = 1
+CACHE_FP8 = 2
+_QUANT = {"cache_int8": CACHE_INT8, "int8": CACHE_INT8, CACHE_INT8: CACHE_INT8,
+          "cache_fp8": CACHE_FP8, "fp8": CACHE_FP8, "fp8_e4m3": CACHE_FP8, CACHE_FP8: CACHE_FP8}
+_ROPE = {"interleaved": 0, 0: 0, False: 0, "neox": 1, 1: 1, True: 1}
+
+
+def _quant(t):
+    if t not in _QUANT:
+        raise ValueError("unknown cache_quant_type %r (cache_int8 | cache_fp8)" % (t,))
+    return _QUANT[t]
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _chk(t, name, dtypes, ndim=None, optional=False):
+    if t is None:
+        if optional:
+            return 0
+        raise ValueError("%s is required" % name)
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise ValueError("%s must be a CUDA/HIP tensor" % name)
+    if not isinstance(dtypes, (tuple, list)):
+        dtypes = (dtypes,)
+    if t.dtype not in dtypes:
+        raise ValueError("%s has dtype %s, expected %s" % (name, t.dtype, "/".join(map(str, dtypes))))
+    if not t.is_contiguous():
+        raise ValueError("%s must be contiguous" % name)
+    if ndim is not None and t.dim() != ndim:
+        raise ValueError("%s must have %d dimensions, has shape %s" % (name, ndim, tuple(t.shape)))
+    return t.data_ptr()
+
+
+_CACHE_DT = (torch.int8, torch.uint8, torch.float8_e4m3fn)
+
+
+def _cache_dims(key_cache, value_cache):
+    if key_cache.shape != value_cache.shape:
+        raise ValueError("key_cache %s and value_cache %s differ in shape" %
+                         (tuple(key_cache.shape), tuple(value_cache.shape)))
+    return key_cache.shape  # num_blocks, hkv, block_size, head_dim
+
+
+def _scales(cache_k_scale, cache_v_scale, hkv, d):
+    pk = _chk(cache_k_scale, "cache_k_scale", torch.float32)
+    pv = _chk(cache_v_scale, "cache_v_scale", torch.float32)
+    if cache_k_scale.numel() != hkv * d or cache_v_scale.numel() != hkv * d:
+        raise ValueError("cache scales must hold kv_num_heads*head_dim = %d values" % (hkv * d))
+    return pk, pv
+
+
+def seq_lens_this_time_of(seq_lens_encoder, seq_lens_decoder):
+    """Tokens each sequence brings this step: its chunk length for a prefill row
+    (seq_lens_encoder > 0), one for a decode row (seq_lens_decoder > 0), else none."""
+    one = (seq_lens_decoder > 0).to(torch.int32)
+    return torch.where(seq_lens_encoder > 0, seq_lens_encoder, one).to(torch.int32)
+
+
+def cu_seqlens_of(seq_lens_this_time):
+    cu = torch.zeros(seq_lens_this_time.numel() + 1, dtype=torch.int32, device=seq_lens_this_time.device)
+    cu[1:] = torch.cumsum(seq_lens_this_time, 0)
+    return cu
+
+
+def write_cache_kv(qkv, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
+                   seq_lens_encoder, seq_lens_decoder, seq_lens_this_time=None, cu_seqlens_q=None,
+                   rotary_embs=None, *, num_heads, kv_num_heads, rope_style="neox",
+                   cache_quant_type="cache_int8", want_kv_out=False):
+    """RoPE on Q/K, quantise K/V into their block-tabled cache slots (in place).
+
+    rotary_embs = (cos, sin) float32 [max_pos, head_dim/2] from rope_table(), or None.
+    Returns (q_out, k_out, v_out); k_out / v_out are None unless want_kv_out.
+    """
+    nb, hkv, bs, d = _cache_dims(key_cache, value_cache)
+    if hkv != kv_num_heads:
+        raise ValueError("cache holds %d KV heads, kv_num_heads=%d" % (hkv, kv_num_heads))
+    p_qkv = _chk(qkv, "qkv", torch.bfloat16, 2)
+    T = qkv.shape[0]
+    if qkv.shape[1] != (num_heads + 2 * hkv) * d:
+        raise ValueError("qkv has %d columns, expected (num_heads+2*kv_num_heads)*head_dim = %d" %
+                         (qkv.shape[1], (num_heads + 2 * hkv) * d))
+    p_kc = _chk(key_cache, "key_cache", _CACHE_DT, 4)
+    p_vc = _chk(value_cache, "value_cache", _CACHE_DT, 4)
+    p_ks, p_vs = _scales(cache_k_scale, cache_v_scale, hkv, d)
+    p_bt = _chk(block_tables, "block_tables", torch.int32, 2)
+    batch, mb = block_tables.shape
+    p_dec = _chk(seq_lens_decoder, "seq_lens_decoder", torch.int32, 1)
+    if seq_lens_decoder.numel() != batch:
+        raise ValueError("seq_lens_decoder has %d entries, block_tables %d rows" % (seq_lens_decoder.numel(), batch))
+    if cu_seqlens_q is None:
+        if seq_lens_this_time is None:
+            _chk(seq_lens_encoder, "seq_lens_encoder", torch.int32, 1)
+            seq_lens_this_time = seq_lens_this_time_of(seq_lens_encoder, seq_lens_decoder)
+        _chk(seq_lens_this_time, "seq_lens_this_time", torch.int32, 1)
+        cu_seqlens_q = cu_seqlens_of(seq_lens_this_time)
+    p_cu = _chk(cu_seqlens_q, "cu_seqlens_q", torch.int32, 1)
+    if cu_seqlens_q.numel() != batch + 1:
+        raise ValueError("cu_seqlens_q must have batch+1 entries")
+    p_cos = p_sin = 0
+    max_pos = 0
+    if rotary_embs is not None:
+        cos, sin = rotary_embs
+        p_cos = _chk(cos, "rotary cos", torch.float32, 2)
+        p_sin = _chk(sin, "rotary sin", torch.float32, 2)
+        if cos.shape != sin.shape or cos.shape[1] != d // 2:
+            raise ValueError("rotary table must be [max_pos, head_dim/2]")
+        max_pos = cos.shape[0]
+    if rope_style not in _ROPE:
+        raise ValueError("unknown rope_style %r (neox | interleaved)" % (rope_style,))
+    q_out = torch.empty((T, num_heads * d), dtype=torch.bfloat16, device=qkv.device)
+    k_out = v_out = None
+    if want_kv_out:
+        k_out = torch.empty((T, hkv * d), dtype=torch.bfloat16, device=qkv.device)
+        v_out = torch.empty((T, hkv * d), dtype=torch.bfloat16, device=qkv.device)
+    rc = _lib.lib().fdattn_write_cache_kv(
+        p_qkv, q_out.data_ptr(), k_out.data_ptr() if want_kv_out else 0,
+        v_out.data_ptr() if want_kv_out else 0, p_kc, p_vc, p_ks, p_vs, p_cos, p_sin, p_bt, p_dec,
+        p_cu, T, batch, num_heads, hkv, d, bs, mb, nb, max_pos, _ROPE[rope_style],
+        _quant(cache_quant_type), _stream())
+    _lib.check(rc, "write_cache_kv")
+    return q_out, k_out, v_out
+
+
+def decode_workspace(batch, num_heads, kv_num_heads, head_dim, device="cuda"):
+    """A workspace tensor large enough for decode_attention(_sparse) at these shapes."""
+    n = _lib.lib().fdattn_decode_workspace_bytes(batch, num_heads, kv_num_heads, head_dim)
+    return torch.empty(n, dtype=torch.uint8, device=device)
+
+
+def _decode_common(q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
+                   seq_lens_decoder, seq_lens_this_time, num_heads, out, workspace):
+    nb, hkv, bs, d = _cache_dims(key_cache, value_cache)
+    p_q = _chk(q, "q", torch.bfloat16)
+    batch, mb = block_tables.shape
+    if q.numel() != batch * num_heads * d:
+        raise ValueError("q holds %d values, expected batch*num_heads*head_dim = %d" %
+                         (q.numel(), batch * num_heads * d))
+    p_kc = _chk(key_cache, "key_cache", _CACHE_DT, 4)
+    p_vc = _chk(value_cache, "value_cache", _CACHE_DT, 4)
+    p_ks, p_vs = _scales(cache_k_scale, cache_v_scale, hkv, d)
+    p_bt = _chk(block_tables, "block_tables", torch.int32, 2)
+    p_dec = _chk(seq_lens_decoder, "seq_lens_decoder", torch.int32, 1)
+    p_tt = _chk(seq_lens_this_time, "seq_lens_this_time", torch.int32, 1, optional=True)
+    if seq_lens_decoder.numel() != batch:
+        raise ValueError("seq_lens_decoder has %d entries, block_tables %d rows" % (seq_lens_decoder.numel(), batch))
+    if out is None:
+        out = torch.empty((batch, num_heads * d), dtype=torch.bfloat16, device=q.device)
+    p_out = _chk(out, "out", torch.bfloat16)
+    if workspace is None:
+        workspace = decode_workspace(batch, num_heads, hkv, d, q.device)
+    p_ws = _chk(workspace, "workspace", torch.uint8)
+    return (p_q, p_kc, p_vc, p_ks, p_vs, p_bt, p_dec, p_tt), out, p_out, p_ws, workspace, \
+        (batch, num_heads, hkv, d, bs, mb, nb)
+
+
+def decode_attention(q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
+                     seq_lens_decoder, seq_lens_this_time=None, *, num_heads,
+                     cache_quant_type="cache_int8", softmax_scale=None, out=None, workspace=None,
+                     impl="auto"):
+    """One query token per sequence against kv_len = seq_lens_decoder (+ seq_lens_this_time)
+    cached tokens.  q bf16 [batch, num_heads*head_dim] -> out bf16 of the same shape.
+    impl: "auto" (MFMA kernel when the shape allows) or "generic"."""
+    ptrs, out, p_out, p_ws, workspace, dims = _decode_common(
+        q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables, seq_lens_decoder,
+        seq_lens_this_time, num_heads, out, workspace)
+    scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(dims[3])
+    if impl == "generic":
+        rc = _lib.lib().fdattn_decode_attention_generic(
+            *ptrs, 0, 0, 0, p_out, p_ws, workspace.numel(), *dims, _quant(cache_quant_type), scale, _stream())
+    elif impl == "auto":
+        rc = _lib.lib().fdattn_decode_attention(
+            *ptrs, p_out, p_ws, workspace.numel(), *dims, _quant(cache_quant_type), scale, _stream())
+    else:
+        raise ValueError("impl must be auto or generic")
+    _lib.check(rc, "decode_attention")
+    return out
+
+
+def decode_attention_sparse(q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
+                            seq_lens_decoder, seq_lens_this_time=None, *, kept_blocks, kept_counts,
+                            num_heads, cache_quant_type="cache_int8", softmax_scale=None, out=None,
+                            workspace=None, impl="auto"):
+    """decode_attention restricted to kept_blocks int32 [batch, kv_num_heads, max_kept]
+    (ascending logical block indices) / kept_counts int32 [batch, kv_num_heads]."""
+    ptrs, out, p_out, p_ws, workspace, dims = _decode_common(
+        q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables, seq_lens_decoder,
+        seq_lens_this_time, num_heads, out, workspace)
+    batch, _, hkv = dims[0], dims[1], dims[2]
+    p_kb = _chk(kept_blocks, "kept_blocks", torch.int32, 3)
+    p_kn = _chk(kept_counts, "kept_counts", torch.int32, 2)
+    if kept_blocks.shape[:2] != (batch, hkv) or kept_counts.shape != (batch, hkv):
+        raise ValueError("kept_blocks must be [batch, kv_num_heads, max_kept], kept_counts [batch, kv_num_heads]")
+    scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(dims[3])
+    fn = _lib.lib().fdattn_decode_attention_sparse if impl == "auto" else _lib.lib().fdattn_decode_attention_generic
+    rc = fn(*ptrs, p_kb, p_kn, kept_blocks.shape[2], p_out, p_ws, workspace.numel(), *dims,
+            _quant(cache_quant_type), scale, _stream())
+    _lib.check(rc, "decode_attention_sparse")
+    return out
+
+
+def splitkv_combine(part_o, part_m, part_l, num_splits=None, out=None):
+    """Merge split-KV partials: part_o f32 [rows, splits, d], part_m / part_l f32 [rows, splits]."""
+    p_o = _chk(part_o, "part_o", torch.float32, 3)
+    p_m = _chk(part_m, "part_m", torch.float32, 2)
+    p_l = _chk(part_l, "part_l", torch.float32, 2)
+    rows, ms, d = part_o.shape
+    if part_m.shape != (rows, ms) or part_l.shape != (rows, ms):
+        raise ValueError("part_m / part_l must be [rows, splits]")
+    p_n = _chk(num_splits, "num_splits", torch.int32, 1, optional=True)
+    if out is None:
+        out = torch.empty((rows, d), dtype=torch.bfloat16, device=part_o.device)
+    rc = _lib.lib().fdattn_splitkv_combine(p_o, p_m, p_l, p_n, _chk(out, "out", torch.bfloat16), rows, ms, d, _stream())
+    _lib.check(rc, "splitkv_combine")
+    return out
+
+
+def sqattn_select(q, key_cache, cache_k_scale, block_tables, seq_lens_decoder, seq_lens_this_time=None, *,
+                  num_heads, top_k, cache_quant_type="cache_fp8", return_scores=False, workspace=None):
+    """SQAttn block selection: per (sequence, KV head) the top_k blocks by block-max q.k score.
+    Returns (kept_blocks int32 [batch, hkv, top_k], kept_counts int32 [batch, hkv][, scores f32])."""
+    nb, hkv, bs, d = key_cache.shape
+    p_q = _chk(q, "q", torch.bfloat16)
+    p_kc = _chk(key_cache, "key_cache", _CACHE_DT, 4)
+    p_ks = _chk(cache_k_scale, "cache_k_scale", torch.float32)
+    p_bt = _chk(block_tables, "block_tables", torch.int32, 2)
+    batch, mb = block_tables.shape
+    p_dec = _chk(seq_lens_decoder, "seq_lens_decoder", torch.int32, 1)
+    p_tt = _chk(seq_lens_this_time, "seq_lens_this_time", torch.int32, 1, optional=True)
+    if q.numel() != batch * num_heads * d:
+        raise ValueError("q holds %d values, expected %d" % (q.numel(), batch * num_heads * d))
+    if top_k <= 0:
+        raise ValueError("top_k must be positive")
+    kept = torch.empty((batch, hkv, top_k), dtype=torch.int32, device=q.device)
+    counts = torch.empty((batch, hkv), dtype=torch.int32, device=q.device)
+    scores = torch.empty((batch, hkv, mb), dtype=torch.float32, device=q.device) if return_scores else None
+    if workspace is None:
+        n = _lib.lib().fdattn_sqattn_workspace_bytes(batch, hkv, mb)
+        workspace = torch.empty(n, dtype=torch.uint8, device=q.device)
+    rc = _lib.lib().fdattn_sqattn_select(
+        p_q, p_kc, p_ks, p_bt, p_dec, p_tt, scores.data_ptr() if return_scores else 0, kept.data_ptr(),
+        counts.data_ptr(), _chk(workspace, "workspace", torch.uint8), workspace.numel(), batch, num_heads,
+        hkv, d, bs, mb, nb, top_k, _quant(cache_quant_type), _stream())
+    _lib.check(rc, "sqattn_select")
+    return (kept, counts, scores) if return_scores else (kept, counts)
+
+
+def append_attention_prefill(q, k_new, v_new, key_cache, value_cache, cache_k_scale, cache_v_scale,
+                             block_tables, seq_lens_decoder, cu_seqlens_q, *, num_heads, max_chunk,
+                             cache_quant_type="cache_int8", softmax_scale=None, out=None, impl="auto"):
+    """Chunked prefill: the chunk's tokens attend to the cached prefix (quantised pages)
+    and causally to the chunk itself (bf16 k_new / v_new)."""
+    nb, hkv, bs, d = _cache_dims(key_cache, value_cache)
+    p_q = _chk(q, "q", torch.bfloat16, 2)
+    p_k = _chk(k_new, "k_new", torch.bfloat16, 2)
+    p_v = _chk(v_new, "v_new", torch.bfloat16, 2)
+    T = q.shape[0]
+    if q.shape[1] != num_heads * d or k_new.shape != (T, hkv * d) or v_new.shape != (T, hkv * d):
+        raise ValueError("q must be [T, num_heads*head_dim], k_new / v_new [T, kv_num_heads*head_dim]")
+    p_kc = _chk(key_cache, "key_cache", _CACHE_DT, 4)
+    p_vc = _chk(value_cache, "value_cache", _CACHE_DT, 4)
+    p_ks, p_vs = _scales(cache_k_scale, cache_v_scale, hkv, d)
+    p_bt = _chk(block_tables, "block_tables", torch.int32, 2)
+    batch, mb = block_tables.shape
+    p_dec = _chk(seq_lens_decoder, "seq_lens_decoder", torch.int32, 1)
+    p_cu = _chk(cu_seqlens_q, "cu_seqlens_q", torch.int32, 1)
+    if cu_seqlens_q.numel() != batch + 1:
+        raise ValueError("cu_seqlens_q must have batch+1 entries")
+    if out is None:
+        out = torch.empty((T, num_heads * d), dtype=torch.bfloat16, device=q.device)
+    scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(d)
+    fn = _lib.lib().fdattn_append_attention_prefill if impl == "auto" else \
+        _lib.lib().fdattn_append_attention_prefill_generic
+    rc = fn(
+        p_q, p_k, p_v, p_kc, p_vc, p_ks, p_vs, p_bt, p_dec, p_cu, _chk(out, "out", torch.bfloat16), T, batch,
+        max_chunk, num_heads, hkv, d, bs, mb, nb, _quant(cache_quant_type), scale, _stream())
+    _lib.check(rc, "append_attention_prefill")
+    return out
+
+
+def append_attention(qkv, key_cache, value_cache, seq_lens_encoder, seq_lens_decoder, seq_lens_this_time,
+                     block_tables, rotary_embs, cache_k_scale, cache_v_scale, *, num_heads, kv_num_heads,
+                     max_chunk, rope_style="neox", cache_quant_type="cache_int8", softmax_scale=None,
+                     workspace=None):
+    """One attention step of a batch that is either all decode rows (one new token
+    each, seq_lens_encoder == 0) or all prefill rows (max_chunk > 1): cache write,
+    then decode attention over the cache, or append attention over prefix + chunk.
+    Returns bf16 [num_tokens, num_heads*head_dim]."""
+    cu = cu_seqlens_of(seq_lens_this_time)
+    prefill = max_chunk > 1
+    q, k_new, v_new = write_cache_kv(
+        qkv, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables, seq_lens_encoder,
+        seq_lens_decoder, seq_lens_this_time, cu, rotary_embs, num_heads=num_heads,
+        kv_num_heads=kv_num_heads, rope_style=rope_style, cache_quant_type=cache_quant_type,
+        want_kv_out=prefill)
+    if prefill:
+        return append_attention_prefill(
+            q, k_new, v_new, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
+            seq_lens_decoder, cu, num_heads=num_heads, max_chunk=max_chunk,
+            cache_quant_type=cache_quant_type, softmax_scale=softmax_scale)
+    if qkv.shape[0] != block_tables.shape[0]:
+        raise ValueError("a decode step needs exactly one token per sequence")
+    return decode_attention(
+        q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables, seq_lens_decoder,
+        seq_lens_this_time, num_heads=num_heads, cache_quant_type=cache_quant_type,
+        softmax_scale=softmax_scale, workspace=workspace)

@@ -1,0 +1,240 @@
+/*
+ * fdattn.h - C ABI of libfdattn.so, the MI355X (gfx950) paged-KV attention path.
+ *
+ * Every entry point takes raw device pointers, explicit integer shapes and an
+ * opaque stream handle (a hipStream_t passed as void*; NULL = the null stream).
+ * Nothing here allocates, frees or synchronises: all buffers, the KV caches and
+ * the workspace included, are owned by the caller ("__fd_keep" in the
+ * reference's C API vocabulary, c_api/fastdeploy_capi/core/fd_common.h:30-56),
+ * and work is only enqueued on the given stream, like the reference's custom
+ * operators enqueue on their input's stream and return without a sync
+ * (fastdeploy/runtime/backends/paddle/ops/voxelize_op.cu:287-351).
+ *
+ * The reference registers the operators it plugs into the engine through
+ * PD_BUILD_OP(name).Inputs(...).Outputs(...).Attrs(...)
+ * (fastdeploy/runtime/backends/paddle/ops/voxelize_op.cc:196-204) with kernel
+ * functions of the form std::vector<paddle::Tensor> fn(const paddle::Tensor&...,
+ * attrs...) (voxelize_op.cc:159-162).  Each function below is the body such a
+ * kernel function would forward to: tensor inputs become pointers, attributes
+ * become ints / floats.
+ *
+ * Errors: the reference's operators throw (PD_THROW, voxelize_op.cc:172) or
+ * abort (FDASSERT, fastdeploy/utils/utils.h:104-111); its C API returns
+ * FD_C_Bool (c_api/fastdeploy_capi/core/fd_common.h:58).  Nothing may unwind
+ * through a C ABI, so every function returns an int:
+ *    0  success (work enqueued)
+ *   <0  argument error (FDATTN_ERR_*), nothing was enqueued
+ *   >0  a hipError_t reported by the launch
+ * and fdattn_last_error() returns the message for the calling thread.
+ *
+ * Data layouts (all row-major, innermost dimension last):
+ *   qkv           bf16  [num_tokens, (hq + 2*hkv) * head_dim]   Q heads, K heads, V heads
+ *   key_cache     u8    [num_blocks, hkv, block_size, head_dim] int8 (two's complement) or fp8 e4m3fn
+ *   value_cache   u8    same
+ *   cache_k_scale f32   [hkv, head_dim]  dequantisation multiplier (max-abs/127 or max-abs/448)
+ *   cache_v_scale f32   [hkv, head_dim]
+ *   block_tables  i32   [batch, max_blocks_per_seq]  physical block per logical block, -1 = none
+ *   seq_lens_*    i32   [batch]
+ *   rope_cos/sin  f32   [max_pos, head_dim/2]  host-built table shared with the CPU oracle
+ */
+#ifndef FDATTN_H_
+#define FDATTN_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FDATTN_API __attribute__((visibility("default")))
+
+/* cache_quant_type */
+#define FDATTN_CACHE_INT8 1     /* q = clamp(rne(x / scale), -127, 127), stored as int8 */
+#define FDATTN_CACHE_FP8_E4M3 2 /* q = e4m3fn(clamp(x / scale, -448, 448)), RNE        */
+
+/* rope_style */
+#define FDATTN_ROPE_INTERLEAVED 0 /* pairs (2j, 2j+1)          */
+#define FDATTN_ROPE_NEOX 1        /* pairs (j, j + head_dim/2) */
+
+/* argument errors */
+#define FDATTN_ERR_NULL -1        /* a required pointer is NULL              */
+#define FDATTN_ERR_SHAPE -2       /* a shape the kernels do not support      */
+#define FDATTN_ERR_QUANT -3       /* unknown cache_quant_type / rope_style   */
+#define FDATTN_ERR_WORKSPACE -4   /* workspace too small                     */
+
+/* Library identification, "fdattn <major>.<minor> gfx950". */
+FDATTN_API const char* fdattn_version(void);
+
+/* Message of the last failing call made by this thread ("" if none). */
+FDATTN_API const char* fdattn_last_error(void);
+
+/*
+ * Cache writer: rotary embedding on Q and K, quantisation of K and V into their
+ * block-tabled cache slots.  Stands where an engine-side custom operator body
+ * would (plug-in pattern: fastdeploy/runtime/backends/paddle/ops/voxelize_op.cc:159-176);
+ * saturation follows function::Clip (fastdeploy/function/clip.cc:20-30).
+ *
+ * Token i belongs to the sequence b with cu_seqlens_q[b] <= i < cu_seqlens_q[b+1]
+ * and sits at position pos = seq_lens_decoder[b] + (i - cu_seqlens_q[b]).
+ *   q_out  bf16 [num_tokens, hq*head_dim]   rotated Q (required)
+ *   k_out  bf16 [num_tokens, hkv*head_dim]  rotated K, rounded to bf16 (optional, may be NULL)
+ *   v_out  bf16 [num_tokens, hkv*head_dim]  V copied through (optional, may be NULL)
+ * rope_cos / rope_sin may both be NULL: no rotation is applied then.
+ * A token whose block-table entry is negative is skipped (no cache store).
+ */
+FDATTN_API int fdattn_write_cache_kv(
+    const void* qkv, void* q_out, void* k_out, void* v_out,
+    void* key_cache, void* value_cache,
+    const float* cache_k_scale, const float* cache_v_scale,
+    const float* rope_cos, const float* rope_sin,
+    const int32_t* block_tables, const int32_t* seq_lens_decoder,
+    const int32_t* cu_seqlens_q,
+    int num_tokens, int batch, int hq, int hkv, int head_dim, int block_size,
+    int max_blocks_per_seq, int num_blocks, int max_pos,
+    int rope_style, int cache_quant_type, void* stream);
+
+/*
+ * Bytes of workspace fdattn_decode_attention / fdattn_decode_attention_sparse
+ * need for these shapes (split-KV partial results).  Never 0.
+ */
+FDATTN_API size_t fdattn_decode_workspace_bytes(int batch, int hq, int hkv, int head_dim);
+
+/*
+ * Decode attention over the quantised paged cache: one query token per sequence,
+ *   out[b, qh, :] = softmax_t(softmax_scale * q[b, qh] . K^[b, t]) . V^[b, t],
+ *   t in [0, kv_len[b]),  kv_len[b] = seq_lens_decoder[b] + (seq_lens_this_time ? seq_lens_this_time[b] : 0),
+ * with K^/V^ the dequantised cache rows of KV head qh / (hq/hkv), gathered through
+ * block_tables.  Rows with kv_len 0 produce zeros.  Softmax follows the
+ * max-shifted form of fastdeploy/function/softmax.cc:58-86 (without its -64 clip).
+ *   q   bf16 [batch, hq*head_dim]     out bf16 [batch, hq*head_dim]
+ * The split-KV partials live in `workspace` and are merged by the library
+ * before the call's work on the stream ends.
+ */
+FDATTN_API int fdattn_decode_attention(
+    const void* q, const void* key_cache, const void* value_cache,
+    const float* cache_k_scale, const float* cache_v_scale,
+    const int32_t* block_tables, const int32_t* seq_lens_decoder,
+    const int32_t* seq_lens_this_time, void* out,
+    void* workspace, size_t workspace_bytes,
+    int batch, int hq, int hkv, int head_dim, int block_size,
+    int max_blocks_per_seq, int num_blocks, int cache_quant_type,
+    float softmax_scale, void* stream);
+
+/*
+ * Same, restricted to a per-(sequence, KV head) list of logical blocks:
+ *   kept_blocks i32 [batch, hkv, max_kept]  logical block indices, ascending, -1 padded
+ *   kept_counts i32 [batch, hkv]
+ * A kept block j covers tokens [j*block_size, min((j+1)*block_size, kv_len)).
+ */
+FDATTN_API int fdattn_decode_attention_sparse(
+    const void* q, const void* key_cache, const void* value_cache,
+    const float* cache_k_scale, const float* cache_v_scale,
+    const int32_t* block_tables, const int32_t* seq_lens_decoder,
+    const int32_t* seq_lens_this_time,
+    const int32_t* kept_blocks, const int32_t* kept_counts, int max_kept,
+    void* out, void* workspace, size_t workspace_bytes,
+    int batch, int hq, int hkv, int head_dim, int block_size,
+    int max_blocks_per_seq, int num_blocks, int cache_quant_type,
+    float softmax_scale, void* stream);
+
+/*
+ * The shape-agnostic decode kernel behind both functions above (any head_dim <= 256
+ * that is a multiple of 4, any hq/hkv, any block_size), callable directly; it is what
+ * they fall back to for shapes the MFMA kernel does not cover (it covers head_dim
+ * 128, hq/hkv 4, block_size 64).  kept_blocks / kept_counts may both be NULL (dense).
+ * Same plug-in position as fdattn_decode_attention.
+ */
+FDATTN_API int fdattn_decode_attention_generic(
+    const void* q, const void* key_cache, const void* value_cache,
+    const float* cache_k_scale, const float* cache_v_scale,
+    const int32_t* block_tables, const int32_t* seq_lens_decoder,
+    const int32_t* seq_lens_this_time,
+    const int32_t* kept_blocks, const int32_t* kept_counts, int max_kept,
+    void* out, void* workspace, size_t workspace_bytes,
+    int batch, int hq, int hkv, int head_dim, int block_size,
+    int max_blocks_per_seq, int num_blocks, int cache_quant_type,
+    float softmax_scale, void* stream);
+
+/*
+ * Split-KV merge of partial attention results (log-sum-exp combine):
+ *   m = max_s m_s,  l = sum_s l_s e^(m_s - m),  out = sum_s o_s e^(m_s - m) / l
+ *   part_o f32 [rows, max_splits, head_dim]  unnormalised partial outputs
+ *   part_m f32 [rows, max_splits]            partial maxima (natural-log domain)
+ *   part_l f32 [rows, max_splits]            partial sums of exponentials
+ *   num_splits i32 [rows] or NULL (= max_splits everywhere)
+ *   out bf16 [rows, head_dim]
+ * Max-shift as in fastdeploy/function/softmax.cc:58-66.
+ */
+FDATTN_API int fdattn_splitkv_combine(
+    const float* part_o, const float* part_m, const float* part_l,
+    const int32_t* num_splits, void* out,
+    int rows, int max_splits, int head_dim, void* stream);
+
+/*
+ * Bytes of workspace fdattn_sqattn_select needs.
+ */
+FDATTN_API size_t fdattn_sqattn_workspace_bytes(int batch, int hkv, int max_blocks_per_seq);
+
+/*
+ * SQAttn block selector.  For every (sequence b, KV head h, logical block j):
+ *   score[b,h,j] = max over the block's valid tokens t and the hq/hkv query heads g of head h
+ *                  of  sum_c (q[b,g,c] * cache_k_scale[h,c]) * K8[t,c]
+ * (reduction as function::Max, fastdeploy/function/reduce.cc:354-357), then the
+ * top_k highest-scoring blocks per (b,h) are kept; equal scores resolve to the
+ * lower block index as in TopKIndices (fastdeploy/vision/utils/utils.h:41-60).
+ *   scores      f32 [batch, hkv, max_blocks_per_seq]  (optional output, may be NULL; -inf for absent blocks)
+ *   kept_blocks i32 [batch, hkv, top_k]  ascending logical block indices, -1 padded
+ *   kept_counts i32 [batch, hkv]         min(top_k, ceil(kv_len / block_size))
+ */
+FDATTN_API int fdattn_sqattn_select(
+    const void* q, const void* key_cache, const float* cache_k_scale,
+    const int32_t* block_tables, const int32_t* seq_lens_decoder,
+    const int32_t* seq_lens_this_time,
+    float* scores, int32_t* kept_blocks, int32_t* kept_counts,
+    void* workspace, size_t workspace_bytes,
+    int batch, int hq, int hkv, int head_dim, int block_size,
+    int max_blocks_per_seq, int num_blocks, int top_k,
+    int cache_quant_type, void* stream);
+
+/*
+ * Chunked-prefill ("append") attention.  Sequence b appends n_b =
+ * cu_seqlens_q[b+1] - cu_seqlens_q[b] new tokens to p_b = seq_lens_decoder[b]
+ * cached ones.  New token i (0-based in the chunk) attends to the p_b cached
+ * tokens (quantised pages, dequantised in-tile) and to the chunk tokens j <= i
+ * (bf16 K/V of this call).
+ *   q     bf16 [num_tokens, hq*head_dim]    rotated Q   (q_out of the cache writer)
+ *   k_new bf16 [num_tokens, hkv*head_dim]   rotated K   (k_out of the cache writer)
+ *   v_new bf16 [num_tokens, hkv*head_dim]   V           (v_out of the cache writer)
+ *   out   bf16 [num_tokens, hq*head_dim]
+ * max_chunk bounds n_b (it sizes the launch grid).
+ */
+FDATTN_API int fdattn_append_attention_prefill(
+    const void* q, const void* k_new, const void* v_new,
+    const void* key_cache, const void* value_cache,
+    const float* cache_k_scale, const float* cache_v_scale,
+    const int32_t* block_tables, const int32_t* seq_lens_decoder,
+    const int32_t* cu_seqlens_q, void* out,
+    int num_tokens, int batch, int max_chunk, int hq, int hkv, int head_dim,
+    int block_size, int max_blocks_per_seq, int num_blocks,
+    int cache_quant_type, float softmax_scale, void* stream);
+
+/*
+ * The shape-agnostic kernel fdattn_append_attention_prefill falls back to when the
+ * MFMA kernel does not cover the shape (it covers head_dim 128, hq/hkv 4,
+ * block_size 64), callable directly.  Same arguments and plug-in position.
+ */
+FDATTN_API int fdattn_append_attention_prefill_generic(
+    const void* q, const void* k_new, const void* v_new,
+    const void* key_cache, const void* value_cache,
+    const float* cache_k_scale, const float* cache_v_scale,
+    const int32_t* block_tables, const int32_t* seq_lens_decoder,
+    const int32_t* cu_seqlens_q, void* out,
+    int num_tokens, int batch, int max_chunk, int hq, int hkv, int head_dim,
+    int block_size, int max_blocks_per_seq, int num_blocks,
+    int cache_quant_type, float softmax_scale, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FDATTN_H_ */
