@@ -1,0 +1,134 @@
+"""Decode attention on the GPU against the CPU oracle (bf16 outputs within 2e-3 abs OR 1e-2 rel)."""
+import numpy as np
+import pytest
+import torch
+
+import fastdeploy_amd as fd
+from conftest import bf16_close, bits, np_of
+from fastdeploy_amd import synthetic as syn
+from fastdeploy_amd.ops import CACHE_FP8, CACHE_INT8
+
+pytestmark = pytest.mark.gpu
+
+ATOL, RTOL = 2e-3, 1e-2     # the path's stated tolerance for bf16 attention outputs
+
+
+def oracle_decode(oracle, case, **kw):
+    return oracle.decode_attention(bits(case["q"]), np_of(case["key_cache"]), np_of(case["value_cache"]),
+                                   np_of(case["cache_k_scale"]), np_of(case["cache_v_scale"]),
+                                   np_of(case["block_tables"]), np_of(case["seq_lens_decoder"]), case["hq"],
+                                   case["hkv"], case["d"], case["quant"], **kw)
+
+
+def gpu_decode(case, impl="auto", **kw):
+    dev = syn.to_device(case, "cuda")
+    out = fd.decode_attention(dev["q"], dev["key_cache"], dev["value_cache"], dev["cache_k_scale"], dev["cache_v_scale"],
+                              dev["block_tables"], dev["seq_lens_decoder"], num_heads=case["hq"],
+                              cache_quant_type=case["quant"], impl=impl, **kw)
+    torch.cuda.synchronize()
+    return bits(out)
+
+
+def check(got, want, what=""):
+    ok, mx, bad = bf16_close(got, want, ATOL, RTOL)
+    assert ok, "%s: %d elements out of tolerance, max abs diff %.4g" % (what, bad, mx)
+
+
+@pytest.mark.parametrize("impl", ["generic", "auto"])
+@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+def test_decode_config1(oracle, impl, quant):
+    """batch 4, 32/8 heads, head_dim 128, ctx 1024, 64 physical blocks in a random permutation."""
+    for seed in range(3):
+        case = syn.decode_case(batch=4, ctx=1024, pool_blocks=64, quant=quant, seed=seed)
+        check(gpu_decode(case, impl), oracle_decode(oracle, case), "cfg1 seed %d" % seed)
+
+
+@pytest.mark.parametrize("impl", ["generic", "auto"])
+@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+def test_decode_ragged_and_edge_lengths(oracle, impl, quant):
+    lens = [1, 2, 63, 64, 65, 127, 128, 129, 700, 0, 1000, 31]
+    case = syn.decode_case(batch=len(lens), ctx=lens, quant=quant, seed=5, extra_blocks=7, max_blocks=20)
+    got, want = gpu_decode(case, impl), oracle_decode(oracle, case)
+    check(got, want, "ragged")
+    assert not got.reshape(len(lens), -1)[9].any()          # kv_len 0 -> zeros
+
+
+@pytest.mark.parametrize("impl", ["generic", "auto"])
+def test_decode_peaked_and_flat_softmax(oracle, impl):
+    """A query aligned with one key (one dominant weight) and constant keys (uniform weights)."""
+    case = syn.decode_case(batch=2, ctx=900, seed=6)
+    q = case["q"].view(2, 32, 128)
+    blk = int(case["block_tables"][0, 3])
+    krow = case["key_cache"][blk, :, 17, :].view(torch.int8).float() * case["cache_k_scale"]
+    q[0] = (krow * 2.0).repeat_interleave(4, 0).to(torch.bfloat16)
+    case["key_cache"][case["block_tables"][1, :15].long()] = 5
+    check(gpu_decode(case, impl), oracle_decode(oracle, case), "peaked/flat")
+
+
+@pytest.mark.parametrize("impl", ["generic", "auto"])
+def test_decode_this_time_adds_to_kv_len(oracle, impl):
+    case = syn.decode_case(batch=3, ctx=[100, 64, 257], seed=7)
+    dev = syn.to_device(case, "cuda")
+    dec = dev["seq_lens_decoder"] - 1
+    one = torch.ones_like(dec)
+    out = fd.decode_attention(dev["q"], dev["key_cache"], dev["value_cache"], dev["cache_k_scale"], dev["cache_v_scale"],
+                              dev["block_tables"], dec, one, num_heads=32, impl=impl)
+    check(bits(out), oracle_decode(oracle, case), "this_time")
+
+
+def test_decode_generic_other_shapes(oracle):
+    """Shapes outside the MFMA kernel: head_dim 64, group 2, block_size 16."""
+    case = syn.decode_case(batch=3, ctx=[50, 200, 333], seed=8, hq=8, hkv=4, d=64, bs=16)
+    got = gpu_decode(case)
+    want = oracle.decode_attention(bits(case["q"]), np_of(case["key_cache"]), np_of(case["value_cache"]),
+                                   np_of(case["cache_k_scale"]), np_of(case["cache_v_scale"]),
+                                   np_of(case["block_tables"]), np_of(case["seq_lens_decoder"]), 8, 4, 64, CACHE_INT8)
+    check(got, want, "d64 g2 bs16")
+
+
+@pytest.mark.parametrize("impl", ["generic", "auto"])
+@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+def test_sparse_decode(oracle, impl, quant):
+    case = syn.decode_case(batch=3, ctx=[2000, 1500, 64 * 40 + 5], quant=quant, seed=9)
+    rng = np.random.default_rng(1)
+    kept = np.full((3, 8, 12), -1, np.int32)
+    cnt = np.zeros((3, 8), np.int32)
+    for b in range(3):
+        nb = (int(case["seq_lens_decoder"][b]) + 63) // 64
+        for h in range(8):
+            k = int(rng.integers(1, 13))
+            kept[b, h, :k] = np.sort(rng.choice(nb, k, replace=False))
+            cnt[b, h] = k
+    kept[2, 0, :3] = [0, 39, 40]      # includes the partial last block
+    kept[2, 0, 3:] = -1
+    cnt[2, 0] = 3
+    dev = syn.to_device(case, "cuda")
+    out = fd.decode_attention_sparse(dev["q"], dev["key_cache"], dev["value_cache"], dev["cache_k_scale"],
+                                     dev["cache_v_scale"], dev["block_tables"], dev["seq_lens_decoder"],
+                                     kept_blocks=torch.from_numpy(kept).cuda(), kept_counts=torch.from_numpy(cnt).cuda(),
+                                     num_heads=32, cache_quant_type=quant, impl=impl)
+    check(bits(out), oracle_decode(oracle, case, kept_blocks=kept, kept_counts=cnt), "sparse")
+
+
+def test_splitkv_combine_entry_point(oracle):
+    g = torch.Generator().manual_seed(0)
+    po = torch.randn((37, 9, 128), generator=g)
+    pm = torch.randn((37, 9), generator=g) * 4
+    pl = torch.rand((37, 9), generator=g) * 50 + 1
+    pm[3, 4:] = -float("inf")
+    ns = torch.randint(1, 10, (37,), generator=g, dtype=torch.int32)
+    for n in (None, ns):
+        out = fd.splitkv_combine(po.cuda(), pm.cuda(), pl.cuda(), None if n is None else n.cuda())
+        want = oracle.splitkv_combine(po.numpy(), pm.numpy(), pl.numpy(), None if n is None else n.numpy())
+        check(bits(out), want, "combine")
+
+
+def test_decode_rejects_bad_arguments():
+    case = syn.to_device(syn.decode_case(batch=2, ctx=64), "cuda")
+    with pytest.raises(ValueError):
+        fd.decode_attention(case["q"][:, :-1].contiguous(), case["key_cache"], case["value_cache"], case["cache_k_scale"],
+                            case["cache_v_scale"], case["block_tables"], case["seq_lens_decoder"], num_heads=32)
+    with pytest.raises(ValueError):
+        fd.decode_attention(case["q"], case["key_cache"], case["value_cache"], case["cache_k_scale"],
+                            case["cache_v_scale"], case["block_tables"], case["seq_lens_decoder"], num_heads=32,
+                            workspace=torch.empty(16, dtype=torch.uint8, device="cuda"))

@@ -1,0 +1,76 @@
+"""SQAttn selector (bit-exact indices) and append/prefill attention on the GPU against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+import fastdeploy_amd as fd
+from conftest import bf16_close, bits, np_of
+from fastdeploy_amd import synthetic as syn
+from fastdeploy_amd.ops import CACHE_FP8, CACHE_INT8
+
+pytestmark = pytest.mark.gpu
+
+
+def oracle_select(oracle, case, top_k):
+    s = oracle.sqattn_block_scores(bits(case["q"]), np_of(case["key_cache"]), np_of(case["cache_k_scale"]),
+                                   np_of(case["block_tables"]), np_of(case["seq_lens_decoder"]), case["hq"],
+                                   case["hkv"], case["d"], case["quant"])
+    kept, cnt = oracle.topk_select(s, np_of(case["seq_lens_decoder"]), case["bs"], top_k)
+    return s, kept, cnt
+
+
+@pytest.mark.parametrize("quant", [CACHE_FP8, CACHE_INT8])
+def test_selector_indices_bit_exact(oracle, quant):
+    for seed in range(2):
+        case = syn.decode_case(batch=3, ctx=[4096, 3000, 64 * 20 + 1], quant=quant, seed=seed, salient=0.05)
+        dev = syn.to_device(case, "cuda")
+        kept, cnt, sc = fd.sqattn_select(dev["q"], dev["key_cache"], dev["cache_k_scale"], dev["block_tables"],
+                                         dev["seq_lens_decoder"], num_heads=32, top_k=8, cache_quant_type=quant,
+                                         return_scores=True)
+        s, okept, ocnt = oracle_select(oracle, case, 8)
+        assert np.array_equal(np_of(cnt), ocnt)
+        assert np.array_equal(np_of(kept), okept)
+        assert np.array_equal(np_of(sc), s.astype(np.float32))
+
+
+def test_selector_ties_and_short_sequences(oracle):
+    case = syn.decode_case(batch=2, ctx=[64 * 12, 100], quant=CACHE_FP8, seed=3)
+    bt = case["block_tables"]
+    # identical K pages -> identical scores -> the lower block index must win
+    for j in (5, 7, 9):
+        case["key_cache"][int(bt[0, j])] = case["key_cache"][int(bt[0, 2])]
+    dev = syn.to_device(case, "cuda")
+    for k in (1, 2, 3, 4, 11, 12, 64):
+        kept, cnt = fd.sqattn_select(dev["q"], dev["key_cache"], dev["cache_k_scale"], dev["block_tables"],
+                                     dev["seq_lens_decoder"], num_heads=32, top_k=k)
+        _, okept, ocnt = oracle_select(oracle, case, k)
+        assert np.array_equal(np_of(kept), okept) and np.array_equal(np_of(cnt), ocnt), k
+
+
+def _prefill_case(seed, prefix, chunks, quant=CACHE_INT8):
+    batch = len(chunks)
+    base = syn.decode_case(batch=batch, ctx=prefix, quant=quant, seed=seed, extra_blocks=4)
+    g = torch.Generator().manual_seed(seed + 100)
+    T = sum(chunks)
+    base["q_new"] = torch.randn((T, 32 * 128), generator=g).to(torch.bfloat16)
+    base["k_new"] = torch.randn((T, 8 * 128), generator=g).to(torch.bfloat16)
+    base["v_new"] = torch.randn((T, 8 * 128), generator=g).to(torch.bfloat16)
+    base["cu_seqlens_q"] = torch.tensor([0] + list(np.cumsum(chunks)), dtype=torch.int32)
+    return base
+
+
+@pytest.mark.parametrize("impl", ["generic", "auto"])
+@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+def test_prefill_small(oracle, impl, quant):
+    c = _prefill_case(1, [200, 64, 0, 333], [70, 128, 5, 1], quant)
+    dev = syn.to_device(c, "cuda")
+    out = fd.append_attention_prefill(dev["q_new"], dev["k_new"], dev["v_new"], dev["key_cache"], dev["value_cache"],
+                                      dev["cache_k_scale"], dev["cache_v_scale"], dev["block_tables"],
+                                      dev["seq_lens_decoder"], dev["cu_seqlens_q"], num_heads=32, max_chunk=128,
+                                      cache_quant_type=quant, impl=impl)
+    want = oracle.append_attention_prefill(bits(c["q_new"]), bits(c["k_new"]), bits(c["v_new"]), np_of(c["key_cache"]),
+                                           np_of(c["value_cache"]), np_of(c["cache_k_scale"]), np_of(c["cache_v_scale"]),
+                                           np_of(c["block_tables"]), np_of(c["seq_lens_decoder"]), np_of(c["cu_seqlens_q"]),
+                                           32, 8, 128, quant)
+    ok, mx, bad = bf16_close(bits(out), want)
+    assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
