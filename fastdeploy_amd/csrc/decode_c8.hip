@@ -1,11 +1,609 @@
-// placeholder until the MFMA kernel lands
+// Decode attention over the int8 / fp8-e4m3 paged cache for head_dim 128, 4 query heads
+// per KV head, block_size 64 - the HBM-bound kernel of the path.
+//
+// Work unit: one (sequence, KV head, cache block) = an 8 KiB K tile + an 8 KiB V tile,
+// each contiguous in HBM.  All units of a launch are laid end to end (sequence-major,
+// head, block) and cut into equal contiguous chunks, one per wavefront, so every
+// wavefront streams the same number of bytes whatever the sequence lengths are.  A
+// wavefront is autonomous: it owns a K slot, a V slot and a P slot in LDS, fills them
+// with direct global->LDS loads (16 B per lane, whole 128-byte rows), and never meets a
+// barrier.  While it works on block i, K(i+1) and V(i+1) are in flight.
+//
+// Arithmetic runs on the MFMA units without dequantising a single cache byte:
+//   int8 cache: v_mfma_i32_16x16x64_i8.  The 4 query heads occupy the 16 MFMA rows as
+//     4 heads x up to 4 byte "limbs": q*k_scale is split into 3 balanced base-128 digits
+//     (21 bits), the softmax weights into 4 base-128 digits (28 bits).  Integer dot
+//     products are exact; the limbs are recombined in fp32.
+//   fp8 cache: v_mfma_f32_16x16x32_fp8_fp8 with q*k_scale and the weights split into 4
+//     e4m3 residual limbs (16 significant bits).
+// The per-channel K scale is folded into q, the V scale is applied once to the output.
+// V tiles are transposed for free by ds_read_b64_tr_b8.
+//
+// Each wavefront leaves one partial (m, l, o[4][128]) per (sequence, KV head) it touched
+// at workspace slot wave + pair; the combine kernel merges the slots of each pair.
 #include "fdattn_common.h"
+
 namespace fdattn {
-size_t c8_workspace_bytes(int, int) { return 0; }
-bool c8_supported(int, int, int, int, int) { return false; }
-int decode_c8_launch(const void*, const void*, const void*, const float*, const float*, const int32_t*,
-                     const int32_t*, const int32_t*, const int32_t*, const int32_t*, int, void*, void*, size_t,
-                     int, int, int, int, int, int, int, int, float, hipStream_t) {
-  return fail(FDATTN_ERR_SHAPE, "decode_c8: not built");
+
+constexpr int kWaves = 4;      // wavefronts per workgroup
+constexpr int kTileB = 8192;   // bytes of one K or V tile (64 tokens x 128 channels)
+constexpr int kD = 128, kG = 4, kBS = 64;
+constexpr int kSlotFloats = kG * kD;  // partial o per slot
+
+struct C8Args {
+  const uint16_t* q;
+  const uint8_t* key_cache;
+  const uint8_t* value_cache;
+  const float* k_scale;
+  const float* v_scale;
+  const int32_t* block_tables;
+  const int32_t* seq_lens_decoder;
+  const int32_t* seq_lens_this_time;
+  const int32_t* kept_blocks;
+  const int32_t* kept_counts;
+  int max_kept;
+  float* part_o;   // [slots][4][128]
+  float* part_ml;  // [slots][8]: m[4] (log2 domain), l[4]
+  uint16_t* out;
+  int batch, hkv, max_blocks, num_blocks, num_waves;
+  float sm_scale_log2;  // softmax_scale * log2(e)
+};
+
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
 }
+// all-reduce within each 16-lane row (row_ror 8, 4, 2, 1)
+__device__ __forceinline__ float row_max16(float v) {
+  v = fmaxf(v, dpp_f<0x128>(v));
+  v = fmaxf(v, dpp_f<0x124>(v));
+  v = fmaxf(v, dpp_f<0x122>(v));
+  v = fmaxf(v, dpp_f<0x121>(v));
+  return v;
+}
+__device__ __forceinline__ float row_sum16(float v) {
+  v += dpp_f<0x128>(v);
+  v += dpp_f<0x124>(v);
+  v += dpp_f<0x122>(v);
+  v += dpp_f<0x121>(v);
+  return v;
+}
+
+template <bool SPARSE>
+__device__ __forceinline__ int pair_count(const C8Args& a, int p) {
+  if (SPARSE) return min(max(a.kept_counts[p], 0), a.max_kept);
+  const int b = p / a.hkv;
+  const int kv = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
+  return min((max(kv, 0) + kBS - 1) / kBS, a.max_blocks);
+}
+
+// Units before pair `upto` (exclusive) summed by one wavefront; all lanes get the result.
+template <bool SPARSE>
+__device__ __forceinline__ int units_before(const C8Args& a, int upto, int lane) {
+  int acc = 0;
+  for (int base = 0; base < upto; base += 64) {
+    const int p = base + lane;
+    acc += p < upto ? pair_count<SPARSE>(a, p) : 0;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+  return acc;
+}
+
+// Direct global->LDS load of one 8 KiB tile: 8 instructions of 64 lanes x 16 B.  LDS
+// receives lane l of instruction i at byte i*1024 + l*16 (row 8i + l/8, position l%8);
+// the lane fetches the 16-byte chunk (l%8) ^ f(row) of that row, so that row r's chunk c
+// sits at position c ^ f(r).  f = (r >> SHIFT) & 7 spreads the later LDS reads over banks.
+// The eight per-lane byte offsets depend on the lane only and are computed once.
+//
+// Written as inline assembly on purpose: the wavefront tracks its own loads with
+// explicit s_waitcnt vmcnt(N) (N = tile loads issued after the one waited for), which
+// stays correct whatever other memory operations the compiler interleaves, because
+// loads return in order and younger operations only make the wait stricter.
+struct DmaOffsets { u32 o[8]; };
+
+template <int SHIFT>
+__device__ __forceinline__ DmaOffsets dma_offsets(int lane) {
+  DmaOffsets d;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int row = 8 * i + (lane >> 3);
+    const int c = (lane & 7) ^ ((row >> SHIFT) & 7);
+    d.o[i] = (u32)(row * 128 + c * 16);
+  }
+  return d;
+}
+
+__device__ __forceinline__ void dma_tile(const uint8_t* gtile, u32 lds_addr, const DmaOffsets& d) {
+  u32 saved_m0;  // m0 (the LDS base of these loads) is put back as it was found
+  asm volatile(
+      "s_mov_b32 %[sv], m0\n\t"
+      "s_mov_b32 m0, %[l]\n\ts_nop 0\n\t"
+      "global_load_lds_dwordx4 %[o0], %[g]\n\t"
+      "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
+      "global_load_lds_dwordx4 %[o1], %[g]\n\t"
+      "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
+      "global_load_lds_dwordx4 %[o2], %[g]\n\t"
+      "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
+      "global_load_lds_dwordx4 %[o3], %[g]\n\t"
+      "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
+      "global_load_lds_dwordx4 %[o4], %[g]\n\t"
+      "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
+      "global_load_lds_dwordx4 %[o5], %[g]\n\t"
+      "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
+      "global_load_lds_dwordx4 %[o6], %[g]\n\t"
+      "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
+      "global_load_lds_dwordx4 %[o7], %[g]\n\t"
+      "s_mov_b32 m0, %[sv]\n\t"
+      : [sv] "=&s"(saved_m0)
+      : [l] "s"(lds_addr), [g] "s"(gtile), [o0] "v"(d.o[0]), [o1] "v"(d.o[1]), [o2] "v"(d.o[2]),
+        [o3] "v"(d.o[3]), [o4] "v"(d.o[4]), [o5] "v"(d.o[5]), [o6] "v"(d.o[6]), [o7] "v"(d.o[7])
+      : "memory", "scc");
+}
+
+__device__ __forceinline__ u32 lds_addr_of(const void* p) {
+  return (u32)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
+}
+
+__device__ __forceinline__ void wait_vm8() { asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); }
+__device__ __forceinline__ void wait_vm0() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+constexpr int kShiftK = 2, kShiftV = 1;
+
+// Per-pair state of a wavefront.
+struct PairState {
+  v4i aq[2];  // Q limbs as the MFMA A operand, two k-steps of 64 channels
+  float rs;   // logit scale of this lane's head (S layout: head = lane / 16)
+  float m, l;
+  float o[8];  // channel 16*ct + lane%16 of head lane/16
+};
+
+// A operand rows: row = head*4 + limb; lane (m = lane%16, g = lane/16) holds channels
+// 16*(g + 4s) .. +15 of k-step s.
+template <int QUANT>
+__device__ __forceinline__ void load_pair(const C8Args& a, int p, int lane, PairState& st) {
+  const int b = p / a.hkv, h = p - b * a.hkv;
+  const int m = lane & 15, g = lane >> 4, head = m >> 2, limb = m & 3;
+  const uint16_t* qrow = a.q + ((size_t)b * a.hkv * kG + h * kG + head) * kD;
+  const float* ks = a.k_scale + (size_t)h * kD;
+  float qs[2][16];
+  float amax = 0.f;
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    const int c0 = 16 * (g + 4 * s);
+    const uint4 w0 = *reinterpret_cast<const uint4*>(qrow + c0);
+    const uint4 w1 = *reinterpret_cast<const uint4*>(qrow + c0 + 8);
+    const u32 w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      qs[s][2 * j] = bf16lo_to_f32(w[j]) * ks[c0 + 2 * j];
+      qs[s][2 * j + 1] = bf16hi_to_f32(w[j]) * ks[c0 + 2 * j + 1];
+      amax = fmaxf(amax, fmaxf(fabsf(qs[s][2 * j]), fabsf(qs[s][2 * j + 1])));
+    }
+  }
+  amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+  amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+  float rsval;
+  if (QUANT == FDATTN_CACHE_INT8) {
+    const float inv = amax > 0.f ? 1048575.0f / amax : 0.f;
+    rsval = amax * (1.0f / 1048575.0f) * a.sm_scale_log2;
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      u32 pk[4] = {0, 0, 0, 0};
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const int X = (int)__builtin_rintf(qs[s][j] * inv);
+        const int x0 = ((X + 64) & 127) - 64;
+        const int X1 = (X - x0) >> 7;
+        const int x1 = ((X1 + 64) & 127) - 64;
+        const int x2 = (X1 - x1) >> 7;
+        const int d = limb == 0 ? x0 : (limb == 1 ? x1 : (limb == 2 ? x2 : 0));
+        pk[j >> 2] |= ((u32)d & 0xffu) << (8 * (j & 3));
+      }
+      st.aq[s] = (v4i){(int)pk[0], (int)pk[1], (int)pk[2], (int)pk[3]};
+    }
+  } else {
+    // residual e4m3 limbs of x = qs * 256 / amax: limb0 = fp8(x), limb1 = fp8(x - limb0), ...
+    const float inv = amax > 0.f ? 256.0f / amax : 0.f;
+    rsval = amax * (1.0f / 256.0f) * a.sm_scale_log2;
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      u32 pk[4] = {0, 0, 0, 0};
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        float x = qs[s][j] * inv;
+        u32 code = 0;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const u32 c = (u32)__builtin_amdgcn_cvt_pk_fp8_f32(x, x, 0, false) & 0xffu;
+          if (t == limb) code = c;
+          x -= __builtin_amdgcn_cvt_f32_fp8((int)c, 0);
+        }
+        pk[j >> 2] |= code << (8 * (j & 3));
+      }
+      st.aq[s] = (v4i){(int)pk[0], (int)pk[1], (int)pk[2], (int)pk[3]};
+    }
+  }
+  // lane 4*head' (g = 0, limb 0) knows head'’s scale; the S layout wants head = lane / 16
+  st.rs = __shfl(rsval, 4 * (lane >> 4), 64);
+  st.m = -INFINITY;
+  st.l = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) st.o[i] = 0.f;
+}
+
+__device__ __forceinline__ void flush_pair(const C8Args& a, int slot, int lane, const PairState& st) {
+  const int n = lane & 15, g = lane >> 4;
+  float* po = a.part_o + (size_t)slot * kSlotFloats + g * kD;
+#pragma unroll
+  for (int ct = 0; ct < 8; ++ct) po[16 * ct + n] = st.o[ct];
+  const float l = row_sum16(st.l);
+  if (n == 0) {
+    a.part_ml[(size_t)slot * 8 + g] = st.m;
+    a.part_ml[(size_t)slot * 8 + 4 + g] = l;
+  }
+}
+
+// The pair that holds unit u and u's index in that pair's block list (wave-uniform).
+template <bool SPARSE>
+__device__ __forceinline__ void locate_unit(const C8Args& a, int P, int u, int lane, int& p_out, int& i_out) {
+  int p = 0, before = 0, running = 0;
+  bool found = false;
+  for (int base = 0; base < P && !found; base += 64) {
+    const int pp = base + lane;
+    const int n = pp < P ? pair_count<SPARSE>(a, pp) : 0;
+    int incl = n;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int t = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += t;
+    }
+    const int tot = __shfl(incl, 63, 64);
+    if (u < running + tot) {
+      const unsigned long long msk = __ballot(running + incl > u);
+      const int first = __ffsll((long long)msk) - 1;
+      p = base + first;
+      before = running + __shfl(incl - n, first, 64);
+      found = true;
+    }
+    running += tot;
+  }
+  p_out = uni(p);
+  i_out = uni(u - before);
+}
+
+template <int QUANT, bool SPARSE>
+__global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
+  __shared__ __attribute__((aligned(16))) uint8_t ldsK[kWaves][kTileB];
+  __shared__ __attribute__((aligned(16))) uint8_t ldsV[kWaves][kTileB];
+  __shared__ __attribute__((aligned(16))) uint8_t ldsP[kWaves][1024];
+  const int lane = threadIdx.x & 63;
+  const int wv = uni(threadIdx.x >> 6);
+  const int w = blockIdx.x * kWaves + wv;
+  uint8_t* const kbuf = ldsK[wv];
+  uint8_t* const vbuf = ldsV[wv];
+  uint8_t* const pbuf = ldsP[wv];
+  const u32 kaddr = uni((int)lds_addr_of(kbuf)), vaddr = uni((int)lds_addr_of(vbuf));
+  const DmaOffsets offK = dma_offsets<kShiftK>(lane), offV = dma_offsets<kShiftV>(lane);
+  const int P = a.batch * a.hkv;
+  const int n16 = lane & 15, g4 = lane >> 4;
+
+  // ---- this wavefront's chunk [u0, u1) of the unit sequence
+  const int U = uni(units_before<SPARSE>(a, P, lane));
+  const int C = (U + a.num_waves - 1) / a.num_waves;
+  const int u0 = w * C, u1 = min(U, u0 + C);
+  if (C == 0 || u0 >= u1) return;
+
+  const size_t tile_stride = (size_t)kBS * kD;  // bytes of one (block, head) tile
+  auto tile_ptr = [&](const uint8_t* cache, int pb, int pp) {
+    return cache + ((size_t)pb * a.hkv + (pp % a.hkv)) * tile_stride;
+  };
+
+  PairState st;
+  int cur_p = -1;
+
+  // The chunk is walked 64 units at a time: lane j first works out unit ub + j (its pair,
+  // physical block and valid-token count) so that the streaming loop below touches no
+  // memory but the tiles themselves.
+  for (int ub = u0; ub < u1; ub += 64) {
+    const int cnt = min(64, u1 - ub);
+    int p0, i0;
+    locate_unit<SPARSE>(a, P, ub, lane, p0, i0);
+    int my_p = p0, my_pb = 0, my_valid = 0;
+    {
+      int off = i0 + lane;
+      int kv = 0, lb = -1, pb = -1;
+      if (lane < cnt) {
+        int n = pair_count<SPARSE>(a, my_p);
+        while (off >= n && my_p < P - 1) {
+          off -= n;
+          ++my_p;
+          n = pair_count<SPARSE>(a, my_p);
+        }
+        const int b = my_p / a.hkv;
+        kv = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
+        lb = off;
+        if (SPARSE) lb = a.kept_blocks[(size_t)my_p * a.max_kept + min(off, a.max_kept - 1)];
+        if (lb >= 0 && lb < a.max_blocks) pb = a.block_tables[(size_t)b * a.max_blocks + lb];
+      }
+      // every load above is consumed here, on every path: nothing of the table build is
+      // left in flight when the streaming loop starts
+      asm volatile("" ::"v"(kv), "v"(lb), "v"(pb));
+      if (pb >= 0 && pb < a.num_blocks) {
+        my_pb = pb;
+        my_valid = min(max(kv - lb * kBS, 0), kBS);
+      }
+    }
+
+    int p = __builtin_amdgcn_readlane(my_p, 0);
+    int pb = __builtin_amdgcn_readlane(my_pb, 0);
+    int valid = __builtin_amdgcn_readlane(my_valid, 0);
+    dma_tile(tile_ptr(a.key_cache, pb, p), kaddr, offK);
+    dma_tile(tile_ptr(a.value_cache, pb, p), vaddr, offV);
+    if (p != cur_p) {
+      if (cur_p >= 0) flush_pair(a, w + cur_p, lane, st);
+      load_pair<QUANT>(a, p, lane, st);
+      cur_p = p;
+    }
+
+    for (int j = 0; j < cnt; ++j) {
+      const bool has_next = j + 1 < cnt;
+      int pn = p, pbn = 0, validn = 0;
+      if (has_next) {
+        pn = __builtin_amdgcn_readlane(my_p, j + 1);
+        pbn = __builtin_amdgcn_readlane(my_pb, j + 1);
+        validn = __builtin_amdgcn_readlane(my_valid, j + 1);
+      }
+
+      // ---------------- S = Q K^T : rows = head*4 + limb, columns = token slots
+      wait_vm8();  // K(j) landed; V(j) may still be in flight
+      v4i S[4];
+      v4f Sf[4];
+#pragma unroll
+      for (int stl = 0; stl < 4; ++stl) {
+        const int tok = 4 * n16 + stl;  // this lane's column of tile stl is token 4n + stl
+        if (QUANT == FDATTN_CACHE_INT8) {
+          v4i acc = {0, 0, 0, 0};
+#pragma unroll
+          for (int s = 0; s < 2; ++s) {
+            const int c = g4 + 4 * s;
+            const v4i kb = *reinterpret_cast<const v4i*>(kbuf + tok * 128 + ((c ^ ((tok >> kShiftK) & 7)) * 16));
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(st.aq[s], kb, acc, 0, 0, 0);
+          }
+          S[stl] = acc;
+        } else {
+          v4f acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int s = 0; s < 2; ++s) {
+            const int c = g4 + 4 * s;
+            const v4i kb = *reinterpret_cast<const v4i*>(kbuf + tok * 128 + ((c ^ ((tok >> kShiftK) & 7)) * 16));
+            const long a0 = ((long)(u32)st.aq[s].y << 32) | (u32)st.aq[s].x;
+            const long a1 = ((long)(u32)st.aq[s].w << 32) | (u32)st.aq[s].z;
+            const long b0 = ((long)(u32)kb.y << 32) | (u32)kb.x;
+            const long b1 = ((long)(u32)kb.w << 32) | (u32)kb.z;
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a0, b0, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a1, b1, acc, 0, 0, 0);
+          }
+          Sf[stl] = acc;
+        }
+      }
+      wait_lgkm0();  // K tile is in registers: its slot may be refilled
+      if (has_next) dma_tile(tile_ptr(a.key_cache, pbn, pn), kaddr, offK);
+
+      // ---------------- online softmax in the S layout: lane = (token slot n, head g)
+      float sv[4];
+      float mb = -INFINITY;
+#pragma unroll
+      for (int stl = 0; stl < 4; ++stl) {
+        float s;
+        if (QUANT == FDATTN_CACHE_INT8)
+          s = st.rs * ((float)S[stl].x + 128.0f * (float)S[stl].y + 16384.0f * (float)S[stl].z);
+        else
+          s = st.rs * ((Sf[stl].x + Sf[stl].y) + (Sf[stl].z + Sf[stl].w));
+        s = (4 * n16 + stl < valid) ? s : -INFINITY;
+        sv[stl] = s;
+        mb = fmaxf(mb, s);
+      }
+      mb = row_max16(mb);
+      const float m_new = fmaxf(st.m, mb);
+      // void unit (no valid token) and nothing seen yet: keep everything at zero
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f(st.m - m_use);
+      st.m = m_new;
+      u32 pw[4] = {0, 0, 0, 0};
+      float lsum = 0.f;
+#pragma unroll
+      for (int stl = 0; stl < 4; ++stl) {
+        const float pr = __builtin_amdgcn_exp2f(sv[stl] - m_use);  // in [0, 1]
+        if (QUANT == FDATTN_CACHE_INT8) {
+          u32 x = (u32)__builtin_rintf(pr * 268435456.0f);  // 2^28
+          x = min(x, 268435455u);
+          lsum += (float)x;
+          pw[0] |= (x & 127u) << (8 * stl);
+          pw[1] |= ((x >> 7) & 127u) << (8 * stl);
+          pw[2] |= ((x >> 14) & 127u) << (8 * stl);
+          pw[3] |= (x >> 21) << (8 * stl);
+        } else {
+          float x = pr * 256.0f, used = 0.f;
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const u32 c = (u32)__builtin_amdgcn_cvt_pk_fp8_f32(x, x, 0, false) & 0xffu;
+            const float dv = __builtin_amdgcn_cvt_f32_fp8((int)c, 0);
+            pw[t] |= c << (8 * stl);
+            x -= dv;
+            used += dv;
+          }
+          lsum += used;
+        }
+      }
+      st.l = st.l * alpha + lsum;
+      // P rows = head*4 + limb, 64 token bytes per row; this lane owns tokens 4n..4n+3
+#pragma unroll
+      for (int r = 0; r < 4; ++r) *reinterpret_cast<u32*>(pbuf + (4 * g4 + r) * 64 + 4 * n16) = pw[r];
+      wave_sync();
+
+      // ---------------- O += P V : V^T operands come transposed out of LDS
+      if (has_next) wait_vm8(); else wait_vm0();  // V(j) landed; K(j+1) may still be in flight
+      if (QUANT != FDATTN_CACHE_INT8 && valid < kBS) {
+        // e4m3 has NaN codes: a stale byte in a row past the sequence end would poison 0 * NaN
+        for (int r = valid + (lane >> 3); r < kBS; r += 8)
+          *reinterpret_cast<uint4*>(vbuf + r * 128 + (lane & 7) * 16) = make_uint4(0, 0, 0, 0);
+        wave_sync();
+      }
+      const v4i pa = *reinterpret_cast<const v4i*>(pbuf + n16 * 64 + 16 * g4);
+#pragma unroll
+      for (int ct = 0; ct < 8; ++ct) {
+        v2i vr[2];
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+          const int tok = 16 * g4 + 8 * r + (n16 >> 1);
+          const uint8_t* src = vbuf + tok * 128 + ((ct ^ ((tok >> kShiftV) & 7)) * 16) + 8 * (n16 & 1);
+          vr[r] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i*)src);
+        }
+        float ob;
+        if (QUANT == FDATTN_CACHE_INT8) {
+          const v4i vb = {vr[0].x, vr[0].y, vr[1].x, vr[1].y};
+          const v4i z = {0, 0, 0, 0};
+          const v4i d = __builtin_amdgcn_mfma_i32_16x16x64_i8(pa, vb, z, 0, 0, 0);
+          ob = (float)d.x + 128.0f * (float)d.y + 16384.0f * (float)d.z + 2097152.0f * (float)d.w;
+        } else {
+          v4f d = {0.f, 0.f, 0.f, 0.f};
+          const long a0 = ((long)(u32)pa.y << 32) | (u32)pa.x, a1 = ((long)(u32)pa.w << 32) | (u32)pa.z;
+          const long b0 = ((long)(u32)vr[0].y << 32) | (u32)vr[0].x, b1 = ((long)(u32)vr[1].y << 32) | (u32)vr[1].x;
+          d = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a0, b0, d, 0, 0, 0);
+          d = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a1, b1, d, 0, 0, 0);
+          ob = (d.x + d.y) + (d.z + d.w);
+        }
+        st.o[ct] = st.o[ct] * alpha + ob;
+      }
+      wait_lgkm0();  // V tile consumed
+      if (has_next) dma_tile(tile_ptr(a.value_cache, pbn, pn), vaddr, offV);
+
+      // ---------------- next unit
+      if (!has_next) break;
+      if (pn != p) {
+        flush_pair(a, w + p, lane, st);
+        load_pair<QUANT>(a, pn, lane, st);
+        cur_p = pn;
+      }
+      p = pn;
+      pb = pbn;
+      valid = validn;
+    }
+  }
+  flush_pair(a, w + cur_p, lane, st);
+}
+
+// One workgroup per (sequence, KV head): merges the slots wave + pair of the wavefronts
+// whose chunks overlap the pair, applies the V scale and writes bf16.
+template <bool SPARSE>
+__global__ __launch_bounds__(256) void decode_c8_combine_kernel(C8Args a) {
+  __shared__ int sh[2];
+  const int p = blockIdx.x, tid = threadIdx.x;
+  const int P = a.batch * a.hkv;
+  if (tid < 64) {
+    const int bef = units_before<SPARSE>(a, p, tid);
+    const int tot = units_before<SPARSE>(a, P, tid);
+    if (tid == 0) { sh[0] = bef; sh[1] = tot; }
+  }
+  __syncthreads();
+  const int before = sh[0], U = sh[1];
+  const int n = pair_count<SPARSE>(a, p);
+  const int b = p / a.hkv, h = p - b * a.hkv;
+  const int head = tid >> 6, c2 = (tid & 63) * 2;
+  uint16_t* o = a.out + ((size_t)b * a.hkv * kG + h * kG + head) * kD + c2;
+  if (n == 0 || U == 0) {
+    *reinterpret_cast<u32*>(o) = 0u;
+    return;
+  }
+  const int C = (U + a.num_waves - 1) / a.num_waves;
+  const int w0 = before / C, w1 = (before + n - 1) / C;
+  float M = -INFINITY;
+  for (int w = w0; w <= w1; ++w) M = fmaxf(M, a.part_ml[(size_t)(w + p) * 8 + head]);
+  float L = 0.f, o0 = 0.f, o1 = 0.f;
+  if (M > -INFINITY) {
+    for (int w = w0; w <= w1; ++w) {
+      const size_t slot = (size_t)(w + p);
+      const float ms = a.part_ml[slot * 8 + head];
+      if (ms == -INFINITY) continue;
+      const float f = exp2f(ms - M);
+      L += a.part_ml[slot * 8 + 4 + head] * f;
+      const float2 v = *reinterpret_cast<const float2*>(a.part_o + slot * kSlotFloats + head * kD + c2);
+      o0 += v.x * f;
+      o1 += v.y * f;
+    }
+  }
+  const float inv = L > 0.f ? 1.0f / L : 0.f;
+  const float r0 = o0 * inv * a.v_scale[h * kD + c2], r1 = o1 * inv * a.v_scale[h * kD + c2 + 1];
+  *reinterpret_cast<u32*>(o) = (u32)f32_to_bf16(r0) | ((u32)f32_to_bf16(r1) << 16);
+}
+
+static int num_cus() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      cus = n;
+    else
+      cus = 256;
+  }
+  return cus;
+}
+
+constexpr int kMaxWaves = 2 * 512 * kWaves;  // workspace is sized for up to 512 CUs
+
+size_t c8_workspace_bytes(int batch, int hkv) {
+  const size_t slots = (size_t)kMaxWaves + (size_t)batch * hkv;
+  return slots * (kSlotFloats + 8) * sizeof(float);
+}
+
+bool c8_supported(int hq, int hkv, int d, int bs, int quant) {
+  return d == kD && hq == kG * hkv && bs == kBS &&
+         (quant == FDATTN_CACHE_INT8 || quant == FDATTN_CACHE_FP8_E4M3);
+}
+
+int decode_c8_launch(const void* q, const void* key_cache, const void* value_cache, const float* k_scale,
+                     const float* v_scale, const int32_t* block_tables, const int32_t* seq_lens_decoder,
+                     const int32_t* seq_lens_this_time, const int32_t* kept_blocks, const int32_t* kept_counts,
+                     int max_kept, void* out, void* workspace, size_t workspace_bytes, int batch, int hq,
+                     int hkv, int d, int bs, int max_blocks, int num_blocks, int quant, float sm_scale,
+                     hipStream_t s) {
+  (void)hq; (void)d; (void)bs;
+  int waves = 2 * num_cus() * kWaves;
+  if (waves > kMaxWaves) waves = kMaxWaves;
+  const size_t slots = (size_t)waves + (size_t)batch * hkv;
+  const size_t need = slots * (kSlotFloats + 8) * sizeof(float);
+  if (workspace_bytes < need)
+    return fail(FDATTN_ERR_WORKSPACE, "fdattn_decode_attention: workspace %zu B < required %zu B", workspace_bytes, need);
+  float* part_o = (float*)workspace;
+  float* part_ml = part_o + slots * kSlotFloats;
+  C8Args a{(const uint16_t*)q, (const uint8_t*)key_cache, (const uint8_t*)value_cache, k_scale, v_scale,
+           block_tables, seq_lens_decoder, seq_lens_this_time, kept_blocks, kept_counts, max_kept, part_o,
+           part_ml, (uint16_t*)out, batch, hkv, max_blocks, num_blocks, waves,
+           sm_scale * 1.4426950408889634f};
+  const dim3 grid(waves / kWaves), block(kWaves * 64);
+  const bool sparse = kept_blocks != nullptr;
+  if (quant == FDATTN_CACHE_INT8) {
+    if (sparse) hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_INT8, true>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_INT8, false>), grid, block, 0, s, a);
+  } else {
+    if (sparse) hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_FP8_E4M3, true>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_FP8_E4M3, false>), grid, block, 0, s, a);
+  }
+  int rc = check_launch("fdattn_decode_attention (mfma)");
+  if (rc) return rc;
+  if (sparse) hipLaunchKernelGGL(decode_c8_combine_kernel<true>, dim3(batch * hkv), dim3(256), 0, s, a);
+  else hipLaunchKernelGGL(decode_c8_combine_kernel<false>, dim3(batch * hkv), dim3(256), 0, s, a);
+  return check_launch("fdattn_decode_attention (combine)");
+}
+
 }  // namespace fdattn
