@@ -1,0 +1,154 @@
+#!/usr/bin/env python3
+"""Benchmark of the paged-KV decode attention hot path on one MI355X.
+
+Workload (BASELINE.json configs[1]): one Llama-3-8B-shaped attention layer in decode,
+batch 64, 32 query / 8 KV heads, head_dim 128, block_size 64, context lengths
+U[3584, 4608], int8 KV cache with per-channel scales, block tables a random
+permutation over a 6000-block pool.  A "step" is one decode-attention pass over the
+batch (split-KV kernel + merge kernel); inputs are resident in HBM.
+
+Prints ONE JSON line.  `value` is microseconds per layer for the whole op;
+`roofline` prices the dominant (split-KV) kernel against the 8 TB/s HBM peak with
+the algorithmic bytes of the pass; `cpu_baseline` is the CPU oracle timed on this
+host's cores on the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def time_events(fn, steps, warmup):
+    """Average milliseconds per call over `steps` back-to-back calls on torch's current stream
+    (the stream the kernels are launched on), bracketed by HIP events and device syncs."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
+    ap.add_argument("--pools", type=int, default=2, help="distinct cache pools rotated between steps")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (the path shards by KV head or by sequence with no "
+                 "exchange; nothing here uses a second device). Run with --gpus 1.")
+
+    import fastdeploy_amd as fd
+    from fastdeploy_amd import synthetic as syn
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    B = 64
+    # distinct pools so that consecutive steps do not re-read the same bytes out of the
+    # last-level cache; every pool has its own block table permutation and contents
+    g = torch.Generator().manual_seed(0)
+    lens = torch.randint(3584, 4609, (B,), generator=g).tolist()
+    cases = [syn.decode_case(batch=B, ctx=lens, pool_blocks=6000, seed=s, device=dev, direct_bytes=True,
+                             max_blocks=72) for s in range(args.pools)]
+    assert fd.decode_uses_mfma(32, 8, 128, 64, "cache_int8")
+    ws = fd.decode_workspace(B, 32, 8, 128, dev)
+    outs = [torch.empty((B, 32 * 128), dtype=torch.bfloat16, device=dev) for _ in cases]
+
+    def run(i, impl):
+        c = cases[i % len(cases)]
+        fd.decode_attention(c["q"], c["key_cache"], c["value_cache"], c["cache_k_scale"], c["cache_v_scale"],
+                            c["block_tables"], c["seq_lens_decoder"], num_heads=32, cache_quant_type="cache_int8",
+                            out=outs[i % len(cases)], workspace=ws, impl=impl)
+
+    counter = [0]
+
+    def step(impl="auto"):
+        run(counter[0], impl)
+        counter[0] += 1
+
+    # whole op: split-KV kernel + merge kernel
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ms_op = time_events(lambda: step("auto"), args.steps, args.warmup)
+    wall = time.perf_counter() - t0
+    # dominant kernel alone (same launches minus the merge), for the roofline line
+    ms_main = time_events(lambda: step("partials"), args.steps, args.warmup)
+    ms_merge = time_events(lambda: step("merge"), args.steps, args.warmup)
+
+    alg_bytes = syn.decode_algorithmic_bytes(lens, B)
+    kv_bytes = syn.decode_kv_bytes(lens)
+    achieved = alg_bytes / (ms_main * 1e-3) / 1e9
+    us_layer = ms_op * 1e3
+    result = {
+        "metric": "decode_attn_us_per_layer", "value": round(us_layer, 3), "unit": "us/layer",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_op, 6),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "configs[1]: Llama-3-8B decode attention, 1 layer, batch 64, 32q/8kv heads, "
+                               "head_dim 128, block_size 64, ctx U[3584,4608], int8 paged KV, 6000-block pool",
+                   "batch": B, "mean_ctx": sum(lens) / B, "kv_bytes": kv_bytes, "pools_rotated": len(cases)},
+        "achieved_hbm_gbps_whole_op": round(alg_bytes / (ms_op * 1e-3) / 1e9, 1),
+        "pct_hbm_peak_whole_op": round(100 * alg_bytes / (ms_op * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
+        "tokens_per_s_1_layer": round(B / (ms_op * 1e-3), 1),
+        "tokens_per_s_32_layers_attention_only": round(B / (32 * ms_op * 1e-3), 1),
+        "kernel_us": {"decode_c8_kernel": round(ms_main * 1e3, 3), "decode_c8_combine_kernel": round(ms_merge * 1e3, 3)},
+        "roofline": {"bound": "hbm", "kernel": "decode_c8_kernel<int8,dense>", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "algorithmic_bytes": alg_bytes, "traffic": None},
+    }
+
+    if not args.no_cpu:
+        from oracle import oracle
+        import numpy as np
+        c = {k: (v.cpu() if isinstance(v, torch.Tensor) else v) for k, v in cases[0].items()}
+        qb = c["q"].view(torch.int16).numpy().view(np.uint16)
+        a = [qb, c["key_cache"].numpy(), c["value_cache"].numpy(), c["cache_k_scale"].numpy(),
+             c["cache_v_scale"].numpy(), c["block_tables"].numpy(), c["seq_lens_decoder"].numpy(), 32, 8, 128, 1]
+        cores = len(os.sched_getaffinity(0))
+        cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+        oracle.decode_attention(*a)                      # warm-up pass (page-in, thread start)
+        reps, t = 0, time.perf_counter()
+        while True:
+            ref = oracle.decode_attention(*a)
+            reps += 1
+            if time.perf_counter() - t > 10.0 or reps >= 5:
+                break
+        cpu_s = (time.perf_counter() - t) / reps
+        result["cpu_baseline"] = {
+            "value": round(cpu_s * 1e6, 1), "unit": "us/layer", "cores": cores, "kind": "port",
+            "sample": "the whole configs[1] workload (pool 0), %d timed passes of the C oracle "
+                      "(fp32, OpenMP over sequence x head); the reference has no CPU attention path" % reps,
+            "gpu_speedup": round(cpu_s * 1e6 / us_layer, 1)}
+        # and the run doubles as a full-size parity check of pool 0
+        got = outs[0].cpu().view(torch.int16).numpy().view(np.uint16)
+        run(0, "auto")
+        torch.cuda.synchronize()
+        got = outs[0].cpu().view(torch.int16).numpy().view(np.uint16)
+        gf = (got.astype(np.uint32) << 16).view(np.float32)
+        rf = (ref.astype(np.uint32) << 16).view(np.float32)
+        d = np.abs(gf - rf)
+        bad = (d > 2e-3) & (d / np.maximum(np.maximum(np.abs(gf), np.abs(rf)), 1e-30) > 1e-2)
+        result["parity_full_size"] = {"max_abs_diff": float(d.max()), "out_of_tolerance": int(bad.sum()),
+                                      "tolerance": "abs 2e-3 OR rel 1e-2"}
+    result["wall_s_timed_region"] = round(wall, 3)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

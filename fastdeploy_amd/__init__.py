@@ -9,6 +9,7 @@ from .ops import (  # noqa: F401
     append_attention_prefill,
     decode_attention,
     decode_attention_sparse,
+    decode_uses_mfma,
     decode_workspace,
     splitkv_combine,
     sqattn_select,

@@ -20,7 +20,7 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
                      const int32_t* kept_blocks, const int32_t* kept_counts, int max_kept,
                      void* out, void* workspace, size_t workspace_bytes, int batch, int hq,
                      int hkv, int d, int bs, int max_blocks, int num_blocks, int quant,
-                     float sm_scale, hipStream_t s);
+                     float sm_scale, hipStream_t s, int stages);
 
 static int check_decode_args(const char* fn, const void* q, const void* kc, const void* vc, const float* ks,
                              const float* vs, const int32_t* bt, const int32_t* dec, const void* out,
@@ -59,11 +59,39 @@ extern "C" int fdattn_decode_attention(
                              cache_v_scale, block_tables, seq_lens_decoder, out, workspace, batch, hq, hkv,
                              head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type);
   if (rc) return rc;
-  auto fn = c8_supported(hq, hkv, head_dim, block_size, cache_quant_type) ? decode_c8_launch : decode_generic_launch;
-  return fn(q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables, seq_lens_decoder,
-            seq_lens_this_time, nullptr, nullptr, 0, out, workspace, workspace_bytes, batch, hq, hkv,
-            head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type, softmax_scale,
-            (hipStream_t)stream);
+  if (c8_supported(hq, hkv, head_dim, block_size, cache_quant_type))
+    return decode_c8_launch(q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
+                            seq_lens_decoder, seq_lens_this_time, nullptr, nullptr, 0, out, workspace,
+                            workspace_bytes, batch, hq, hkv, head_dim, block_size, max_blocks_per_seq,
+                            num_blocks, cache_quant_type, softmax_scale, (hipStream_t)stream, 3);
+  return decode_generic_launch(q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
+                               seq_lens_decoder, seq_lens_this_time, nullptr, nullptr, 0, out, workspace,
+                               workspace_bytes, batch, hq, hkv, head_dim, block_size, max_blocks_per_seq,
+                               num_blocks, cache_quant_type, softmax_scale, (hipStream_t)stream);
+}
+
+extern "C" int fdattn_decode_uses_mfma(int hq, int hkv, int head_dim, int block_size, int cache_quant_type) {
+  return c8_supported(hq, hkv, head_dim, block_size, cache_quant_type) ? 1 : 0;
+}
+
+extern "C" int fdattn_decode_attention_stages(
+    const void* q, const void* key_cache, const void* value_cache, const float* cache_k_scale,
+    const float* cache_v_scale, const int32_t* block_tables, const int32_t* seq_lens_decoder,
+    const int32_t* seq_lens_this_time, void* out, void* workspace, size_t workspace_bytes, int batch,
+    int hq, int hkv, int head_dim, int block_size, int max_blocks_per_seq, int num_blocks,
+    int cache_quant_type, float softmax_scale, int stages, void* stream) {
+  int rc = check_decode_args("fdattn_decode_attention_stages", q, key_cache, value_cache, cache_k_scale,
+                             cache_v_scale, block_tables, seq_lens_decoder, out, workspace, batch, hq, hkv,
+                             head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type);
+  if (rc) return rc;
+  if (!c8_supported(hq, hkv, head_dim, block_size, cache_quant_type))
+    return fail(FDATTN_ERR_SHAPE, "fdattn_decode_attention_stages: shape not covered by the MFMA kernel");
+  if (stages < 1 || stages > 3)
+    return fail(FDATTN_ERR_SHAPE, "fdattn_decode_attention_stages: stages must be 1, 2 or 3");
+  return decode_c8_launch(q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
+                          seq_lens_decoder, seq_lens_this_time, nullptr, nullptr, 0, out, workspace,
+                          workspace_bytes, batch, hq, hkv, head_dim, block_size, max_blocks_per_seq,
+                          num_blocks, cache_quant_type, softmax_scale, (hipStream_t)stream, stages);
 }
 
 extern "C" int fdattn_decode_attention_generic(
@@ -99,9 +127,15 @@ extern "C" int fdattn_decode_attention_sparse(
   if (rc) return rc;
   if (!kept_blocks || !kept_counts || max_kept <= 0)
     return fail(FDATTN_ERR_NULL, "fdattn_decode_attention_sparse: kept_blocks / kept_counts / max_kept missing");
-  auto fn = c8_supported(hq, hkv, head_dim, block_size, cache_quant_type) ? decode_c8_launch : decode_generic_launch;
-  return fn(q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables, seq_lens_decoder,
-            seq_lens_this_time, kept_blocks, kept_counts, max_kept, out, workspace, workspace_bytes, batch,
-            hq, hkv, head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type, softmax_scale,
-            (hipStream_t)stream);
+  if (c8_supported(hq, hkv, head_dim, block_size, cache_quant_type))
+    return decode_c8_launch(q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
+                            seq_lens_decoder, seq_lens_this_time, kept_blocks, kept_counts, max_kept, out,
+                            workspace, workspace_bytes, batch, hq, hkv, head_dim, block_size,
+                            max_blocks_per_seq, num_blocks, cache_quant_type, softmax_scale,
+                            (hipStream_t)stream, 3);
+  return decode_generic_launch(q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
+                               seq_lens_decoder, seq_lens_this_time, kept_blocks, kept_counts, max_kept, out,
+                               workspace, workspace_bytes, batch, hq, hkv, head_dim, block_size,
+                               max_blocks_per_seq, num_blocks, cache_quant_type, softmax_scale,
+                               (hipStream_t)stream);
 }

@@ -576,7 +576,7 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
                      const int32_t* seq_lens_this_time, const int32_t* kept_blocks, const int32_t* kept_counts,
                      int max_kept, void* out, void* workspace, size_t workspace_bytes, int batch, int hq,
                      int hkv, int d, int bs, int max_blocks, int num_blocks, int quant, float sm_scale,
-                     hipStream_t s) {
+                     hipStream_t s, int stages) {
   (void)hq; (void)d; (void)bs;
   int waves = 2 * num_cus() * kWaves;
   if (waves > kMaxWaves) waves = kMaxWaves;
@@ -592,7 +592,8 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
            sm_scale * 1.4426950408889634f};
   const dim3 grid(waves / kWaves), block(kWaves * 64);
   const bool sparse = kept_blocks != nullptr;
-  if (quant == FDATTN_CACHE_INT8) {
+  if (!(stages & 1)) {
+  } else if (quant == FDATTN_CACHE_INT8) {
     if (sparse) hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_INT8, true>), grid, block, 0, s, a);
     else hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_INT8, false>), grid, block, 0, s, a);
   } else {
@@ -600,7 +601,7 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
     else hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_FP8_E4M3, false>), grid, block, 0, s, a);
   }
   int rc = check_launch("fdattn_decode_attention (mfma)");
-  if (rc) return rc;
+  if (rc || !(stages & 2)) return rc;
   if (sparse) hipLaunchKernelGGL(decode_c8_combine_kernel<true>, dim3(batch * hkv), dim3(256), 0, s, a);
   else hipLaunchKernelGGL(decode_c8_combine_kernel<false>, dim3(batch * hkv), dim3(256), 0, s, a);
   return check_launch("fdattn_decode_attention (combine)");

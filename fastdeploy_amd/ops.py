@@ -148,6 +148,12 @@ def decode_workspace(batch, num_heads, kv_num_heads, head_dim, device="cuda"):
     return torch.empty(n, dtype=torch.uint8, device=device)
 
 
+def decode_uses_mfma(num_heads, kv_num_heads, head_dim, block_size, cache_quant_type="cache_int8"):
+    """True if decode_attention runs these shapes on the MFMA kernel."""
+    return bool(_lib.lib().fdattn_decode_uses_mfma(num_heads, kv_num_heads, head_dim, block_size,
+                                                   _quant(cache_quant_type)))
+
+
 def _decode_common(q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
                    seq_lens_decoder, seq_lens_this_time, num_heads, out, workspace):
     nb, hkv, bs, d = _cache_dims(key_cache, value_cache)
@@ -191,8 +197,12 @@ def decode_attention(q, key_cache, value_cache, cache_k_scale, cache_v_scale, bl
     elif impl == "auto":
         rc = _lib.lib().fdattn_decode_attention(
             *ptrs, p_out, p_ws, workspace.numel(), *dims, _quant(cache_quant_type), scale, _stream())
+    elif impl in ("partials", "merge"):   # the two kernels of the MFMA path, one at a time
+        rc = _lib.lib().fdattn_decode_attention_stages(
+            *ptrs, p_out, p_ws, workspace.numel(), *dims, _quant(cache_quant_type), scale,
+            1 if impl == "partials" else 2, _stream())
     else:
-        raise ValueError("impl must be auto or generic")
+        raise ValueError("impl must be auto, generic, partials or merge")
     _lib.check(rc, "decode_attention")
     return out
 

@@ -122,6 +122,29 @@ FDATTN_API int fdattn_decode_attention(
     float softmax_scale, void* stream);
 
 /*
+ * 1 if fdattn_decode_attention(_sparse) runs these shapes on the MFMA kernel (head_dim
+ * 128, hq/hkv 4, block_size 64, either cache type), 0 if on the shape-agnostic one.
+ */
+FDATTN_API int fdattn_decode_uses_mfma(int hq, int hkv, int head_dim, int block_size, int cache_quant_type);
+
+/*
+ * fdattn_decode_attention split into its two kernels, for profiling and for callers
+ * that overlap other work with the merge: stages = 1 runs only the split-KV kernel
+ * (partials into `workspace`), 2 only the merge (workspace -> out), 3 both.  MFMA
+ * shapes only (FDATTN_ERR_SHAPE otherwise).  Same plug-in position as
+ * fdattn_decode_attention.
+ */
+FDATTN_API int fdattn_decode_attention_stages(
+    const void* q, const void* key_cache, const void* value_cache,
+    const float* cache_k_scale, const float* cache_v_scale,
+    const int32_t* block_tables, const int32_t* seq_lens_decoder,
+    const int32_t* seq_lens_this_time, void* out,
+    void* workspace, size_t workspace_bytes,
+    int batch, int hq, int hkv, int head_dim, int block_size,
+    int max_blocks_per_seq, int num_blocks, int cache_quant_type,
+    float softmax_scale, int stages, void* stream);
+
+/*
  * Same, restricted to a per-(sequence, KV head) list of logical blocks:
  *   kept_blocks i32 [batch, hkv, max_kept]  logical block indices, ascending, -1 padded
  *   kept_counts i32 [batch, hkv]
