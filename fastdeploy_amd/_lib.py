@@ -13,7 +13,7 @@ SIGNATURES = {
     "fdattn_version": (ctypes.c_char_p, []),
     "fdattn_last_error": (ctypes.c_char_p, []),
     "fdattn_write_cache_kv": (_i, [_vp] * 13 + [_i] * 11 + [_vp]),
-    "fdattn_decode_workspace_bytes": (_sz, [_i] * 4),
+    "fdattn_decode_workspace_bytes": (_sz, [_i] * 5),
     "fdattn_decode_attention": (_i, [_vp] * 10 + [_sz] + [_i] * 8 + [_f, _vp]),
     "fdattn_decode_uses_mfma": (_i, [_i] * 5),
     "fdattn_decode_attention_stages": (_i, [_vp] * 10 + [_sz] + [_i] * 8 + [_f, _i, _vp]),

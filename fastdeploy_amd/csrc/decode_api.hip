@@ -12,7 +12,7 @@ int decode_generic_launch(const void* q, const void* key_cache, const void* valu
                           void* out, void* workspace, size_t workspace_bytes, int batch, int hq,
                           int hkv, int d, int bs, int max_blocks, int num_blocks, int quant,
                           float sm_scale, hipStream_t s);
-size_t c8_workspace_bytes(int batch, int hkv);
+size_t c8_workspace_bytes(int batch, int hkv, int max_units);
 bool c8_supported(int hq, int hkv, int d, int bs, int quant);
 int decode_c8_launch(const void* q, const void* key_cache, const void* value_cache,
                      const float* k_scale, const float* v_scale, const int32_t* block_tables,
@@ -41,10 +41,10 @@ static int check_decode_args(const char* fn, const void* q, const void* kc, cons
 
 using namespace fdattn;
 
-extern "C" size_t fdattn_decode_workspace_bytes(int batch, int hq, int hkv, int head_dim) {
-  if (batch <= 0 || hq <= 0 || hkv <= 0 || head_dim <= 0) return 256;
+extern "C" size_t fdattn_decode_workspace_bytes(int batch, int hq, int hkv, int head_dim, int max_blocks_per_seq) {
+  if (batch <= 0 || hq <= 0 || hkv <= 0 || head_dim <= 0 || max_blocks_per_seq <= 0) return 256;
   size_t a = generic_workspace_bytes(batch, hq, head_dim);
-  size_t b = c8_workspace_bytes(batch, hkv);
+  size_t b = c8_workspace_bytes(batch, hkv, max_blocks_per_seq);
   size_t n = a > b ? a : b;
   return (n + 255) & ~(size_t)255;
 }

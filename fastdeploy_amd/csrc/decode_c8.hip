@@ -2,12 +2,17 @@
 // per KV head, block_size 64 - the HBM-bound kernel of the path.
 //
 // Work unit: one (sequence, KV head, cache block) = an 8 KiB K tile + an 8 KiB V tile,
-// each contiguous in HBM.  All units of a launch are laid end to end (sequence-major,
-// head, block) and cut into equal contiguous chunks, one per wavefront, so every
-// wavefront streams the same number of bytes whatever the sequence lengths are.  A
-// wavefront is autonomous: it owns a K slot, a V slot and a P slot in LDS, fills them
-// with direct global->LDS loads (16 B per lane, whole 128-byte rows), and never meets a
-// barrier.  While it works on block i, K(i+1) and V(i+1) are in flight.
+// each contiguous in HBM.  The block list of every (sequence, KV head) pair is cut into
+// chunks of `chunk` units; one workgroup of 4 wavefronts takes one chunk (grid = chunks
+// per pair x pairs, workgroups past the end of a list do nothing).  Chunks are short
+// (24 units = 384 KiB by default), so the hardware dispatcher balances uneven sequence
+// lengths, and they need no scan to be found: pair and chunk follow from the block index,
+// the physical blocks from one coalesced read of the block table.
+//
+// Inside a workgroup every wavefront is autonomous: it takes units wave, wave+4, ... of
+// the chunk, owns a K slot, a V slot and a P slot in LDS, fills them with direct
+// global->LDS loads (16 B per lane, whole 128-byte rows) and meets no barrier until the
+// chunk is done.  While it works on unit j, K(j+1) and V(j+1) are in flight.
 //
 // Arithmetic runs on the MFMA units without dequantising a single cache byte:
 //   int8 cache: v_mfma_i32_16x16x64_i8.  The 4 query heads occupy the 16 MFMA rows as
@@ -19,9 +24,18 @@
 // The per-channel K scale is folded into q, the V scale is applied once to the output.
 // V tiles are transposed for free by ds_read_b64_tr_b8.
 //
-// Each wavefront leaves one partial (m, l, o[4][128]) per (sequence, KV head) it touched
-// at workspace slot wave + pair; the combine kernel merges the slots of each pair.
+// At the end the 4 wavefronts merge their (m, l, o) through LDS.  A pair with a single
+// chunk is finished on the spot (bf16 output written); otherwise the workgroup leaves one
+// partial at workspace slot pair*chunks_per_pair + chunk and the merge kernel combines
+// them.  Two variants were measured slower and dropped: merging inside the main kernel
+// (the last workgroup to arrive at a pair combines it: the device-scope stores, the atomic
+// and the barrier sit at the end of every workgroup, where nothing hides their latency),
+// and handing chunks out through an atomic ticket counter instead of the block index.
 #include "fdattn_common.h"
+
+#ifndef TRACE
+#define TRACE(slot)  // timestamp hook of the perf harness; nothing in the library
+#endif
 
 namespace fdattn {
 
@@ -29,6 +43,7 @@ constexpr int kWaves = 4;      // wavefronts per workgroup
 constexpr int kTileB = 8192;   // bytes of one K or V tile (64 tokens x 128 channels)
 constexpr int kD = 128, kG = 4, kBS = 64;
 constexpr int kSlotFloats = kG * kD;  // partial o per slot
+constexpr int kMaxChunk = 64;         // units per chunk: one unit-table entry per lane
 
 struct C8Args {
   const uint16_t* q;
@@ -42,10 +57,12 @@ struct C8Args {
   const int32_t* kept_blocks;
   const int32_t* kept_counts;
   int max_kept;
-  float* part_o;   // [slots][4][128]
-  float* part_ml;  // [slots][8]: m[4] (log2 domain), l[4]
+  float* part_o;   // [pairs * chunks_per_pair][4][128]
+  float* part_ml;  // [pairs * chunks_per_pair][8]: m[4] (log2 domain), l[4]
   uint16_t* out;
-  int batch, hkv, max_blocks, num_blocks, num_waves;
+  int batch, hkv, max_blocks, num_blocks;
+  int chunk;            // units per workgroup
+  int chunks_per_pair;  // grid.x
   float sm_scale_log2;  // softmax_scale * log2(e)
 };
 
@@ -71,25 +88,11 @@ __device__ __forceinline__ float row_sum16(float v) {
   return v;
 }
 
+// Length of the pair's block list: every block of the sequence, or the kept ones.
 template <bool SPARSE>
-__device__ __forceinline__ int pair_count(const C8Args& a, int p) {
+__device__ __forceinline__ int pair_units(const C8Args& a, int p, int kv_len) {
   if (SPARSE) return min(max(a.kept_counts[p], 0), a.max_kept);
-  const int b = p / a.hkv;
-  const int kv = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
-  return min((max(kv, 0) + kBS - 1) / kBS, a.max_blocks);
-}
-
-// Units before pair `upto` (exclusive) summed by one wavefront; all lanes get the result.
-template <bool SPARSE>
-__device__ __forceinline__ int units_before(const C8Args& a, int upto, int lane) {
-  int acc = 0;
-  for (int base = 0; base < upto; base += 64) {
-    const int p = base + lane;
-    acc += p < upto ? pair_count<SPARSE>(a, p) : 0;
-  }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
-  return acc;
+  return min((max(kv_len, 0) + kBS - 1) / kBS, a.max_blocks);
 }
 
 // Direct global->LDS load of one 8 KiB tile: 8 instructions of 64 lanes x 16 B.  LDS
@@ -116,7 +119,11 @@ __device__ __forceinline__ DmaOffsets dma_offsets(int lane) {
   return d;
 }
 
-__device__ __forceinline__ void dma_tile(const uint8_t* gtile, u32 lds_addr, const DmaOffsets& d) {
+__device__ __forceinline__ void dma_tile(const uint8_t* gtile_in, u32 lds_addr, const DmaOffsets& d) {
+  // the tile address is wave-uniform by construction; make that explicit so it sits in SGPRs
+  const unsigned long long gp = (unsigned long long)gtile_in;
+  const u32 glo = __builtin_amdgcn_readfirstlane((u32)gp), ghi = __builtin_amdgcn_readfirstlane((u32)(gp >> 32));
+  const uint8_t* gtile = (const uint8_t*)(((unsigned long long)ghi << 32) | glo);
   u32 saved_m0;  // m0 (the LDS base of these loads) is put back as it was found
   asm volatile(
       "s_mov_b32 %[sv], m0\n\t"
@@ -240,131 +247,98 @@ __device__ __forceinline__ void load_pair(const C8Args& a, int p, int lane, Pair
   for (int i = 0; i < 8; ++i) st.o[i] = 0.f;
 }
 
-__device__ __forceinline__ void flush_pair(const C8Args& a, int slot, int lane, const PairState& st) {
-  const int n = lane & 15, g = lane >> 4;
-  float* po = a.part_o + (size_t)slot * kSlotFloats + g * kD;
-#pragma unroll
-  for (int ct = 0; ct < 8; ++ct) po[16 * ct + n] = st.o[ct];
-  const float l = row_sum16(st.l);
-  if (n == 0) {
-    a.part_ml[(size_t)slot * 8 + g] = st.m;
-    a.part_ml[(size_t)slot * 8 + 4 + g] = l;
-  }
-}
-
-// The pair that holds unit u and u's index in that pair's block list (wave-uniform).
-template <bool SPARSE>
-__device__ __forceinline__ void locate_unit(const C8Args& a, int P, int u, int lane, int& p_out, int& i_out) {
-  int p = 0, before = 0, running = 0;
-  bool found = false;
-  for (int base = 0; base < P && !found; base += 64) {
-    const int pp = base + lane;
-    const int n = pp < P ? pair_count<SPARSE>(a, pp) : 0;
-    int incl = n;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-      const int t = __shfl_up(incl, o, 64);
-      if (lane >= o) incl += t;
-    }
-    const int tot = __shfl(incl, 63, 64);
-    if (u < running + tot) {
-      const unsigned long long msk = __ballot(running + incl > u);
-      const int first = __ffsll((long long)msk) - 1;
-      p = base + first;
-      before = running + __shfl(incl - n, first, 64);
-      found = true;
-    }
-    running += tot;
-  }
-  p_out = uni(p);
-  i_out = uni(u - before);
-}
-
 template <int QUANT, bool SPARSE>
 __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
   __shared__ __attribute__((aligned(16))) uint8_t ldsK[kWaves][kTileB];
   __shared__ __attribute__((aligned(16))) uint8_t ldsV[kWaves][kTileB];
   __shared__ __attribute__((aligned(16))) uint8_t ldsP[kWaves][1024];
+  TRACE(0);
   const int lane = threadIdx.x & 63;
   const int wv = uni(threadIdx.x >> 6);
-  const int w = blockIdx.x * kWaves + wv;
+  const int ticket = blockIdx.x;
+  const int p = ticket / a.chunks_per_pair, ck = ticket - p * a.chunks_per_pair;
+  const int b = p / a.hkv, h = p - b * a.hkv;
+  const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
+  const int n_p = pair_units<SPARSE>(a, p, kv_len);
+  const int first = ck * a.chunk;
+  const int cnt = min(a.chunk, n_p - first);  // <= 0: past the end of this pair's list
+  const bool single = n_p <= a.chunk;
+  if (cnt <= 0) {
+    if (n_p == 0 && ck == 0) {  // empty sequence: its output rows are zeros
+      uint16_t* o = a.out + ((size_t)b * a.hkv * kG + h * kG + (threadIdx.x >> 6)) * kD + (threadIdx.x & 63) * 2;
+      *reinterpret_cast<u32*>(o) = 0u;
+    }
+    return;
+  }
+
   uint8_t* const kbuf = ldsK[wv];
   uint8_t* const vbuf = ldsV[wv];
   uint8_t* const pbuf = ldsP[wv];
   const u32 kaddr = uni((int)lds_addr_of(kbuf)), vaddr = uni((int)lds_addr_of(vbuf));
   const DmaOffsets offK = dma_offsets<kShiftK>(lane), offV = dma_offsets<kShiftV>(lane);
-  const int P = a.batch * a.hkv;
   const int n16 = lane & 15, g4 = lane >> 4;
 
-  // ---- this wavefront's chunk [u0, u1) of the unit sequence
-  const int U = uni(units_before<SPARSE>(a, P, lane));
-  const int C = (U + a.num_waves - 1) / a.num_waves;
-  const int u0 = w * C, u1 = min(U, u0 + C);
-  if (C == 0 || u0 >= u1) return;
+  // ---- unit table: lane j describes unit first + j (physical block, valid tokens)
+  int my_pb = 0, my_valid = 0;
+  {
+    int lb = -1, pb = -1;
+    if (lane < cnt) {
+      lb = first + lane;
+      if (SPARSE) lb = a.kept_blocks[(size_t)p * a.max_kept + lb];
+      if (lb >= 0 && lb < a.max_blocks) pb = a.block_tables[(size_t)b * a.max_blocks + lb];
+    }
+    // both loads are consumed here on every path: nothing of the table build stays in
+    // flight when the streaming loop starts
+    asm volatile("" ::"v"(lb), "v"(pb));
+    if (pb >= 0 && pb < a.num_blocks) {
+      my_pb = pb;
+      my_valid = min(max(kv_len - lb * kBS, 0), kBS);
+    }
+  }
+  TRACE(2);
 
   const size_t tile_stride = (size_t)kBS * kD;  // bytes of one (block, head) tile
-  auto tile_ptr = [&](const uint8_t* cache, int pb, int pp) {
-    return cache + ((size_t)pb * a.hkv + (pp % a.hkv)) * tile_stride;
-  };
+  const uint8_t* const kbase = a.key_cache + (size_t)h * tile_stride;
+  const uint8_t* const vbase = a.value_cache + (size_t)h * tile_stride;
+  const size_t blk_stride = (size_t)a.hkv * tile_stride;
 
   PairState st;
-  int cur_p = -1;
+  st.m = -INFINITY;
+  st.l = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) st.o[i] = 0.f;
 
-  // The chunk is walked 64 units at a time: lane j first works out unit ub + j (its pair,
-  // physical block and valid-token count) so that the streaming loop below touches no
-  // memory but the tiles themselves.
-  for (int ub = u0; ub < u1; ub += 64) {
-    const int cnt = min(64, u1 - ub);
-    int p0, i0;
-    locate_unit<SPARSE>(a, P, ub, lane, p0, i0);
-    int my_p = p0, my_pb = 0, my_valid = 0;
-    {
-      int off = i0 + lane;
-      int kv = 0, lb = -1, pb = -1;
-      if (lane < cnt) {
-        int n = pair_count<SPARSE>(a, my_p);
-        while (off >= n && my_p < P - 1) {
-          off -= n;
-          ++my_p;
-          n = pair_count<SPARSE>(a, my_p);
-        }
-        const int b = my_p / a.hkv;
-        kv = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
-        lb = off;
-        if (SPARSE) lb = a.kept_blocks[(size_t)my_p * a.max_kept + min(off, a.max_kept - 1)];
-        if (lb >= 0 && lb < a.max_blocks) pb = a.block_tables[(size_t)b * a.max_blocks + lb];
-      }
-      // every load above is consumed here, on every path: nothing of the table build is
-      // left in flight when the streaming loop starts
-      asm volatile("" ::"v"(kv), "v"(lb), "v"(pb));
-      if (pb >= 0 && pb < a.num_blocks) {
-        my_pb = pb;
-        my_valid = min(max(kv - lb * kBS, 0), kBS);
-      }
-    }
+  if (wv < cnt) {  // this wavefront has units wv, wv + 4, ...
+    int pb = __builtin_amdgcn_readlane(my_pb, wv);
+    int valid = __builtin_amdgcn_readlane(my_valid, wv);
+    dma_tile(kbase + (size_t)pb * blk_stride, kaddr, offK);
+    dma_tile(vbase + (size_t)pb * blk_stride, vaddr, offV);
+    TRACE(3);
+    load_pair<QUANT>(a, p, lane, st);
 
-    int p = __builtin_amdgcn_readlane(my_p, 0);
-    int pb = __builtin_amdgcn_readlane(my_pb, 0);
-    int valid = __builtin_amdgcn_readlane(my_valid, 0);
-    dma_tile(tile_ptr(a.key_cache, pb, p), kaddr, offK);
-    dma_tile(tile_ptr(a.value_cache, pb, p), vaddr, offV);
-    if (p != cur_p) {
-      if (cur_p >= 0) flush_pair(a, w + cur_p, lane, st);
-      load_pair<QUANT>(a, p, lane, st);
-      cur_p = p;
-    }
-
-    for (int j = 0; j < cnt; ++j) {
-      const bool has_next = j + 1 < cnt;
-      int pn = p, pbn = 0, validn = 0;
+    for (int j = wv; j < cnt; j += kWaves) {
+      const bool has_next = j + kWaves < cnt;
+      int pbn = 0, validn = 0;
       if (has_next) {
-        pn = __builtin_amdgcn_readlane(my_p, j + 1);
-        pbn = __builtin_amdgcn_readlane(my_pb, j + 1);
-        validn = __builtin_amdgcn_readlane(my_valid, j + 1);
+        pbn = __builtin_amdgcn_readlane(my_pb, j + kWaves);
+        validn = __builtin_amdgcn_readlane(my_valid, j + kWaves);
       }
 
+#ifdef FDATTN_EXP_NOCOMPUTE
+      wait_vm8();
+      st.l += (float)kbuf[lane * 4];
+      wait_lgkm0();
+      if (has_next) dma_tile(kbase + (size_t)pbn * blk_stride, kaddr, offK);
+      if (has_next) wait_vm8(); else wait_vm0();
+      st.l += (float)vbuf[lane * 4];
+      wait_lgkm0();
+      if (has_next) dma_tile(vbase + (size_t)pbn * blk_stride, vaddr, offV);
+      pb = pbn; valid = validn;
+      continue;
+#endif
       // ---------------- S = Q K^T : rows = head*4 + limb, columns = token slots
       wait_vm8();  // K(j) landed; V(j) may still be in flight
+      if (j == wv) TRACE(4);
       v4i S[4];
       v4f Sf[4];
 #pragma unroll
@@ -396,7 +370,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
         }
       }
       wait_lgkm0();  // K tile is in registers: its slot may be refilled
-      if (has_next) dma_tile(tile_ptr(a.key_cache, pbn, pn), kaddr, offK);
+      if (has_next) dma_tile(kbase + (size_t)pbn * blk_stride, kaddr, offK);
 
       // ---------------- online softmax in the S layout: lane = (token slot n, head g)
       float sv[4];
@@ -485,84 +459,115 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
         st.o[ct] = st.o[ct] * alpha + ob;
       }
       wait_lgkm0();  // V tile consumed
-      if (has_next) dma_tile(tile_ptr(a.value_cache, pbn, pn), vaddr, offV);
+      if (has_next) dma_tile(vbase + (size_t)pbn * blk_stride, vaddr, offV);
 
-      // ---------------- next unit
-      if (!has_next) break;
-      if (pn != p) {
-        flush_pair(a, w + p, lane, st);
-        load_pair<QUANT>(a, pn, lane, st);
-        cur_p = pn;
-      }
-      p = pn;
       pb = pbn;
       valid = validn;
     }
   }
-  flush_pair(a, w + cur_p, lane, st);
-}
+  TRACE(5);
 
-// One workgroup per (sequence, KV head): merges the slots wave + pair of the wavefronts
-// whose chunks overlap the pair, applies the V scale and writes bf16.
-template <bool SPARSE>
-__global__ __launch_bounds__(256) void decode_c8_combine_kernel(C8Args a) {
-  __shared__ int sh[2];
-  const int p = blockIdx.x, tid = threadIdx.x;
-  const int P = a.batch * a.hkv;
-  if (tid < 64) {
-    const int bef = units_before<SPARSE>(a, p, tid);
-    const int tot = units_before<SPARSE>(a, P, tid);
-    if (tid == 0) { sh[0] = bef; sh[1] = tot; }
+  // ---- merge the 4 wavefronts through LDS (their K slots are free now)
+  {
+    float* const mo = reinterpret_cast<float*>(kbuf);  // [4 heads][128] of this wavefront
+    float* const mml = reinterpret_cast<float*>(pbuf);  // m[4], l[4]
+    const float l = row_sum16(st.l);
+#pragma unroll
+    for (int ct = 0; ct < 8; ++ct) mo[g4 * kD + 16 * ct + n16] = st.o[ct];
+    if (n16 == 0) {
+      mml[g4] = st.m;
+      mml[4 + g4] = l;
+    }
   }
   __syncthreads();
-  const int before = sh[0], U = sh[1];
-  const int n = pair_count<SPARSE>(a, p);
-  const int b = p / a.hkv, h = p - b * a.hkv;
-  const int head = tid >> 6, c2 = (tid & 63) * 2;
-  uint16_t* o = a.out + ((size_t)b * a.hkv * kG + h * kG + head) * kD + c2;
-  if (n == 0 || U == 0) {
-    *reinterpret_cast<u32*>(o) = 0u;
-    return;
+  {
+    const int tid = threadIdx.x, head = tid >> 6, c2 = (tid & 63) * 2;
+    float M = -INFINITY;
+#pragma unroll
+    for (int w2 = 0; w2 < kWaves; ++w2) M = fmaxf(M, reinterpret_cast<const float*>(ldsP[w2])[head]);
+    float L = 0.f, o0 = 0.f, o1 = 0.f;
+    if (M > -INFINITY) {
+#pragma unroll
+      for (int w2 = 0; w2 < kWaves; ++w2) {
+        const float* ml = reinterpret_cast<const float*>(ldsP[w2]);
+        const float ms = ml[head];
+        const float f = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - M);
+        L += ml[4 + head] * f;
+        const float2 v = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(ldsK[w2]) + head * kD + c2);
+        o0 += v.x * f;
+        o1 += v.y * f;
+      }
+    }
+    if (single) {
+      // the only chunk of this pair: finish here
+      const float inv = L > 0.f ? 1.0f / L : 0.f;
+      const float r0 = o0 * inv * a.v_scale[h * kD + c2], r1 = o1 * inv * a.v_scale[h * kD + c2 + 1];
+      uint16_t* o = a.out + ((size_t)b * a.hkv * kG + h * kG + head) * kD + c2;
+      *reinterpret_cast<u32*>(o) = (u32)f32_to_bf16(r0) | ((u32)f32_to_bf16(r1) << 16);
+    } else {
+      const size_t slot = (size_t)p * a.chunks_per_pair + ck;
+      *reinterpret_cast<float2*>(a.part_o + slot * kSlotFloats + head * kD + c2) = make_float2(o0, o1);
+      if ((tid & 63) == 0) {
+        a.part_ml[slot * 8 + head] = M;
+        a.part_ml[slot * 8 + 4 + head] = L;
+      }
+    }
   }
-  const int C = (U + a.num_waves - 1) / a.num_waves;
-  const int w0 = before / C, w1 = (before + n - 1) / C;
+  TRACE(6);
+}
+
+// One workgroup per (sequence, KV head) whose list spans several chunks: merges their
+// partials, applies the V scale and writes bf16.  Single-chunk pairs were finished by the
+// main kernel.
+template <bool SPARSE>
+__global__ __launch_bounds__(256) void decode_c8_combine_kernel(C8Args a) {
+  const int p = blockIdx.x, tid = threadIdx.x;
+  const int b = p / a.hkv, h = p - b * a.hkv;
+  const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
+  const int n_p = pair_units<SPARSE>(a, p, kv_len);
+  if (n_p <= a.chunk) return;
+  const int head = tid >> 6, c2 = (tid & 63) * 2;
+  const int nch = (n_p + a.chunk - 1) / a.chunk;
+  const size_t s0 = (size_t)p * a.chunks_per_pair;
   float M = -INFINITY;
-  for (int w = w0; w <= w1; ++w) M = fmaxf(M, a.part_ml[(size_t)(w + p) * 8 + head]);
+  for (int c = 0; c < nch; ++c) M = fmaxf(M, a.part_ml[(s0 + c) * 8 + head]);
   float L = 0.f, o0 = 0.f, o1 = 0.f;
   if (M > -INFINITY) {
-    for (int w = w0; w <= w1; ++w) {
-      const size_t slot = (size_t)(w + p);
-      const float ms = a.part_ml[slot * 8 + head];
+    for (int c = 0; c < nch; ++c) {
+      const float ms = a.part_ml[(s0 + c) * 8 + head];
       if (ms == -INFINITY) continue;
-      const float f = exp2f(ms - M);
-      L += a.part_ml[slot * 8 + 4 + head] * f;
-      const float2 v = *reinterpret_cast<const float2*>(a.part_o + slot * kSlotFloats + head * kD + c2);
+      const float f = __builtin_amdgcn_exp2f(ms - M);
+      L += a.part_ml[(s0 + c) * 8 + 4 + head] * f;
+      const float2 v = *reinterpret_cast<const float2*>(a.part_o + (s0 + c) * kSlotFloats + head * kD + c2);
       o0 += v.x * f;
       o1 += v.y * f;
     }
   }
   const float inv = L > 0.f ? 1.0f / L : 0.f;
   const float r0 = o0 * inv * a.v_scale[h * kD + c2], r1 = o1 * inv * a.v_scale[h * kD + c2 + 1];
+  uint16_t* o = a.out + ((size_t)b * a.hkv * kG + h * kG + head) * kD + c2;
   *reinterpret_cast<u32*>(o) = (u32)f32_to_bf16(r0) | ((u32)f32_to_bf16(r1) << 16);
 }
 
-static int num_cus() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-      cus = n;
-    else
-      cus = 256;
-  }
-  return cus;
+#ifndef FDATTN_CHUNK
+#define FDATTN_CHUNK 24
+#endif
+
+// Units per workgroup: 24 (384 KiB of cache) keeps workgroups short enough for the
+// dispatcher to balance and long enough to amortise their start; small launches get
+// smaller chunks so that the grid still covers the GPU.
+static int pick_chunk(int pairs, int max_units) {
+  int chunk = FDATTN_CHUNK;  // at most kMaxChunk
+  while (chunk > 4 && (long long)pairs * ((max_units + chunk - 1) / chunk) < 1024) chunk /= 2;
+  return chunk;
 }
 
-constexpr int kMaxWaves = 2 * 512 * kWaves;  // workspace is sized for up to 512 CUs
+constexpr int kMaxPairs = 1 << 20;
 
-size_t c8_workspace_bytes(int batch, int hkv) {
-  const size_t slots = (size_t)kMaxWaves + (size_t)batch * hkv;
+size_t c8_workspace_bytes(int batch, int hkv, int max_units) {
+  const int pairs = batch * hkv;
+  const int chunk = pick_chunk(pairs, max_units);
+  const size_t slots = (size_t)pairs * ((max_units + chunk - 1) / chunk);
   return slots * (kSlotFloats + 8) * sizeof(float);
 }
 
@@ -578,9 +583,16 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
                      int hkv, int d, int bs, int max_blocks, int num_blocks, int quant, float sm_scale,
                      hipStream_t s, int stages) {
   (void)hq; (void)d; (void)bs;
-  int waves = 2 * num_cus() * kWaves;
-  if (waves > kMaxWaves) waves = kMaxWaves;
-  const size_t slots = (size_t)waves + (size_t)batch * hkv;
+  const bool sparse = kept_blocks != nullptr;
+  const int pairs = batch * hkv;
+  const int max_units = sparse ? (max_kept < max_blocks ? max_kept : max_blocks) : max_blocks;
+  const int chunk = pick_chunk(pairs, max_units);
+  const int cpp = ((max_units + chunk - 1) / chunk);
+  if (pairs > kMaxPairs)
+    return fail(FDATTN_ERR_SHAPE, "fdattn_decode_attention: batch*kv_heads = %d exceeds %d", pairs, kMaxPairs);
+  if ((long long)pairs * cpp > 0x7fffffffLL)
+    return fail(FDATTN_ERR_SHAPE, "fdattn_decode_attention: %d pairs x %d chunks exceed the grid limit", pairs, cpp);
+  const size_t slots = (size_t)pairs * cpp;
   const size_t need = slots * (kSlotFloats + 8) * sizeof(float);
   if (workspace_bytes < need)
     return fail(FDATTN_ERR_WORKSPACE, "fdattn_decode_attention: workspace %zu B < required %zu B", workspace_bytes, need);
@@ -588,10 +600,9 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
   float* part_ml = part_o + slots * kSlotFloats;
   C8Args a{(const uint16_t*)q, (const uint8_t*)key_cache, (const uint8_t*)value_cache, k_scale, v_scale,
            block_tables, seq_lens_decoder, seq_lens_this_time, kept_blocks, kept_counts, max_kept, part_o,
-           part_ml, (uint16_t*)out, batch, hkv, max_blocks, num_blocks, waves,
+           part_ml, (uint16_t*)out, batch, hkv, max_blocks, num_blocks, chunk, cpp,
            sm_scale * 1.4426950408889634f};
-  const dim3 grid(waves / kWaves), block(kWaves * 64);
-  const bool sparse = kept_blocks != nullptr;
+  const dim3 grid(cpp * pairs), block(kWaves * 64);
   if (!(stages & 1)) {
   } else if (quant == FDATTN_CACHE_INT8) {
     if (sparse) hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_INT8, true>), grid, block, 0, s, a);
@@ -602,9 +613,9 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
   }
   int rc = check_launch("fdattn_decode_attention (mfma)");
   if (rc || !(stages & 2)) return rc;
-  if (sparse) hipLaunchKernelGGL(decode_c8_combine_kernel<true>, dim3(batch * hkv), dim3(256), 0, s, a);
-  else hipLaunchKernelGGL(decode_c8_combine_kernel<false>, dim3(batch * hkv), dim3(256), 0, s, a);
-  return check_launch("fdattn_decode_attention (combine)");
+  if (sparse) hipLaunchKernelGGL(decode_c8_combine_kernel<true>, dim3(pairs), dim3(256), 0, s, a);
+  else hipLaunchKernelGGL(decode_c8_combine_kernel<false>, dim3(pairs), dim3(256), 0, s, a);
+  return check_launch("fdattn_decode_attention (merge)");
 }
 
 }  // namespace fdattn

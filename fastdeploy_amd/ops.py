@@ -142,9 +142,9 @@ def write_cache_kv(qkv, key_cache, value_cache, cache_k_scale, cache_v_scale, bl
     return q_out, k_out, v_out
 
 
-def decode_workspace(batch, num_heads, kv_num_heads, head_dim, device="cuda"):
+def decode_workspace(batch, num_heads, kv_num_heads, head_dim, max_blocks_per_seq, device="cuda"):
     """A workspace tensor large enough for decode_attention(_sparse) at these shapes."""
-    n = _lib.lib().fdattn_decode_workspace_bytes(batch, num_heads, kv_num_heads, head_dim)
+    n = _lib.lib().fdattn_decode_workspace_bytes(batch, num_heads, kv_num_heads, head_dim, max_blocks_per_seq)
     return torch.empty(n, dtype=torch.uint8, device=device)
 
 
@@ -174,7 +174,7 @@ def _decode_common(q, key_cache, value_cache, cache_k_scale, cache_v_scale, bloc
         out = torch.empty((batch, num_heads * d), dtype=torch.bfloat16, device=q.device)
     p_out = _chk(out, "out", torch.bfloat16)
     if workspace is None:
-        workspace = decode_workspace(batch, num_heads, hkv, d, q.device)
+        workspace = decode_workspace(batch, num_heads, hkv, d, mb, q.device)
     p_ws = _chk(workspace, "workspace", torch.uint8)
     return (p_q, p_kc, p_vc, p_ks, p_vs, p_bt, p_dec, p_tt), out, p_out, p_ws, workspace, \
         (batch, num_heads, hkv, d, bs, mb, nb)

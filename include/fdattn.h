@@ -96,9 +96,11 @@ FDATTN_API int fdattn_write_cache_kv(
 
 /*
  * Bytes of workspace fdattn_decode_attention / fdattn_decode_attention_sparse
- * need for these shapes (split-KV partial results).  Never 0.
+ * need for these shapes (split-KV partial results).  Never 0.  The workspace needs
+ * no initialisation; calls that overlap on the GPU must not share one.
  */
-FDATTN_API size_t fdattn_decode_workspace_bytes(int batch, int hq, int hkv, int head_dim);
+FDATTN_API size_t fdattn_decode_workspace_bytes(int batch, int hq, int hkv, int head_dim,
+                                                int max_blocks_per_seq);
 
 /*
  * Decode attention over the quantised paged cache: one query token per sequence,
@@ -108,8 +110,8 @@ FDATTN_API size_t fdattn_decode_workspace_bytes(int batch, int hq, int hkv, int 
  * block_tables.  Rows with kv_len 0 produce zeros.  Softmax follows the
  * max-shifted form of fastdeploy/function/softmax.cc:58-86 (without its -64 clip).
  *   q   bf16 [batch, hq*head_dim]     out bf16 [batch, hq*head_dim]
- * The split-KV partials live in `workspace` and are merged by the library
- * before the call's work on the stream ends.
+ * The split-KV partials live in `workspace` and are merged by a second, small kernel
+ * enqueued behind the first.
  */
 FDATTN_API int fdattn_decode_attention(
     const void* q, const void* key_cache, const void* value_cache,
@@ -130,9 +132,9 @@ FDATTN_API int fdattn_decode_uses_mfma(int hq, int hkv, int head_dim, int block_
 /*
  * fdattn_decode_attention split into its two kernels, for profiling and for callers
  * that overlap other work with the merge: stages = 1 runs only the split-KV kernel
- * (partials into `workspace`), 2 only the merge (workspace -> out), 3 both.  MFMA
- * shapes only (FDATTN_ERR_SHAPE otherwise).  Same plug-in position as
- * fdattn_decode_attention.
+ * (partials into `workspace`; sequences that fit one chunk are finished by it), 2 only
+ * the merge (workspace -> out), 3 both.  MFMA shapes only (FDATTN_ERR_SHAPE otherwise).
+ * Same plug-in position as fdattn_decode_attention.
  */
 FDATTN_API int fdattn_decode_attention_stages(
     const void* q, const void* key_cache, const void* value_cache,

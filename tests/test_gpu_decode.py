@@ -132,3 +132,16 @@ def test_decode_rejects_bad_arguments():
         fd.decode_attention(case["q"], case["key_cache"], case["value_cache"], case["cache_k_scale"],
                             case["cache_v_scale"], case["block_tables"], case["seq_lens_decoder"], num_heads=32,
                             workspace=torch.empty(16, dtype=torch.uint8, device="cuda"))
+
+
+def test_workspace_is_reusable_across_calls_and_shapes(oracle):
+    """One workspace serves calls of different batch sizes, lengths and cache types back to back."""
+    ws = fd.decode_workspace(12, 32, 8, 128, 64, "cuda")
+    ws.fill_(0xAB)   # the kernels must not rely on its contents
+    cases = [syn.decode_case(batch=12, ctx=[1, 2, 63, 64, 65, 127, 128, 129, 700, 0, 1000, 31], seed=5, max_blocks=20),
+             syn.decode_case(batch=3, ctx=[4000, 64 * 17, 5], seed=6, max_blocks=64),
+             syn.decode_case(batch=12, ctx=2048, seed=7, max_blocks=40, quant=CACHE_FP8)]
+    for rep in range(3):
+        for case in cases:
+            got = gpu_decode(case, workspace=ws)
+            check(got, oracle_decode(oracle, case), "reuse rep %d" % rep)
