@@ -24,6 +24,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes of one decode_c8_kernel launch on this workload, from the TCC counters
+# (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB copy: summary in
+# profiles/decode_c8_kernel_configs1_b64_ctx4k.md); it cannot be measured from inside this script.
+MEASURED_TRAFFIC_BYTES = 527_798_000 + 3_195_000
 
 
 def time_events(fn, steps, warmup):
@@ -48,6 +52,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--pools", type=int, default=2, help="distinct cache pools rotated between steps")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run a plain 1 GiB device copy, the yardstick the HBM byte counters are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the path shards by KV head or by sequence with no "
@@ -91,6 +97,14 @@ def main():
     ms_main = time_events(lambda: step("partials"), args.steps, args.warmup)
     ms_merge = time_events(lambda: step("merge"), args.steps, args.warmup)
 
+    if args.calibrate:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)       # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
+
     alg_bytes = syn.decode_algorithmic_bytes(lens, B)
     kv_bytes = syn.decode_kv_bytes(lens)
     achieved = alg_bytes / (ms_main * 1e-3) / 1e9
@@ -110,7 +124,7 @@ def main():
                       "decode_c8_combine_kernel_incl_launch": round(ms_merge * 1e3, 3)},
         "roofline": {"bound": "hbm", "kernel": "decode_c8_kernel<int8,dense>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "algorithmic_bytes": alg_bytes, "traffic": None},
+                     "algorithmic_bytes": alg_bytes, "traffic": MEASURED_TRAFFIC_BYTES},
     }
 
     if not args.no_cpu:
