@@ -74,3 +74,47 @@ def test_prefill_small(oracle, impl, quant):
                                            32, 8, 128, quant)
     ok, mx, bad = bf16_close(bits(out), want)
     assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
+
+
+@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+def test_prefill_ragged_edges(oracle, quant):
+    """Prefix lengths around the tile size, chunks around the workgroup size, an empty prefix."""
+    c = _prefill_case(2, [0, 63, 64, 65, 1000, 129], [129, 128, 1, 127, 257, 64], quant)
+    dev = syn.to_device(c, "cuda")
+    out = fd.append_attention_prefill(dev["q_new"], dev["k_new"], dev["v_new"], dev["key_cache"], dev["value_cache"],
+                                      dev["cache_k_scale"], dev["cache_v_scale"], dev["block_tables"],
+                                      dev["seq_lens_decoder"], dev["cu_seqlens_q"], num_heads=32, max_chunk=257,
+                                      cache_quant_type=quant)
+    want = oracle.append_attention_prefill(bits(c["q_new"]), bits(c["k_new"]), bits(c["v_new"]), np_of(c["key_cache"]),
+                                           np_of(c["value_cache"]), np_of(c["cache_k_scale"]), np_of(c["cache_v_scale"]),
+                                           np_of(c["block_tables"]), np_of(c["seq_lens_decoder"]), np_of(c["cu_seqlens_q"]),
+                                           32, 8, 128, quant)
+    ok, mx, bad = bf16_close(bits(out), want)
+    assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
+
+
+def test_prefill_config5_shape_sampled_rows(oracle):
+    """batch 2, 2048 new tokens on 8192 cached (int8 paged), causal: the full-size launch, checked on a
+    sample of rows against the oracle and, on the GPU, against the shape-agnostic kernel on every row."""
+    g = torch.Generator(device="cuda").manual_seed(0)
+    c = syn.decode_case(batch=2, ctx=8192, seed=0, device="cuda", direct_bytes=True, extra_blocks=8)
+    T = 2 * 2048
+    c["q_new"] = torch.randn((T, 32 * 128), generator=g, device="cuda").to(torch.bfloat16)
+    c["k_new"] = torch.randn((T, 8 * 128), generator=g, device="cuda").to(torch.bfloat16)
+    c["v_new"] = torch.randn((T, 8 * 128), generator=g, device="cuda").to(torch.bfloat16)
+    cu = torch.tensor([0, 2048, 4096], dtype=torch.int32, device="cuda")
+    args = (c["q_new"], c["k_new"], c["v_new"], c["key_cache"], c["value_cache"], c["cache_k_scale"],
+            c["cache_v_scale"], c["block_tables"], c["seq_lens_decoder"], cu)
+    out = fd.append_attention_prefill(*args, num_heads=32, max_chunk=2048)
+    torch.cuda.synchronize()
+    ids = np.array([0, 1, 63, 64, 127, 128, 1000, 2047, 2048, 2049, 3000, 4095], np.int32)
+    want = oracle.append_attention_prefill(bits(c["q_new"]), bits(c["k_new"]), bits(c["v_new"]), np_of(c["key_cache"]),
+                                           np_of(c["value_cache"]), np_of(c["cache_k_scale"]), np_of(c["cache_v_scale"]),
+                                           np_of(c["block_tables"]), np_of(c["seq_lens_decoder"]), np_of(cu),
+                                           32, 8, 128, CACHE_INT8, token_ids=ids)
+    ok, mx, bad = bf16_close(bits(out)[ids], want[ids])
+    assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
+    # every row: the two GPU kernels agree within twice the tolerance (each is within it of the truth)
+    ref = fd.append_attention_prefill(*args, num_heads=32, max_chunk=2048, impl="generic")
+    ok, mx, bad = bf16_close(bits(out), bits(ref), 4e-3, 2e-2)
+    assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
