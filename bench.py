@@ -45,6 +45,83 @@ def time_events(fn, steps, warmup):
     return e0.elapsed_time(e1) / steps
 
 
+def other_workloads(args):
+    """The rows of the path that are not the headline metric (configs[2], [3], [4]): one JSON line each
+    with the kernel time and its roofline fraction.  Not part of the default run."""
+    import fastdeploy_amd as fd
+    from fastdeploy_amd import synthetic as syn
+    dev = "cuda:0"
+    res = []
+    g = torch.Generator(device=dev).manual_seed(0)
+
+    def line(name, ms, bound, work, peak, unit, extra=None):
+        ach = work / (ms * 1e-3) / (1e9 if unit == "GB/s" else 1e12)
+        d = {"workload": name, "us": round(ms * 1e3, 2),
+             "roofline": {"bound": bound, "achieved": round(ach, 1), "peak": peak, "unit": unit, "frac": round(ach / peak, 4)}}
+        if extra:
+            d.update(extra)
+        print(json.dumps(d))
+        res.append(d)
+
+    if args.workload in ("write_decode", "all"):
+        # configs[2]: 256 new tokens, positions U{0..8191}, RoPE theta 500000, int8 write, then decode over ctx = pos + 1
+        c = syn.write_case(num_seqs=256, max_pos=8192, seed=0, device=dev, blocks_per_seq=128)
+        rot = (c["rope_cos"], c["rope_sin"])
+        ws = fd.decode_workspace(256, 32, 8, 128, 128, dev)
+
+        def wr():
+            return fd.write_cache_kv(c["qkv"], c["key_cache"], c["value_cache"], c["cache_k_scale"], c["cache_v_scale"],
+                                     c["block_tables"], c["seq_lens_encoder"], c["seq_lens_decoder"], c["seq_lens_this_time"],
+                                     c["cu_seqlens_q"], rot, num_heads=32, kv_num_heads=8)
+        q = wr()[0]
+        ms = time_events(wr, args.steps, args.warmup)
+        line("configs[2] cache write (256 tokens, RoPE + int8)", ms, "hbm", 256 * (48 * 128 * 2 + 2 * 8 * 128 + 32 * 128 * 2),
+             HBM_PEAK_GBPS, "GB/s", {"note": "5.8 MB of traffic: launch-bound"})
+        lens = (c["seq_lens_decoder"] + 1).tolist()
+
+        def dec():
+            fd.decode_attention(q, c["key_cache"], c["value_cache"], c["cache_k_scale"], c["cache_v_scale"],
+                                c["block_tables"], c["seq_lens_decoder"], c["seq_lens_this_time"], num_heads=32, workspace=ws)
+        ms = time_events(dec, args.steps, args.warmup)
+        line("configs[2] decode (batch 256, ctx = pos+1, mean 4k)", ms, "hbm", syn.decode_algorithmic_bytes(lens, 256),
+             HBM_PEAK_GBPS, "GB/s")
+
+    if args.workload in ("sqattn", "all"):
+        # configs[3]: batch 16, ctx 32768, fp8 KV, top-64 of 512 blocks per KV head
+        c = syn.decode_case(batch=16, ctx=32768, quant=2, seed=0, device=dev, direct_bytes=True)
+        sel = lambda: fd.sqattn_select(c["q"], c["key_cache"], c["cache_k_scale"], c["block_tables"], c["seq_lens_decoder"],
+                                       num_heads=32, top_k=64, cache_quant_type="cache_fp8")
+        kept, cnt = sel()
+        ms = time_events(sel, max(args.steps // 10, 5), 2)
+        line("configs[3] SQAttn selector (scores + top-64 of 512)", ms, "hbm", 16 * 32768 * 8 * 128, HBM_PEAK_GBPS, "GB/s")
+        ws = fd.decode_workspace(16, 32, 8, 128, 512, dev)
+        sp = lambda: fd.decode_attention_sparse(c["q"], c["key_cache"], c["value_cache"], c["cache_k_scale"], c["cache_v_scale"],
+                                                c["block_tables"], c["seq_lens_decoder"], kept_blocks=kept, kept_counts=cnt,
+                                                num_heads=32, cache_quant_type="cache_fp8", workspace=ws)
+        ms = time_events(sp, args.steps, args.warmup)
+        line("configs[3] sparse decode (64 of 512 blocks)", ms, "hbm", 16 * 8 * 64 * 64 * 128 * 2, HBM_PEAK_GBPS, "GB/s")
+        de = lambda: fd.decode_attention(c["q"], c["key_cache"], c["value_cache"], c["cache_k_scale"], c["cache_v_scale"],
+                                         c["block_tables"], c["seq_lens_decoder"], num_heads=32, cache_quant_type="cache_fp8", workspace=ws)
+        ms = time_events(de, max(args.steps // 4, 5), 3)
+        line("configs[3] dense fp8 decode, for comparison", ms, "hbm", 16 * 32768 * 8 * 128 * 2, HBM_PEAK_GBPS, "GB/s")
+
+    if args.workload in ("prefill", "all"):
+        # configs[4]: batch 2, 2048 new tokens on 8192 cached (int8 paged), causal
+        c = syn.decode_case(batch=2, ctx=8192, seed=0, device=dev, direct_bytes=True, extra_blocks=8)
+        T = 4096
+        q = torch.randn((T, 4096), generator=g, device=dev).to(torch.bfloat16)
+        k = torch.randn((T, 1024), generator=g, device=dev).to(torch.bfloat16)
+        v = torch.randn((T, 1024), generator=g, device=dev).to(torch.bfloat16)
+        cu = torch.tensor([0, 2048, 4096], dtype=torch.int32, device=dev)
+        out = torch.empty_like(q)
+        pf = lambda: fd.append_attention_prefill(q, k, v, c["key_cache"], c["value_cache"], c["cache_k_scale"], c["cache_v_scale"],
+                                                 c["block_tables"], c["seq_lens_decoder"], cu, num_heads=32, max_chunk=2048, out=out)
+        ms = time_events(pf, max(args.steps // 10, 5), 3)
+        line("configs[4] append attention (2 x 2048 new on 8192 cached)", ms, "mfma", 2 * syn.prefill_flops(8192, 2048),
+             2500.0, "TFLOP/s")
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -52,6 +129,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--pools", type=int, default=2, help="distinct cache pools rotated between steps")
+    ap.add_argument("--workload", default="decode", choices=["decode", "write_decode", "sqattn", "prefill", "all"],
+                    help="decode = the headline metric (default); the others print one line per kernel of that row")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain 1 GiB device copy, the yardstick the HBM byte counters are scaled by")
     args = ap.parse_args()
@@ -66,6 +145,9 @@ def main():
         sys.exit("bench.py: no GPU visible")
     dev = "cuda:0"
     torch.cuda.set_device(0)
+    if args.workload != "decode":
+        other_workloads(args)
+        return
     B = 64
     # distinct pools so that consecutive steps do not re-read the same bytes out of the
     # last-level cache; every pool has its own block table permutation and contents

@@ -22,6 +22,7 @@ SIGNATURES = {
     "fdattn_splitkv_combine": (_i, [_vp] * 5 + [_i] * 3 + [_vp]),
     "fdattn_sqattn_workspace_bytes": (_sz, [_i] * 3),
     "fdattn_sqattn_select": (_i, [_vp] * 10 + [_sz] + [_i] * 9 + [_vp]),
+    "fdattn_sqattn_select_exact": (_i, [_vp] * 10 + [_sz] + [_i] * 9 + [_vp]),
     "fdattn_append_attention_prefill": (_i, [_vp] * 11 + [_i] * 10 + [_f, _vp]),
     "fdattn_append_attention_prefill_generic": (_i, [_vp] * 11 + [_i] * 10 + [_f, _vp]),
 }

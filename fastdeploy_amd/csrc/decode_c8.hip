@@ -31,19 +31,13 @@
 // (the last workgroup to arrive at a pair combines it: the device-scope stores, the atomic
 // and the barrier sit at the end of every workgroup, where nothing hides their latency),
 // and handing chunks out through an atomic ticket counter instead of the block index.
-#include "fdattn_common.h"
+#include "c8_common.h"
 
 #ifndef TRACE
 #define TRACE(slot)  // timestamp hook of the perf harness; nothing in the library
 #endif
 
 namespace fdattn {
-
-constexpr int kWaves = 4;      // wavefronts per workgroup
-constexpr int kTileB = 8192;   // bytes of one K or V tile (64 tokens x 128 channels)
-constexpr int kD = 128, kG = 4, kBS = 64;
-constexpr int kSlotFloats = kG * kD;  // partial o per slot
-constexpr int kMaxChunk = 64;         // units per chunk: one unit-table entry per lane
 
 struct C8Args {
   const uint16_t* q;
@@ -66,185 +60,11 @@ struct C8Args {
   float sm_scale_log2;  // softmax_scale * log2(e)
 };
 
-__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
-
-template <int CTRL>
-__device__ __forceinline__ float dpp_f(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
-}
-// all-reduce within each 16-lane row (row_ror 8, 4, 2, 1)
-__device__ __forceinline__ float row_max16(float v) {
-  v = fmaxf(v, dpp_f<0x128>(v));
-  v = fmaxf(v, dpp_f<0x124>(v));
-  v = fmaxf(v, dpp_f<0x122>(v));
-  v = fmaxf(v, dpp_f<0x121>(v));
-  return v;
-}
-__device__ __forceinline__ float row_sum16(float v) {
-  v += dpp_f<0x128>(v);
-  v += dpp_f<0x124>(v);
-  v += dpp_f<0x122>(v);
-  v += dpp_f<0x121>(v);
-  return v;
-}
-
 // Length of the pair's block list: every block of the sequence, or the kept ones.
 template <bool SPARSE>
 __device__ __forceinline__ int pair_units(const C8Args& a, int p, int kv_len) {
   if (SPARSE) return min(max(a.kept_counts[p], 0), a.max_kept);
   return min((max(kv_len, 0) + kBS - 1) / kBS, a.max_blocks);
-}
-
-// Direct global->LDS load of one 8 KiB tile: 8 instructions of 64 lanes x 16 B.  LDS
-// receives lane l of instruction i at byte i*1024 + l*16 (row 8i + l/8, position l%8);
-// the lane fetches the 16-byte chunk (l%8) ^ f(row) of that row, so that row r's chunk c
-// sits at position c ^ f(r).  f = (r >> SHIFT) & 7 spreads the later LDS reads over banks.
-// The eight per-lane byte offsets depend on the lane only and are computed once.
-//
-// Written as inline assembly on purpose: the wavefront tracks its own loads with
-// explicit s_waitcnt vmcnt(N) (N = tile loads issued after the one waited for), which
-// stays correct whatever other memory operations the compiler interleaves, because
-// loads return in order and younger operations only make the wait stricter.
-struct DmaOffsets { u32 o[8]; };
-
-template <int SHIFT>
-__device__ __forceinline__ DmaOffsets dma_offsets(int lane) {
-  DmaOffsets d;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int row = 8 * i + (lane >> 3);
-    const int c = (lane & 7) ^ ((row >> SHIFT) & 7);
-    d.o[i] = (u32)(row * 128 + c * 16);
-  }
-  return d;
-}
-
-__device__ __forceinline__ void dma_tile(const uint8_t* gtile_in, u32 lds_addr, const DmaOffsets& d) {
-  // the tile address is wave-uniform by construction; make that explicit so it sits in SGPRs
-  const unsigned long long gp = (unsigned long long)gtile_in;
-  const u32 glo = __builtin_amdgcn_readfirstlane((u32)gp), ghi = __builtin_amdgcn_readfirstlane((u32)(gp >> 32));
-  const uint8_t* gtile = (const uint8_t*)(((unsigned long long)ghi << 32) | glo);
-  u32 saved_m0;  // m0 (the LDS base of these loads) is put back as it was found
-  asm volatile(
-      "s_mov_b32 %[sv], m0\n\t"
-      "s_mov_b32 m0, %[l]\n\ts_nop 0\n\t"
-      "global_load_lds_dwordx4 %[o0], %[g]\n\t"
-      "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
-      "global_load_lds_dwordx4 %[o1], %[g]\n\t"
-      "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
-      "global_load_lds_dwordx4 %[o2], %[g]\n\t"
-      "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
-      "global_load_lds_dwordx4 %[o3], %[g]\n\t"
-      "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
-      "global_load_lds_dwordx4 %[o4], %[g]\n\t"
-      "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
-      "global_load_lds_dwordx4 %[o5], %[g]\n\t"
-      "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
-      "global_load_lds_dwordx4 %[o6], %[g]\n\t"
-      "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
-      "global_load_lds_dwordx4 %[o7], %[g]\n\t"
-      "s_mov_b32 m0, %[sv]\n\t"
-      : [sv] "=&s"(saved_m0)
-      : [l] "s"(lds_addr), [g] "s"(gtile), [o0] "v"(d.o[0]), [o1] "v"(d.o[1]), [o2] "v"(d.o[2]),
-        [o3] "v"(d.o[3]), [o4] "v"(d.o[4]), [o5] "v"(d.o[5]), [o6] "v"(d.o[6]), [o7] "v"(d.o[7])
-      : "memory", "scc");
-}
-
-__device__ __forceinline__ u32 lds_addr_of(const void* p) {
-  return (u32)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
-}
-
-__device__ __forceinline__ void wait_vm8() { asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); }
-__device__ __forceinline__ void wait_vm0() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-__device__ __forceinline__ void wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
-__device__ __forceinline__ void wave_sync() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
-constexpr int kShiftK = 2, kShiftV = 1;
-
-// Per-pair state of a wavefront.
-struct PairState {
-  v4i aq[2];  // Q limbs as the MFMA A operand, two k-steps of 64 channels
-  float rs;   // logit scale of this lane's head (S layout: head = lane / 16)
-  float m, l;
-  float o[8];  // channel 16*ct + lane%16 of head lane/16
-};
-
-// A operand rows: row = head*4 + limb; lane (m = lane%16, g = lane/16) holds channels
-// 16*(g + 4s) .. +15 of k-step s.
-template <int QUANT>
-__device__ __forceinline__ void load_pair(const C8Args& a, int p, int lane, PairState& st) {
-  const int b = p / a.hkv, h = p - b * a.hkv;
-  const int m = lane & 15, g = lane >> 4, head = m >> 2, limb = m & 3;
-  const uint16_t* qrow = a.q + ((size_t)b * a.hkv * kG + h * kG + head) * kD;
-  const float* ks = a.k_scale + (size_t)h * kD;
-  float qs[2][16];
-  float amax = 0.f;
-#pragma unroll
-  for (int s = 0; s < 2; ++s) {
-    const int c0 = 16 * (g + 4 * s);
-    const uint4 w0 = *reinterpret_cast<const uint4*>(qrow + c0);
-    const uint4 w1 = *reinterpret_cast<const uint4*>(qrow + c0 + 8);
-    const u32 w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      qs[s][2 * j] = bf16lo_to_f32(w[j]) * ks[c0 + 2 * j];
-      qs[s][2 * j + 1] = bf16hi_to_f32(w[j]) * ks[c0 + 2 * j + 1];
-      amax = fmaxf(amax, fmaxf(fabsf(qs[s][2 * j]), fabsf(qs[s][2 * j + 1])));
-    }
-  }
-  amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-  amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
-  float rsval;
-  if (QUANT == FDATTN_CACHE_INT8) {
-    const float inv = amax > 0.f ? 1048575.0f / amax : 0.f;
-    rsval = amax * (1.0f / 1048575.0f) * a.sm_scale_log2;
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      u32 pk[4] = {0, 0, 0, 0};
-#pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        const int X = (int)__builtin_rintf(qs[s][j] * inv);
-        const int x0 = ((X + 64) & 127) - 64;
-        const int X1 = (X - x0) >> 7;
-        const int x1 = ((X1 + 64) & 127) - 64;
-        const int x2 = (X1 - x1) >> 7;
-        const int d = limb == 0 ? x0 : (limb == 1 ? x1 : (limb == 2 ? x2 : 0));
-        pk[j >> 2] |= ((u32)d & 0xffu) << (8 * (j & 3));
-      }
-      st.aq[s] = (v4i){(int)pk[0], (int)pk[1], (int)pk[2], (int)pk[3]};
-    }
-  } else {
-    // residual e4m3 limbs of x = qs * 256 / amax: limb0 = fp8(x), limb1 = fp8(x - limb0), ...
-    const float inv = amax > 0.f ? 256.0f / amax : 0.f;
-    rsval = amax * (1.0f / 256.0f) * a.sm_scale_log2;
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      u32 pk[4] = {0, 0, 0, 0};
-#pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        float x = qs[s][j] * inv;
-        u32 code = 0;
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const u32 c = (u32)__builtin_amdgcn_cvt_pk_fp8_f32(x, x, 0, false) & 0xffu;
-          if (t == limb) code = c;
-          x -= __builtin_amdgcn_cvt_f32_fp8((int)c, 0);
-        }
-        pk[j >> 2] |= code << (8 * (j & 3));
-      }
-      st.aq[s] = (v4i){(int)pk[0], (int)pk[1], (int)pk[2], (int)pk[3]};
-    }
-  }
-  // lane 4*head' (g = 0, limb 0) knows head'’s scale; the S layout wants head = lane / 16
-  st.rs = __shfl(rsval, 4 * (lane >> 4), 64);
-  st.m = -INFINITY;
-  st.l = 0.f;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) st.o[i] = 0.f;
 }
 
 template <int QUANT, bool SPARSE>
@@ -314,7 +134,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
     dma_tile(kbase + (size_t)pb * blk_stride, kaddr, offK);
     dma_tile(vbase + (size_t)pb * blk_stride, vaddr, offV);
     TRACE(3);
-    load_pair<QUANT>(a, p, lane, st);
+    load_pair<QUANT>(a.q, a.k_scale, a.hkv, a.sm_scale_log2, p, lane, st);
 
     for (int j = wv; j < cnt; j += kWaves) {
       const bool has_next = j + kWaves < cnt;

@@ -1,11 +1,21 @@
 // SQAttn block selector: per-block max q.k scores over the quantised K pages and a
 // per-(sequence, KV head) top-k with ties to the lower block index.
 //
-// Scores are computed in fp64 with the channels summed in ascending order, one
-// token per lane.  Every product (fp32 q*scale times an int8 / e4m3 value) is exact
-// in fp64, so only the order of the additions matters for the bits of the result,
-// and that order is fixed: the selection is reproducible bit for bit on a CPU.
-#include "fdattn_common.h"
+// The selection is DEFINED on scores computed in fp64 with the channels summed in
+// ascending order.  Every product (fp32 q*scale times an int8 / e4m3 value) is exact in
+// fp64, so only the order of the additions matters for the bits of a score, and that
+// order is fixed: the kept indices are reproducible bit for bit on a CPU.
+//
+// Two implementations give the same indices:
+//  * exact: every block scored in fp64, one token per lane (any shape; fp64-VALU bound);
+//  * fast (head_dim 128, 4 query heads per KV head, block_size 64): every block scored on
+//    the MFMA units straight from the cache bytes (the streaming machinery of the decode
+//    kernel, K tiles only - HBM bound), together with a bound eps on the error of those
+//    scores.  The top-k kernel then classifies each block as surely kept (fewer than k
+//    blocks could beat it even if every score were off by eps), surely dropped (k blocks
+//    beat it whatever the errors are) or undecided; only the undecided blocks - those
+//    within 2*eps of the k-th score, a handful - are re-scored in fp64 and ranked exactly.
+#include "c8_common.h"
 
 namespace fdattn {
 
@@ -136,6 +146,249 @@ __global__ __launch_bounds__(256) void sqattn_topk_kernel(const double* __restri
   if (tid == 0) kept_counts[blockIdx.x] = k;
 }
 
+// ---------------------------------------------------------------- fast path
+
+struct SelArgs {
+  const uint16_t* q;
+  const uint8_t* key_cache;
+  const float* k_scale;
+  const int32_t* block_tables;
+  const int32_t* seq_lens_decoder;
+  const int32_t* seq_lens_this_time;
+  float* approx;  // [pairs][max_blocks]
+  float* eps;     // [pairs]
+  float* scores_out;  // optional copy of approx
+  int32_t* kept_blocks;
+  int32_t* kept_counts;
+  int batch, hkv, max_blocks, num_blocks, chunk, chunks_per_pair, top_k;
+};
+
+// One workgroup = `chunk` consecutive blocks of one (sequence, KV head); each wavefront
+// streams blocks wave, wave+4, ... through two LDS slots (one tile computing, one or two
+// in flight) and leaves one fp32 score per block.
+template <int QUANT>
+__global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelArgs a) {
+  __shared__ __attribute__((aligned(16))) uint8_t ldsA[kWaves][kTileB];
+  __shared__ __attribute__((aligned(16))) uint8_t ldsB[kWaves][kTileB];
+  const int lane = threadIdx.x & 63;
+  const int wv = uni(threadIdx.x >> 6);
+  const int p = blockIdx.x / a.chunks_per_pair, ck = blockIdx.x - p * a.chunks_per_pair;
+  const int b = p / a.hkv, h = p - b * a.hkv;
+  const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
+  const int n_p = min((max(kv_len, 0) + kBS - 1) / kBS, a.max_blocks);
+  const int first = ck * a.chunk;
+  const int cnt = min(a.chunk, n_p - first);
+  float* const srow = a.approx + (size_t)p * a.max_blocks;
+  // blocks of this chunk past the sequence: -inf
+  for (int j = max(first, n_p) + (int)threadIdx.x; j < min(first + a.chunk, a.max_blocks); j += blockDim.x) {
+    srow[j] = -INFINITY;
+    if (a.scores_out) a.scores_out[(size_t)p * a.max_blocks + j] = -INFINITY;
+  }
+  if (cnt <= 0) return;
+
+  if (ck == 0 && wv == 0) {
+    // error bound of the MFMA scores of this pair (see the top of the file): q*scale is cut to
+    // 21 bits (int8) or 16 significant bits in e4m3 limbs (fp8), and sums are kept in fp32
+    float amax = 0.f, sabs = 0.f;
+    for (int g = 0; g < kG; ++g) {
+      float sa = 0.f, am = 0.f;
+      for (int c = lane; c < kD; c += 64) {
+        const float qs = fabsf(bf16_to_f32(a.q[((size_t)b * a.hkv * kG + h * kG + g) * kD + c]) * a.k_scale[h * kD + c]);
+        sa += qs;
+        am = fmaxf(am, qs);
+      }
+      sabs = fmaxf(sabs, wave_sum(sa));
+      amax = fmaxf(amax, wave_max(am));
+    }
+    float e;
+    if (QUANT == FDATTN_CACHE_INT8) e = amax * (128.0f * 127.0f / 2097150.0f) + sabs * 127.0f * 9.5367431640625e-7f;
+    else e = sabs * 448.0f * 4.8828125e-4f;  // 2^-11
+    if (lane == 0) a.eps[p] = e * 1.0001f;
+  }
+
+  uint8_t* const slot[2] = {ldsA[wv], ldsB[wv]};
+  const u32 saddr[2] = {(u32)uni((int)lds_addr_of(slot[0])), (u32)uni((int)lds_addr_of(slot[1]))};
+  const DmaOffsets offK = dma_offsets<kShiftK>(lane);
+  const int n16 = lane & 15, g4 = lane >> 4;
+
+  int my_pb = 0, my_valid = 0;
+  {
+    int pb = -1;
+    if (lane < cnt) pb = a.block_tables[(size_t)b * a.max_blocks + first + lane];
+    asm volatile("" ::"v"(pb));
+    if (pb >= 0 && pb < a.num_blocks) {
+      my_pb = pb;
+      my_valid = min(max(kv_len - (first + lane) * kBS, 0), kBS);
+    }
+  }
+  if (wv >= cnt) return;
+  const size_t tile_stride = (size_t)kBS * kD;
+  const uint8_t* const kbase = a.key_cache + (size_t)h * tile_stride;
+  const size_t blk_stride = (size_t)a.hkv * tile_stride;
+
+  dma_tile(kbase + (size_t)__builtin_amdgcn_readlane(my_pb, wv) * blk_stride, saddr[0], offK);
+  if (wv + kWaves < cnt)
+    dma_tile(kbase + (size_t)__builtin_amdgcn_readlane(my_pb, wv + kWaves) * blk_stride, saddr[1], offK);
+  PairState st;
+  load_pair<QUANT>(a.q, a.k_scale, a.hkv, 1.0f, p, lane, st);  // scores in natural units
+
+  int it = 0;
+  for (int j = wv; j < cnt; j += kWaves, ++it) {
+    const int valid = __builtin_amdgcn_readlane(my_valid, j);
+    const uint8_t* kbuf = slot[it & 1];
+    if (j + kWaves < cnt) wait_vm8(); else wait_vm0();
+    float sv = -INFINITY;
+#pragma unroll
+    for (int stl = 0; stl < 4; ++stl) {
+      const int tok = 4 * n16 + stl;
+      float s;
+      if (QUANT == FDATTN_CACHE_INT8) {
+        v4i acc = {0, 0, 0, 0};
+#pragma unroll
+        for (int k2 = 0; k2 < 2; ++k2) {
+          const int c = g4 + 4 * k2;
+          const v4i kb = *reinterpret_cast<const v4i*>(kbuf + tok * 128 + ((c ^ ((tok >> kShiftK) & 7)) * 16));
+          acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(st.aq[k2], kb, acc, 0, 0, 0);
+        }
+        s = st.rs * ((float)acc.x + 128.0f * (float)acc.y + 16384.0f * (float)acc.z);
+      } else {
+        v4f acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int k2 = 0; k2 < 2; ++k2) {
+          const int c = g4 + 4 * k2;
+          const v4i kb = *reinterpret_cast<const v4i*>(kbuf + tok * 128 + ((c ^ ((tok >> kShiftK) & 7)) * 16));
+          const long a0 = ((long)(u32)st.aq[k2].y << 32) | (u32)st.aq[k2].x;
+          const long a1 = ((long)(u32)st.aq[k2].w << 32) | (u32)st.aq[k2].z;
+          const long b0 = ((long)(u32)kb.y << 32) | (u32)kb.x;
+          const long b1 = ((long)(u32)kb.w << 32) | (u32)kb.z;
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a0, b0, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a1, b1, acc, 0, 0, 0);
+        }
+        s = st.rs * ((acc.x + acc.y) + (acc.z + acc.w));
+      }
+      sv = fmaxf(sv, tok < valid ? s : -INFINITY);
+    }
+    wait_lgkm0();  // tile consumed: refill its slot with the block two steps ahead
+    if (j + 2 * kWaves < cnt)
+      dma_tile(kbase + (size_t)__builtin_amdgcn_readlane(my_pb, j + 2 * kWaves) * blk_stride, saddr[it & 1], offK);
+    sv = row_max16(sv);                          // over the tokens of this head
+    sv = fmaxf(sv, __shfl_xor(sv, 16, 64));      // over the 4 heads of the group
+    sv = fmaxf(sv, __shfl_xor(sv, 32, 64));
+    if (lane == 0) {
+      srow[first + j] = sv;
+      if (a.scores_out) a.scores_out[(size_t)p * a.max_blocks + first + j] = sv;
+    }
+  }
+}
+
+// One workgroup per (sequence, KV head): classify, re-score the undecided blocks in fp64, emit.
+template <int QUANT>
+__global__ __launch_bounds__(256) void sqattn_resolve_kernel(SelArgs a) {
+  extern __shared__ double smd[];                  // exact scores of undecided blocks [max_blocks]
+  float* sf = reinterpret_cast<float*>(smd + a.max_blocks);      // approx scores [max_blocks]
+  int* state = reinterpret_cast<int*>(sf + a.max_blocks);         // 0 dropped, 1 kept, 2 undecided -> list index
+  int* ulist = state + a.max_blocks;                              // undecided block ids
+  __shared__ float qs[kG][kD];
+  __shared__ int n_in, n_unc, wave_tot[4], running;
+  const int p = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int b = p / a.hkv, h = p - b * a.hkv;
+  const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
+  const int nblk = min((max(kv_len, 0) + kBS - 1) / kBS, a.max_blocks);
+  const int k = min(a.top_k, nblk);
+  int32_t* out = a.kept_blocks + (size_t)p * a.top_k;
+  if (tid == 0) { n_in = 0; n_unc = 0; running = 0; }
+  const float* s = a.approx + (size_t)p * a.max_blocks;
+  for (int j = tid; j < nblk; j += 256) sf[j] = s[j];
+  __syncthreads();
+  if (k < nblk) {
+    const float eps = a.eps[p];
+    for (int j = tid; j < nblk; j += 256) {
+      const float lo = sf[j] - eps, hi = sf[j] + eps;
+      int sure_better = 0, maybe_better = 0;
+      for (int i = 0; i < nblk; ++i) {
+        const float si = sf[i];
+        sure_better += (si - eps > hi);
+        maybe_better += (i != j) && (si + eps >= lo);
+      }
+      int stt = 2;
+      if (maybe_better < k) stt = 1;
+      else if (sure_better >= k) stt = 0;
+      state[j] = stt;
+      if (stt == 1) atomicAdd(&n_in, 1);
+      if (stt == 2) ulist[atomicAdd(&n_unc, 1)] = j;
+    }
+    __syncthreads();
+    const int nu = n_unc, need = k - n_in;
+    if (nu > 0) {
+      for (int i = tid; i < kG * kD; i += 256) {
+        const int g = i / kD, c = i % kD;
+        qs[g][c] = __fmul_rn(bf16_to_f32(a.q[((size_t)b * a.hkv * kG + h * kG + g) * kD + c]), a.k_scale[h * kD + c]);
+      }
+      __syncthreads();
+      // exact score of each undecided block: fp64, channels in ascending order, lane = token
+      for (int u = wv; u < nu; u += 4) {
+        const int j = ulist[u];
+        const int pb = a.block_tables[(size_t)b * a.max_blocks + j];
+        double best = -INFINITY;
+        if (pb >= 0 && pb < a.num_blocks && j * kBS + lane < kv_len) {
+          const uint8_t* kr = a.key_cache + (((size_t)pb * a.hkv + h) * kBS + lane) * kD;
+          double acc[kG] = {0.0, 0.0, 0.0, 0.0};
+          for (int c = 0; c < kD; c += 4) {
+            const u32 w = *reinterpret_cast<const u32*>(kr + c);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const double kv = dq64<QUANT>((w >> (8 * e)) & 0xff);
+#pragma unroll
+              for (int g = 0; g < kG; ++g) acc[g] = __dadd_rn(acc[g], __dmul_rn((double)qs[g][c + e], kv));
+            }
+          }
+          best = fmax(fmax(acc[0], acc[1]), fmax(acc[2], acc[3]));
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) best = fmax(best, __shfl_xor(best, off, 64));
+        if (lane == 0) smd[u] = best;
+      }
+      __syncthreads();
+      // the `need` best undecided blocks: exact score descending, block index ascending
+      for (int u = tid; u < nu; u += 256) {
+        const double su = smd[u];
+        const int ju = ulist[u];
+        int rank = 0;
+        for (int i = 0; i < nu; ++i) {
+          const double si = smd[i];
+          rank += (si > su) || (si == su && ulist[i] < ju);
+        }
+        state[ju] = rank < need ? 1 : 0;
+      }
+      __syncthreads();
+    }
+  } else {
+    for (int j = tid; j < nblk; j += 256) state[j] = 1;
+    __syncthreads();
+  }
+  // ordered compaction of the kept blocks
+  for (int base = 0; base < nblk; base += 256) {
+    const int j = base + tid;
+    const int f = j < nblk ? (state[j] == 1) : 0;
+    const unsigned long long bal = __ballot(f);
+    const int before = __popcll(bal & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_tot[wv] = __popcll(bal);
+    __syncthreads();
+    int off = running;
+    for (int ww = 0; ww < wv; ++ww) off += wave_tot[ww];
+    if (f && off + before < a.top_k) out[off + before] = j;
+    __syncthreads();
+    if (tid == 0) running += wave_tot[0] + wave_tot[1] + wave_tot[2] + wave_tot[3];
+    __syncthreads();
+  }
+  for (int j = k + tid; j < a.top_k; j += 256) out[j] = -1;
+  if (tid == 0) a.kept_counts[p] = k;
+}
+
+static bool sel_fast_supported(int hq, int hkv, int d, int bs, int max_blocks) {
+  return d == kD && hq == kG * hkv && bs == kBS && max_blocks <= 2048;  // 20 B of LDS per block in the top-k kernel
+}
+
 }  // namespace fdattn
 
 using namespace fdattn;
@@ -146,7 +399,7 @@ extern "C" size_t fdattn_sqattn_workspace_bytes(int batch, int hkv, int max_bloc
   return (n + 255) & ~(size_t)255;
 }
 
-extern "C" int fdattn_sqattn_select(const void* q, const void* key_cache, const float* cache_k_scale,
+static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_cache, const float* cache_k_scale,
                                     const int32_t* block_tables, const int32_t* seq_lens_decoder,
                                     const int32_t* seq_lens_this_time, float* scores, int32_t* kept_blocks,
                                     int32_t* kept_counts, void* workspace, size_t workspace_bytes, int batch,
@@ -168,6 +421,26 @@ extern "C" int fdattn_sqattn_select(const void* q, const void* key_cache, const 
   if (workspace_bytes < need)
     return fail(FDATTN_ERR_WORKSPACE, "fdattn_sqattn_select: workspace %zu B < required %zu B", workspace_bytes, need);
   hipStream_t s = (hipStream_t)stream;
+  if (allow_fast && sel_fast_supported(hq, hkv, head_dim, block_size, max_blocks_per_seq)) {
+    const int pairs = batch * hkv;
+    int chunk = 32;
+    while (chunk > 4 && (long long)pairs * ((max_blocks_per_seq + chunk - 1) / chunk) < 1024) chunk /= 2;
+    const int cpp = (max_blocks_per_seq + chunk - 1) / chunk;
+    float* approx = (float*)workspace;
+    float* eps = approx + (size_t)pairs * max_blocks_per_seq;  // fits: the workspace holds 8 bytes per block
+    SelArgs sa{(const uint16_t*)q, (const uint8_t*)key_cache, cache_k_scale, block_tables, seq_lens_decoder,
+               seq_lens_this_time, approx, eps, scores, kept_blocks, kept_counts, batch, hkv,
+               max_blocks_per_seq, num_blocks, chunk, cpp, top_k};
+    const size_t shm2 = (size_t)max_blocks_per_seq * (sizeof(double) + sizeof(float) + 2 * sizeof(int));
+    if (cache_quant_type == FDATTN_CACHE_INT8) {
+      hipLaunchKernelGGL(sqattn_scores_mfma_kernel<FDATTN_CACHE_INT8>, dim3(pairs * cpp), dim3(256), 0, s, sa);
+      hipLaunchKernelGGL(sqattn_resolve_kernel<FDATTN_CACHE_INT8>, dim3(pairs), dim3(256), shm2, s, sa);
+    } else {
+      hipLaunchKernelGGL(sqattn_scores_mfma_kernel<FDATTN_CACHE_FP8_E4M3>, dim3(pairs * cpp), dim3(256), 0, s, sa);
+      hipLaunchKernelGGL(sqattn_resolve_kernel<FDATTN_CACHE_FP8_E4M3>, dim3(pairs), dim3(256), shm2, s, sa);
+    }
+    return check_launch("fdattn_sqattn_select (mfma)");
+  }
   ScoreArgs a{(const uint16_t*)q, (const uint8_t*)key_cache, cache_k_scale, block_tables, seq_lens_decoder,
               seq_lens_this_time, (double*)workspace, scores, batch, hq, hkv, head_dim, block_size,
               max_blocks_per_seq, num_blocks};
@@ -183,4 +456,26 @@ extern "C" int fdattn_sqattn_select(const void* q, const void* key_cache, const 
                      seq_lens_decoder, seq_lens_this_time, kept_blocks, kept_counts, hkv, block_size,
                      max_blocks_per_seq, top_k);
   return check_launch("fdattn_sqattn_select (top-k)");
+}
+
+extern "C" int fdattn_sqattn_select(const void* q, const void* key_cache, const float* cache_k_scale,
+                                    const int32_t* block_tables, const int32_t* seq_lens_decoder,
+                                    const int32_t* seq_lens_this_time, float* scores, int32_t* kept_blocks,
+                                    int32_t* kept_counts, void* workspace, size_t workspace_bytes, int batch,
+                                    int hq, int hkv, int head_dim, int block_size, int max_blocks_per_seq,
+                                    int num_blocks, int top_k, int cache_quant_type, void* stream) {
+  return sqattn_select_impl(true, q, key_cache, cache_k_scale, block_tables, seq_lens_decoder, seq_lens_this_time,
+                            scores, kept_blocks, kept_counts, workspace, workspace_bytes, batch, hq, hkv, head_dim,
+                            block_size, max_blocks_per_seq, num_blocks, top_k, cache_quant_type, stream);
+}
+
+extern "C" int fdattn_sqattn_select_exact(const void* q, const void* key_cache, const float* cache_k_scale,
+                                          const int32_t* block_tables, const int32_t* seq_lens_decoder,
+                                          const int32_t* seq_lens_this_time, float* scores, int32_t* kept_blocks,
+                                          int32_t* kept_counts, void* workspace, size_t workspace_bytes, int batch,
+                                          int hq, int hkv, int head_dim, int block_size, int max_blocks_per_seq,
+                                          int num_blocks, int top_k, int cache_quant_type, void* stream) {
+  return sqattn_select_impl(false, q, key_cache, cache_k_scale, block_tables, seq_lens_decoder, seq_lens_this_time,
+                            scores, kept_blocks, kept_counts, workspace, workspace_bytes, batch, hq, hkv, head_dim,
+                            block_size, max_blocks_per_seq, num_blocks, top_k, cache_quant_type, stream);
 }

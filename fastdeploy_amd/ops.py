@@ -246,7 +246,7 @@ def splitkv_combine(part_o, part_m, part_l, num_splits=None, out=None):
 
 
 def sqattn_select(q, key_cache, cache_k_scale, block_tables, seq_lens_decoder, seq_lens_this_time=None, *,
-                  num_heads, top_k, cache_quant_type="cache_fp8", return_scores=False, workspace=None):
+                  num_heads, top_k, cache_quant_type="cache_fp8", return_scores=False, workspace=None, impl="auto"):
     """SQAttn block selection: per (sequence, KV head) the top_k blocks by block-max q.k score.
     Returns (kept_blocks int32 [batch, hkv, top_k], kept_counts int32 [batch, hkv][, scores f32])."""
     nb, hkv, bs, d = key_cache.shape
@@ -267,7 +267,8 @@ def sqattn_select(q, key_cache, cache_k_scale, block_tables, seq_lens_decoder, s
     if workspace is None:
         n = _lib.lib().fdattn_sqattn_workspace_bytes(batch, hkv, mb)
         workspace = torch.empty(n, dtype=torch.uint8, device=q.device)
-    rc = _lib.lib().fdattn_sqattn_select(
+    fn = _lib.lib().fdattn_sqattn_select if impl == "auto" else _lib.lib().fdattn_sqattn_select_exact
+    rc = fn(
         p_q, p_kc, p_ks, p_bt, p_dec, p_tt, scores.data_ptr() if return_scores else 0, kept.data_ptr(),
         counts.data_ptr(), _chk(workspace, "workspace", torch.uint8), workspace.numel(), batch, num_heads,
         hkv, d, bs, mb, nb, top_k, _quant(cache_quant_type), _stream())

@@ -208,11 +208,30 @@ FDATTN_API size_t fdattn_sqattn_workspace_bytes(int batch, int hkv, int max_bloc
  * (reduction as function::Max, fastdeploy/function/reduce.cc:354-357), then the
  * top_k highest-scoring blocks per (b,h) are kept; equal scores resolve to the
  * lower block index as in TopKIndices (fastdeploy/vision/utils/utils.h:41-60).
- *   scores      f32 [batch, hkv, max_blocks_per_seq]  (optional output, may be NULL; -inf for absent blocks)
+ *   scores      f32 [batch, hkv, max_blocks_per_seq]  (optional output, may be NULL; -inf for absent blocks).
+ *               For head_dim 128, hq/hkv 4, block_size 64 these are the MFMA scores the selection starts
+ *               from (within a small relative error of the fp64 ones; blocks too close to the k-th score to
+ *               call are re-scored in fp64 internally, so the kept indices are those of the fp64 scores);
+ *               otherwise the fp64 scores rounded to fp32.
  *   kept_blocks i32 [batch, hkv, top_k]  ascending logical block indices, -1 padded
  *   kept_counts i32 [batch, hkv]         min(top_k, ceil(kv_len / block_size))
  */
 FDATTN_API int fdattn_sqattn_select(
+    const void* q, const void* key_cache, const float* cache_k_scale,
+    const int32_t* block_tables, const int32_t* seq_lens_decoder,
+    const int32_t* seq_lens_this_time,
+    float* scores, int32_t* kept_blocks, int32_t* kept_counts,
+    void* workspace, size_t workspace_bytes,
+    int batch, int hq, int hkv, int head_dim, int block_size,
+    int max_blocks_per_seq, int num_blocks, int top_k,
+    int cache_quant_type, void* stream);
+
+/*
+ * The selector with every block scored in fp64 (any head_dim <= 256, hq/hkv <= 8, any block_size):
+ * what fdattn_sqattn_select falls back to for shapes its MFMA scoring does not cover; same kept
+ * indices, `scores` = the fp64 scores rounded to fp32.  Same arguments and plug-in position.
+ */
+FDATTN_API int fdattn_sqattn_select_exact(
     const void* q, const void* key_cache, const float* cache_k_scale,
     const int32_t* block_tables, const int32_t* seq_lens_decoder,
     const int32_t* seq_lens_this_time,

@@ -19,32 +19,69 @@ def oracle_select(oracle, case, top_k):
     return s, kept, cnt
 
 
+@pytest.mark.parametrize("impl", ["auto", "exact"])
 @pytest.mark.parametrize("quant", [CACHE_FP8, CACHE_INT8])
-def test_selector_indices_bit_exact(oracle, quant):
+def test_selector_indices_bit_exact(oracle, quant, impl):
     for seed in range(2):
         case = syn.decode_case(batch=3, ctx=[4096, 3000, 64 * 20 + 1], quant=quant, seed=seed, salient=0.05)
         dev = syn.to_device(case, "cuda")
-        kept, cnt, sc = fd.sqattn_select(dev["q"], dev["key_cache"], dev["cache_k_scale"], dev["block_tables"],
-                                         dev["seq_lens_decoder"], num_heads=32, top_k=8, cache_quant_type=quant,
-                                         return_scores=True)
-        s, okept, ocnt = oracle_select(oracle, case, 8)
-        assert np.array_equal(np_of(cnt), ocnt)
-        assert np.array_equal(np_of(kept), okept)
-        assert np.array_equal(np_of(sc), s.astype(np.float32))
+        for k in (8, 17):
+            kept, cnt, sc = fd.sqattn_select(dev["q"], dev["key_cache"], dev["cache_k_scale"], dev["block_tables"],
+                                             dev["seq_lens_decoder"], num_heads=32, top_k=k, cache_quant_type=quant,
+                                             return_scores=True, impl=impl)
+            s, okept, ocnt = oracle_select(oracle, case, k)
+            assert np.array_equal(np_of(cnt), ocnt)
+            assert np.array_equal(np_of(kept), okept)
+            if impl == "exact":
+                assert np.array_equal(np_of(sc), s.astype(np.float32))
+            else:   # the MFMA scores the selection starts from: close to the fp64 ones, -inf in the same places
+                got = np_of(sc).astype(np.float64)
+                fin = np.isfinite(s)
+                assert np.array_equal(np.isfinite(got), fin)
+                assert np.abs(got[fin] - s[fin]).max() <= 2e-3 * np.abs(s[fin]).max()
 
 
-def test_selector_ties_and_short_sequences(oracle):
-    case = syn.decode_case(batch=2, ctx=[64 * 12, 100], quant=CACHE_FP8, seed=3)
+@pytest.mark.parametrize("impl", ["auto", "exact"])
+@pytest.mark.parametrize("quant", [CACHE_FP8, CACHE_INT8])
+def test_selector_ties_near_ties_and_short_sequences(oracle, quant, impl):
+    case = syn.decode_case(batch=2, ctx=[64 * 12, 100], quant=quant, seed=3)
     bt = case["block_tables"]
     # identical K pages -> identical scores -> the lower block index must win
     for j in (5, 7, 9):
         case["key_cache"][int(bt[0, j])] = case["key_cache"][int(bt[0, 2])]
+    # near ties: copies that differ by one code step in one channel of every token
+    for j, ch in ((3, 0), (10, 77)):
+        page = case["key_cache"][int(bt[0, 2])].clone()
+        page[:, :, ch] = torch.where((page[:, :, ch] & 0x7F) < 0x70, page[:, :, ch] + 1, page[:, :, ch])
+        case["key_cache"][int(bt[0, j])] = page
     dev = syn.to_device(case, "cuda")
-    for k in (1, 2, 3, 4, 11, 12, 64):
+    for k in (1, 2, 3, 4, 5, 6, 7, 11, 12, 64):
         kept, cnt = fd.sqattn_select(dev["q"], dev["key_cache"], dev["cache_k_scale"], dev["block_tables"],
-                                     dev["seq_lens_decoder"], num_heads=32, top_k=k)
+                                     dev["seq_lens_decoder"], num_heads=32, top_k=k, cache_quant_type=quant, impl=impl)
         _, okept, ocnt = oracle_select(oracle, case, k)
         assert np.array_equal(np_of(kept), okept) and np.array_equal(np_of(cnt), ocnt), k
+
+
+def test_selector_config4_shape_indices_bit_exact(oracle):
+    """batch 16, ctx 32768, fp8 KV, top-64 of 512 blocks per KV head, 5 % salient blocks (scaled x4):
+    the full-size launch against the oracle."""
+    case = syn.decode_case(batch=16, ctx=32768, quant=CACHE_FP8, seed=0, device="cuda", salient=0.05)
+    kept, cnt = fd.sqattn_select(case["q"], case["key_cache"], case["cache_k_scale"], case["block_tables"],
+                                 case["seq_lens_decoder"], num_heads=32, top_k=64)
+    torch.cuda.synchronize()
+    cpu = syn.to_device(case, "cpu")
+    _, okept, ocnt = oracle_select(oracle, cpu, 64)
+    assert np.array_equal(np_of(cnt), ocnt)
+    assert np.array_equal(np_of(kept), okept)
+    # and the sparse decode over the kept blocks equals the oracle's
+    out = fd.decode_attention_sparse(case["q"], case["key_cache"], case["value_cache"], case["cache_k_scale"],
+                                     case["cache_v_scale"], case["block_tables"], case["seq_lens_decoder"],
+                                     kept_blocks=kept, kept_counts=cnt, num_heads=32, cache_quant_type=CACHE_FP8)
+    want = oracle.decode_attention(bits(cpu["q"]), np_of(cpu["key_cache"]), np_of(cpu["value_cache"]),
+                                   np_of(cpu["cache_k_scale"]), np_of(cpu["cache_v_scale"]), np_of(cpu["block_tables"]),
+                                   np_of(cpu["seq_lens_decoder"]), 32, 8, 128, CACHE_FP8, kept_blocks=okept, kept_counts=ocnt)
+    ok, mx, bad = bf16_close(bits(out), want)
+    assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
 
 
 def _prefill_case(seed, prefix, chunks, quant=CACHE_INT8):
