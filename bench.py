@@ -88,7 +88,7 @@ def other_workloads(args):
 
     if args.workload in ("sqattn", "all"):
         # configs[3]: batch 16, ctx 32768, fp8 KV, top-64 of 512 blocks per KV head
-        c = syn.decode_case(batch=16, ctx=32768, quant=2, seed=0, device=dev, direct_bytes=True)
+        c = syn.decode_case(batch=16, ctx=32768, quant=2, seed=0, device=dev, salient=0.05)   # K ~ N(0,1), 5 % of blocks x4
         sel = lambda: fd.sqattn_select(c["q"], c["key_cache"], c["cache_k_scale"], c["block_tables"], c["seq_lens_decoder"],
                                        num_heads=32, top_k=64, cache_quant_type="cache_fp8")
         kept, cnt = sel()

@@ -156,7 +156,8 @@ struct SelArgs {
   const int32_t* seq_lens_decoder;
   const int32_t* seq_lens_this_time;
   float* approx;  // [pairs][max_blocks]
-  float* eps;     // [pairs]
+  float* eps;     // [pairs]: bound that holds for every block of the pair
+  float* ebound;  // [pairs][max_blocks]: per-block bound (fp8 only, else NULL)
   float* scores_out;  // optional copy of approx
   int32_t* kept_blocks;
   int32_t* kept_counts;
@@ -200,9 +201,15 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
       sabs = fmaxf(sabs, wave_sum(sa));
       amax = fmaxf(amax, wave_max(am));
     }
+    // int8: q*scale is rounded to a multiple of step = amax/1048575, at most step/2 off per channel, times
+    //   |k| <= 127 over 128 channels; the integer dot products are exact and the fp32 recombination of the
+    //   three limbs adds at most a few 2^-24 of the leading term (covered by the 2048).
+    // fp8: four e4m3 residual limbs leave at most 2^-16 of |q*scale| per channel (or the subnormal floor,
+    //   2^-10 in units of amax/256), and the fp32 accumulation of the products adds at most 2^-17 of
+    //   sum |q*scale||k|; with |k| <= 448 that is below 2^-15 * 448 * sum |q*scale| + amax * 2^-18 * 128 * 448.
     float e;
-    if (QUANT == FDATTN_CACHE_INT8) e = amax * (128.0f * 127.0f / 2097150.0f) + sabs * 127.0f * 9.5367431640625e-7f;
-    else e = sabs * 448.0f * 4.8828125e-4f;  // 2^-11
+    if (QUANT == FDATTN_CACHE_INT8) e = amax * ((128.0f * 127.0f * 0.5f + 2048.0f) / 1048575.0f);
+    else e = sabs * 448.0f * 3.0517578125e-5f + amax * (128.0f * 448.0f * 3.814697265625e-6f);
     if (lane == 0) a.eps[p] = e * 1.0001f;
   }
 
@@ -231,13 +238,37 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
     dma_tile(kbase + (size_t)__builtin_amdgcn_readlane(my_pb, wv + kWaves) * blk_stride, saddr[1], offK);
   PairState st;
   load_pair<QUANT>(a.q, a.k_scale, a.hkv, 1.0f, p, lane, st);  // scores in natural units
+  // fp8: a second operand, |q*scale| in one e4m3 limb, gives sum_c |q*scale||k| per token next to the score;
+  // the error of a block's score is a small multiple of that sum (see the bound below)
+  v4i aabs[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+  float amax_pair = 0.f;
+  if (QUANT != FDATTN_CACHE_INT8) {
+    const int m = lane & 15, g = lane >> 4, head = m >> 2, limb = m & 3;
+    const uint16_t* qrow = a.q + ((size_t)b * a.hkv * kG + h * kG + head) * kD;
+    // st.rs = amax / 256 of this lane's S-layout head; the A layout wants the head of row m
+    const float rs_row = __shfl(st.rs, 16 * head, 64);
+    const float inv = rs_row > 0.f ? 1.0f / rs_row : 0.f;
+#pragma unroll
+    for (int k2 = 0; k2 < 2; ++k2) {
+      const int c0 = 16 * (g + 4 * k2);
+      u32 pk[4] = {0, 0, 0, 0};
+#pragma unroll
+      for (int jj = 0; jj < 16; ++jj) {
+        const float x = fabsf(bf16_to_f32(qrow[c0 + jj]) * a.k_scale[h * kD + c0 + jj]) * inv;
+        const u32 code = limb == 0 ? ((u32)__builtin_amdgcn_cvt_pk_fp8_f32(x, x, 0, false) & 0xffu) : 0u;
+        pk[jj >> 2] |= code << (8 * (jj & 3));
+      }
+      aabs[k2] = (v4i){(int)pk[0], (int)pk[1], (int)pk[2], (int)pk[3]};
+    }
+    amax_pair = fmaxf(fmaxf(__shfl(st.rs, 0, 64), __shfl(st.rs, 16, 64)), fmaxf(__shfl(st.rs, 32, 64), __shfl(st.rs, 48, 64))) * 256.0f;
+  }
 
   int it = 0;
   for (int j = wv; j < cnt; j += kWaves, ++it) {
     const int valid = __builtin_amdgcn_readlane(my_valid, j);
     const uint8_t* kbuf = slot[it & 1];
     if (j + kWaves < cnt) wait_vm8(); else wait_vm0();
-    float sv = -INFINITY;
+    float sv = -INFINITY, bv = 0.f;
 #pragma unroll
     for (int stl = 0; stl < 4; ++stl) {
       const int tok = 4 * n16 + stl;
@@ -252,7 +283,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
         }
         s = st.rs * ((float)acc.x + 128.0f * (float)acc.y + 16384.0f * (float)acc.z);
       } else {
-        v4f acc = {0.f, 0.f, 0.f, 0.f};
+        v4f acc = {0.f, 0.f, 0.f, 0.f}, ab = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int k2 = 0; k2 < 2; ++k2) {
           const int c = g4 + 4 * k2;
@@ -263,8 +294,13 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
           const long b1 = ((long)(u32)kb.w << 32) | (u32)kb.z;
           acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a0, b0, acc, 0, 0, 0);
           acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a1, b1, acc, 0, 0, 0);
+          const long m0 = ((long)(u32)aabs[k2].y << 32) | (u32)aabs[k2].x;
+          const long m1 = ((long)(u32)aabs[k2].w << 32) | (u32)aabs[k2].z;
+          ab = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(m0, b0 & 0x7f7f7f7f7f7f7f7fL, ab, 0, 0, 0);
+          ab = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(m1, b1 & 0x7f7f7f7f7f7f7f7fL, ab, 0, 0, 0);
         }
         s = st.rs * ((acc.x + acc.y) + (acc.z + acc.w));
+        bv = fmaxf(bv, tok < valid ? st.rs * ab.x : 0.f);
       }
       sv = fmaxf(sv, tok < valid ? s : -INFINITY);
     }
@@ -274,11 +310,76 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
     sv = row_max16(sv);                          // over the tokens of this head
     sv = fmaxf(sv, __shfl_xor(sv, 16, 64));      // over the 4 heads of the group
     sv = fmaxf(sv, __shfl_xor(sv, 32, 64));
+    if (QUANT != FDATTN_CACHE_INT8) {
+      bv = row_max16(bv);
+      bv = fmaxf(bv, __shfl_xor(bv, 16, 64));
+      bv = fmaxf(bv, __shfl_xor(bv, 32, 64));
+      // residual of the four limbs <= 2^-16 |q*scale| per channel (or the e4m3 subnormal floor, 2^-10 in units
+      // of amax/256); fp32 accumulation <= 2^-17 of sum |q*scale||k|; the one-limb |q*scale| is itself up to
+      // 2^-4 low: (2^-16 + 2^-17) * (1 + 2^-4) < 2^-15.3 -> 2.5e-5
+      bv = bv * 2.5e-5f + amax_pair * (128.0f * 448.0f * 3.814697265625e-6f) * 1.0001f;
+    }
     if (lane == 0) {
       srow[first + j] = sv;
+      if (QUANT != FDATTN_CACHE_INT8) a.ebound[(size_t)p * a.max_blocks + first + j] = bv;
       if (a.scores_out) a.scores_out[(size_t)p * a.max_blocks + first + j] = sv;
     }
   }
+}
+
+__device__ __forceinline__ unsigned order_key(float f) {
+  const unsigned u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);  // unsigned order == float order
+}
+__device__ __forceinline__ float key_to_float(unsigned k) {
+  return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+// The r-th largest (r = 1 is the maximum) of v[j] + sign * e[j], j < n, found by a whole 256-thread
+// workgroup; every thread returns the value.  hist: 256 ints, sel: 2 unsigneds of shared memory.
+__device__ float radix_select_desc(const float* v, const float* e, float sign, int n, int r, int* hist, unsigned* sel) {
+  const int tid = threadIdx.x;
+  unsigned prefix = 0, mask = 0;
+  int remaining = r;
+  for (int shift = 24; shift >= 0; shift -= 8) {
+    hist[tid] = 0;
+    __syncthreads();
+    for (int j = tid; j < n; j += 256) {
+      const unsigned key = order_key(v[j] + sign * e[j]);
+      if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1);
+    }
+    __syncthreads();
+    if (tid < 64) {
+      // bins 255 .. 0 in 4 groups of 64 handled by one wavefront: find the bin where the count from the
+      // top reaches `remaining`
+      int rem = remaining, found = -1;
+      for (int grp = 3; grp >= 0 && found < 0; --grp) {
+        const int bin = grp * 64 + (63 - tid);  // lane 0 holds the highest bin of the group
+        const int c = hist[bin];
+        int incl = c;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+          const int t = __shfl_up(incl, o, 64);
+          if (tid >= o) incl += t;
+        }
+        const unsigned long long hit = __ballot(incl >= rem);
+        if (hit) {
+          const int l = __ffsll((long long)hit) - 1;
+          found = grp * 64 + (63 - l);
+          rem -= __shfl(incl - c, l, 64);
+        } else {
+          rem -= __shfl(incl, 63, 64);
+        }
+      }
+      if (tid == 0) { sel[0] = (unsigned)found; sel[1] = (unsigned)rem; }
+    }
+    __syncthreads();
+    prefix |= sel[0] << shift;
+    mask |= 255u << shift;
+    remaining = (int)sel[1];
+    __syncthreads();
+  }
+  return key_to_float(prefix);
 }
 
 // One workgroup per (sequence, KV head): classify, re-score the undecided blocks in fp64, emit.
@@ -286,10 +387,14 @@ template <int QUANT>
 __global__ __launch_bounds__(256) void sqattn_resolve_kernel(SelArgs a) {
   extern __shared__ double smd[];                  // exact scores of undecided blocks [max_blocks]
   float* sf = reinterpret_cast<float*>(smd + a.max_blocks);      // approx scores [max_blocks]
-  int* state = reinterpret_cast<int*>(sf + a.max_blocks);         // 0 dropped, 1 kept, 2 undecided -> list index
+  float* se = sf + a.max_blocks;                                  // error bounds [max_blocks]
+  int* state = reinterpret_cast<int*>(se + a.max_blocks);         // 0 dropped, 1 kept, 2 undecided
   int* ulist = state + a.max_blocks;                              // undecided block ids
   __shared__ float qs[kG][kD];
   __shared__ int n_in, n_unc, wave_tot[4], running;
+  __shared__ float thr[2];
+  __shared__ int hist[256];
+  __shared__ unsigned sel[2];
   const int p = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int b = p / a.hkv, h = p - b * a.hkv;
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
@@ -301,18 +406,23 @@ __global__ __launch_bounds__(256) void sqattn_resolve_kernel(SelArgs a) {
   for (int j = tid; j < nblk; j += 256) sf[j] = s[j];
   __syncthreads();
   if (k < nblk) {
+    // With score i known to within e_i (L_i = s_i - e_i, U_i = s_i + e_i): block j is surely kept if
+    // L_j > the (k+1)-th largest U (then at most k blocks, itself included, can reach it) and surely
+    // dropped if U_j < the k-th largest L (then k blocks beat it for certain); the rest is undecided.
     const float eps = a.eps[p];
+    const float* eb = a.ebound ? a.ebound + (size_t)p * a.max_blocks : nullptr;
+    for (int j = tid; j < nblk; j += 256) se[j] = eb ? eb[j] : eps;
+    __syncthreads();
+    // k-th largest lower bound and (k+1)-th largest upper bound by radix selection (4 passes of 8 bits
+    // over order-preserving integer keys), not by ranking every block against every other
+    thr[0] = radix_select_desc(sf, se, -1.0f, nblk, k, hist, sel);
+    thr[1] = radix_select_desc(sf, se, +1.0f, nblk, k + 1, hist, sel);
+    const float lk = thr[0], uk1 = thr[1];
     for (int j = tid; j < nblk; j += 256) {
-      const float lo = sf[j] - eps, hi = sf[j] + eps;
-      int sure_better = 0, maybe_better = 0;
-      for (int i = 0; i < nblk; ++i) {
-        const float si = sf[i];
-        sure_better += (si - eps > hi);
-        maybe_better += (i != j) && (si + eps >= lo);
-      }
+      const float lj = sf[j] - se[j], uj = sf[j] + se[j];
       int stt = 2;
-      if (maybe_better < k) stt = 1;
-      else if (sure_better >= k) stt = 0;
+      if (lj > uk1) stt = 1;
+      else if (uj < lk) stt = 0;
       state[j] = stt;
       if (stt == 1) atomicAdd(&n_in, 1);
       if (stt == 2) ulist[atomicAdd(&n_unc, 1)] = j;
@@ -386,7 +496,7 @@ __global__ __launch_bounds__(256) void sqattn_resolve_kernel(SelArgs a) {
 }
 
 static bool sel_fast_supported(int hq, int hkv, int d, int bs, int max_blocks) {
-  return d == kD && hq == kG * hkv && bs == kBS && max_blocks <= 2048;  // 20 B of LDS per block in the top-k kernel
+  return d == kD && hq == kG * hkv && bs == kBS && max_blocks <= 2048;  // 24 B of LDS per block in the top-k kernel
 }
 
 }  // namespace fdattn
@@ -395,7 +505,7 @@ using namespace fdattn;
 
 extern "C" size_t fdattn_sqattn_workspace_bytes(int batch, int hkv, int max_blocks_per_seq) {
   if (batch <= 0 || hkv <= 0 || max_blocks_per_seq <= 0) return 256;
-  size_t n = (size_t)batch * hkv * max_blocks_per_seq * sizeof(double);
+  size_t n = (size_t)batch * hkv * ((size_t)max_blocks_per_seq * sizeof(double) + sizeof(float));
   return (n + 255) & ~(size_t)255;
 }
 
@@ -417,7 +527,7 @@ static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_ca
                 batch, hq, hkv, head_dim, block_size, max_blocks_per_seq, top_k, kSelMaxG, kSelMaxD);
   if (cache_quant_type != FDATTN_CACHE_INT8 && cache_quant_type != FDATTN_CACHE_FP8_E4M3)
     return fail(FDATTN_ERR_QUANT, "fdattn_sqattn_select: unknown cache_quant_type %d", cache_quant_type);
-  const size_t need = (size_t)batch * hkv * max_blocks_per_seq * sizeof(double);
+  const size_t need = (size_t)batch * hkv * ((size_t)max_blocks_per_seq * sizeof(double) + sizeof(float));
   if (workspace_bytes < need)
     return fail(FDATTN_ERR_WORKSPACE, "fdattn_sqattn_select: workspace %zu B < required %zu B", workspace_bytes, need);
   hipStream_t s = (hipStream_t)stream;
@@ -427,11 +537,12 @@ static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_ca
     while (chunk > 4 && (long long)pairs * ((max_blocks_per_seq + chunk - 1) / chunk) < 1024) chunk /= 2;
     const int cpp = (max_blocks_per_seq + chunk - 1) / chunk;
     float* approx = (float*)workspace;
-    float* eps = approx + (size_t)pairs * max_blocks_per_seq;  // fits: the workspace holds 8 bytes per block
+    float* ebound = approx + (size_t)pairs * max_blocks_per_seq;
+    float* eps = ebound + (size_t)pairs * max_blocks_per_seq;
     SelArgs sa{(const uint16_t*)q, (const uint8_t*)key_cache, cache_k_scale, block_tables, seq_lens_decoder,
-               seq_lens_this_time, approx, eps, scores, kept_blocks, kept_counts, batch, hkv,
+               seq_lens_this_time, approx, eps, cache_quant_type == FDATTN_CACHE_INT8 ? nullptr : ebound, scores, kept_blocks, kept_counts, batch, hkv,
                max_blocks_per_seq, num_blocks, chunk, cpp, top_k};
-    const size_t shm2 = (size_t)max_blocks_per_seq * (sizeof(double) + sizeof(float) + 2 * sizeof(int));
+    const size_t shm2 = (size_t)max_blocks_per_seq * (sizeof(double) + 2 * sizeof(float) + 2 * sizeof(int));
     if (cache_quant_type == FDATTN_CACHE_INT8) {
       hipLaunchKernelGGL(sqattn_scores_mfma_kernel<FDATTN_CACHE_INT8>, dim3(pairs * cpp), dim3(256), 0, s, sa);
       hipLaunchKernelGGL(sqattn_resolve_kernel<FDATTN_CACHE_INT8>, dim3(pairs), dim3(256), shm2, s, sa);
