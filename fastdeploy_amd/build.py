@@ -18,7 +18,7 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-fvisibility=hidden", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
-]
+] + os.environ.get("FDATTN_EXTRA_FLAGS", "").split()
 
 SOURCES = ["api.hip", "cache_writer.hip", "decode_generic.hip", "decode_c8.hip", "decode_api.hip",
            "sqattn.hip", "prefill.hip", "prefill_mfma.hip"]

@@ -169,8 +169,7 @@ struct SelArgs {
 // in flight) and leaves one fp32 score per block.
 template <int QUANT>
 __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelArgs a) {
-  __shared__ __attribute__((aligned(16))) uint8_t ldsA[kWaves][kTileB];
-  __shared__ __attribute__((aligned(16))) uint8_t ldsB[kWaves][kTileB];
+  __shared__ __attribute__((aligned(16))) uint8_t ldsK[kWaves][2][kTileB];  // two K slots per wavefront
   const int lane = threadIdx.x & 63;
   const int wv = uni(threadIdx.x >> 6);
   const int p = blockIdx.x / a.chunks_per_pair, ck = blockIdx.x - p * a.chunks_per_pair;
@@ -213,8 +212,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
     if (lane == 0) a.eps[p] = e * 1.0001f;
   }
 
-  uint8_t* const slot[2] = {ldsA[wv], ldsB[wv]};
-  const u32 saddr[2] = {(u32)uni((int)lds_addr_of(slot[0])), (u32)uni((int)lds_addr_of(slot[1]))};
+  const u32 saddr0 = (u32)uni((int)lds_addr_of(ldsK[wv][0]));
   const DmaOffsets offK = dma_offsets<kShiftK>(lane);
   const int n16 = lane & 15, g4 = lane >> 4;
 
@@ -233,9 +231,9 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
   const uint8_t* const kbase = a.key_cache + (size_t)h * tile_stride;
   const size_t blk_stride = (size_t)a.hkv * tile_stride;
 
-  dma_tile(kbase + (size_t)__builtin_amdgcn_readlane(my_pb, wv) * blk_stride, saddr[0], offK);
+  dma_tile(kbase + (size_t)__builtin_amdgcn_readlane(my_pb, wv) * blk_stride, saddr0, offK);
   if (wv + kWaves < cnt)
-    dma_tile(kbase + (size_t)__builtin_amdgcn_readlane(my_pb, wv + kWaves) * blk_stride, saddr[1], offK);
+    dma_tile(kbase + (size_t)__builtin_amdgcn_readlane(my_pb, wv + kWaves) * blk_stride, saddr0 + kTileB, offK);
   PairState st;
   load_pair<QUANT>(a.q, a.k_scale, a.hkv, 1.0f, p, lane, st);  // scores in natural units
   // fp8: a second operand, |q*scale| in one e4m3 limb, gives sum_c |q*scale||k| per token next to the score;
@@ -266,7 +264,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
   int it = 0;
   for (int j = wv; j < cnt; j += kWaves, ++it) {
     const int valid = __builtin_amdgcn_readlane(my_valid, j);
-    const uint8_t* kbuf = slot[it & 1];
+    const uint8_t* kbuf = ldsK[wv][it & 1];  // indexed, not picked from a pointer array: stays an LDS address
     if (j + kWaves < cnt) wait_vm8(); else wait_vm0();
     float sv = -INFINITY, bv = 0.f;
 #pragma unroll
@@ -306,7 +304,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
     }
     wait_lgkm0();  // tile consumed: refill its slot with the block two steps ahead
     if (j + 2 * kWaves < cnt)
-      dma_tile(kbase + (size_t)__builtin_amdgcn_readlane(my_pb, j + 2 * kWaves) * blk_stride, saddr[it & 1], offK);
+      dma_tile(kbase + (size_t)__builtin_amdgcn_readlane(my_pb, j + 2 * kWaves) * blk_stride, saddr0 + (u32)(it & 1) * kTileB, offK);
     sv = row_max16(sv);                          // over the tokens of this head
     sv = fmaxf(sv, __shfl_xor(sv, 16, 64));      // over the 4 heads of the group
     sv = fmaxf(sv, __shfl_xor(sv, 32, 64));
@@ -428,7 +426,14 @@ __global__ __launch_bounds__(256) void sqattn_resolve_kernel(SelArgs a) {
       if (stt == 2) ulist[atomicAdd(&n_unc, 1)] = j;
     }
     __syncthreads();
+#ifdef FDATTN_EXP_NORESCORE
+    const int nu = 0, need = k - n_in;
+#else
     const int nu = n_unc, need = k - n_in;
+#endif
+#ifdef FDATTN_EXP_COUNT
+    if (tid == 0) a.eps[p] = (float)n_unc;
+#endif
     if (nu > 0) {
       for (int i = tid; i < kG * kD; i += 256) {
         const int g = i / kD, c = i % kD;
@@ -443,13 +448,15 @@ __global__ __launch_bounds__(256) void sqattn_resolve_kernel(SelArgs a) {
         if (pb >= 0 && pb < a.num_blocks && j * kBS + lane < kv_len) {
           const uint8_t* kr = a.key_cache + (((size_t)pb * a.hkv + h) * kBS + lane) * kD;
           double acc[kG] = {0.0, 0.0, 0.0, 0.0};
-          for (int c = 0; c < kD; c += 4) {
-            const u32 w = *reinterpret_cast<const u32*>(kr + c);
+          // the products are exact in fp64, so fma(q, k, acc) rounds exactly like add(acc, mul(q, k))
+          for (int c = 0; c < kD; c += 16) {
+            const uint4 w4 = *reinterpret_cast<const uint4*>(kr + c);
+            const u32 ws[4] = {w4.x, w4.y, w4.z, w4.w};
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const double kv = dq64<QUANT>((w >> (8 * e)) & 0xff);
+            for (int e = 0; e < 16; ++e) {
+              const double kv = dq64<QUANT>((ws[e >> 2] >> (8 * (e & 3))) & 0xff);
 #pragma unroll
-              for (int g = 0; g < kG; ++g) acc[g] = __dadd_rn(acc[g], __dmul_rn((double)qs[g][c + e], kv));
+              for (int g = 0; g < kG; ++g) acc[g] = __fma_rn((double)qs[g][c + e], kv, acc[g]);
             }
           }
           best = fmax(fmax(acc[0], acc[1]), fmax(acc[2], acc[3]));
@@ -533,7 +540,7 @@ static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_ca
   hipStream_t s = (hipStream_t)stream;
   if (allow_fast && sel_fast_supported(hq, hkv, head_dim, block_size, max_blocks_per_seq)) {
     const int pairs = batch * hkv;
-    int chunk = 32;
+    int chunk = 64;
     while (chunk > 4 && (long long)pairs * ((max_blocks_per_seq + chunk - 1) / chunk) < 1024) chunk /= 2;
     const int cpp = (max_blocks_per_seq + chunk - 1) / chunk;
     float* approx = (float*)workspace;
