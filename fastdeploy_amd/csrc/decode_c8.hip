@@ -144,18 +144,6 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
         validn = __builtin_amdgcn_readlane(my_valid, j + kWaves);
       }
 
-#ifdef FDATTN_EXP_NOCOMPUTE
-      wait_vm8();
-      st.l += (float)kbuf[lane * 4];
-      wait_lgkm0();
-      if (has_next) dma_tile(kbase + (size_t)pbn * blk_stride, kaddr, offK);
-      if (has_next) wait_vm8(); else wait_vm0();
-      st.l += (float)vbuf[lane * 4];
-      wait_lgkm0();
-      if (has_next) dma_tile(vbase + (size_t)pbn * blk_stride, vaddr, offV);
-      pb = pbn; valid = validn;
-      continue;
-#endif
       // ---------------- S = Q K^T : rows = head*4 + limb, columns = token slots
       wait_vm8();  // K(j) landed; V(j) may still be in flight
       if (j == wv) TRACE(4);

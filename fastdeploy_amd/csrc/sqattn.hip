@@ -426,14 +426,7 @@ __global__ __launch_bounds__(256) void sqattn_resolve_kernel(SelArgs a) {
       if (stt == 2) ulist[atomicAdd(&n_unc, 1)] = j;
     }
     __syncthreads();
-#ifdef FDATTN_EXP_NORESCORE
-    const int nu = 0, need = k - n_in;
-#else
     const int nu = n_unc, need = k - n_in;
-#endif
-#ifdef FDATTN_EXP_COUNT
-    if (tid == 0) a.eps[p] = (float)n_unc;
-#endif
     if (nu > 0) {
       for (int i = tid; i < kG * kD; i += 256) {
         const int g = i / kD, c = i % kD;
