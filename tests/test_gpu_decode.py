@@ -145,3 +145,57 @@ def test_workspace_is_reusable_across_calls_and_shapes(oracle):
         for case in cases:
             got = gpu_decode(case, workspace=ws)
             check(got, oracle_decode(oracle, case), "reuse rep %d" % rep)
+
+
+def test_decode_config2_full_size(oracle):
+    """batch 64, ctx U[3584, 4608], int8 KV, block tables a random permutation over a 6000-block pool:
+    the full-size launch against the oracle, plus two size-independent properties: the result does not
+    depend on where the blocks sit in the pool, and it is the same whatever the split-KV chunking is
+    (dense call == sparse call that keeps every block)."""
+    g = torch.Generator().manual_seed(0)
+    lens = torch.randint(3584, 4609, (64,), generator=g).tolist()
+    case = syn.decode_case(batch=64, ctx=lens, pool_blocks=6000, seed=1, device="cuda", max_blocks=72)
+    out = fd.decode_attention(case["q"], case["key_cache"], case["value_cache"], case["cache_k_scale"],
+                              case["cache_v_scale"], case["block_tables"], case["seq_lens_decoder"], num_heads=32)
+    torch.cuda.synchronize()
+    cpu = syn.to_device(case, "cpu")
+    check(bits(out), oracle_decode(oracle, cpu), "cfg2")
+    # move every block somewhere else in the pool: bit-identical output
+    perm = torch.randperm(6000, generator=torch.Generator().manual_seed(5)).cuda()
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(6000, device="cuda")
+    bt2 = torch.where(case["block_tables"] >= 0, inv[case["block_tables"].clamp(min=0).long()].to(torch.int32), -1)
+    out2 = fd.decode_attention(case["q"], case["key_cache"][perm], case["value_cache"][perm], case["cache_k_scale"],
+                               case["cache_v_scale"], bt2.contiguous(), case["seq_lens_decoder"], num_heads=32)
+    assert torch.equal(out, out2)
+    # keep-everything sparse call: same blocks, different chunk geometry -> same within a bf16 ulp of rounding noise
+    nb = torch.tensor([(n + 63) // 64 for n in lens], dtype=torch.int32, device="cuda")
+    kept = torch.arange(72, dtype=torch.int32, device="cuda")[None, None, :].repeat(64, 8, 1)
+    kept = torch.where(kept < nb[:, None, None], kept, -1).contiguous()
+    cnt = nb[:, None].repeat(1, 8).contiguous()
+    out3 = fd.decode_attention_sparse(case["q"], case["key_cache"], case["value_cache"], case["cache_k_scale"],
+                                      case["cache_v_scale"], case["block_tables"], case["seq_lens_decoder"],
+                                      kept_blocks=kept, kept_counts=cnt, num_heads=32)
+    check(bits(out3), bits(out), "dense vs keep-all sparse")
+
+
+def test_write_then_decode_config3_full_size(oracle):
+    """256 new tokens (bf16 qkv ~ N(0,1)), RoPE theta 500000 at positions U{0..8191}, int8 write into the
+    block-tabled slots, then decode over ctx = pos + 1: cache bytes bit-exact, outputs within tolerance."""
+    case = syn.write_case(num_seqs=256, max_pos=8192, seed=2, blocks_per_seq=128)
+    # the prior cache contents are random bytes: use scales that keep the logits moderate
+    dev = syn.to_device(case, "cuda")
+    out = fd.append_attention(dev["qkv"], dev["key_cache"], dev["value_cache"], dev["seq_lens_encoder"],
+                              dev["seq_lens_decoder"], dev["seq_lens_this_time"], dev["block_tables"],
+                              (dev["rope_cos"], dev["rope_sin"]), dev["cache_k_scale"], dev["cache_v_scale"],
+                              num_heads=32, kv_num_heads=8, max_chunk=1)
+    torch.cuda.synchronize()
+    kc, vc = np_of(case["key_cache"]).copy(), np_of(case["value_cache"]).copy()
+    q, _, _ = oracle.write_cache_kv(bits(case["qkv"]), kc, vc, np_of(case["cache_k_scale"]), np_of(case["cache_v_scale"]),
+                                    np_of(case["rope_cos"]), np_of(case["rope_sin"]), np_of(case["block_tables"]),
+                                    np_of(case["seq_lens_decoder"]), np_of(case["cu_seqlens_q"]), 32, 8, 128, 1, CACHE_INT8,
+                                    want_kv_out=False)
+    assert np.array_equal(np_of(dev["key_cache"]), kc) and np.array_equal(np_of(dev["value_cache"]), vc)
+    want = oracle.decode_attention(q, kc, vc, np_of(case["cache_k_scale"]), np_of(case["cache_v_scale"]),
+                                   np_of(case["block_tables"]), np_of(case["seq_lens_decoder"]) + 1, 32, 8, 128, CACHE_INT8)
+    check(bits(out), want, "cfg3")
