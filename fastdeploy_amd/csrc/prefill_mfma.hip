@@ -1,35 +1,53 @@
-// Chunked-prefill ("append") attention on the bf16 MFMA units, head_dim 128, block_size 64.
+// Chunked-prefill ("append") attention on the MFMA units, head_dim 128, block_size 64.
 //
-// One workgroup = 128 new tokens of one query head (4 wavefronts x 32 tokens); it walks
-// the keys in tiles of 64: first the cached prefix, one cache block per tile (int8 / fp8
-// bytes converted to bf16 once per workgroup while they are staged into LDS - "dequantised
-// in-tile"), then the chunk's own bf16 K/V up to the causal diagonal.
+// One workgroup = NW wavefronts x 32 new tokens of one query head (NW = 8 -> 256 tokens, or
+// 4 -> 128 for short chunks); it walks the keys in tiles of 64: first the cached prefix, one
+// cache block per tile (int8 / fp8 bytes turned into fp16 once per workgroup while they are
+// staged into LDS - "dequantised in-tile"), then the chunk's own bf16 K/V up to the causal
+// diagonal.
 //
-// Number formats: cache bytes (int8, e4m3) are exact in fp16, so the prefix tiles run on
-// v_mfma_f32_32x32x16_f16 with Q*k_scale rounded to fp16 (11 significant bits); the chunk's
-// own K stays bf16 and meets the bf16 Q on v_mfma_f32_32x32x16_bf16 (exact inputs).  The
-// softmax weights and V always go through fp16 (V of the chunk is converted, saturating at
-// +-65504): bf16 weights (8 bits) would not hold the 2e-3 / 1e-2 output tolerance on rows
-// with few keys.
+// Number formats.  The prefix tiles run on v_mfma_f32_32x32x16_f16.  An int8 byte b becomes
+// the fp16 SUBNORMAL with mantissa b ^ 0x80, i.e. the value 2^-24 (b + 128): one xor per four
+// bytes and one byte permute per two, no int->float conversion.  The MFMA treats fp16
+// subnormals exactly, so the products are exact; the factor 2^24 goes into the softmax scale
+// and the offset 128 drops out algebraically:
+//   scores:  sum_c q_c 2^-24 (k_c + 128)  =  2^-24 (q.k + 128 sum_c q_c)  - the second term is a
+//            per-query constant, folded into the exponent's additive constant;
+//   output:  sum_j p_j 2^-24 (v_j + 128)  =  2^-24 (sum_j p_j v_j + 128 l),  l = sum_j p_j -
+//            removed once, when the walk leaves the prefix, with l summed from the same
+//            fp16-rounded weights the MFMA multiplied (v_dot2_f32_f16).
+// e4m3 bytes are converted by v_cvt_pk_f32_fp8 (exact in fp16).  Q * k_scale is rounded to
+// fp16 (11 significant bits).  The chunk's own K stays bf16 and meets the bf16 Q on
+// v_mfma_f32_32x32x16_bf16 (exact inputs).  The softmax weights and V always go through fp16
+// (V of the chunk is converted, saturating at +-65504): bf16 weights (8 bits) would not hold
+// the 2e-3 / 1e-2 output tolerance on rows with few keys.
 //
-// The scores are computed transposed, S^T = K Q^T: in the
-// result layout a lane owns one query and 16 of every 32 keys, so the softmax row
-// reductions are in-lane plus one exchange with lane^32, and P^T is already laid out as
-// the B operand of the second product O^T = V^T P^T - no trip through LDS.  V^T operands
-// come transposed out of LDS by ds_read_b64_tr_b16.  The per-channel K scale is folded
-// into Q for the prefix tiles; the V scale is applied to the accumulator once, when the
-// walk passes from the prefix to the chunk.  K/V tiles are double-buffered in LDS with
-// the next tile's global loads in flight during the current tile's MFMAs; one barrier
-// per tile.
+// The scores are computed transposed, S^T = K Q^T: in the result layout a lane owns one query
+// and 16 of every 32 keys, so the softmax row reductions are in-lane plus one exchange with
+// lane^32, and P^T is already laid out as the B operand of the second product
+// O^T = V^T P^T - no trip through LDS.  V^T operands come transposed out of LDS by
+// ds_read_b64_tr_b16.  The running maximum is only raised when a tile exceeds it by more than
+// 2^6 (the weights then stay below 64, far inside fp16), so the accumulator is rescaled on a
+// handful of tiles instead of every one.  The per-channel K scale is folded into Q for the
+// prefix tiles; the V scale is applied to the accumulator once, when the walk passes from
+// the prefix to the chunk.  K/V tiles are double-buffered in LDS with the next tile's
+// global loads in flight during the current tile's MFMAs; one barrier per tile.
+//
+// LDS rows: K 272 B apart (the 32 rows a ds_read_b128 touches fall on distinct banks), V
+// 320 B apart (the 4 rows x 64 B a ds_read_b64_tr_b16 half-wave touches fall on distinct
+// banks); both tiles are written as whole 256 B rows by 16 consecutive lanes.
 #include "prefill.h"
 
 namespace fdattn {
 
 namespace {
 
-constexpr int BM = 128, BN = 64, HD = 128;
-constexpr int LDK = 136;  // bf16 elements per LDS row (272 B: 16-byte aligned, off the 256 B bank period)
-constexpr int TILE_ELEMS = BN * LDK;
+constexpr int BN = 64, HD = 128;
+constexpr int LDK = 136;  // 16-bit elements per K row in LDS (272 B)
+constexpr int LDV = 160;  // 16-bit elements per V row in LDS (320 B)
+constexpr int K_ELEMS = BN * LDK, BUF_ELEMS = BN * (LDK + LDV);
+constexpr int kSlots = 3;  // K/V tiles resident in LDS
+constexpr float kRaise = 6.0f;  // log2 of the largest softmax weight tolerated before the maximum is raised
 
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
@@ -37,6 +55,14 @@ typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 typedef short v4s __attribute__((ext_vector_type(4)));
 typedef short v8s __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+
+// how a cache byte sits in fp16: value = kMul^-1 (byte value + kOff)
+template <int QUANT>
+struct ByteFmt {
+  static constexpr float kMul = QUANT == FDATTN_CACHE_INT8 ? 16777216.0f : 1.0f;
+  static constexpr float kOff = QUANT == FDATTN_CACHE_INT8 ? 128.0f : 0.0f;
+};
 
 __device__ __forceinline__ u32 pack_bf16(float lo, float hi) {
   return (u32)f32_to_bf16(lo) | ((u32)f32_to_bf16(hi) << 16);
@@ -46,42 +72,241 @@ __device__ __forceinline__ u32 pack_f16(float lo, float hi) {
   const v2h v = {(_Float16)lo, (_Float16)hi};
   return __builtin_bit_cast(u32, v);
 }
-// two floats -> packed fp16 in one instruction (round toward zero): exact for cache values
-// (integers up to 127, e4m3 values), a 2^-11 downward nudge for softmax weights
+// two floats -> packed fp16 in one instruction (round toward zero): exact for e4m3 values,
+// a 2^-11 downward nudge for softmax weights
 __device__ __forceinline__ u32 pack_f16_fast(float lo, float hi) {
   return __builtin_bit_cast(u32, __builtin_amdgcn_cvt_pkrtz(lo, hi));
 }
-__device__ __forceinline__ float sat_f16(float x) { return fminf(fmaxf(x, -65504.0f), 65504.0f); }
+__device__ __forceinline__ float sat_f16(float x) { return __builtin_amdgcn_fmed3f(x, -65504.0f, 65504.0f); }
 
+// 8 cache bytes -> 8 fp16
 template <int QUANT>
-__device__ __forceinline__ float cvt8(u32 byte) {
-  if (QUANT == FDATTN_CACHE_INT8) return (float)(int)(int8_t)byte;
-  return __builtin_amdgcn_cvt_f32_fp8((int)byte, 0);
-}
-
-// 16 cache bytes -> 16 fp16 (two 16-byte LDS stores)
-template <int QUANT>
-__device__ __forceinline__ void cvt16_store(uint4 w, uint16_t* dst) {
-  const u32 ws[4] = {w.x, w.y, w.z, w.w};
-  u32 o[8];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    o[2 * i] = pack_f16_fast(cvt8<QUANT>(ws[i] & 0xff), cvt8<QUANT>((ws[i] >> 8) & 0xff));
-    o[2 * i + 1] = pack_f16_fast(cvt8<QUANT>((ws[i] >> 16) & 0xff), cvt8<QUANT>(ws[i] >> 24));
+__device__ __forceinline__ uint4 cvt8(u32 w0, u32 w1) {
+  if (QUANT == FDATTN_CACHE_INT8) {
+    const u32 x0 = w0 ^ 0x80808080u, x1 = w1 ^ 0x80808080u;
+    return make_uint4(__builtin_amdgcn_perm(0u, x0, 0x0c010c00u), __builtin_amdgcn_perm(0u, x0, 0x0c030c02u),
+                      __builtin_amdgcn_perm(0u, x1, 0x0c010c00u), __builtin_amdgcn_perm(0u, x1, 0x0c030c02u));
   }
-  *reinterpret_cast<uint4*>(dst) = make_uint4(o[0], o[1], o[2], o[3]);
-  *reinterpret_cast<uint4*>(dst + 8) = make_uint4(o[4], o[5], o[6], o[7]);
+  const v2f a = __builtin_amdgcn_cvt_pk_f32_fp8((int)w0, false), b = __builtin_amdgcn_cvt_pk_f32_fp8((int)w0, true);
+  const v2f c = __builtin_amdgcn_cvt_pk_f32_fp8((int)w1, false), d = __builtin_amdgcn_cvt_pk_f32_fp8((int)w1, true);
+  return make_uint4(pack_f16_fast(a[0], a[1]), pack_f16_fast(b[0], b[1]), pack_f16_fast(c[0], c[1]),
+                    pack_f16_fast(d[0], d[1]));
 }
 
-struct Stage {  // one thread's share of a K tile and a V tile on its way to LDS
-  uint4 k[4], v[4];
-};
+// ---- the matrix phase, hand-scheduled.  Operands stream from LDS through six 4-register
+// buffers (v232..v255): up to twelve reads are in flight while an MFMA runs, a buffer is
+// refilled right after the MFMA that consumed it has issued, and every wait names exactly
+// the reads that may still be outstanding.  The blocks open with lgkmcnt(0) so that nothing
+// else (a scalar load returns out of order) disturbs the count.
+typedef u32 u4v __attribute__((ext_vector_type(4)));
+#define FD_OPERAND_REGS                                                                                       \
+  "v232", "v233", "v234", "v235", "v236", "v237", "v238", "v239", "v240", "v241", "v242", "v243", "v244", "v245", \
+      "v246", "v247", "v248", "v249", "v250", "v251", "v252", "v253", "v254", "v255", "memory"
+
+// O^T[ct] += V^T P^T over one 64-key tile; va = LDS byte address of this lane's first V row
+__device__ __forceinline__ void pv_tile(v16f (&o)[4], const v8h (&pf)[2][2], u32 va) {
+  asm volatile(
+      "s_waitcnt lgkmcnt(0)\n\t"
+      "ds_read_b64_tr_b16 v[232:233], %[va] offset:0\n\t"
+      "ds_read_b64_tr_b16 v[234:235], %[va] offset:2560\n\t"
+      "ds_read_b64_tr_b16 v[236:237], %[va] offset:64\n\t"
+      "ds_read_b64_tr_b16 v[238:239], %[va] offset:2624\n\t"
+      "ds_read_b64_tr_b16 v[240:241], %[va] offset:128\n\t"
+      "ds_read_b64_tr_b16 v[242:243], %[va] offset:2688\n\t"
+      "ds_read_b64_tr_b16 v[244:245], %[va] offset:192\n\t"
+      "ds_read_b64_tr_b16 v[246:247], %[va] offset:2752\n\t"
+      "ds_read_b64_tr_b16 v[248:249], %[va] offset:5120\n\t"
+      "ds_read_b64_tr_b16 v[250:251], %[va] offset:7680\n\t"
+      "ds_read_b64_tr_b16 v[252:253], %[va] offset:5184\n\t"
+      "ds_read_b64_tr_b16 v[254:255], %[va] offset:7744\n\t"
+      "s_waitcnt lgkmcnt(10)\n\t"
+      "v_mfma_f32_32x32x16_f16 %[o0], v[232:235], %[p00], %[o0]\n\t"
+      "ds_read_b64_tr_b16 v[232:233], %[va] offset:5248\n\t"
+      "ds_read_b64_tr_b16 v[234:235], %[va] offset:7808\n\t"
+      "s_waitcnt lgkmcnt(10)\n\t"
+      "v_mfma_f32_32x32x16_f16 %[o1], v[236:239], %[p00], %[o1]\n\t"
+      "ds_read_b64_tr_b16 v[236:237], %[va] offset:5312\n\t"
+      "ds_read_b64_tr_b16 v[238:239], %[va] offset:7872\n\t"
+      "s_waitcnt lgkmcnt(10)\n\t"
+      "v_mfma_f32_32x32x16_f16 %[o2], v[240:243], %[p00], %[o2]\n\t"
+      "ds_read_b64_tr_b16 v[240:241], %[va] offset:10240\n\t"
+      "ds_read_b64_tr_b16 v[242:243], %[va] offset:12800\n\t"
+      "s_waitcnt lgkmcnt(10)\n\t"
+      "v_mfma_f32_32x32x16_f16 %[o3], v[244:247], %[p00], %[o3]\n\t"
+      "ds_read_b64_tr_b16 v[244:245], %[va] offset:10304\n\t"
+      "ds_read_b64_tr_b16 v[246:247], %[va] offset:12864\n\t"
+      "s_waitcnt lgkmcnt(10)\n\t"
+      "v_mfma_f32_32x32x16_f16 %[o0], v[248:251], %[p01], %[o0]\n\t"
+      "ds_read_b64_tr_b16 v[248:249], %[va] offset:10368\n\t"
+      "ds_read_b64_tr_b16 v[250:251], %[va] offset:12928\n\t"
+      "s_waitcnt lgkmcnt(10)\n\t"
+      "v_mfma_f32_32x32x16_f16 %[o1], v[252:255], %[p01], %[o1]\n\t"
+      "ds_read_b64_tr_b16 v[252:253], %[va] offset:10432\n\t"
+      "ds_read_b64_tr_b16 v[254:255], %[va] offset:12992\n\t"
+      "s_waitcnt lgkmcnt(10)\n\t"
+      "v_mfma_f32_32x32x16_f16 %[o2], v[232:235], %[p01], %[o2]\n\t"
+      "ds_read_b64_tr_b16 v[232:233], %[va] offset:15360\n\t"
+      "ds_read_b64_tr_b16 v[234:235], %[va] offset:17920\n\t"
+      "s_waitcnt lgkmcnt(10)\n\t"
+      "v_mfma_f32_32x32x16_f16 %[o3], v[236:239], %[p01], %[o3]\n\t"
+      "ds_read_b64_tr_b16 v[236:237], %[va] offset:15424\n\t"
+      "ds_read_b64_tr_b16 v[238:239], %[va] offset:17984\n\t"
+      "s_waitcnt lgkmcnt(10)\n\t"
+      "v_mfma_f32_32x32x16_f16 %[o0], v[240:243], %[p10], %[o0]\n\t"
+      "ds_read_b64_tr_b16 v[240:241], %[va] offset:15488\n\t"
+      "ds_read_b64_tr_b16 v[242:243], %[va] offset:18048\n\t"
+      "s_waitcnt lgkmcnt(10)\n\t"
+      "v_mfma_f32_32x32x16_f16 %[o1], v[244:247], %[p10], %[o1]\n\t"
+      "ds_read_b64_tr_b16 v[244:245], %[va] offset:15552\n\t"
+      "ds_read_b64_tr_b16 v[246:247], %[va] offset:18112\n\t"
+      "s_waitcnt lgkmcnt(10)\n\t"
+      "v_mfma_f32_32x32x16_f16 %[o2], v[248:251], %[p10], %[o2]\n\t"
+      "s_waitcnt lgkmcnt(8)\n\t"
+      "v_mfma_f32_32x32x16_f16 %[o3], v[252:255], %[p10], %[o3]\n\t"
+      "s_waitcnt lgkmcnt(6)\n\t"
+      "v_mfma_f32_32x32x16_f16 %[o0], v[232:235], %[p11], %[o0]\n\t"
+      "s_waitcnt lgkmcnt(4)\n\t"
+      "v_mfma_f32_32x32x16_f16 %[o1], v[236:239], %[p11], %[o1]\n\t"
+      "s_waitcnt lgkmcnt(2)\n\t"
+      "v_mfma_f32_32x32x16_f16 %[o2], v[240:243], %[p11], %[o2]\n\t"
+      "s_waitcnt lgkmcnt(0)\n\t"
+      "v_mfma_f32_32x32x16_f16 %[o3], v[244:247], %[p11], %[o3]\n\t"
+      : [o0] "+v"(o[0]), [o1] "+v"(o[1]), [o2] "+v"(o[2]), [o3] "+v"(o[3])
+      : [va] "v"(va), [p00] "v"(pf[0][0]), [p01] "v"(pf[0][1]), [p10] "v"(pf[1][0]), [p11] "v"(pf[1][1])
+      : FD_OPERAND_REGS);
+}
+// S^T = K Q^T over one 64-key tile (two 32-key accumulators); ka = LDS byte address of this
+// lane's first K row; F16 picks the fp16 MFMA (prefix tiles), else bf16 (the chunk's own keys)
+template <bool F16>
+__device__ __forceinline__ void qk_tile(v16f& a0, v16f& a1, const uint4 (&qf)[8], u32 ka) {
+  const u4v q0 = {qf[0].x, qf[0].y, qf[0].z, qf[0].w}, q1 = {qf[1].x, qf[1].y, qf[1].z, qf[1].w};
+  const u4v q2 = {qf[2].x, qf[2].y, qf[2].z, qf[2].w}, q3 = {qf[3].x, qf[3].y, qf[3].z, qf[3].w};
+  const u4v q4 = {qf[4].x, qf[4].y, qf[4].z, qf[4].w}, q5 = {qf[5].x, qf[5].y, qf[5].z, qf[5].w};
+  const u4v q6 = {qf[6].x, qf[6].y, qf[6].z, qf[6].w}, q7 = {qf[7].x, qf[7].y, qf[7].z, qf[7].w};
+  if (F16) {
+    asm volatile(
+        "s_waitcnt lgkmcnt(0)\n\t"
+        "ds_read_b128 v[232:235], %[ka] offset:0\n\t"
+        "ds_read_b128 v[236:239], %[ka] offset:8704\n\t"
+        "ds_read_b128 v[240:243], %[ka] offset:32\n\t"
+        "ds_read_b128 v[244:247], %[ka] offset:8736\n\t"
+        "ds_read_b128 v[248:251], %[ka] offset:64\n\t"
+        "ds_read_b128 v[252:255], %[ka] offset:8768\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_f16 %[a0], v[232:235], %[q0], 0\n\t"
+        "ds_read_b128 v[232:235], %[ka] offset:96\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_f16 %[a1], v[236:239], %[q0], 0\n\t"
+        "ds_read_b128 v[236:239], %[ka] offset:8800\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_f16 %[a0], v[240:243], %[q1], %[a0]\n\t"
+        "ds_read_b128 v[240:243], %[ka] offset:128\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_f16 %[a1], v[244:247], %[q1], %[a1]\n\t"
+        "ds_read_b128 v[244:247], %[ka] offset:8832\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_f16 %[a0], v[248:251], %[q2], %[a0]\n\t"
+        "ds_read_b128 v[248:251], %[ka] offset:160\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_f16 %[a1], v[252:255], %[q2], %[a1]\n\t"
+        "ds_read_b128 v[252:255], %[ka] offset:8864\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_f16 %[a0], v[232:235], %[q3], %[a0]\n\t"
+        "ds_read_b128 v[232:235], %[ka] offset:192\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_f16 %[a1], v[236:239], %[q3], %[a1]\n\t"
+        "ds_read_b128 v[236:239], %[ka] offset:8896\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_f16 %[a0], v[240:243], %[q4], %[a0]\n\t"
+        "ds_read_b128 v[240:243], %[ka] offset:224\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_f16 %[a1], v[244:247], %[q4], %[a1]\n\t"
+        "ds_read_b128 v[244:247], %[ka] offset:8928\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_f16 %[a0], v[248:251], %[q5], %[a0]\n\t"
+        "s_waitcnt lgkmcnt(4)\n\t"
+        "v_mfma_f32_32x32x16_f16 %[a1], v[252:255], %[q5], %[a1]\n\t"
+        "s_waitcnt lgkmcnt(3)\n\t"
+        "v_mfma_f32_32x32x16_f16 %[a0], v[232:235], %[q6], %[a0]\n\t"
+        "s_waitcnt lgkmcnt(2)\n\t"
+        "v_mfma_f32_32x32x16_f16 %[a1], v[236:239], %[q6], %[a1]\n\t"
+        "s_waitcnt lgkmcnt(1)\n\t"
+        "v_mfma_f32_32x32x16_f16 %[a0], v[240:243], %[q7], %[a0]\n\t"
+        "s_waitcnt lgkmcnt(0)\n\t"
+        "v_mfma_f32_32x32x16_f16 %[a1], v[244:247], %[q7], %[a1]\n\t"
+        : [a0] "=&v"(a0), [a1] "=&v"(a1)
+        : [ka] "v"(ka), [q0] "v"(q0), [q1] "v"(q1), [q2] "v"(q2), [q3] "v"(q3), [q4] "v"(q4), [q5] "v"(q5),
+          [q6] "v"(q6), [q7] "v"(q7)
+        : FD_OPERAND_REGS);
+  } else {
+    asm volatile(
+        "s_waitcnt lgkmcnt(0)\n\t"
+        "ds_read_b128 v[232:235], %[ka] offset:0\n\t"
+        "ds_read_b128 v[236:239], %[ka] offset:8704\n\t"
+        "ds_read_b128 v[240:243], %[ka] offset:32\n\t"
+        "ds_read_b128 v[244:247], %[ka] offset:8736\n\t"
+        "ds_read_b128 v[248:251], %[ka] offset:64\n\t"
+        "ds_read_b128 v[252:255], %[ka] offset:8768\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[a0], v[232:235], %[q0], 0\n\t"
+        "ds_read_b128 v[232:235], %[ka] offset:96\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[a1], v[236:239], %[q0], 0\n\t"
+        "ds_read_b128 v[236:239], %[ka] offset:8800\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[a0], v[240:243], %[q1], %[a0]\n\t"
+        "ds_read_b128 v[240:243], %[ka] offset:128\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[a1], v[244:247], %[q1], %[a1]\n\t"
+        "ds_read_b128 v[244:247], %[ka] offset:8832\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[a0], v[248:251], %[q2], %[a0]\n\t"
+        "ds_read_b128 v[248:251], %[ka] offset:160\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[a1], v[252:255], %[q2], %[a1]\n\t"
+        "ds_read_b128 v[252:255], %[ka] offset:8864\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[a0], v[232:235], %[q3], %[a0]\n\t"
+        "ds_read_b128 v[232:235], %[ka] offset:192\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[a1], v[236:239], %[q3], %[a1]\n\t"
+        "ds_read_b128 v[236:239], %[ka] offset:8896\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[a0], v[240:243], %[q4], %[a0]\n\t"
+        "ds_read_b128 v[240:243], %[ka] offset:224\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[a1], v[244:247], %[q4], %[a1]\n\t"
+        "ds_read_b128 v[244:247], %[ka] offset:8928\n\t"
+        "s_waitcnt lgkmcnt(5)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[a0], v[248:251], %[q5], %[a0]\n\t"
+        "s_waitcnt lgkmcnt(4)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[a1], v[252:255], %[q5], %[a1]\n\t"
+        "s_waitcnt lgkmcnt(3)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[a0], v[232:235], %[q6], %[a0]\n\t"
+        "s_waitcnt lgkmcnt(2)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[a1], v[236:239], %[q6], %[a1]\n\t"
+        "s_waitcnt lgkmcnt(1)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[a0], v[240:243], %[q7], %[a0]\n\t"
+        "s_waitcnt lgkmcnt(0)\n\t"
+        "v_mfma_f32_32x32x16_bf16 %[a1], v[244:247], %[q7], %[a1]\n\t"
+        : [a0] "=&v"(a0), [a1] "=&v"(a1)
+        : [ka] "v"(ka), [q0] "v"(q0), [q1] "v"(q1), [q2] "v"(q2), [q3] "v"(q3), [q4] "v"(q4), [q5] "v"(q5),
+          [q6] "v"(q6), [q7] "v"(q7)
+        : FD_OPERAND_REGS);
+  }
+}
+__device__ __forceinline__ u32 lds_addr(const void* p) {
+  return (u32)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
+}
 
 }  // namespace
 
-template <int QUANT>
-__global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs a) {
-  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];  // [2 buffers][K tile, V tile][64][LDK] 16-bit
+template <int QUANT, int NW>
+__global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
+  constexpr int BM = 32 * NW;       // queries per workgroup
+  constexpr int PASSES = 16 / NW;   // 16-byte LDS chunks a thread stages per tile and tensor
+  constexpr int ROWS = 2 * NW;      // tile rows covered by one staging pass of one wavefront group
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];  // [kSlots][K tile | V tile]
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int b = blockIdx.z, qh = blockIdx.y, h = qh / (a.hq / a.hkv);
   const int tok0 = a.cu_seqlens_q[b], n_b = a.cu_seqlens_q[b + 1] - tok0, p = a.seq_lens_decoder[b];
@@ -100,10 +325,12 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs a) {
   const int n_chk = (min(n_b, q0 + BM) + BN - 1) / BN;
   const int n_tiles = n_pre + n_chk;
   const int32_t* table = a.block_tables + (size_t)b * a.max_blocks;
+  const float sc = a.sm_scale * 1.4426950408889634f;  // logits go to the log2 domain
 
   // ---- Q as the B operand: lane = query, 8 channels per k-step
   const uint16_t* qrow = a.q + ((size_t)(tok0 + ci) * a.hq + qh) * HD;
-  uint4 qf[8];  // fp16 (q * k_scale) while the prefix is walked, bf16 q for the chunk
+  uint4 qf[8];       // fp16 (q * k_scale) while the prefix is walked, bf16 q for the chunk
+  float qsum = 0.f;  // sum over this lane's 64 channels of the rounded q * k_scale
   auto load_q = [&](bool scaled) {
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
@@ -112,59 +339,77 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs a) {
       if (scaled) {
         const float4 s0 = *reinterpret_cast<const float4*>(a.k_scale + h * HD + c0);
         const float4 s1 = *reinterpret_cast<const float4*>(a.k_scale + h * HD + c0 + 4);
-        w.x = pack_f16(bf16lo_to_f32(w.x) * s0.x, bf16hi_to_f32(w.x) * s0.y);
-        w.y = pack_f16(bf16lo_to_f32(w.y) * s0.z, bf16hi_to_f32(w.y) * s0.w);
-        w.z = pack_f16(bf16lo_to_f32(w.z) * s1.x, bf16hi_to_f32(w.z) * s1.y);
-        w.w = pack_f16(bf16lo_to_f32(w.w) * s1.z, bf16hi_to_f32(w.w) * s1.w);
+        const v2h h0 = {(_Float16)(bf16lo_to_f32(w.x) * s0.x), (_Float16)(bf16hi_to_f32(w.x) * s0.y)};
+        const v2h h1 = {(_Float16)(bf16lo_to_f32(w.y) * s0.z), (_Float16)(bf16hi_to_f32(w.y) * s0.w)};
+        const v2h h2 = {(_Float16)(bf16lo_to_f32(w.z) * s1.x), (_Float16)(bf16hi_to_f32(w.z) * s1.y)};
+        const v2h h3 = {(_Float16)(bf16lo_to_f32(w.w) * s1.z), (_Float16)(bf16hi_to_f32(w.w) * s1.w)};
+        qsum += ((float)h0[0] + (float)h0[1]) + ((float)h1[0] + (float)h1[1]) + ((float)h2[0] + (float)h2[1]) +
+                ((float)h3[0] + (float)h3[1]);
+        w = make_uint4(__builtin_bit_cast(u32, h0), __builtin_bit_cast(u32, h1), __builtin_bit_cast(u32, h2),
+                       __builtin_bit_cast(u32, h3));
       }
       qf[s] = w;
     }
   };
 
-  // ---- staging: thread tid moves key tid/4, channels 32*(tid%4) .. +31 of a tile
-  const int skey = tid >> 2, sc0 = (tid & 3) * 32;
-  Stage stg;
+  // ---- the two wavefront groups.  Group 0 (the first NW/2 wavefronts) and group 1 run the
+  // same per-tile sequence  [matrix phase: O += V P of the previous tile, S = K Q of this
+  // tile]  barrier  [vector phase: softmax of this tile, staging]  barrier,  but group 1
+  // starts one barrier late: while one group keeps the MFMA units busy the other one keeps
+  // the vector ALU busy (wavefronts w and w + NW/2 share a SIMD).
+  const int grp = wv / (NW / 2);
+  const int gtid = tid - grp * 32 * NW;
+  const int lead = 1 + grp;  // in the vector phase of tile t a group stages its rows of tile t + lead
+
+  // ---- staging: a group's 32*NW threads move rows 32*grp .. 32*grp+31 of a tile, one
+  // 16-byte LDS chunk (8 channels) per thread and pass
+  const int srow = 32 * grp + (gtid >> 4), scc = (gtid & 15) * 8;
+  uint4 stg_k[PASSES], stg_v[PASSES];
   auto fetch = [&](int t) {
+    if (t >= n_tiles) return;
     if (t < n_pre) {
       int pb = table[t];
       pb = (pb >= 0 && pb < a.num_blocks) ? pb : 0;
-      const size_t off = (((size_t)pb * a.hkv + h) * BN + skey) * HD + sc0;
-      stg.k[0] = *reinterpret_cast<const uint4*>(a.key_cache + off);
-      stg.k[1] = *reinterpret_cast<const uint4*>(a.key_cache + off + 16);
-      stg.v[0] = *reinterpret_cast<const uint4*>(a.value_cache + off);
-      stg.v[1] = *reinterpret_cast<const uint4*>(a.value_cache + off + 16);
-    } else {
-      const int j = min((t - n_pre) * BN + skey, n_b - 1);  // keys past the chunk are masked later
-      const size_t off = ((size_t)(tok0 + j) * a.hkv + h) * HD + sc0;
+      const size_t off = (((size_t)pb * a.hkv + h) * BN + srow) * HD + scc;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        stg.k[i] = *reinterpret_cast<const uint4*>(a.k_new + off + 8 * i);
-        stg.v[i] = *reinterpret_cast<const uint4*>(a.v_new + off + 8 * i);
+      for (int i = 0; i < PASSES; ++i) {
+        const uint2 kk = *reinterpret_cast<const uint2*>(a.key_cache + off + (size_t)i * ROWS * HD);
+        const uint2 vv = *reinterpret_cast<const uint2*>(a.value_cache + off + (size_t)i * ROWS * HD);
+        stg_k[i].x = kk.x, stg_k[i].y = kk.y, stg_v[i].x = vv.x, stg_v[i].y = vv.y;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < PASSES; ++i) {
+        const int j = min((t - n_pre) * BN + srow + i * ROWS, n_b - 1);  // keys past the chunk are masked later
+        const size_t off = ((size_t)(tok0 + j) * a.hkv + h) * HD + scc;
+        stg_k[i] = *reinterpret_cast<const uint4*>(a.k_new + off);
+        stg_v[i] = *reinterpret_cast<const uint4*>(a.v_new + off);
       }
     }
   };
-  auto commit = [&](int t, int buf) {
-    uint16_t* kd = lds + (size_t)buf * 2 * TILE_ELEMS + skey * LDK + sc0;
-    uint16_t* vd = kd + TILE_ELEMS;
+  auto commit = [&](int t) {
+    if (t >= n_tiles) return;
+    uint16_t* kd = lds + (size_t)(t % kSlots) * BUF_ELEMS + srow * LDK + scc;
+    uint16_t* vd = lds + (size_t)(t % kSlots) * BUF_ELEMS + K_ELEMS + srow * LDV + scc;
     if (t < n_pre) {
-      if (t * BN + skey >= p) {
-        // rows past the cached prefix hold stale bytes (fp8 has NaN codes, and 0 * NaN would
-        // poison the second product): stage zeros for them
-        stg.k[0] = stg.k[1] = stg.v[0] = stg.v[1] = make_uint4(0, 0, 0, 0);
+      // rows past the cached prefix hold stale bytes (fp8 has NaN codes, and 0 * NaN would
+      // poison the second product): zero bytes are staged for them
+      const bool ragged = (t + 1) * BN > p;
+#pragma unroll
+      for (int i = 0; i < PASSES; ++i) {
+        if (ragged && t * BN + srow + i * ROWS >= p) stg_k[i].x = stg_k[i].y = stg_v[i].x = stg_v[i].y = 0u;
+        *reinterpret_cast<uint4*>(kd + i * ROWS * LDK) = cvt8<QUANT>(stg_k[i].x, stg_k[i].y);
+        *reinterpret_cast<uint4*>(vd + i * ROWS * LDV) = cvt8<QUANT>(stg_v[i].x, stg_v[i].y);
       }
-      cvt16_store<QUANT>(stg.k[0], kd);
-      cvt16_store<QUANT>(stg.k[1], kd + 16);
-      cvt16_store<QUANT>(stg.v[0], vd);
-      cvt16_store<QUANT>(stg.v[1], vd + 16);
     } else {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        *reinterpret_cast<uint4*>(kd + 8 * i) = stg.k[i];
-        const u32 vw[4] = {stg.v[i].x, stg.v[i].y, stg.v[i].z, stg.v[i].w};
+      for (int i = 0; i < PASSES; ++i) {
+        *reinterpret_cast<uint4*>(kd + i * ROWS * LDK) = stg_k[i];
+        const u32 vw[4] = {stg_v[i].x, stg_v[i].y, stg_v[i].z, stg_v[i].w};
         u32 hw[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) hw[e] = pack_f16(sat_f16(bf16lo_to_f32(vw[e])), sat_f16(bf16hi_to_f32(vw[e])));
-        *reinterpret_cast<uint4*>(vd + 8 * i) = make_uint4(hw[0], hw[1], hw[2], hw[3]);
+        *reinterpret_cast<uint4*>(vd + i * ROWS * LDV) = make_uint4(hw[0], hw[1], hw[2], hw[3]);
       }
     }
   };
@@ -174,77 +419,103 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs a) {
   for (int ct = 0; ct < 4; ++ct)
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[ct][r] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
-  const float sc = a.sm_scale * 1.4426950408889634f;  // logits go to the log2 domain
+  float m_ref = -INFINITY;  // exponent reference of the weights (at most kRaise below the true maximum)
+  float l_run = 0.f;        // this lane's share (its 16 of every 32 keys) of the weight sum
+
+  // tiles this wavefront computes on; chunk tiles wholly above its diagonal contribute
+  // nothing and it only helps staging them
+  const int my_tiles = wave_active ? n_pre + ci_wave_max / BN + 1 : 0;
+  const int q16 = lane >> 4, i16 = lane & 15;
 
   load_q(n_pre > 0);
+  // log2-domain constant that removes the byte offset from the prefix scores
+  const float qbias = -ByteFmt<QUANT>::kOff * sc * (qsum + __shfl_xor(qsum, 32, 64));
+
+  // prologue: tile 0 (and group 1's rows of tile 1) into LDS, the next one into registers
   fetch(0);
-  for (int t = 0; t < n_tiles; ++t) {
-    const int buf = t & 1;
-    commit(t, buf);
-    __syncthreads();
-    if (t + 1 < n_tiles) fetch(t + 1);
-    if (t == n_pre && n_pre > 0) {
-      // leaving the quantised prefix: o holds sums over int8/fp8 values, give them their scale
-      load_q(false);
-#pragma unroll
-      for (int ct = 0; ct < 4; ++ct)
-#pragma unroll
-        for (int rb = 0; rb < 4; ++rb) {
-          const float4 vs = *reinterpret_cast<const float4*>(a.v_scale + h * HD + 32 * ct + 8 * rb + 4 * hf);
-          o[ct][4 * rb + 0] *= vs.x;
-          o[ct][4 * rb + 1] *= vs.y;
-          o[ct][4 * rb + 2] *= vs.z;
-          o[ct][4 * rb + 3] *= vs.w;
-        }
+  commit(0);
+  if (grp == 1) {
+    fetch(1);
+    commit(1);
+  }
+  fetch(lead);
+  __syncthreads();
+  if (grp == 1) __syncthreads();  // group 1 trails by one phase
+
+  v16f st[2];
+  v8h pf[2][2];
+  for (int t = 0; t <= n_tiles; ++t) {
+    // ================= matrix phase =================
+    if (t == n_pre && n_pre > 0 && t < my_tiles) load_q(false);  // the chunk's scores meet the bf16 q
+    if (t >= 1 && t <= my_tiles) {
+      // ---- O^T += V^T P^T, tile t-1.  k-slot e of lane group hf is key 32kb + 16ss + 8(e/4) +
+      // 4hf + e%4 (the P^T layout); lane i16 supplies the row (key kbase + i16/4, channels
+      // cbase + 4(i16%4)..+3)
+      pv_tile(o, pf, lds_addr(lds + (size_t)((t - 1) % kSlots) * BUF_ELEMS + K_ELEMS + (4 * hf + (i16 >> 2)) * LDV +
+                              16 * (q16 & 1) + 4 * (i16 & 3)));
     }
-    const bool is_pre = t < n_pre;
-    const int key0 = is_pre ? t * BN : (t - n_pre) * BN;  // index of the tile's first key in its segment
-    // a chunk tile wholly above this wavefront's diagonal contributes nothing
-    const bool skip = !wave_active || (!is_pre && key0 > ci_wave_max);
-    if (!skip) {
-      const uint16_t* kt = lds + (size_t)buf * 2 * TILE_ELEMS;
-      const uint16_t* vt = kt + TILE_ELEMS;
-      // ---- S^T = K Q^T
-      v16f st[2];
+    if (t < my_tiles) {
+      // ---- S^T = K Q^T, tile t
+      const u32 ka = lds_addr(lds + (size_t)(t % kSlots) * BUF_ELEMS + j32 * LDK + 8 * hf);
+      if (t < n_pre)
+        qk_tile<true>(st[0], st[1], qf, ka);
+      else
+        qk_tile<false>(st[0], st[1], qf, ka);
+    }
+    __syncthreads();
+    // ================= vector phase =================
+    if (t < my_tiles) {
+      if (t == n_pre && n_pre > 0) {
+        // leaving the quantised prefix: o holds sums over offset bytes; remove the offset
+        // and give the channels their scale
+        const float l_off = -ByteFmt<QUANT>::kOff * (l_run + __shfl_xor(l_run, 32, 64));
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        v16f acc;
+        for (int ct = 0; ct < 4; ++ct)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-#pragma unroll
-        for (int s = 0; s < 8; ++s) {
-          const uint4 w = *reinterpret_cast<const uint4*>(kt + (32 * kb + j32) * LDK + 16 * s + 8 * hf);
-          if (is_pre)
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, w), __builtin_bit_cast(v8h, qf[s]), acc, 0, 0, 0);
-          else
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, w), __builtin_bit_cast(v8bf, qf[s]), acc, 0, 0, 0);
-        }
-        st[kb] = acc;
+          for (int rb = 0; rb < 4; ++rb) {
+            const float4 vs = *reinterpret_cast<const float4*>(a.v_scale + h * HD + 32 * ct + 8 * rb + 4 * hf);
+            o[ct][4 * rb + 0] = (o[ct][4 * rb + 0] * ByteFmt<QUANT>::kMul + l_off) * vs.x;
+            o[ct][4 * rb + 1] = (o[ct][4 * rb + 1] * ByteFmt<QUANT>::kMul + l_off) * vs.y;
+            o[ct][4 * rb + 2] = (o[ct][4 * rb + 2] * ByteFmt<QUANT>::kMul + l_off) * vs.z;
+            o[ct][4 * rb + 3] = (o[ct][4 * rb + 3] * ByteFmt<QUANT>::kMul + l_off) * vs.w;
+          }
       }
       // ---- mask + online softmax; this lane: one query, keys 32kb + (r%4) + 8(r/4) + 4hf
-      const int limit = is_pre ? p - key0 : ci - key0 + 1;  // keys [0, limit) of the tile are visible
-      const bool need_mask = is_pre ? (key0 + BN > p) : (key0 + BN > q0 + 32 * wv + 1);
+      const bool pre = t < n_pre;
+      const int key0 = pre ? t * BN : (t - n_pre) * BN;  // index of the tile's first key in its segment
+      const int limit = pre ? p - key0 : ci - key0 + 1;  // keys [0, limit) of the tile are visible
+      const bool need_mask = pre ? (key0 + BN > p) : (key0 + BN > q0 + 32 * wv + 1);
+      if (need_mask) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int key = 32 * kb + (r & 3) + 8 * (r >> 2) + 4 * hf;
+            st[kb][r] = key < limit ? st[kb][r] : -INFINITY;
+          }
+      }
       float mx = -INFINITY;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          float s = st[kb][r] * sc;
-          if (need_mask) {
-            const int key = 32 * kb + (r & 3) + 8 * (r >> 2) + 4 * hf;
-            s = key < limit ? s : -INFINITY;
-          }
-          st[kb][r] = s;
-          mx = fmaxf(mx, s);
-        }
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, st[kb][r]);
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m_run, mx);
-      const float m_use = m_new == -INFINITY ? 0.f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
-      m_run = m_new;
-      float psum = 0.f;
-      v8h pf[2][2];
+      // logit (log2 domain) = accumulator * scl + add
+      const float scl = pre ? sc * ByteFmt<QUANT>::kMul : sc;
+      const float add = pre ? qbias : 0.f;
+      mx = mx * scl + add;
+      const bool raise = mx > m_ref + kRaise;  // always true for the first visible key (m_ref = -inf)
+      if (__any(raise)) {
+        const float alpha = raise ? __builtin_amdgcn_exp2f(m_ref - mx) : 1.0f;
+        m_ref = raise ? mx : m_ref;
+        l_run *= alpha;
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[ct][r] *= alpha;
+      }
+      const float cst = add - (m_ref == -INFINITY ? 0.f : m_ref);
+      const v2h ones = {(_Float16)1.0f, (_Float16)1.0f};
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -252,37 +523,20 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs a) {
           u32 w[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const float p0 = __builtin_amdgcn_exp2f(st[kb][8 * ss + 2 * e] - m_use);
-            const float p1 = __builtin_amdgcn_exp2f(st[kb][8 * ss + 2 * e + 1] - m_use);
-            psum += p0 + p1;
+            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[kb][8 * ss + 2 * e], scl, cst));
+            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[kb][8 * ss + 2 * e + 1], scl, cst));
             w[e] = pack_f16_fast(p0, p1);
+            // the sum is taken over the rounded weights, the ones the MFMA multiplies
+            l_run = __builtin_amdgcn_fdot2(__builtin_bit_cast(v2h, w[e]), ones, l_run, false);
           }
           pf[kb][ss] = __builtin_bit_cast(v8h, make_uint4(w[0], w[1], w[2], w[3]));
         }
-      l_run = l_run * alpha + psum;
-      // ---- O^T = O^T * alpha + V^T P^T
-      const int q16 = lane >> 4, i16 = lane & 15;
-#pragma unroll
-      for (int ct = 0; ct < 4; ++ct) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) o[ct][r] *= alpha;
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int ss = 0; ss < 2; ++ss) {
-            // k-slot e of lane group hf is key 32kb + 16ss + 8(e/4) + 4hf + e%4 (the P^T layout);
-            // lane i16 supplies the row (key kbase + i16/4, channels cbase + 4(i16%4)..+3)
-            const int kbase = 32 * kb + 16 * ss + 4 * hf + (i16 >> 2);
-            const int cbase = 32 * ct + 16 * (q16 & 1) + 4 * (i16 & 3);
-            const uint16_t* src = vt + kbase * LDK + cbase;
-            const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)src);
-            const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(src + 8 * LDK));
-            const v8s vv = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-            o[ct] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, vv), pf[kb][ss], o[ct], 0, 0, 0);
-          }
-      }
     }
+    commit(t + lead);
+    fetch(t + lead + 1);
+    __syncthreads();
   }
+  if (grp == 0) __syncthreads();  // the barrier group 1 took before its first phase
 
   // ---- epilogue: normalise and store bf16 (every query saw at least its own chunk tile)
   if (!wave_active || ci_raw >= n_b) return;
@@ -305,28 +559,38 @@ bool prefill_mfma_supported(int hq, int hkv, int d, int bs, int quant) {
          (quant == FDATTN_CACHE_INT8 || quant == FDATTN_CACHE_FP8_E4M3);
 }
 
+namespace {
+
+template <int QUANT, int NW>
+hipError_t launch_one(const PrefillArgs& a, int max_chunk, hipStream_t s) {
+  constexpr int BM = 32 * NW;
+  const dim3 grid((max_chunk + BM - 1) / BM, a.hq, a.batch), block(64 * NW);
+  const size_t shm = (size_t)kSlots * BUF_ELEMS * sizeof(uint16_t);  // 113,664 B
+  static bool attr_set = false;  // one flag per instantiation
+  if (!attr_set) {
+    const hipError_t e = hipFuncSetAttribute((const void*)prefill_mfma_kernel<QUANT, NW>,
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((prefill_mfma_kernel<QUANT, NW>), grid, block, shm, s, a);
+  return hipSuccess;
+}
+
+}  // namespace
+
 int prefill_mfma_launch(const PrefillArgs& a, int max_chunk, int quant, hipStream_t s) {
-  const dim3 grid((max_chunk + BM - 1) / BM, a.hq, a.batch), block(256);
-  const size_t shm = (size_t)2 * 2 * TILE_ELEMS * sizeof(uint16_t);  // 69,632 B
   if (a.batch > 65535 || a.hq > 65535)
     return fail(FDATTN_ERR_SHAPE, "fdattn_append_attention_prefill: batch or head count exceeds the grid limit");
-  static bool attr_set[2] = {false, false};
-  hipError_t e = hipSuccess;
-  if (quant == FDATTN_CACHE_INT8) {
-    if (!attr_set[0]) {
-      e = hipFuncSetAttribute((const void*)prefill_mfma_kernel<FDATTN_CACHE_INT8>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);
-      attr_set[0] = e == hipSuccess;
-    }
-    if (e == hipSuccess) hipLaunchKernelGGL(prefill_mfma_kernel<FDATTN_CACHE_INT8>, grid, block, shm, s, a);
-  } else {
-    if (!attr_set[1]) {
-      e = hipFuncSetAttribute((const void*)prefill_mfma_kernel<FDATTN_CACHE_FP8_E4M3>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);
-      attr_set[1] = e == hipSuccess;
-    }
-    if (e == hipSuccess) hipLaunchKernelGGL(prefill_mfma_kernel<FDATTN_CACHE_FP8_E4M3>, grid, block, shm, s, a);
-  }
+  // 256-token workgroups share each staged tile among 8 wavefronts; short chunks keep 128
+  static const char* nw_env = getenv("FDATTN_PREFILL_NW");
+  const bool wide = nw_env ? atoi(nw_env) == 8 : max_chunk > 128;
+  hipError_t e;
+  if (quant == FDATTN_CACHE_INT8)
+    e = wide ? launch_one<FDATTN_CACHE_INT8, 8>(a, max_chunk, s) : launch_one<FDATTN_CACHE_INT8, 4>(a, max_chunk, s);
+  else
+    e = wide ? launch_one<FDATTN_CACHE_FP8_E4M3, 8>(a, max_chunk, s)
+             : launch_one<FDATTN_CACHE_FP8_E4M3, 4>(a, max_chunk, s);
   if (e != hipSuccess) return fail((int)e, "fdattn_append_attention_prefill: %s", hipGetErrorString(e));
   return check_launch("fdattn_append_attention_prefill (mfma)");
 }
