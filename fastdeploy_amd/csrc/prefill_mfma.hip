@@ -30,8 +30,14 @@
 // 2^6 (the weights then stay below 64, far inside fp16), so the accumulator is rescaled on a
 // handful of tiles instead of every one.  The per-channel K scale is folded into Q for the
 // prefix tiles; the V scale is applied to the accumulator once, when the walk passes from
-// the prefix to the chunk.  K/V tiles are double-buffered in LDS with the next tile's
-// global loads in flight during the current tile's MFMAs; one barrier per tile.
+// the prefix to the chunk.
+//
+// Schedule.  The wavefronts form two groups that alternate between a matrix phase (the two
+// MFMA streams of a tile, hand-scheduled: LDS operand reads six deep in flight, exact
+// s_waitcnt counts) and a vector phase (staging of a later tile, then the softmax), half a
+// tile out of step with each other, so that the MFMA units and the vector ALU of a SIMD are
+// fed by different wavefronts at the same time.  Three K/V tiles are resident in LDS; the
+// global loads of a tile are issued a whole tile before its bytes are converted.
 //
 // LDS rows: K 272 B apart (the 32 rows a ds_read_b128 touches fall on distinct banks), V
 // 320 B apart (the 4 rows x 64 B a ds_read_b64_tr_b16 half-wave touches fall on distinct
@@ -93,207 +99,20 @@ __device__ __forceinline__ uint4 cvt8(u32 w0, u32 w1) {
                     pack_f16_fast(d[0], d[1]));
 }
 
-// ---- the matrix phase, hand-scheduled.  Operands stream from LDS through six 4-register
-// buffers (v232..v255): up to twelve reads are in flight while an MFMA runs, a buffer is
-// refilled right after the MFMA that consumed it has issued, and every wait names exactly
-// the reads that may still be outstanding.  The blocks open with lgkmcnt(0) so that nothing
-// else (a scalar load returns out of order) disturbs the count.
+// ---- the matrix phase, hand-scheduled (generated by gen_prefill_sched.py).  Operands stream
+// from LDS through six 4-register buffers: up to twelve reads are in flight while an MFMA
+// runs, a buffer is refilled right after the MFMA that consumed it has issued, and every
+// wait names exactly the reads that may still be outstanding.  The blocks open with
+// lgkmcnt(0) so that nothing else (a scalar load returns out of order) disturbs the count.
 typedef u32 u4v __attribute__((ext_vector_type(4)));
-#define FD_OPERAND_REGS                                                                                       \
-  "v232", "v233", "v234", "v235", "v236", "v237", "v238", "v239", "v240", "v241", "v242", "v243", "v244", "v245", \
-      "v246", "v247", "v248", "v249", "v250", "v251", "v252", "v253", "v254", "v255", "memory"
+typedef u32 u2v __attribute__((ext_vector_type(2)));
+#include "prefill_mfma_sched.inc"
 
-// O^T[ct] += V^T P^T over one 64-key tile; va = LDS byte address of this lane's first V row
-__device__ __forceinline__ void pv_tile(v16f (&o)[4], const v8h (&pf)[2][2], u32 va) {
-  asm volatile(
-      "s_waitcnt lgkmcnt(0)\n\t"
-      "ds_read_b64_tr_b16 v[232:233], %[va] offset:0\n\t"
-      "ds_read_b64_tr_b16 v[234:235], %[va] offset:2560\n\t"
-      "ds_read_b64_tr_b16 v[236:237], %[va] offset:64\n\t"
-      "ds_read_b64_tr_b16 v[238:239], %[va] offset:2624\n\t"
-      "ds_read_b64_tr_b16 v[240:241], %[va] offset:128\n\t"
-      "ds_read_b64_tr_b16 v[242:243], %[va] offset:2688\n\t"
-      "ds_read_b64_tr_b16 v[244:245], %[va] offset:192\n\t"
-      "ds_read_b64_tr_b16 v[246:247], %[va] offset:2752\n\t"
-      "ds_read_b64_tr_b16 v[248:249], %[va] offset:5120\n\t"
-      "ds_read_b64_tr_b16 v[250:251], %[va] offset:7680\n\t"
-      "ds_read_b64_tr_b16 v[252:253], %[va] offset:5184\n\t"
-      "ds_read_b64_tr_b16 v[254:255], %[va] offset:7744\n\t"
-      "s_waitcnt lgkmcnt(10)\n\t"
-      "v_mfma_f32_32x32x16_f16 %[o0], v[232:235], %[p00], %[o0]\n\t"
-      "ds_read_b64_tr_b16 v[232:233], %[va] offset:5248\n\t"
-      "ds_read_b64_tr_b16 v[234:235], %[va] offset:7808\n\t"
-      "s_waitcnt lgkmcnt(10)\n\t"
-      "v_mfma_f32_32x32x16_f16 %[o1], v[236:239], %[p00], %[o1]\n\t"
-      "ds_read_b64_tr_b16 v[236:237], %[va] offset:5312\n\t"
-      "ds_read_b64_tr_b16 v[238:239], %[va] offset:7872\n\t"
-      "s_waitcnt lgkmcnt(10)\n\t"
-      "v_mfma_f32_32x32x16_f16 %[o2], v[240:243], %[p00], %[o2]\n\t"
-      "ds_read_b64_tr_b16 v[240:241], %[va] offset:10240\n\t"
-      "ds_read_b64_tr_b16 v[242:243], %[va] offset:12800\n\t"
-      "s_waitcnt lgkmcnt(10)\n\t"
-      "v_mfma_f32_32x32x16_f16 %[o3], v[244:247], %[p00], %[o3]\n\t"
-      "ds_read_b64_tr_b16 v[244:245], %[va] offset:10304\n\t"
-      "ds_read_b64_tr_b16 v[246:247], %[va] offset:12864\n\t"
-      "s_waitcnt lgkmcnt(10)\n\t"
-      "v_mfma_f32_32x32x16_f16 %[o0], v[248:251], %[p01], %[o0]\n\t"
-      "ds_read_b64_tr_b16 v[248:249], %[va] offset:10368\n\t"
-      "ds_read_b64_tr_b16 v[250:251], %[va] offset:12928\n\t"
-      "s_waitcnt lgkmcnt(10)\n\t"
-      "v_mfma_f32_32x32x16_f16 %[o1], v[252:255], %[p01], %[o1]\n\t"
-      "ds_read_b64_tr_b16 v[252:253], %[va] offset:10432\n\t"
-      "ds_read_b64_tr_b16 v[254:255], %[va] offset:12992\n\t"
-      "s_waitcnt lgkmcnt(10)\n\t"
-      "v_mfma_f32_32x32x16_f16 %[o2], v[232:235], %[p01], %[o2]\n\t"
-      "ds_read_b64_tr_b16 v[232:233], %[va] offset:15360\n\t"
-      "ds_read_b64_tr_b16 v[234:235], %[va] offset:17920\n\t"
-      "s_waitcnt lgkmcnt(10)\n\t"
-      "v_mfma_f32_32x32x16_f16 %[o3], v[236:239], %[p01], %[o3]\n\t"
-      "ds_read_b64_tr_b16 v[236:237], %[va] offset:15424\n\t"
-      "ds_read_b64_tr_b16 v[238:239], %[va] offset:17984\n\t"
-      "s_waitcnt lgkmcnt(10)\n\t"
-      "v_mfma_f32_32x32x16_f16 %[o0], v[240:243], %[p10], %[o0]\n\t"
-      "ds_read_b64_tr_b16 v[240:241], %[va] offset:15488\n\t"
-      "ds_read_b64_tr_b16 v[242:243], %[va] offset:18048\n\t"
-      "s_waitcnt lgkmcnt(10)\n\t"
-      "v_mfma_f32_32x32x16_f16 %[o1], v[244:247], %[p10], %[o1]\n\t"
-      "ds_read_b64_tr_b16 v[244:245], %[va] offset:15552\n\t"
-      "ds_read_b64_tr_b16 v[246:247], %[va] offset:18112\n\t"
-      "s_waitcnt lgkmcnt(10)\n\t"
-      "v_mfma_f32_32x32x16_f16 %[o2], v[248:251], %[p10], %[o2]\n\t"
-      "s_waitcnt lgkmcnt(8)\n\t"
-      "v_mfma_f32_32x32x16_f16 %[o3], v[252:255], %[p10], %[o3]\n\t"
-      "s_waitcnt lgkmcnt(6)\n\t"
-      "v_mfma_f32_32x32x16_f16 %[o0], v[232:235], %[p11], %[o0]\n\t"
-      "s_waitcnt lgkmcnt(4)\n\t"
-      "v_mfma_f32_32x32x16_f16 %[o1], v[236:239], %[p11], %[o1]\n\t"
-      "s_waitcnt lgkmcnt(2)\n\t"
-      "v_mfma_f32_32x32x16_f16 %[o2], v[240:243], %[p11], %[o2]\n\t"
-      "s_waitcnt lgkmcnt(0)\n\t"
-      "v_mfma_f32_32x32x16_f16 %[o3], v[244:247], %[p11], %[o3]\n\t"
-      : [o0] "+v"(o[0]), [o1] "+v"(o[1]), [o2] "+v"(o[2]), [o3] "+v"(o[3])
-      : [va] "v"(va), [p00] "v"(pf[0][0]), [p01] "v"(pf[0][1]), [p10] "v"(pf[1][0]), [p11] "v"(pf[1][1])
-      : FD_OPERAND_REGS);
-}
-// S^T = K Q^T over one 64-key tile (two 32-key accumulators); ka = LDS byte address of this
-// lane's first K row; F16 picks the fp16 MFMA (prefix tiles), else bf16 (the chunk's own keys)
-template <bool F16>
-__device__ __forceinline__ void qk_tile(v16f& a0, v16f& a1, const uint4 (&qf)[8], u32 ka) {
-  const u4v q0 = {qf[0].x, qf[0].y, qf[0].z, qf[0].w}, q1 = {qf[1].x, qf[1].y, qf[1].z, qf[1].w};
-  const u4v q2 = {qf[2].x, qf[2].y, qf[2].z, qf[2].w}, q3 = {qf[3].x, qf[3].y, qf[3].z, qf[3].w};
-  const u4v q4 = {qf[4].x, qf[4].y, qf[4].z, qf[4].w}, q5 = {qf[5].x, qf[5].y, qf[5].z, qf[5].w};
-  const u4v q6 = {qf[6].x, qf[6].y, qf[6].z, qf[6].w}, q7 = {qf[7].x, qf[7].y, qf[7].z, qf[7].w};
-  if (F16) {
-    asm volatile(
-        "s_waitcnt lgkmcnt(0)\n\t"
-        "ds_read_b128 v[232:235], %[ka] offset:0\n\t"
-        "ds_read_b128 v[236:239], %[ka] offset:8704\n\t"
-        "ds_read_b128 v[240:243], %[ka] offset:32\n\t"
-        "ds_read_b128 v[244:247], %[ka] offset:8736\n\t"
-        "ds_read_b128 v[248:251], %[ka] offset:64\n\t"
-        "ds_read_b128 v[252:255], %[ka] offset:8768\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_f16 %[a0], v[232:235], %[q0], 0\n\t"
-        "ds_read_b128 v[232:235], %[ka] offset:96\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_f16 %[a1], v[236:239], %[q0], 0\n\t"
-        "ds_read_b128 v[236:239], %[ka] offset:8800\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_f16 %[a0], v[240:243], %[q1], %[a0]\n\t"
-        "ds_read_b128 v[240:243], %[ka] offset:128\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_f16 %[a1], v[244:247], %[q1], %[a1]\n\t"
-        "ds_read_b128 v[244:247], %[ka] offset:8832\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_f16 %[a0], v[248:251], %[q2], %[a0]\n\t"
-        "ds_read_b128 v[248:251], %[ka] offset:160\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_f16 %[a1], v[252:255], %[q2], %[a1]\n\t"
-        "ds_read_b128 v[252:255], %[ka] offset:8864\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_f16 %[a0], v[232:235], %[q3], %[a0]\n\t"
-        "ds_read_b128 v[232:235], %[ka] offset:192\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_f16 %[a1], v[236:239], %[q3], %[a1]\n\t"
-        "ds_read_b128 v[236:239], %[ka] offset:8896\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_f16 %[a0], v[240:243], %[q4], %[a0]\n\t"
-        "ds_read_b128 v[240:243], %[ka] offset:224\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_f16 %[a1], v[244:247], %[q4], %[a1]\n\t"
-        "ds_read_b128 v[244:247], %[ka] offset:8928\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_f16 %[a0], v[248:251], %[q5], %[a0]\n\t"
-        "s_waitcnt lgkmcnt(4)\n\t"
-        "v_mfma_f32_32x32x16_f16 %[a1], v[252:255], %[q5], %[a1]\n\t"
-        "s_waitcnt lgkmcnt(3)\n\t"
-        "v_mfma_f32_32x32x16_f16 %[a0], v[232:235], %[q6], %[a0]\n\t"
-        "s_waitcnt lgkmcnt(2)\n\t"
-        "v_mfma_f32_32x32x16_f16 %[a1], v[236:239], %[q6], %[a1]\n\t"
-        "s_waitcnt lgkmcnt(1)\n\t"
-        "v_mfma_f32_32x32x16_f16 %[a0], v[240:243], %[q7], %[a0]\n\t"
-        "s_waitcnt lgkmcnt(0)\n\t"
-        "v_mfma_f32_32x32x16_f16 %[a1], v[244:247], %[q7], %[a1]\n\t"
-        : [a0] "=&v"(a0), [a1] "=&v"(a1)
-        : [ka] "v"(ka), [q0] "v"(q0), [q1] "v"(q1), [q2] "v"(q2), [q3] "v"(q3), [q4] "v"(q4), [q5] "v"(q5),
-          [q6] "v"(q6), [q7] "v"(q7)
-        : FD_OPERAND_REGS);
-  } else {
-    asm volatile(
-        "s_waitcnt lgkmcnt(0)\n\t"
-        "ds_read_b128 v[232:235], %[ka] offset:0\n\t"
-        "ds_read_b128 v[236:239], %[ka] offset:8704\n\t"
-        "ds_read_b128 v[240:243], %[ka] offset:32\n\t"
-        "ds_read_b128 v[244:247], %[ka] offset:8736\n\t"
-        "ds_read_b128 v[248:251], %[ka] offset:64\n\t"
-        "ds_read_b128 v[252:255], %[ka] offset:8768\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[a0], v[232:235], %[q0], 0\n\t"
-        "ds_read_b128 v[232:235], %[ka] offset:96\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[a1], v[236:239], %[q0], 0\n\t"
-        "ds_read_b128 v[236:239], %[ka] offset:8800\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[a0], v[240:243], %[q1], %[a0]\n\t"
-        "ds_read_b128 v[240:243], %[ka] offset:128\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[a1], v[244:247], %[q1], %[a1]\n\t"
-        "ds_read_b128 v[244:247], %[ka] offset:8832\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[a0], v[248:251], %[q2], %[a0]\n\t"
-        "ds_read_b128 v[248:251], %[ka] offset:160\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[a1], v[252:255], %[q2], %[a1]\n\t"
-        "ds_read_b128 v[252:255], %[ka] offset:8864\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[a0], v[232:235], %[q3], %[a0]\n\t"
-        "ds_read_b128 v[232:235], %[ka] offset:192\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[a1], v[236:239], %[q3], %[a1]\n\t"
-        "ds_read_b128 v[236:239], %[ka] offset:8896\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[a0], v[240:243], %[q4], %[a0]\n\t"
-        "ds_read_b128 v[240:243], %[ka] offset:224\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[a1], v[244:247], %[q4], %[a1]\n\t"
-        "ds_read_b128 v[244:247], %[ka] offset:8928\n\t"
-        "s_waitcnt lgkmcnt(5)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[a0], v[248:251], %[q5], %[a0]\n\t"
-        "s_waitcnt lgkmcnt(4)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[a1], v[252:255], %[q5], %[a1]\n\t"
-        "s_waitcnt lgkmcnt(3)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[a0], v[232:235], %[q6], %[a0]\n\t"
-        "s_waitcnt lgkmcnt(2)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[a1], v[236:239], %[q6], %[a1]\n\t"
-        "s_waitcnt lgkmcnt(1)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[a0], v[240:243], %[q7], %[a0]\n\t"
-        "s_waitcnt lgkmcnt(0)\n\t"
-        "v_mfma_f32_32x32x16_bf16 %[a1], v[244:247], %[q7], %[a1]\n\t"
-        : [a0] "=&v"(a0), [a1] "=&v"(a1)
-        : [ka] "v"(ka), [q0] "v"(q0), [q1] "v"(q1), [q2] "v"(q2), [q3] "v"(q3), [q4] "v"(q4), [q5] "v"(q5),
-          [q6] "v"(q6), [q7] "v"(q7)
-        : FD_OPERAND_REGS);
-  }
+// the value held by lane ^ 32
+__device__ __forceinline__ float swap32(float x) {
+  typedef u32 u2v __attribute__((ext_vector_type(2)));
+  const u2v r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(threadIdx.x & 32 ? r[0] : r[1]);
 }
 __device__ __forceinline__ u32 lds_addr(const void* p) {
   return (u32)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
@@ -307,7 +126,8 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   constexpr int PASSES = 16 / NW;   // 16-byte LDS chunks a thread stages per tile and tensor
   constexpr int ROWS = 2 * NW;      // tile rows covered by one staging pass of one wavefront group
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];  // [kSlots][K tile | V tile]
-  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // in a scalar register: what depends on it stays uniform
   const int b = blockIdx.z, qh = blockIdx.y, h = qh / (a.hq / a.hkv);
   const int tok0 = a.cu_seqlens_q[b], n_b = a.cu_seqlens_q[b + 1] - tok0, p = a.seq_lens_decoder[b];
   const int qt = (int)gridDim.x - 1 - (int)blockIdx.x;  // long rows (late tokens) first
@@ -354,27 +174,42 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
 
   // ---- the two wavefront groups.  Group 0 (the first NW/2 wavefronts) and group 1 run the
   // same per-tile sequence  [matrix phase: O += V P of the previous tile, S = K Q of this
-  // tile]  barrier  [vector phase: softmax of this tile, staging]  barrier,  but group 1
+  // tile]  barrier  [vector phase: staging, softmax of this tile]  barrier,  but group 1
   // starts one barrier late: while one group keeps the MFMA units busy the other one keeps
-  // the vector ALU busy (wavefronts w and w + NW/2 share a SIMD).
+  // the vector ALU busy (wavefronts w and w + NW/2 share a SIMD).  Tile u lives in LDS slot
+  // u % 3: group 0 writes its rows in its vector phase of tile u-1 and group 1 in its vector
+  // phase of tile u-2 (both end before group 0's matrix phase of tile u starts); K is read in
+  // the matrix phases of tile u and V in those of tile u+1.
   const int grp = wv / (NW / 2);
   const int gtid = tid - grp * 32 * NW;
   const int lead = 1 + grp;  // in the vector phase of tile t a group stages its rows of tile t + lead
-
   // ---- staging: a group's 32*NW threads move rows 32*grp .. 32*grp+31 of a tile, one
   // 16-byte LDS chunk (8 channels) per thread and pass
   const int srow = 32 * grp + (gtid >> 4), scc = (gtid & 15) * 8;
+  const u32 goff = (u32)(srow * HD + scc);  // this thread's byte offset inside a cache block
   uint4 stg_k[PASSES], stg_v[PASSES];
+  // The physical block of the next prefix tile to fetch is requested one fetch ahead and kept
+  // in a vector register until it is needed (vzero hides from the compiler that the index is
+  // uniform: it would otherwise move the value to a scalar register - and wait for the load -
+  // straight away).
+  int vzero;
+  asm("v_mov_b32 %0, 0" : "=v"(vzero));
+  int pb_next = n_pre > 0 ? table[vzero] : 0;
   auto fetch = [&](int t) {
     if (t >= n_tiles) return;
     if (t < n_pre) {
-      int pb = table[t];
-      pb = (pb >= 0 && pb < a.num_blocks) ? pb : 0;
-      const size_t off = (((size_t)pb * a.hkv + h) * BN + srow) * HD + scc;
+      // the block id was requested one fetch earlier: its scalar load has long returned
+      const int pb_u = __builtin_amdgcn_readfirstlane(pb_next);
+      const int pb = (pb_u >= 0 && pb_u < a.num_blocks) ? pb_u : 0;
+      pb_next = table[min(t + 1, n_pre - 1) + vzero];  // every group fetches its tiles in order 0, 1, 2, ...
+      // a scalar block base plus this thread's fixed 32-bit offset: no per-tile vector arithmetic
+      const size_t blk = ((size_t)pb * a.hkv + h) * (BN * HD);
+      const uint8_t* kb = a.key_cache + blk;
+      const uint8_t* vb = a.value_cache + blk;
 #pragma unroll
       for (int i = 0; i < PASSES; ++i) {
-        const uint2 kk = *reinterpret_cast<const uint2*>(a.key_cache + off + (size_t)i * ROWS * HD);
-        const uint2 vv = *reinterpret_cast<const uint2*>(a.value_cache + off + (size_t)i * ROWS * HD);
+        const uint2 kk = *reinterpret_cast<const uint2*>(kb + (goff + (u32)(i * ROWS * HD)));
+        const uint2 vv = *reinterpret_cast<const uint2*>(vb + (goff + (u32)(i * ROWS * HD)));
         stg_k[i].x = kk.x, stg_k[i].y = kk.y, stg_v[i].x = vv.x, stg_v[i].y = vv.y;
       }
     } else {
@@ -387,6 +222,8 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
       }
     }
   };
+  // this thread's fetched chunks of tile t into its LDS slot: fp16 for cache bytes and for the
+  // chunk's V, the chunk's bf16 K as it is
   auto commit = [&](int t) {
     if (t >= n_tiles) return;
     uint16_t* kd = lds + (size_t)(t % kSlots) * BUF_ELEMS + srow * LDK + scc;
@@ -394,10 +231,13 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
     if (t < n_pre) {
       // rows past the cached prefix hold stale bytes (fp8 has NaN codes, and 0 * NaN would
       // poison the second product): zero bytes are staged for them
-      const bool ragged = (t + 1) * BN > p;
+      if ((t + 1) * BN > p) {
+#pragma unroll
+        for (int i = 0; i < PASSES; ++i)
+          if (t * BN + srow + i * ROWS >= p) stg_k[i].x = stg_k[i].y = stg_v[i].x = stg_v[i].y = 0u;
+      }
 #pragma unroll
       for (int i = 0; i < PASSES; ++i) {
-        if (ragged && t * BN + srow + i * ROWS >= p) stg_k[i].x = stg_k[i].y = stg_v[i].x = stg_v[i].y = 0u;
         *reinterpret_cast<uint4*>(kd + i * ROWS * LDK) = cvt8<QUANT>(stg_k[i].x, stg_k[i].y);
         *reinterpret_cast<uint4*>(vd + i * ROWS * LDV) = cvt8<QUANT>(stg_v[i].x, stg_v[i].y);
       }
@@ -434,11 +274,11 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   // prologue: tile 0 (and group 1's rows of tile 1) into LDS, the next one into registers
   fetch(0);
   commit(0);
+  fetch(1);
   if (grp == 1) {
-    fetch(1);
     commit(1);
+    fetch(2);
   }
-  fetch(lead);
   __syncthreads();
   if (grp == 1) __syncthreads();  // group 1 trails by one phase
 
@@ -447,23 +287,25 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   for (int t = 0; t <= n_tiles; ++t) {
     // ================= matrix phase =================
     if (t == n_pre && n_pre > 0 && t < my_tiles) load_q(false);  // the chunk's scores meet the bf16 q
-    if (t >= 1 && t <= my_tiles) {
-      // ---- O^T += V^T P^T, tile t-1.  k-slot e of lane group hf is key 32kb + 16ss + 8(e/4) +
-      // 4hf + e%4 (the P^T layout); lane i16 supplies the row (key kbase + i16/4, channels
-      // cbase + 4(i16%4)..+3)
-      pv_tile(o, pf, lds_addr(lds + (size_t)((t - 1) % kSlots) * BUF_ELEMS + K_ELEMS + (4 * hf + (i16 >> 2)) * LDV +
-                              16 * (q16 & 1) + 4 * (i16 & 3)));
-    }
-    if (t < my_tiles) {
-      // ---- S^T = K Q^T, tile t
-      const u32 ka = lds_addr(lds + (size_t)(t % kSlots) * BUF_ELEMS + j32 * LDK + 8 * hf);
+    // ---- O^T += V^T P^T, tile t-1, then S^T = K Q^T, tile t.  In the first product k-slot e of
+    // lane group hf is key 32kb + 16ss + 8(e/4) + 4hf + e%4 (the P^T layout); lane i16 supplies
+    // the row (key kbase + i16/4, channels cbase + 4(i16%4)..+3)
+    const bool do_pv = t >= 1 && t <= my_tiles, do_qk = t < my_tiles;
+    const u32 va = lds_addr(lds + (size_t)((t + kSlots - 1) % kSlots) * BUF_ELEMS + K_ELEMS + (4 * hf + (i16 >> 2)) * LDV +
+                            16 * (q16 & 1) + 4 * (i16 & 3));
+    const u32 ka = lds_addr(lds + (size_t)(t % kSlots) * BUF_ELEMS + j32 * LDK + 8 * hf);
+    if (do_pv) mm_pv(o, pf, va);
+    if (do_qk) {
       if (t < n_pre)
-        qk_tile<true>(st[0], st[1], qf, ka);
+        mm_qk<true>(st[0], st[1], qf, ka);
       else
-        qk_tile<false>(st[0], st[1], qf, ka);
+        mm_qk<false>(st[0], st[1], qf, ka);
     }
     __syncthreads();
     // ================= vector phase =================
+    // staging first: its LDS writes and global loads then run under the softmax arithmetic
+    commit(t + lead);
+    fetch(t + lead + 1);
     if (t < my_tiles) {
       if (t == n_pre && n_pre > 0) {
         // leaving the quantised prefix: o holds sums over offset bytes; remove the offset
@@ -494,12 +336,15 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
             st[kb][r] = key < limit ? st[kb][r] : -INFINITY;
           }
       }
-      float mx = -INFINITY;
+      float m4[4];  // four independent chains, not one of 32 dependent maxima
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
+      for (int c = 0; c < 4; ++c) {
+        m4[c] = fmaxf(st[c >> 1][8 * (c & 1)], st[c >> 1][8 * (c & 1) + 1]);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, st[kb][r]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        for (int r = 2; r < 8; ++r) m4[c] = fmaxf(m4[c], st[c >> 1][8 * (c & 1) + r]);
+      }
+      float mx = fmaxf(fmaxf(m4[0], m4[1]), fmaxf(m4[2], m4[3]));
+      mx = fmaxf(mx, swap32(mx));
       // logit (log2 domain) = accumulator * scl + add
       const float scl = pre ? sc * ByteFmt<QUANT>::kMul : sc;
       const float add = pre ? qbias : 0.f;
@@ -516,24 +361,27 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
       }
       const float cst = add - (m_ref == -INFINITY ? 0.f : m_ref);
       const v2h ones = {(_Float16)1.0f, (_Float16)1.0f};
+      float ls[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int ss = 0; ss < 2; ++ss) {
+          // eight exponentials in flight at a time: the transcendental unit's latency is
+          // paid once per batch, not once per pair
+          float e8[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) e8[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(st[kb][8 * ss + e], scl, cst));
           u32 w[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[kb][8 * ss + 2 * e], scl, cst));
-            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[kb][8 * ss + 2 * e + 1], scl, cst));
-            w[e] = pack_f16_fast(p0, p1);
+            w[e] = pack_f16_fast(e8[2 * e], e8[2 * e + 1]);
             // the sum is taken over the rounded weights, the ones the MFMA multiplies
-            l_run = __builtin_amdgcn_fdot2(__builtin_bit_cast(v2h, w[e]), ones, l_run, false);
+            ls[e] = __builtin_amdgcn_fdot2(__builtin_bit_cast(v2h, w[e]), ones, ls[e], false);
           }
           pf[kb][ss] = __builtin_bit_cast(v8h, make_uint4(w[0], w[1], w[2], w[3]));
         }
+      l_run += (ls[0] + ls[1]) + (ls[2] + ls[3]);
     }
-    commit(t + lead);
-    fetch(t + lead + 1);
     __syncthreads();
   }
   if (grp == 0) __syncthreads();  // the barrier group 1 took before its first phase
@@ -583,8 +431,7 @@ int prefill_mfma_launch(const PrefillArgs& a, int max_chunk, int quant, hipStrea
   if (a.batch > 65535 || a.hq > 65535)
     return fail(FDATTN_ERR_SHAPE, "fdattn_append_attention_prefill: batch or head count exceeds the grid limit");
   // 256-token workgroups share each staged tile among 8 wavefronts; short chunks keep 128
-  static const char* nw_env = getenv("FDATTN_PREFILL_NW");
-  const bool wide = nw_env ? atoi(nw_env) == 8 : max_chunk > 128;
+  const bool wide = max_chunk > 128;
   hipError_t e;
   if (quant == FDATTN_CACHE_INT8)
     e = wide ? launch_one<FDATTN_CACHE_INT8, 8>(a, max_chunk, s) : launch_one<FDATTN_CACHE_INT8, 4>(a, max_chunk, s);
