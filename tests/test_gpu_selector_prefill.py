@@ -130,6 +130,55 @@ def test_prefill_ragged_edges(oracle, quant):
     assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
 
 
+def _run_prefill_vs_oracle(oracle, c, quant, max_chunk):
+    dev = syn.to_device(c, "cuda")
+    out = fd.append_attention_prefill(dev["q_new"], dev["k_new"], dev["v_new"], dev["key_cache"], dev["value_cache"],
+                                      dev["cache_k_scale"], dev["cache_v_scale"], dev["block_tables"],
+                                      dev["seq_lens_decoder"], dev["cu_seqlens_q"], num_heads=32, max_chunk=max_chunk,
+                                      cache_quant_type=quant)
+    want = oracle.append_attention_prefill(bits(c["q_new"]), bits(c["k_new"]), bits(c["v_new"]), np_of(c["key_cache"]),
+                                           np_of(c["value_cache"]), np_of(c["cache_k_scale"]), np_of(c["cache_v_scale"]),
+                                           np_of(c["block_tables"]), np_of(c["seq_lens_decoder"]), np_of(c["cu_seqlens_q"]),
+                                           32, 8, 128, quant)
+    ok, mx, bad = bf16_close(bits(out), want)
+    assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
+
+
+@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+@pytest.mark.parametrize("order", ["ascending", "descending"])
+def test_prefill_scores_trending_along_the_prefix(oracle, quant, order):
+    """Keys whose score grows (or falls) steadily from block to block: the running maximum is raised
+    again and again (or never after the first tile), the case the deferred rescaling has to get right.
+    Sharp softmax on top: q is scaled up."""
+    c = _prefill_case(3, [1536, 700], [260, 90], quant)
+    bt, kc = c["block_tables"], c["key_cache"]
+    sgn = torch.where(torch.arange(128) % 3 == 0, -1, 1)
+    top = 120 if quant == CACHE_INT8 else 0x6e  # int8 magnitude / e4m3 code of 240
+    for b, n in enumerate(c["seq_lens_decoder"].tolist()):
+        nb = (n + 63) // 64
+        for j in range(nb):
+            frac = (j + 1) / nb if order == "ascending" else (nb - j) / nb
+            if quant == CACHE_INT8:
+                mag = int(round(top * frac))
+                row = (sgn * mag).to(torch.int8).view(torch.uint8)
+            else:
+                code = max(1, int(round(top * frac)))          # e4m3 codes are monotonic in magnitude
+                row = torch.where(sgn < 0, code | 0x80, code).to(torch.uint8)
+            kc[int(bt[b, j])] = row                              # every head, every token of the block
+    c["q_new"] = (c["q_new"].float().abs() * sgn.repeat(32).float() * 1.5).to(torch.bfloat16)
+    _run_prefill_vs_oracle(oracle, c, quant, 260)
+
+
+@pytest.mark.parametrize("fill", [127, -127, 0])
+def test_prefill_constant_value_bytes(oracle, fill):
+    """V bytes all equal: the output is fill * v_scale whatever the weights are - exactly the case where the
+    kernel's byte offset (it stages b + 128) must cancel against the weight sum."""
+    c = _prefill_case(4, [2048, 65], [300, 20], CACHE_INT8)
+    c["value_cache"][:] = torch.tensor(fill, dtype=torch.int8).view(torch.uint8)
+    c["v_new"] = torch.zeros_like(c["v_new"])
+    _run_prefill_vs_oracle(oracle, c, CACHE_INT8, 300)
+
+
 def test_prefill_config5_shape_sampled_rows(oracle):
     """batch 2, 2048 new tokens on 8192 cached (int8 paged), causal: the full-size launch, checked on a
     sample of rows against the oracle and, on the GPU, against the shape-agnostic kernel on every row."""
