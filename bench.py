@@ -132,7 +132,8 @@ def main():
     ap.add_argument("--workload", default="decode", choices=["decode", "write_decode", "sqattn", "prefill", "all"],
                     help="decode = the headline metric (default); the others print one line per kernel of that row")
     ap.add_argument("--calibrate", action="store_true",
-                    help="also run a plain 1 GiB device copy, the yardstick the HBM byte counters are scaled by")
+                    help="kept for the profiling command line: the 1 GiB device copy (the yardstick the HBM byte "
+                         "counters are scaled by) now always runs")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the path shards by KV head or by sequence with no "
@@ -179,13 +180,24 @@ def main():
     ms_main = time_events(lambda: step("partials"), args.steps, args.warmup)
     ms_merge = time_events(lambda: step("merge"), args.steps, args.warmup)
 
-    if args.calibrate:
-        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)       # reads 1 GiB, writes 1 GiB
-        torch.cuda.synchronize()
-        del src, dst
+    # single launches timed one by one (event pair each): the spread behind the average
+    singles = []
+    for _ in range(min(args.steps, 100)):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        step("partials")
+        e1.record()
+        e1.synchronize()
+        singles.append(e0.elapsed_time(e1) * 1e3)
+    singles.sort()
+
+    # yardstick of the same run: a plain 1 GiB device copy (reads 1 GiB, writes 1 GiB) - what the
+    # memory system of this box gives a trivial kernel, beside the nominal 8 TB/s
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    ms_copy = time_events(lambda: dst.copy_(src), 10, 3)
+    copy_gbps = 2.0 * (1 << 30) / (ms_copy * 1e-3) / 1e9
+    del src, dst
 
     alg_bytes = syn.decode_algorithmic_bytes(lens, B)
     kv_bytes = syn.decode_kv_bytes(lens)
@@ -206,7 +218,11 @@ def main():
                       "decode_c8_combine_kernel_incl_launch": round(ms_merge * 1e3, 3)},
         "roofline": {"bound": "hbm", "kernel": "decode_c8_kernel<int8,dense>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "algorithmic_bytes": alg_bytes, "traffic": MEASURED_TRAFFIC_BYTES},
+                     "algorithmic_bytes": alg_bytes, "traffic": MEASURED_TRAFFIC_BYTES,
+                     "device_copy_gbps_same_run": round(copy_gbps, 1),
+                     "frac_of_device_copy": round(achieved / copy_gbps, 4)},
+        "kernel_us_single_launches": {"min": round(singles[0], 2), "median": round(singles[len(singles) // 2], 2),
+                                      "max": round(singles[-1], 2), "n": len(singles)},
     }
 
     if not args.no_cpu:
