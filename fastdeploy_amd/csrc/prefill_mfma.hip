@@ -26,9 +26,9 @@
 // and 16 of every 32 keys, so the softmax row reductions are in-lane plus one exchange with
 // lane^32, and P^T is already laid out as the B operand of the second product
 // O^T = V^T P^T - no trip through LDS.  V^T operands come transposed out of LDS by
-// ds_read_b64_tr_b16.  The running maximum is only raised when a tile exceeds it by more than
-// 2^6 (the weights then stay below 64, far inside fp16), so the accumulator is rescaled on a
-// handful of tiles instead of every one.  The per-channel K scale is folded into Q for the
+// ds_read_b64_tr_b16.  The exponent reference of a query is raised only when its weight sum
+// over a tile exceeds 1024 (every weight then stays far inside fp16): the tile's maximum is
+// not even computed on the other tiles, and the accumulator is rescaled on a handful of them.  The per-channel K scale is folded into Q for the
 // prefix tiles; the V scale is applied to the accumulator once, when the walk passes from
 // the prefix to the chunk.
 //
@@ -53,7 +53,7 @@ constexpr int LDK = 136;  // 16-bit elements per K row in LDS (272 B)
 constexpr int LDV = 160;  // 16-bit elements per V row in LDS (320 B)
 constexpr int K_ELEMS = BN * LDK, BUF_ELEMS = BN * (LDK + LDV);
 constexpr int kSlots = 3;  // K/V tiles resident in LDS
-constexpr float kRaise = 6.0f;  // log2 of the largest softmax weight tolerated before the maximum is raised
+constexpr float kSumLimit = 1024.0f;  // a query's weight sum over one tile above which its exponent reference is raised
 
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
@@ -259,7 +259,7 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   for (int ct = 0; ct < 4; ++ct)
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[ct][r] = 0.f;
-  float m_ref = -INFINITY;  // exponent reference of the weights (at most kRaise below the true maximum)
+  float m_ref = -INFINITY;  // exponent reference of the weights: a maximum seen so far, at most ~10 (log2) below the largest score
   float l_run = 0.f;        // this lane's share (its 16 of every 32 keys) of the weight sum
 
   // tiles this wavefront computes on; chunk tiles wholly above its diagonal contribute
@@ -336,21 +336,57 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
             st[kb][r] = key < limit ? st[kb][r] : -INFINITY;
           }
       }
-      float m4[4];  // four independent chains, not one of 32 dependent maxima
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        m4[c] = fmaxf(st[c >> 1][8 * (c & 1)], st[c >> 1][8 * (c & 1) + 1]);
-#pragma unroll
-        for (int r = 2; r < 8; ++r) m4[c] = fmaxf(m4[c], st[c >> 1][8 * (c & 1) + r]);
-      }
-      float mx = fmaxf(fmaxf(m4[0], m4[1]), fmaxf(m4[2], m4[3]));
-      mx = fmaxf(mx, swap32(mx));
       // logit (log2 domain) = accumulator * scl + add
       const float scl = pre ? sc * ByteFmt<QUANT>::kMul : sc;
       const float add = pre ? qbias : 0.f;
-      mx = mx * scl + add;
-      const bool raise = mx > m_ref + kRaise;  // always true for the first visible key (m_ref = -inf)
-      if (__any(raise)) {
+      // fp16 P^T operands and this lane's weight sum for the exponent reference m_ref
+      float tsum;
+      auto weights = [&]() {
+        const float cst = add - (m_ref == -INFINITY ? 0.f : m_ref);
+        const v2h ones = {(_Float16)1.0f, (_Float16)1.0f};
+        float ls[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int ss = 0; ss < 2; ++ss) {
+            // eight exponentials in flight at a time: the transcendental unit's latency is
+            // paid once per batch, not once per pair
+            float e8[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) e8[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(st[kb][8 * ss + e], scl, cst));
+            u32 w[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              w[e] = pack_f16_fast(e8[2 * e], e8[2 * e + 1]);
+              // the sum is taken over the rounded weights, the ones the MFMA multiplies
+              ls[e] = __builtin_amdgcn_fdot2(__builtin_bit_cast(v2h, w[e]), ones, ls[e], false);
+            }
+            pf[kb][ss] = __builtin_bit_cast(v8h, make_uint4(w[0], w[1], w[2], w[3]));
+          }
+        tsum = (ls[0] + ls[1]) + (ls[2] + ls[3]);
+      };
+      // Optimistic pass: weights against the reference as it stands.  Their sum over the
+      // query's 64 keys bounds every one of them, so a sum within kSumLimit proves that the
+      // reference was good enough (no weight beyond fp16, none worth rescaling for) without
+      // ever looking for the tile's maximum.
+      weights();
+      const float qsum64 = tsum + swap32(tsum);
+      const bool redo = !(qsum64 <= kSumLimit) || m_ref == -INFINITY;  // also true for inf / NaN sums
+      if (__any(redo)) {
+        // Rare (the first tile, and tiles whose scores outgrow the reference): take the exact
+        // maximum, raise the reference of the queries that asked for it, rescale what they
+        // have accumulated, and compute the weights again.
+        float m4[4];  // four independent chains, not one of 32 dependent maxima
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          m4[c] = fmaxf(st[c >> 1][8 * (c & 1)], st[c >> 1][8 * (c & 1) + 1]);
+#pragma unroll
+          for (int r = 2; r < 8; ++r) m4[c] = fmaxf(m4[c], st[c >> 1][8 * (c & 1) + r]);
+        }
+        float mx = fmaxf(fmaxf(m4[0], m4[1]), fmaxf(m4[2], m4[3]));
+        mx = fmaxf(mx, swap32(mx));
+        mx = mx * scl + add;
+        const bool raise = redo && mx > m_ref;
         const float alpha = raise ? __builtin_amdgcn_exp2f(m_ref - mx) : 1.0f;
         m_ref = raise ? mx : m_ref;
         l_run *= alpha;
@@ -358,29 +394,9 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
         for (int ct = 0; ct < 4; ++ct)
 #pragma unroll
           for (int r = 0; r < 16; ++r) o[ct][r] *= alpha;
+        weights();
       }
-      const float cst = add - (m_ref == -INFINITY ? 0.f : m_ref);
-      const v2h ones = {(_Float16)1.0f, (_Float16)1.0f};
-      float ls[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int ss = 0; ss < 2; ++ss) {
-          // eight exponentials in flight at a time: the transcendental unit's latency is
-          // paid once per batch, not once per pair
-          float e8[8];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) e8[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(st[kb][8 * ss + e], scl, cst));
-          u32 w[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            w[e] = pack_f16_fast(e8[2 * e], e8[2 * e + 1]);
-            // the sum is taken over the rounded weights, the ones the MFMA multiplies
-            ls[e] = __builtin_amdgcn_fdot2(__builtin_bit_cast(v2h, w[e]), ones, ls[e], false);
-          }
-          pf[kb][ss] = __builtin_bit_cast(v8h, make_uint4(w[0], w[1], w[2], w[3]));
-        }
-      l_run += (ls[0] + ls[1]) + (ls[2] + ls[3]);
+      l_run += tsum;
     }
     __syncthreads();
   }
