@@ -52,7 +52,7 @@ constexpr int BN = 64, HD = 128;
 constexpr int LDK = 136;  // 16-bit elements per K row in LDS (272 B)
 constexpr int LDV = 160;  // 16-bit elements per V row in LDS (320 B)
 constexpr int K_ELEMS = BN * LDK, BUF_ELEMS = BN * (LDK + LDV);
-constexpr int kSlots = 3;  // K/V tiles resident in LDS
+constexpr int kSlots = 4;  // K/V tile slots in LDS (three are live at a time; four make the slot of a tile a mask)
 constexpr float kSumLimit = 1024.0f;  // a query's weight sum over one tile above which its exponent reference is raised
 
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
@@ -113,6 +113,10 @@ __device__ __forceinline__ float swap32(float x) {
   typedef u32 u2v __attribute__((ext_vector_type(2)));
   const u2v r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
   return __uint_as_float(threadIdx.x & 32 ? r[0] : r[1]);
+}
+__device__ __forceinline__ void lds_store16(u32 addr, uint4 v) {
+  const u4v w = {v.x, v.y, v.z, v.w};
+  *(__attribute__((address_space(3))) u4v*)(uintptr_t)addr = w;
 }
 __device__ __forceinline__ u32 lds_addr(const void* p) {
   return (u32)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
@@ -177,7 +181,7 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   // tile]  barrier  [vector phase: staging, softmax of this tile]  barrier,  but group 1
   // starts one barrier late: while one group keeps the MFMA units busy the other one keeps
   // the vector ALU busy (wavefronts w and w + NW/2 share a SIMD).  Tile u lives in LDS slot
-  // u % 3: group 0 writes its rows in its vector phase of tile u-1 and group 1 in its vector
+  // u % 4: group 0 writes its rows in its vector phase of tile u-1 and group 1 in its vector
   // phase of tile u-2 (both end before group 0's matrix phase of tile u starts); K is read in
   // the matrix phases of tile u and V in those of tile u+1.
   const int grp = wv / (NW / 2);
@@ -187,6 +191,8 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   // 16-byte LDS chunk (8 channels) per thread and pass
   const int srow = 32 * grp + (gtid >> 4), scc = (gtid & 15) * 8;
   const u32 goff = (u32)(srow * HD + scc);  // this thread's byte offset inside a cache block
+  // LDS byte addresses of its K and V chunk of pass 0 in slot 0
+  const u32 kw0 = lds_addr(lds + srow * LDK + scc), vw0 = lds_addr(lds + K_ELEMS + srow * LDV + scc);
   uint4 stg_k[PASSES], stg_v[PASSES];
   // The physical block of the next prefix tile to fetch is requested one fetch ahead and kept
   // in a vector register until it is needed (vzero hides from the compiler that the index is
@@ -226,8 +232,8 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   // chunk's V, the chunk's bf16 K as it is
   auto commit = [&](int t) {
     if (t >= n_tiles) return;
-    uint16_t* kd = lds + (size_t)(t % kSlots) * BUF_ELEMS + srow * LDK + scc;
-    uint16_t* vd = lds + (size_t)(t % kSlots) * BUF_ELEMS + K_ELEMS + srow * LDV + scc;
+    const u32 slot_off = (u32)(t & (kSlots - 1)) * (u32)(BUF_ELEMS * sizeof(uint16_t));
+    const u32 kd = kw0 + slot_off, vd = vw0 + slot_off;
     if (t < n_pre) {
       // rows past the cached prefix hold stale bytes (fp8 has NaN codes, and 0 * NaN would
       // poison the second product): zero bytes are staged for them
@@ -238,18 +244,18 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
       }
 #pragma unroll
       for (int i = 0; i < PASSES; ++i) {
-        *reinterpret_cast<uint4*>(kd + i * ROWS * LDK) = cvt8<QUANT>(stg_k[i].x, stg_k[i].y);
-        *reinterpret_cast<uint4*>(vd + i * ROWS * LDV) = cvt8<QUANT>(stg_v[i].x, stg_v[i].y);
+        lds_store16(kd + i * ROWS * LDK * 2, cvt8<QUANT>(stg_k[i].x, stg_k[i].y));
+        lds_store16(vd + i * ROWS * LDV * 2, cvt8<QUANT>(stg_v[i].x, stg_v[i].y));
       }
     } else {
 #pragma unroll
       for (int i = 0; i < PASSES; ++i) {
-        *reinterpret_cast<uint4*>(kd + i * ROWS * LDK) = stg_k[i];
+        lds_store16(kd + i * ROWS * LDK * 2, stg_k[i]);
         const u32 vw[4] = {stg_v[i].x, stg_v[i].y, stg_v[i].z, stg_v[i].w};
         u32 hw[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) hw[e] = pack_f16(sat_f16(bf16lo_to_f32(vw[e])), sat_f16(bf16hi_to_f32(vw[e])));
-        *reinterpret_cast<uint4*>(vd + i * ROWS * LDV) = make_uint4(hw[0], hw[1], hw[2], hw[3]);
+        lds_store16(vd + i * ROWS * LDV * 2, make_uint4(hw[0], hw[1], hw[2], hw[3]));
       }
     }
   };
@@ -271,13 +277,12 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   // log2-domain constant that removes the byte offset from the prefix scores
   const float qbias = -ByteFmt<QUANT>::kOff * sc * (qsum + __shfl_xor(qsum, 32, 64));
 
-  // prologue: tile 0 (and group 1's rows of tile 1) into LDS, the next one into registers
+  // prologue: tile 0 (and group 1's rows of tile 1) into LDS
   fetch(0);
   commit(0);
-  fetch(1);
   if (grp == 1) {
+    fetch(1);
     commit(1);
-    fetch(2);
   }
   __syncthreads();
   if (grp == 1) __syncthreads();  // group 1 trails by one phase
@@ -287,13 +292,14 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   for (int t = 0; t <= n_tiles; ++t) {
     // ================= matrix phase =================
     if (t == n_pre && n_pre > 0 && t < my_tiles) load_q(false);  // the chunk's scores meet the bf16 q
+    fetch(t + lead);  // converted and written to LDS in the vector phase that follows
     // ---- O^T += V^T P^T, tile t-1, then S^T = K Q^T, tile t.  In the first product k-slot e of
     // lane group hf is key 32kb + 16ss + 8(e/4) + 4hf + e%4 (the P^T layout); lane i16 supplies
     // the row (key kbase + i16/4, channels cbase + 4(i16%4)..+3)
     const bool do_pv = t >= 1 && t <= my_tiles, do_qk = t < my_tiles;
-    const u32 va = lds_addr(lds + (size_t)((t + kSlots - 1) % kSlots) * BUF_ELEMS + K_ELEMS + (4 * hf + (i16 >> 2)) * LDV +
+    const u32 va = lds_addr(lds + (size_t)((t + kSlots - 1) & (kSlots - 1)) * BUF_ELEMS + K_ELEMS + (4 * hf + (i16 >> 2)) * LDV +
                             16 * (q16 & 1) + 4 * (i16 & 3));
-    const u32 ka = lds_addr(lds + (size_t)(t % kSlots) * BUF_ELEMS + j32 * LDK + 8 * hf);
+    const u32 ka = lds_addr(lds + (size_t)(t & (kSlots - 1)) * BUF_ELEMS + j32 * LDK + 8 * hf);
     if (do_pv) mm_pv(o, pf, va);
     if (do_qk) {
       if (t < n_pre)
@@ -305,7 +311,6 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
     // ================= vector phase =================
     // staging first: its LDS writes and global loads then run under the softmax arithmetic
     commit(t + lead);
-    fetch(t + lead + 1);
     if (t < my_tiles) {
       if (t == n_pre && n_pre > 0) {
         // leaving the quantised prefix: o holds sums over offset bytes; remove the offset
@@ -429,7 +434,7 @@ template <int QUANT, int NW>
 hipError_t launch_one(const PrefillArgs& a, int max_chunk, hipStream_t s) {
   constexpr int BM = 32 * NW;
   const dim3 grid((max_chunk + BM - 1) / BM, a.hq, a.batch), block(64 * NW);
-  const size_t shm = (size_t)kSlots * BUF_ELEMS * sizeof(uint16_t);  // 113,664 B
+  const size_t shm = (size_t)kSlots * BUF_ELEMS * sizeof(uint16_t);  // 151,552 B
   static bool attr_set = false;  // one flag per instantiation
   if (!attr_set) {
     const hipError_t e = hipFuncSetAttribute((const void*)prefill_mfma_kernel<QUANT, NW>,
