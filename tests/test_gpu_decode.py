@@ -199,3 +199,48 @@ def test_write_then_decode_config3_full_size(oracle):
     want = oracle.decode_attention(q, kc, vc, np_of(case["cache_k_scale"]), np_of(case["cache_v_scale"]),
                                    np_of(case["block_tables"]), np_of(case["seq_lens_decoder"]) + 1, 32, 8, 128, CACHE_INT8)
     check(bits(out), want, "cfg3")
+
+
+def test_decode_step_replays_from_a_hip_graph():
+    """One decode step of a layer (cache write + decode attention + the length update) captured in a HIP
+    graph and replayed with eager work and synchronisations between the replays: every replay must equal
+    the same step run eagerly on a copy of the state (outputs and cache bytes, bit for bit).  The path
+    allocates nothing of its own and clears nothing with memsets, which is what makes it capturable."""
+    case = syn.write_case(num_seqs=48, max_pos=2048, seed=5, blocks_per_seq=34)
+    dev = syn.to_device(case, "cuda")
+    eag = {k: (v.clone() if isinstance(v, torch.Tensor) else v) for k, v in dev.items()}
+    rot_g, rot_e = (dev["rope_cos"], dev["rope_sin"]), (eag["rope_cos"], eag["rope_sin"])
+    ws_g = fd.decode_workspace(48, 32, 8, 128, 34, "cuda")
+    ws_e = fd.decode_workspace(48, 32, 8, 128, 34, "cuda")
+
+    def step(c, rot, ws):
+        out = fd.append_attention(c["qkv"], c["key_cache"], c["value_cache"], c["seq_lens_encoder"],
+                                  c["seq_lens_decoder"], c["seq_lens_this_time"], c["block_tables"], rot,
+                                  c["cache_k_scale"], c["cache_v_scale"], num_heads=32, kv_num_heads=8, max_chunk=1,
+                                  workspace=ws)
+        c["seq_lens_decoder"].add_(1)
+        return out
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):            # warm-up outside the capture, on a throw-away copy
+        tmp = {k: (v.clone() if isinstance(v, torch.Tensor) else v) for k, v in dev.items()}
+        step(tmp, rot_g, ws_g)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_g = step(dev, rot_g, ws_g)
+    # the capture itself runs nothing: state is still the initial one
+    gen = torch.Generator(device="cuda").manual_seed(11)
+    for r in range(4):
+        new_qkv = torch.randn(dev["qkv"].shape, generator=gen, device="cuda").to(torch.bfloat16)
+        dev["qkv"].copy_(new_qkv)            # eager work between the replays
+        eag["qkv"].copy_(new_qkv)
+        torch.cuda.synchronize()
+        graph.replay()
+        want = step(eag, rot_e, ws_e)
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, want), "replay %d: outputs differ" % r
+        assert torch.equal(dev["key_cache"], eag["key_cache"]) and torch.equal(dev["value_cache"], eag["value_cache"]), r
+        assert torch.equal(dev["seq_lens_decoder"], eag["seq_lens_decoder"])
