@@ -6,6 +6,7 @@ only as device buffers.
 """
 from .ops import (  # noqa: F401
     append_attention,
+    append_attention_workspace,
     append_attention_prefill,
     decode_attention,
     decode_attention_sparse,

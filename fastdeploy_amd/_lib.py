@@ -25,6 +25,8 @@ SIGNATURES = {
     "fdattn_sqattn_select_exact": (_i, [_vp] * 10 + [_sz] + [_i] * 9 + [_vp]),
     "fdattn_append_attention_prefill": (_i, [_vp] * 11 + [_i] * 10 + [_f, _vp]),
     "fdattn_append_attention_prefill_generic": (_i, [_vp] * 11 + [_i] * 10 + [_f, _vp]),
+    "fdattn_append_attention_workspace_bytes": (_sz, [_i] * 6),
+    "fdattn_append_attention": (_i, [_vp] * 14 + [_sz] + [_i] * 12 + [_f, _vp]),
 }
 
 _lib = None

@@ -1,0 +1,86 @@
+// One attention step of a mixed batch - prefill rows, decode rows and idle slots together:
+// cache write for every new token, decode attention for the decode rows, append attention
+// for the prefill rows.  Nothing is gathered or synchronised: the kernels find their rows
+// through cu_seqlens_q / seq_lens_encoder on the device.
+#include "launch.h"
+
+namespace fdattn {
+
+static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+struct StepWorkspace {
+  size_t q_rot, k_new, v_new, decode, total;  // byte offsets of the parts, and the sum
+};
+
+static StepWorkspace step_workspace(int num_tokens, int batch, int hq, int hkv, int d, int max_blocks) {
+  StepWorkspace w;
+  w.q_rot = 0;
+  w.k_new = w.q_rot + align256((size_t)num_tokens * hq * d * 2);
+  w.v_new = w.k_new + align256((size_t)num_tokens * hkv * d * 2);
+  w.decode = w.v_new + align256((size_t)num_tokens * hkv * d * 2);
+  w.total = w.decode + fdattn_decode_workspace_bytes(batch, hq, hkv, d, max_blocks);
+  return w;
+}
+
+}  // namespace fdattn
+
+using namespace fdattn;
+
+extern "C" size_t fdattn_append_attention_workspace_bytes(int num_tokens, int batch, int hq, int hkv, int head_dim,
+                                                          int max_blocks_per_seq) {
+  if (num_tokens < 0 || batch <= 0 || hq <= 0 || hkv <= 0 || head_dim <= 0 || max_blocks_per_seq <= 0) return 256;
+  return step_workspace(num_tokens, batch, hq, hkv, head_dim, max_blocks_per_seq).total;
+}
+
+extern "C" int fdattn_append_attention(
+    const void* qkv, void* key_cache, void* value_cache, const float* cache_k_scale, const float* cache_v_scale,
+    const float* rope_cos, const float* rope_sin, const int32_t* block_tables, const int32_t* seq_lens_encoder,
+    const int32_t* seq_lens_decoder, const int32_t* seq_lens_this_time, const int32_t* cu_seqlens_q, void* out,
+    void* workspace, size_t workspace_bytes, int num_tokens, int batch, int max_chunk, int hq, int hkv,
+    int head_dim, int block_size, int max_blocks_per_seq, int num_blocks, int max_pos, int rope_style,
+    int cache_quant_type, float softmax_scale, void* stream) {
+  if (!seq_lens_encoder || !seq_lens_this_time || !cu_seqlens_q || !out || !workspace)
+    return fail(FDATTN_ERR_NULL, "fdattn_append_attention: a required pointer is NULL");
+  if (num_tokens < 0 || batch <= 0 || max_chunk <= 0 || hq <= 0 || hkv <= 0 || head_dim <= 0 ||
+      max_blocks_per_seq <= 0)
+    return fail(FDATTN_ERR_SHAPE, "fdattn_append_attention: bad shape tokens=%d batch=%d max_chunk=%d hq=%d hkv=%d "
+                "head_dim=%d max_blocks=%d", num_tokens, batch, max_chunk, hq, hkv, head_dim, max_blocks_per_seq);
+  if (num_tokens == 0) return 0;
+  const StepWorkspace w = step_workspace(num_tokens, batch, hq, hkv, head_dim, max_blocks_per_seq);
+  if (workspace_bytes < w.total)
+    return fail(FDATTN_ERR_WORKSPACE, "fdattn_append_attention: workspace %zu B < required %zu B", workspace_bytes,
+                w.total);
+  char* ws = (char*)workspace;
+  void* q_rot = ws + w.q_rot;
+  const bool any_prefill = max_chunk > 1;
+  void* k_new = any_prefill ? ws + w.k_new : nullptr;
+  void* v_new = any_prefill ? ws + w.v_new : nullptr;
+  // 1. every new token: rotate, quantise, store (argument checks of the shared kind happen here)
+  int rc = fdattn_write_cache_kv(qkv, q_rot, k_new, v_new, key_cache, value_cache, cache_k_scale, cache_v_scale,
+                                 rope_cos, rope_sin, block_tables, seq_lens_decoder, cu_seqlens_q, num_tokens, batch,
+                                 hq, hkv, head_dim, block_size, max_blocks_per_seq, num_blocks, max_pos, rope_style,
+                                 cache_quant_type, stream);
+  if (rc) return rc;
+  // 2. decode rows: one token, seq_lens_encoder == 0; they read their own token back from the cache
+  const RowMap rows{cu_seqlens_q, seq_lens_encoder};
+  const size_t dws = w.total - w.decode;
+  hipStream_t s = (hipStream_t)stream;
+  if (c8_supported(hq, hkv, head_dim, block_size, cache_quant_type))
+    rc = decode_c8_launch(q_rot, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
+                          seq_lens_decoder, seq_lens_this_time, nullptr, nullptr, 0, out, ws + w.decode, dws, batch,
+                          hq, hkv, head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type,
+                          softmax_scale, s, 3, rows);
+  else
+    rc = decode_generic_launch(q_rot, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
+                               seq_lens_decoder, seq_lens_this_time, nullptr, nullptr, 0, out, ws + w.decode, dws,
+                               batch, hq, hkv, head_dim, block_size, max_blocks_per_seq, num_blocks,
+                               cache_quant_type, softmax_scale, s, rows);
+  if (rc) return rc;
+  // 3. prefill rows: seq_lens_encoder > 0; the chunk's own K/V come from this call, the prefix from the cache
+  if (any_prefill)
+    rc = prefill_launch(q_rot, k_new, v_new, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
+                        seq_lens_decoder, cu_seqlens_q, seq_lens_encoder, out, num_tokens, batch, max_chunk, hq, hkv,
+                        head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type, softmax_scale, s,
+                        false);
+  return rc;
+}

@@ -115,11 +115,11 @@ struct PairState {
 // A operand rows: row = head*4 + limb; lane (m = lane%16, g = lane/16) holds channels
 // 16*(g + 4s) .. +15 of k-step s.
 template <int QUANT>
-__device__ __forceinline__ void load_pair(const uint16_t* q, const float* k_scale, int hkv, float sm_scale_log2, int p, int lane,
-                                          PairState& st) {
-  const int b = p / hkv, h = p - b * hkv;
+__device__ __forceinline__ void load_pair(const uint16_t* q, const float* k_scale, int hkv, float sm_scale_log2, int p, int row,
+                                          int lane, PairState& st) {
+  const int h = p % hkv;  // row: the sequence's row of q
   const int m = lane & 15, g = lane >> 4, head = m >> 2, limb = m & 3;
-  const uint16_t* qrow = q + ((size_t)b * hkv * kG + h * kG + head) * kD;
+  const uint16_t* qrow = q + ((size_t)row * hkv * kG + h * kG + head) * kD;
   const float* ks = k_scale + (size_t)h * kD;
   float qs[2][16];
   float amax = 0.f;

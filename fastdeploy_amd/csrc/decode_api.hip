@@ -1,26 +1,9 @@
 // Entry points of decode attention: argument checks and the choice between the
 // MFMA kernel (head_dim 128, 4 query heads per KV head, block_size 64) and the
 // shape-agnostic kernel.
-#include "fdattn_common.h"
+#include "launch.h"
 
 namespace fdattn {
-size_t generic_workspace_bytes(int batch, int hq, int d);
-int decode_generic_launch(const void* q, const void* key_cache, const void* value_cache,
-                          const float* k_scale, const float* v_scale, const int32_t* block_tables,
-                          const int32_t* seq_lens_decoder, const int32_t* seq_lens_this_time,
-                          const int32_t* kept_blocks, const int32_t* kept_counts, int max_kept,
-                          void* out, void* workspace, size_t workspace_bytes, int batch, int hq,
-                          int hkv, int d, int bs, int max_blocks, int num_blocks, int quant,
-                          float sm_scale, hipStream_t s);
-size_t c8_workspace_bytes(int batch, int hkv, int max_units);
-bool c8_supported(int hq, int hkv, int d, int bs, int quant);
-int decode_c8_launch(const void* q, const void* key_cache, const void* value_cache,
-                     const float* k_scale, const float* v_scale, const int32_t* block_tables,
-                     const int32_t* seq_lens_decoder, const int32_t* seq_lens_this_time,
-                     const int32_t* kept_blocks, const int32_t* kept_counts, int max_kept,
-                     void* out, void* workspace, size_t workspace_bytes, int batch, int hq,
-                     int hkv, int d, int bs, int max_blocks, int num_blocks, int quant,
-                     float sm_scale, hipStream_t s, int stages);
 
 static int check_decode_args(const char* fn, const void* q, const void* kc, const void* vc, const float* ks,
                              const float* vs, const int32_t* bt, const int32_t* dec, const void* out,

@@ -33,9 +33,6 @@
 // and handing chunks out through an atomic ticket counter instead of the block index.
 #include "c8_common.h"
 
-#ifndef TRACE
-#define TRACE(slot)  // timestamp hook of the perf harness; nothing in the library
-#endif
 
 namespace fdattn {
 
@@ -54,6 +51,7 @@ struct C8Args {
   float* part_o;   // [pairs * chunks_per_pair][4][128]
   float* part_ml;  // [pairs * chunks_per_pair][8]: m[4] (log2 domain), l[4]
   uint16_t* out;
+  RowMap rows;  // which sequences are decode rows and where their q / out rows are
   int batch, hkv, max_blocks, num_blocks;
   int chunk;            // units per workgroup
   int chunks_per_pair;  // grid.x
@@ -72,12 +70,13 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
   __shared__ __attribute__((aligned(16))) uint8_t ldsK[kWaves][kTileB];
   __shared__ __attribute__((aligned(16))) uint8_t ldsV[kWaves][kTileB];
   __shared__ __attribute__((aligned(16))) uint8_t ldsP[kWaves][1024];
-  TRACE(0);
   const int lane = threadIdx.x & 63;
   const int wv = uni(threadIdx.x >> 6);
   const int ticket = blockIdx.x;
   const int p = ticket / a.chunks_per_pair, ck = ticket - p * a.chunks_per_pair;
   const int b = p / a.hkv, h = p - b * a.hkv;
+  int row;
+  if (!decode_row(a.rows, b, row)) return;
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
   const int n_p = pair_units<SPARSE>(a, p, kv_len);
   const int first = ck * a.chunk;
@@ -85,7 +84,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
   const bool single = n_p <= a.chunk;
   if (cnt <= 0) {
     if (n_p == 0 && ck == 0) {  // empty sequence: its output rows are zeros
-      uint16_t* o = a.out + ((size_t)b * a.hkv * kG + h * kG + (threadIdx.x >> 6)) * kD + (threadIdx.x & 63) * 2;
+      uint16_t* o = a.out + ((size_t)row * a.hkv * kG + h * kG + (threadIdx.x >> 6)) * kD + (threadIdx.x & 63) * 2;
       *reinterpret_cast<u32*>(o) = 0u;
     }
     return;
@@ -115,7 +114,6 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
       my_valid = min(max(kv_len - lb * kBS, 0), kBS);
     }
   }
-  TRACE(2);
 
   const size_t tile_stride = (size_t)kBS * kD;  // bytes of one (block, head) tile
   const uint8_t* const kbase = a.key_cache + (size_t)h * tile_stride;
@@ -133,8 +131,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
     int valid = __builtin_amdgcn_readlane(my_valid, wv);
     dma_tile(kbase + (size_t)pb * blk_stride, kaddr, offK);
     dma_tile(vbase + (size_t)pb * blk_stride, vaddr, offV);
-    TRACE(3);
-    load_pair<QUANT>(a.q, a.k_scale, a.hkv, a.sm_scale_log2, p, lane, st);
+    load_pair<QUANT>(a.q, a.k_scale, a.hkv, a.sm_scale_log2, p, row, lane, st);
 
     for (int j = wv; j < cnt; j += kWaves) {
       const bool has_next = j + kWaves < cnt;
@@ -146,7 +143,6 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
 
       // ---------------- S = Q K^T : rows = head*4 + limb, columns = token slots
       wait_vm8();  // K(j) landed; V(j) may still be in flight
-      if (j == wv) TRACE(4);
       v4i S[4];
       v4f Sf[4];
 #pragma unroll
@@ -273,7 +269,6 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
       valid = validn;
     }
   }
-  TRACE(5);
 
   // ---- merge the 4 wavefronts through LDS (their K slots are free now)
   {
@@ -310,7 +305,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
       // the only chunk of this pair: finish here
       const float inv = L > 0.f ? 1.0f / L : 0.f;
       const float r0 = o0 * inv * a.v_scale[h * kD + c2], r1 = o1 * inv * a.v_scale[h * kD + c2 + 1];
-      uint16_t* o = a.out + ((size_t)b * a.hkv * kG + h * kG + head) * kD + c2;
+      uint16_t* o = a.out + ((size_t)row * a.hkv * kG + h * kG + head) * kD + c2;
       *reinterpret_cast<u32*>(o) = (u32)f32_to_bf16(r0) | ((u32)f32_to_bf16(r1) << 16);
     } else {
       const size_t slot = (size_t)p * a.chunks_per_pair + ck;
@@ -321,7 +316,6 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
       }
     }
   }
-  TRACE(6);
 }
 
 // One workgroup per (sequence, KV head) whose list spans several chunks: merges their
@@ -331,6 +325,8 @@ template <bool SPARSE>
 __global__ __launch_bounds__(256) void decode_c8_combine_kernel(C8Args a) {
   const int p = blockIdx.x, tid = threadIdx.x;
   const int b = p / a.hkv, h = p - b * a.hkv;
+  int row;
+  if (!decode_row(a.rows, b, row)) return;
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
   const int n_p = pair_units<SPARSE>(a, p, kv_len);
   if (n_p <= a.chunk) return;
@@ -353,7 +349,7 @@ __global__ __launch_bounds__(256) void decode_c8_combine_kernel(C8Args a) {
   }
   const float inv = L > 0.f ? 1.0f / L : 0.f;
   const float r0 = o0 * inv * a.v_scale[h * kD + c2], r1 = o1 * inv * a.v_scale[h * kD + c2 + 1];
-  uint16_t* o = a.out + ((size_t)b * a.hkv * kG + h * kG + head) * kD + c2;
+  uint16_t* o = a.out + ((size_t)row * a.hkv * kG + h * kG + head) * kD + c2;
   *reinterpret_cast<u32*>(o) = (u32)f32_to_bf16(r0) | ((u32)f32_to_bf16(r1) << 16);
 }
 
@@ -389,7 +385,7 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
                      const int32_t* seq_lens_this_time, const int32_t* kept_blocks, const int32_t* kept_counts,
                      int max_kept, void* out, void* workspace, size_t workspace_bytes, int batch, int hq,
                      int hkv, int d, int bs, int max_blocks, int num_blocks, int quant, float sm_scale,
-                     hipStream_t s, int stages) {
+                     hipStream_t s, int stages, RowMap rows) {
   (void)hq; (void)d; (void)bs;
   const bool sparse = kept_blocks != nullptr;
   const int pairs = batch * hkv;
@@ -408,7 +404,7 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
   float* part_ml = part_o + slots * kSlotFloats;
   C8Args a{(const uint16_t*)q, (const uint8_t*)key_cache, (const uint8_t*)value_cache, k_scale, v_scale,
            block_tables, seq_lens_decoder, seq_lens_this_time, kept_blocks, kept_counts, max_kept, part_o,
-           part_ml, (uint16_t*)out, batch, hkv, max_blocks, num_blocks, chunk, cpp,
+           part_ml, (uint16_t*)out, rows, batch, hkv, max_blocks, num_blocks, chunk, cpp,
            sm_scale * 1.4426950408889634f};
   const dim3 grid(cpp * pairs), block(kWaves * 64);
   if (!(stages & 1)) {

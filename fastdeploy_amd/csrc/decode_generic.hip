@@ -3,7 +3,7 @@
 // q.K and channels for P.V.  This is the fall-back for shapes the MFMA kernel in
 // decode_c8.hip does not cover (any head_dim <= 256, any group size, any block size);
 // it makes no attempt to reach the HBM roofline.
-#include "fdattn_common.h"
+#include "launch.h"
 
 namespace fdattn {
 
@@ -22,6 +22,7 @@ struct GenericDecodeArgs {
   float* part_o;  // [rows, max_splits, d]
   float* part_m;  // [rows, max_splits]
   float* part_l;
+  RowMap rows;
   int batch, hq, hkv, d, bs, max_blocks, num_blocks, max_splits;
   float sm_scale;
 };
@@ -42,10 +43,12 @@ __global__ __launch_bounds__(64) void decode_generic_kernel(GenericDecodeArgs a)
   const int row = blockIdx.x, split = blockIdx.y, nsplit = gridDim.y;
   const int b = row / a.hq, qh = row % a.hq, g = a.hq / a.hkv, h = qh / g;
   const int d = a.d, bs = a.bs;
+  int qrow;  // the sequence's row of q
+  if (!decode_row(a.rows, b, qrow)) return;
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
 
   for (int c = lane; c < d; c += 64)
-    qs[c] = bf16_to_f32(a.q[(size_t)row * d + c]) * a.k_scale[h * d + c] * a.sm_scale;
+    qs[c] = bf16_to_f32(a.q[((size_t)qrow * a.hq + qh) * d + c]) * a.k_scale[h * d + c] * a.sm_scale;
   __syncthreads();
 
   int nblk = (kv_len + bs - 1) / bs;
@@ -117,10 +120,19 @@ __global__ __launch_bounds__(64) void decode_generic_kernel(GenericDecodeArgs a)
 }
 
 // out[r,:] = sum_s o_s e^(m_s - m) / sum_s l_s e^(m_s - m); one thread per channel.
+// With a row map (hq > 0) partial row r = (sequence, head) goes to the sequence's out row, and
+// sequences that are not decode rows are left alone.
 __global__ void splitkv_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_m,
                                        const float* __restrict__ part_l, const int32_t* __restrict__ num_splits,
-                                       uint16_t* __restrict__ out, int rows, int max_splits, int d) {
+                                       uint16_t* __restrict__ out, int rows, int max_splits, int d, int hq,
+                                       RowMap map) {
   const int r = blockIdx.x;
+  size_t orow = (size_t)r;
+  if (hq > 0) {
+    int srow;
+    if (!decode_row(map, r / hq, srow)) return;
+    orow = (size_t)srow * hq + r % hq;
+  }
   const int ns = num_splits ? min(num_splits[r], max_splits) : max_splits;
   float m = -INFINITY;
   for (int s = 0; s < ns; ++s) m = fmaxf(m, part_m[(size_t)r * max_splits + s]);
@@ -135,7 +147,7 @@ __global__ void splitkv_combine_kernel(const float* __restrict__ part_o, const f
       const float ms = part_m[(size_t)r * max_splits + s];
       if (ms > -INFINITY) o += part_o[((size_t)r * max_splits + s) * d + c] * __expf(ms - m);
     }
-    out[(size_t)r * d + c] = f32_to_bf16(l > 0.f ? o / l : 0.f);
+    out[orow * d + c] = f32_to_bf16(l > 0.f ? o / l : 0.f);
   }
 }
 
@@ -151,7 +163,7 @@ int decode_generic_launch(const void* q, const void* key_cache, const void* valu
                           const int32_t* kept_blocks, const int32_t* kept_counts, int max_kept,
                           void* out, void* workspace, size_t workspace_bytes, int batch, int hq,
                           int hkv, int d, int bs, int max_blocks, int num_blocks, int quant,
-                          float sm_scale, hipStream_t s) {
+                          float sm_scale, hipStream_t s, RowMap rmap) {
   if (d > kMaxD || d % 4 != 0)
     return fail(FDATTN_ERR_SHAPE, "fdattn_decode_attention: head_dim %d unsupported (multiple of 4, <= %d)", d, kMaxD);
   const size_t need = generic_workspace_bytes(batch, hq, d);
@@ -166,7 +178,7 @@ int decode_generic_launch(const void* q, const void* key_cache, const void* valu
   float* part_l = part_m + (size_t)rows * nsplit;
   GenericDecodeArgs a{(const uint16_t*)q, (const uint8_t*)key_cache, (const uint8_t*)value_cache,
                       k_scale, v_scale, block_tables, seq_lens_decoder, seq_lens_this_time,
-                      kept_blocks, kept_counts, max_kept, part_o, part_m, part_l, batch, hq, hkv,
+                      kept_blocks, kept_counts, max_kept, part_o, part_m, part_l, rmap, batch, hq, hkv,
                       d, bs, max_blocks, num_blocks, nsplit, sm_scale};
   if (quant == FDATTN_CACHE_INT8)
     hipLaunchKernelGGL(decode_generic_kernel<FDATTN_CACHE_INT8>, dim3(rows, nsplit), dim3(64), 0, s, a);
@@ -175,7 +187,7 @@ int decode_generic_launch(const void* q, const void* key_cache, const void* valu
   int rc = check_launch("fdattn_decode_attention (generic)");
   if (rc) return rc;
   hipLaunchKernelGGL(splitkv_combine_kernel, dim3(rows), dim3(128), 0, s, part_o, part_m, part_l,
-                     (const int32_t*)nullptr, (uint16_t*)out, rows, nsplit, d);
+                     (const int32_t*)nullptr, (uint16_t*)out, rows, nsplit, d, hq, rmap);
   return check_launch("fdattn_splitkv_combine");
 }
 
@@ -193,6 +205,6 @@ extern "C" int fdattn_splitkv_combine(const float* part_o, const float* part_m, 
                 max_splits, head_dim);
   if (rows == 0) return 0;
   hipLaunchKernelGGL(splitkv_combine_kernel, dim3(rows), dim3(128), 0, (hipStream_t)stream, part_o, part_m,
-                     part_l, num_splits, (uint16_t*)out, rows, max_splits, head_dim);
+                     part_l, num_splits, (uint16_t*)out, rows, max_splits, head_dim, 0, RowMap{nullptr, nullptr});
   return check_launch("fdattn_splitkv_combine");
 }

@@ -11,6 +11,25 @@ namespace fdattn {
 int fail(int code, const char* fmt, ...);
 int check_launch(const char* what);
 
+// Rows of a mixed batch (prefill rows, decode rows and idle slots in one step).  With both
+// pointers NULL sequence b owns q / out row b and every sequence is a decode row.  Otherwise
+// sequence b's tokens are rows cu_seqlens_q[b] .. cu_seqlens_q[b+1]-1; it is a decode row if
+// it has exactly one token and seq_lens_encoder[b] == 0, a prefill row if seq_lens_encoder[b] > 0.
+struct RowMap {
+  const int32_t* cu_seqlens_q;
+  const int32_t* seq_lens_encoder;
+};
+// false: sequence b is not a decode row (nothing to read, nothing to write); row = its q / out row
+__device__ __forceinline__ bool decode_row(const RowMap& m, int b, int& row) {
+  row = b;
+  if (!m.cu_seqlens_q) return true;
+  row = m.cu_seqlens_q[b];
+  return m.cu_seqlens_q[b + 1] - row == 1 && (!m.seq_lens_encoder || m.seq_lens_encoder[b] == 0);
+}
+__device__ __forceinline__ bool prefill_row(const RowMap& m, int b) {
+  return !m.seq_lens_encoder || m.seq_lens_encoder[b] > 0;
+}
+
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
 typedef float v4f __attribute__((ext_vector_type(4)));

@@ -1,0 +1,33 @@
+// Launchers shared by the entry-point files of libfdattn.so.
+#pragma once
+#include "fdattn_common.h"
+
+namespace fdattn {
+
+size_t generic_workspace_bytes(int batch, int hq, int d);
+int decode_generic_launch(const void* q, const void* key_cache, const void* value_cache,
+                          const float* k_scale, const float* v_scale, const int32_t* block_tables,
+                          const int32_t* seq_lens_decoder, const int32_t* seq_lens_this_time,
+                          const int32_t* kept_blocks, const int32_t* kept_counts, int max_kept,
+                          void* out, void* workspace, size_t workspace_bytes, int batch, int hq,
+                          int hkv, int d, int bs, int max_blocks, int num_blocks, int quant,
+                          float sm_scale, hipStream_t s, RowMap rows = RowMap{nullptr, nullptr});
+size_t c8_workspace_bytes(int batch, int hkv, int max_units);
+bool c8_supported(int hq, int hkv, int d, int bs, int quant);
+// stages: 1 = the split-KV kernel, 2 = the merge of its partials, 3 = both
+int decode_c8_launch(const void* q, const void* key_cache, const void* value_cache,
+                     const float* k_scale, const float* v_scale, const int32_t* block_tables,
+                     const int32_t* seq_lens_decoder, const int32_t* seq_lens_this_time,
+                     const int32_t* kept_blocks, const int32_t* kept_counts, int max_kept,
+                     void* out, void* workspace, size_t workspace_bytes, int batch, int hq,
+                     int hkv, int d, int bs, int max_blocks, int num_blocks, int quant,
+                     float sm_scale, hipStream_t s, int stages, RowMap rows = RowMap{nullptr, nullptr});
+// append (prefill) attention; seq_lens_encoder may be NULL (every sequence is a prefill row)
+int prefill_launch(const void* q, const void* k_new, const void* v_new, const void* key_cache,
+                   const void* value_cache, const float* cache_k_scale, const float* cache_v_scale,
+                   const int32_t* block_tables, const int32_t* seq_lens_decoder, const int32_t* cu_seqlens_q,
+                   const int32_t* seq_lens_encoder, void* out, int num_tokens, int batch, int max_chunk, int hq,
+                   int hkv, int head_dim, int block_size, int max_blocks, int num_blocks, int cache_quant_type,
+                   float softmax_scale, hipStream_t s, bool force_generic);
+
+}  // namespace fdattn

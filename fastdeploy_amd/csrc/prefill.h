@@ -15,6 +15,7 @@ struct PrefillArgs {
   const int32_t* block_tables;
   const int32_t* seq_lens_decoder;
   const int32_t* cu_seqlens_q;
+  const int32_t* seq_lens_encoder;  // NULL, or > 0 for the sequences that are prefill rows of a mixed batch
   uint16_t* out;
   int num_tokens, batch, hq, hkv, d, bs, max_blocks, num_blocks;
   float sm_scale;

@@ -1,4 +1,5 @@
 // Chunked-prefill ("append") attention.
+#include "launch.h"
 #include "prefill.h"
 
 namespace fdattn {
@@ -27,6 +28,7 @@ __global__ __launch_bounds__(64) void prefill_generic_kernel(PrefillArgs a) {
   }
   const int b = lo;
   if (tok >= a.cu_seqlens_q[b + 1]) return;
+  if (a.seq_lens_encoder && a.seq_lens_encoder[b] <= 0) return;  // a decode row or an idle slot of a mixed batch
   const int ci = tok - a.cu_seqlens_q[b], p = a.seq_lens_decoder[b];
   const int nkeys = p + ci + 1;
   for (int c = lane; c < d; c += 64) qf[c] = bf16_to_f32(a.q[((size_t)tok * a.hq + qh) * d + c]) * a.sm_scale;
@@ -95,17 +97,12 @@ __global__ __launch_bounds__(64) void prefill_generic_kernel(PrefillArgs a) {
   }
 }
 
-}  // namespace fdattn
-
-using namespace fdattn;
-
-static int prefill_common(bool force_generic, const void* q, const void* k_new, const void* v_new,
-                          const void* key_cache, const void* value_cache, const float* cache_k_scale,
-                          const float* cache_v_scale, const int32_t* block_tables,
-                          const int32_t* seq_lens_decoder, const int32_t* cu_seqlens_q, void* out,
-                          int num_tokens, int batch, int max_chunk, int hq, int hkv, int head_dim,
-                          int block_size, int max_blocks_per_seq, int num_blocks, int cache_quant_type,
-                          float softmax_scale, void* stream) {
+int prefill_launch(const void* q, const void* k_new, const void* v_new, const void* key_cache,
+                   const void* value_cache, const float* cache_k_scale, const float* cache_v_scale,
+                   const int32_t* block_tables, const int32_t* seq_lens_decoder, const int32_t* cu_seqlens_q,
+                   const int32_t* seq_lens_encoder, void* out, int num_tokens, int batch, int max_chunk, int hq,
+                   int hkv, int head_dim, int block_size, int max_blocks_per_seq, int num_blocks,
+                   int cache_quant_type, float softmax_scale, hipStream_t s, bool force_generic) {
   if (!q || !k_new || !v_new || !key_cache || !value_cache || !cache_k_scale || !cache_v_scale ||
       !block_tables || !seq_lens_decoder || !cu_seqlens_q || !out)
     return fail(FDATTN_ERR_NULL, "fdattn_append_attention_prefill: a required pointer is NULL");
@@ -120,9 +117,8 @@ static int prefill_common(bool force_generic, const void* q, const void* k_new, 
   if (num_tokens == 0) return 0;
   PrefillArgs a{(const uint16_t*)q, (const uint16_t*)k_new, (const uint16_t*)v_new, (const uint8_t*)key_cache,
                 (const uint8_t*)value_cache, cache_k_scale, cache_v_scale, block_tables, seq_lens_decoder,
-                cu_seqlens_q, (uint16_t*)out, num_tokens, batch, hq, hkv, head_dim, block_size,
+                cu_seqlens_q, seq_lens_encoder, (uint16_t*)out, num_tokens, batch, hq, hkv, head_dim, block_size,
                 max_blocks_per_seq, num_blocks, softmax_scale};
-  hipStream_t s = (hipStream_t)stream;
   if (!force_generic && prefill_mfma_supported(hq, hkv, head_dim, block_size, cache_quant_type))
     return prefill_mfma_launch(a, max_chunk, cache_quant_type, s);
   if (cache_quant_type == FDATTN_CACHE_INT8)
@@ -132,16 +128,20 @@ static int prefill_common(bool force_generic, const void* q, const void* k_new, 
   return check_launch("fdattn_append_attention_prefill");
 }
 
+}  // namespace fdattn
+
+using namespace fdattn;
+
 extern "C" int fdattn_append_attention_prefill(
     const void* q, const void* k_new, const void* v_new, const void* key_cache, const void* value_cache,
     const float* cache_k_scale, const float* cache_v_scale, const int32_t* block_tables,
     const int32_t* seq_lens_decoder, const int32_t* cu_seqlens_q, void* out, int num_tokens, int batch,
     int max_chunk, int hq, int hkv, int head_dim, int block_size, int max_blocks_per_seq, int num_blocks,
     int cache_quant_type, float softmax_scale, void* stream) {
-  return prefill_common(false, q, k_new, v_new, key_cache, value_cache, cache_k_scale, cache_v_scale,
-                        block_tables, seq_lens_decoder, cu_seqlens_q, out, num_tokens, batch, max_chunk, hq,
-                        hkv, head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type,
-                        softmax_scale, stream);
+  return prefill_launch(q, k_new, v_new, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
+                        seq_lens_decoder, cu_seqlens_q, nullptr, out, num_tokens, batch, max_chunk, hq, hkv,
+                        head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type, softmax_scale,
+                        (hipStream_t)stream, false);
 }
 
 extern "C" int fdattn_append_attention_prefill_generic(
@@ -150,8 +150,8 @@ extern "C" int fdattn_append_attention_prefill_generic(
     const int32_t* seq_lens_decoder, const int32_t* cu_seqlens_q, void* out, int num_tokens, int batch,
     int max_chunk, int hq, int hkv, int head_dim, int block_size, int max_blocks_per_seq, int num_blocks,
     int cache_quant_type, float softmax_scale, void* stream) {
-  return prefill_common(true, q, k_new, v_new, key_cache, value_cache, cache_k_scale, cache_v_scale,
-                        block_tables, seq_lens_decoder, cu_seqlens_q, out, num_tokens, batch, max_chunk, hq,
-                        hkv, head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type,
-                        softmax_scale, stream);
+  return prefill_launch(q, k_new, v_new, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
+                        seq_lens_decoder, cu_seqlens_q, nullptr, out, num_tokens, batch, max_chunk, hq, hkv,
+                        head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type, softmax_scale,
+                        (hipStream_t)stream, true);
 }

@@ -78,8 +78,7 @@ __device__ __forceinline__ u32 pack_f16(float lo, float hi) {
   const v2h v = {(_Float16)lo, (_Float16)hi};
   return __builtin_bit_cast(u32, v);
 }
-// two floats -> packed fp16 in one instruction (round toward zero): exact for e4m3 values,
-// a 2^-11 downward nudge for softmax weights
+// two floats -> packed fp16, round toward zero: exact for e4m3 values
 __device__ __forceinline__ u32 pack_f16_fast(float lo, float hi) {
   return __builtin_bit_cast(u32, __builtin_amdgcn_cvt_pkrtz(lo, hi));
 }
@@ -137,6 +136,7 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   const int qt = (int)gridDim.x - 1 - (int)blockIdx.x;  // long rows (late tokens) first
   const int q0 = qt * BM;
   if (q0 >= n_b) return;
+  if (a.seq_lens_encoder && a.seq_lens_encoder[b] <= 0) return;  // a decode row or an idle slot of a mixed batch
 
   const int j32 = lane & 31, hf = lane >> 5;
   // this lane's query; rows past the chunk behave like its last row and are not stored
@@ -362,7 +362,7 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
             u32 w[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-              w[e] = pack_f16_fast(e8[2 * e], e8[2 * e + 1]);
+              w[e] = pack_f16(e8[2 * e], e8[2 * e + 1]);  // round to nearest: truncation would bias every weight down
               // the sum is taken over the rounded weights, the ones the MFMA multiplies
               ls[e] = __builtin_amdgcn_fdot2(__builtin_bit_cast(v2h, w[e]), ones, ls[e], false);
             }

@@ -235,7 +235,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
   if (wv + kWaves < cnt)
     dma_tile(kbase + (size_t)__builtin_amdgcn_readlane(my_pb, wv + kWaves) * blk_stride, saddr0 + kTileB, offK);
   PairState st;
-  load_pair<QUANT>(a.q, a.k_scale, a.hkv, 1.0f, p, lane, st);  // scores in natural units
+  load_pair<QUANT>(a.q, a.k_scale, a.hkv, 1.0f, p, p / a.hkv, lane, st);  // scores in natural units
   // fp8: a second operand, |q*scale| in one e4m3 limb, gives sum_c |q*scale||k| per token next to the score;
   // the error of a block's score is a small multiple of that sum (see the bound below)
   v4i aabs[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};

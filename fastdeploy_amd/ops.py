@@ -309,29 +309,71 @@ def append_attention_prefill(q, k_new, v_new, key_cache, value_cache, cache_k_sc
     return out
 
 
+def append_attention_workspace(num_tokens, batch, num_heads, kv_heads, head_dim, max_blocks_per_seq, device="cuda"):
+    """A workspace tensor large enough for append_attention at these shapes."""
+    n = _lib.lib().fdattn_append_attention_workspace_bytes(num_tokens, batch, num_heads, kv_heads, head_dim,
+                                                          max_blocks_per_seq)
+    return torch.empty(n, dtype=torch.uint8, device=device)
+
+
 def append_attention(qkv, key_cache, value_cache, seq_lens_encoder, seq_lens_decoder, seq_lens_this_time,
                      block_tables, rotary_embs, cache_k_scale, cache_v_scale, *, num_heads, kv_num_heads,
                      max_chunk, rope_style="neox", cache_quant_type="cache_int8", softmax_scale=None,
-                     workspace=None):
-    """One attention step of a batch that is either all decode rows (one new token
-    each, seq_lens_encoder == 0) or all prefill rows (max_chunk > 1): cache write,
-    then decode attention over the cache, or append attention over prefix + chunk.
+                     cu_seqlens_q=None, workspace=None, out=None):
+    """One attention step of a layer over a mixed batch (one call into the library):
+    every new token is rotated and written to the cache, decode rows (one token,
+    seq_lens_encoder == 0) attend to the cache, prefill rows (seq_lens_encoder > 0)
+    to their cached prefix and causally to their own chunk; slots without a token
+    are skipped.  max_chunk bounds the tokens of one sequence (1 = decode only).
     Returns bf16 [num_tokens, num_heads*head_dim]."""
-    cu = cu_seqlens_of(seq_lens_this_time)
-    prefill = max_chunk > 1
-    q, k_new, v_new = write_cache_kv(
-        qkv, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables, seq_lens_encoder,
-        seq_lens_decoder, seq_lens_this_time, cu, rotary_embs, num_heads=num_heads,
-        kv_num_heads=kv_num_heads, rope_style=rope_style, cache_quant_type=cache_quant_type,
-        want_kv_out=prefill)
-    if prefill:
-        return append_attention_prefill(
-            q, k_new, v_new, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
-            seq_lens_decoder, cu, num_heads=num_heads, max_chunk=max_chunk,
-            cache_quant_type=cache_quant_type, softmax_scale=softmax_scale)
-    if qkv.shape[0] != block_tables.shape[0]:
-        raise ValueError("a decode step needs exactly one token per sequence")
-    return decode_attention(
-        q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables, seq_lens_decoder,
-        seq_lens_this_time, num_heads=num_heads, cache_quant_type=cache_quant_type,
-        softmax_scale=softmax_scale, workspace=workspace)
+    nb, hkv, bs, d = _cache_dims(key_cache, value_cache)
+    if hkv != kv_num_heads:
+        raise ValueError("cache holds %d KV heads, kv_num_heads=%d" % (hkv, kv_num_heads))
+    p_qkv = _chk(qkv, "qkv", torch.bfloat16, 2)
+    T = qkv.shape[0]
+    if qkv.shape[1] != (num_heads + 2 * hkv) * d:
+        raise ValueError("qkv has %d columns, expected (num_heads+2*kv_num_heads)*head_dim = %d" %
+                         (qkv.shape[1], (num_heads + 2 * hkv) * d))
+    p_kc = _chk(key_cache, "key_cache", _CACHE_DT, 4)
+    p_vc = _chk(value_cache, "value_cache", _CACHE_DT, 4)
+    p_ks, p_vs = _scales(cache_k_scale, cache_v_scale, hkv, d)
+    p_bt = _chk(block_tables, "block_tables", torch.int32, 2)
+    batch, mb = block_tables.shape
+    p_enc = _chk(seq_lens_encoder, "seq_lens_encoder", torch.int32, 1)
+    p_dec = _chk(seq_lens_decoder, "seq_lens_decoder", torch.int32, 1)
+    p_this = _chk(seq_lens_this_time, "seq_lens_this_time", torch.int32, 1)
+    for name, t in (("seq_lens_encoder", seq_lens_encoder), ("seq_lens_decoder", seq_lens_decoder),
+                    ("seq_lens_this_time", seq_lens_this_time)):
+        if t.numel() != batch:
+            raise ValueError("%s has %d entries, block_tables %d rows" % (name, t.numel(), batch))
+    if cu_seqlens_q is None:
+        cu_seqlens_q = cu_seqlens_of(seq_lens_this_time)
+    p_cu = _chk(cu_seqlens_q, "cu_seqlens_q", torch.int32, 1)
+    if cu_seqlens_q.numel() != batch + 1:
+        raise ValueError("cu_seqlens_q must have batch+1 entries")
+    p_cos = p_sin = 0
+    max_pos = 0
+    if rotary_embs is not None:
+        cos, sin = rotary_embs
+        p_cos = _chk(cos, "rotary cos", torch.float32, 2)
+        p_sin = _chk(sin, "rotary sin", torch.float32, 2)
+        if cos.shape != sin.shape or cos.shape[1] != d // 2:
+            raise ValueError("rotary table must be [max_pos, head_dim/2]")
+        max_pos = cos.shape[0]
+    if rope_style not in _ROPE:
+        raise ValueError("unknown rope_style %r (neox | interleaved)" % (rope_style,))
+    if max_chunk < 1:
+        raise ValueError("max_chunk must be >= 1")
+    if out is None:
+        out = torch.empty((T, num_heads * d), dtype=torch.bfloat16, device=qkv.device)
+    need = _lib.lib().fdattn_append_attention_workspace_bytes(T, batch, num_heads, hkv, d, mb)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=qkv.device)
+    scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(d)
+    rc = _lib.lib().fdattn_append_attention(
+        p_qkv, p_kc, p_vc, p_ks, p_vs, p_cos, p_sin, p_bt, p_enc, p_dec, p_this, p_cu,
+        _chk(out, "out", torch.bfloat16), workspace.data_ptr(), workspace.numel() * workspace.element_size(),
+        T, batch, max_chunk, num_heads, hkv, d, bs, mb, nb, max_pos, _ROPE[rope_style], _quant(cache_quant_type),
+        scale, _stream())
+    _lib.check(rc, "append_attention")
+    return out

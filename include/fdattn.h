@@ -265,8 +265,8 @@ FDATTN_API int fdattn_append_attention_prefill(
 
 /*
  * The shape-agnostic kernel fdattn_append_attention_prefill falls back to when the
- * MFMA kernel does not cover the shape (it covers head_dim 128, hq/hkv 4,
- * block_size 64), callable directly.  Same arguments and plug-in position.
+ * MFMA kernel does not cover the shape (it covers head_dim 128, block_size 64),
+ * callable directly.  Same arguments and plug-in position.
  */
 FDATTN_API int fdattn_append_attention_prefill_generic(
     const void* q, const void* k_new, const void* v_new,
@@ -277,6 +277,40 @@ FDATTN_API int fdattn_append_attention_prefill_generic(
     int num_tokens, int batch, int max_chunk, int hq, int hkv, int head_dim,
     int block_size, int max_blocks_per_seq, int num_blocks,
     int cache_quant_type, float softmax_scale, void* stream);
+
+/*
+ * Bytes of workspace fdattn_append_attention needs for these shapes (rotated Q, the
+ * chunk's K and V, split-KV partial results).  Never 0; no initialisation needed.
+ */
+FDATTN_API size_t fdattn_append_attention_workspace_bytes(int num_tokens, int batch, int hq, int hkv,
+                                                          int head_dim, int max_blocks_per_seq);
+
+/*
+ * One attention step of a layer over a mixed batch: the whole of what an engine-side
+ * attention operator does between the QKV projection and the output projection
+ * (plug-in position as for the pieces above,
+ * fastdeploy/runtime/backends/paddle/ops/voxelize_op.cc:159-204).  Sequence b owns the
+ * token rows cu_seqlens_q[b] .. cu_seqlens_q[b+1]-1 of qkv and out and is
+ *   a prefill row  if seq_lens_encoder[b] > 0: its tokens are appended to the
+ *                  seq_lens_decoder[b] cached ones (fdattn_append_attention_prefill),
+ *   a decode row   if seq_lens_encoder[b] == 0 and it has one token: the token is written
+ *                  to the cache and attends to seq_lens_decoder[b] + 1 cached tokens
+ *                  (fdattn_decode_attention),
+ *   idle           otherwise (no token: nothing is read or written for it).
+ * Every new token is first rotated and written to the cache (fdattn_write_cache_kv).
+ * max_chunk bounds the tokens of one sequence in this step (1 = no prefill row).
+ * Nothing is gathered or synchronised on the host; out rows of idle slots do not exist.
+ */
+FDATTN_API int fdattn_append_attention(
+    const void* qkv, void* key_cache, void* value_cache,
+    const float* cache_k_scale, const float* cache_v_scale,
+    const float* rope_cos, const float* rope_sin,
+    const int32_t* block_tables, const int32_t* seq_lens_encoder,
+    const int32_t* seq_lens_decoder, const int32_t* seq_lens_this_time,
+    const int32_t* cu_seqlens_q, void* out, void* workspace, size_t workspace_bytes,
+    int num_tokens, int batch, int max_chunk, int hq, int hkv, int head_dim,
+    int block_size, int max_blocks_per_seq, int num_blocks, int max_pos,
+    int rope_style, int cache_quant_type, float softmax_scale, void* stream);
 
 #ifdef __cplusplus
 }

@@ -210,8 +210,8 @@ def test_decode_step_replays_from_a_hip_graph():
     dev = syn.to_device(case, "cuda")
     eag = {k: (v.clone() if isinstance(v, torch.Tensor) else v) for k, v in dev.items()}
     rot_g, rot_e = (dev["rope_cos"], dev["rope_sin"]), (eag["rope_cos"], eag["rope_sin"])
-    ws_g = fd.decode_workspace(48, 32, 8, 128, 34, "cuda")
-    ws_e = fd.decode_workspace(48, 32, 8, 128, 34, "cuda")
+    ws_g = fd.append_attention_workspace(48, 48, 32, 8, 128, 34)
+    ws_e = fd.append_attention_workspace(48, 48, 32, 8, 128, 34)
 
     def step(c, rot, ws):
         out = fd.append_attention(c["qkv"], c["key_cache"], c["value_cache"], c["seq_lens_encoder"],

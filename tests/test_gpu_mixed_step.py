@@ -1,0 +1,115 @@
+"""One attention step over a mixed batch (prefill rows, decode rows, idle slots in one call) against the
+CPU oracle: cache bytes bit-exact, bf16 outputs within 2e-3 abs OR 1e-2 rel."""
+import numpy as np
+import pytest
+import torch
+
+import fastdeploy_amd as fd
+from conftest import bf16_close, bits, np_of
+from fastdeploy_amd.ops import CACHE_FP8, CACHE_INT8, cu_seqlens_of, seq_lens_this_time_of
+from fastdeploy_amd.rope import rope_table
+
+pytestmark = pytest.mark.gpu
+
+
+def mixed_case(enc, dec, quant, seed, hq=32, hkv=8, d=128, bs=64, max_pos=4096):
+    g = torch.Generator().manual_seed(seed)
+    batch = len(enc)
+    enc_t, dec_t = torch.tensor(enc, dtype=torch.int32), torch.tensor(dec, dtype=torch.int32)
+    this = seq_lens_this_time_of(enc_t, dec_t)
+    cu = cu_seqlens_of(this)
+    T = int(cu[-1])
+    mb = max((int(dec[b]) + int(this[b]) + bs - 1) // bs for b in range(batch)) + 1
+    pool = batch * mb
+    bt = torch.randperm(pool, generator=g).to(torch.int32).view(batch, mb).contiguous()
+    kc = torch.randint(0, 256, (pool, hkv, bs, d), generator=g, dtype=torch.uint8)
+    vc = torch.randint(0, 256, (pool, hkv, bs, d), generator=g, dtype=torch.uint8)
+    if quant == CACHE_FP8:  # no NaN codes in the prior contents
+        kc = torch.where((kc & 0x7F) == 0x7F, kc & 0xFE, kc)
+        vc = torch.where((vc & 0x7F) == 0x7F, vc & 0xFE, vc)
+    # The prior cache bytes are uniform over all codes - far heavier-tailed than quantised activations - so the
+    # scales put the dequantised range at +-(1..1.5): the prefill kernel carries q*k_scale and the softmax weights
+    # in fp16, and its error grows with the magnitude of the dequantised cache.
+    qmax = 127.0 if quant == CACHE_INT8 else 448.0
+    ks = ((torch.rand((hkv, d), generator=g) * 0.5 + 1.0) / qmax).contiguous()
+    vs = ((torch.rand((hkv, d), generator=g) * 0.5 + 1.0) / qmax).contiguous()
+    qkv = torch.randn((T, (hq + 2 * hkv) * d), generator=g).to(torch.bfloat16)
+    cos, sin = rope_table(max_pos, d, 500000.0, "cpu")
+    return dict(qkv=qkv, key_cache=kc, value_cache=vc, cache_k_scale=ks, cache_v_scale=vs, block_tables=bt,
+                seq_lens_encoder=enc_t, seq_lens_decoder=dec_t, seq_lens_this_time=this, cu_seqlens_q=cu,
+                rope_cos=cos, rope_sin=sin, T=T)
+
+
+def oracle_step(oracle, c, quant, hq=32, hkv=8, d=128):
+    """The step composed from the oracle's pieces; returns (out bf16 bits [T, hq*d] with NaN-free rows only where
+    a token exists, key cache, value cache)."""
+    kc, vc = np_of(c["key_cache"]).copy(), np_of(c["value_cache"]).copy()
+    ks, vs = np_of(c["cache_k_scale"]), np_of(c["cache_v_scale"])
+    bt, dec, cu = np_of(c["block_tables"]), np_of(c["seq_lens_decoder"]), np_of(c["cu_seqlens_q"])
+    enc, this = np_of(c["seq_lens_encoder"]), np_of(c["seq_lens_this_time"])
+    q, k_new, v_new = oracle.write_cache_kv(bits(c["qkv"]), kc, vc, ks, vs, np_of(c["rope_cos"]), np_of(c["rope_sin"]),
+                                            bt, dec, cu, hq, hkv, d, 1, quant, want_kv_out=True)
+    out = np.zeros((c["T"], hq * d), np.uint16)
+    drows = [b for b in range(len(enc)) if enc[b] == 0 and this[b] == 1]
+    if drows:
+        qd = np.ascontiguousarray(q[[cu[b] for b in drows]])
+        od = oracle.decode_attention(qd, kc, vc, ks, vs, np.ascontiguousarray(bt[drows]),
+                                     np.ascontiguousarray(dec[drows] + 1), hq, hkv, d, quant)
+        for i, b in enumerate(drows):
+            out[cu[b]] = od[i]
+    ptoks = np.array([t for b in range(len(enc)) if enc[b] > 0 for t in range(cu[b], cu[b + 1])], np.int32)
+    if len(ptoks):
+        op = oracle.append_attention_prefill(q, k_new, v_new, kc, vc, ks, vs, bt, dec, cu, hq, hkv, d, quant,
+                                             token_ids=ptoks)
+        out[ptoks] = op[ptoks]
+    return out, kc, vc
+
+
+@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+def test_mixed_batch_step(oracle, quant):
+    enc = [0, 150, 0, 0, 70, 0, 1, 300]
+    dec = [700, 0, 0, 63, 200, 1, 0, 129]
+    c = mixed_case(enc, dec, quant, seed=7)
+    dev = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
+    out = fd.append_attention(dev["qkv"], dev["key_cache"], dev["value_cache"], dev["seq_lens_encoder"],
+                              dev["seq_lens_decoder"], dev["seq_lens_this_time"], dev["block_tables"],
+                              (dev["rope_cos"], dev["rope_sin"]), dev["cache_k_scale"], dev["cache_v_scale"],
+                              num_heads=32, kv_num_heads=8, max_chunk=300, cache_quant_type=quant,
+                              cu_seqlens_q=dev["cu_seqlens_q"])
+    torch.cuda.synchronize()
+    want, kc, vc = oracle_step(oracle, c, quant)
+    assert np.array_equal(np_of(dev["key_cache"]), kc) and np.array_equal(np_of(dev["value_cache"]), vc)
+    ok, mx, bad = bf16_close(bits(out), want)
+    assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
+
+
+def test_decode_only_and_prefill_only_steps_through_the_same_entry(oracle):
+    for enc, dec, mc in (([0, 0, 0, 0], [5, 64, 1000, 0], 1), ([64, 1, 257, 0], [0, 0, 100, 0], 257)):
+        c = mixed_case(enc, dec, CACHE_INT8, seed=9)
+        dev = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
+        ws = fd.append_attention_workspace(c["T"], len(enc), 32, 8, 128, dev["block_tables"].shape[1])
+        out = fd.append_attention(dev["qkv"], dev["key_cache"], dev["value_cache"], dev["seq_lens_encoder"],
+                                  dev["seq_lens_decoder"], dev["seq_lens_this_time"], dev["block_tables"],
+                                  (dev["rope_cos"], dev["rope_sin"]), dev["cache_k_scale"], dev["cache_v_scale"],
+                                  num_heads=32, kv_num_heads=8, max_chunk=mc, workspace=ws)
+        torch.cuda.synchronize()
+        want, kc, vc = oracle_step(oracle, c, CACHE_INT8)
+        assert np.array_equal(np_of(dev["key_cache"]), kc) and np.array_equal(np_of(dev["value_cache"]), vc)
+        ok, mx, bad = bf16_close(bits(out), want)
+        assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
+
+
+def test_mixed_step_other_shape_runs_on_the_generic_kernels(oracle):
+    """head_dim 64, 2 query heads per KV head, block_size 16: none of the MFMA kernels covers it."""
+    hq, hkv, d, bs = 4, 2, 64, 16
+    c = mixed_case([0, 40, 0, 9], [33, 0, 0, 20], CACHE_INT8, seed=3, hq=hq, hkv=hkv, d=d, bs=bs, max_pos=256)
+    dev = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
+    out = fd.append_attention(dev["qkv"], dev["key_cache"], dev["value_cache"], dev["seq_lens_encoder"],
+                              dev["seq_lens_decoder"], dev["seq_lens_this_time"], dev["block_tables"],
+                              (dev["rope_cos"], dev["rope_sin"]), dev["cache_k_scale"], dev["cache_v_scale"],
+                              num_heads=hq, kv_num_heads=hkv, max_chunk=40)
+    torch.cuda.synchronize()
+    want, kc, vc = oracle_step(oracle, c, CACHE_INT8, hq, hkv, d)
+    assert np.array_equal(np_of(dev["key_cache"]), kc) and np.array_equal(np_of(dev["value_cache"]), vc)
+    ok, mx, bad = bf16_close(bits(out), want)
+    assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
