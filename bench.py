@@ -85,6 +85,18 @@ def other_workloads(args):
         ms = time_events(dec, args.steps, args.warmup)
         line("configs[2] decode (batch 256, ctx = pos+1, mean 4k)", ms, "hbm", syn.decode_algorithmic_bytes(lens, 256),
              HBM_PEAK_GBPS, "GB/s")
+        # the same two pieces as ONE library call (the cache keeps being rewritten at the same positions)
+        sws = fd.append_attention_workspace(256, 256, 32, 8, 128, 128, dev)
+        sout = torch.empty((256, 32 * 128), dtype=torch.bfloat16, device=dev)
+
+        def fused():
+            fd.append_attention(c["qkv"], c["key_cache"], c["value_cache"], c["seq_lens_encoder"], c["seq_lens_decoder"],
+                                c["seq_lens_this_time"], c["block_tables"], rot, c["cache_k_scale"], c["cache_v_scale"],
+                                num_heads=32, kv_num_heads=8, max_chunk=1, cu_seqlens_q=c["cu_seqlens_q"], workspace=sws,
+                                out=sout)
+        ms = time_events(fused, args.steps, args.warmup)
+        line("configs[2] fused step: cache write + decode in one call", ms, "hbm",
+             syn.decode_algorithmic_bytes(lens, 256) + 256 * (48 * 128 * 2 + 2 * 8 * 128 + 32 * 128 * 2), HBM_PEAK_GBPS, "GB/s")
 
     if args.workload in ("sqattn", "all"):
         # configs[3]: batch 16, ctx 32768, fp8 KV, top-64 of 512 blocks per KV head
