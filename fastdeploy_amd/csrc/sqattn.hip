@@ -333,32 +333,37 @@ __device__ __forceinline__ float key_to_float(unsigned k) {
   return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
 }
 
-// The r-th largest (r = 1 is the maximum) of v[j] + sign * e[j], j < n, found by a whole 256-thread
-// workgroup; every thread returns the value.  hist: 256 ints, sel: 2 unsigneds of shared memory.
-__device__ float radix_select_desc(const float* v, const float* e, float sign, int n, int r, int* hist, unsigned* sel) {
-  const int tid = threadIdx.x;
-  unsigned prefix = 0, mask = 0;
-  int remaining = r;
+// Two order statistics in one sweep, by a whole 256-thread workgroup: out[0] = the r0-th largest
+// (r = 1 is the maximum) of v[j] - e[j] and out[1] = the r1-th largest of v[j] + e[j], j < n.  Radix
+// selection over order-preserving integer keys, 4 passes of 8 bits; wavefront w < 2 scans the
+// histogram of selection w.  hist: 2 x 256 ints, sel: 2 x 2 unsigneds of shared memory.
+__device__ void radix_select2_desc(const float* v, const float* e, int n, int r0, int r1, int* hist, unsigned* sel,
+                                   float* out) {
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  unsigned prefix[2] = {0u, 0u}, mask = 0;
+  int remaining[2] = {r0, r1};
   for (int shift = 24; shift >= 0; shift -= 8) {
     hist[tid] = 0;
+    hist[256 + tid] = 0;
     __syncthreads();
     for (int j = tid; j < n; j += 256) {
-      const unsigned key = order_key(v[j] + sign * e[j]);
-      if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1);
+      const unsigned k0 = order_key(v[j] - e[j]), k1 = order_key(v[j] + e[j]);
+      if ((k0 & mask) == prefix[0]) atomicAdd(&hist[(k0 >> shift) & 255u], 1);
+      if ((k1 & mask) == prefix[1]) atomicAdd(&hist[256 + ((k1 >> shift) & 255u)], 1);
     }
     __syncthreads();
-    if (tid < 64) {
-      // bins 255 .. 0 in 4 groups of 64 handled by one wavefront: find the bin where the count from the
-      // top reaches `remaining`
-      int rem = remaining, found = -1;
+    if (wv < 2) {
+      // bins 255 .. 0 in 4 groups of 64: find the bin where the count from the top reaches `remaining`
+      const int* hs = hist + 256 * wv;
+      int rem = remaining[wv], found = -1;
       for (int grp = 3; grp >= 0 && found < 0; --grp) {
-        const int bin = grp * 64 + (63 - tid);  // lane 0 holds the highest bin of the group
-        const int c = hist[bin];
+        const int bin = grp * 64 + (63 - lane);  // lane 0 holds the highest bin of the group
+        const int c = hs[bin];
         int incl = c;
 #pragma unroll
         for (int o = 1; o < 64; o <<= 1) {
           const int t = __shfl_up(incl, o, 64);
-          if (tid >= o) incl += t;
+          if (lane >= o) incl += t;
         }
         const unsigned long long hit = __ballot(incl >= rem);
         if (hit) {
@@ -369,15 +374,18 @@ __device__ float radix_select_desc(const float* v, const float* e, float sign, i
           rem -= __shfl(incl, 63, 64);
         }
       }
-      if (tid == 0) { sel[0] = (unsigned)found; sel[1] = (unsigned)rem; }
+      if (lane == 0) { sel[2 * wv] = (unsigned)found; sel[2 * wv + 1] = (unsigned)rem; }
     }
     __syncthreads();
-    prefix |= sel[0] << shift;
+    prefix[0] |= sel[0] << shift;
+    prefix[1] |= sel[2] << shift;
     mask |= 255u << shift;
-    remaining = (int)sel[1];
+    remaining[0] = (int)sel[1];
+    remaining[1] = (int)sel[3];
     __syncthreads();
   }
-  return key_to_float(prefix);
+  out[0] = key_to_float(prefix[0]);
+  out[1] = key_to_float(prefix[1]);
 }
 
 // One workgroup per (sequence, KV head): classify, re-score the undecided blocks in fp64, emit.
@@ -390,9 +398,8 @@ __global__ __launch_bounds__(256) void sqattn_resolve_kernel(SelArgs a) {
   int* ulist = state + a.max_blocks;                              // undecided block ids
   __shared__ float qs[kG][kD];
   __shared__ int n_in, n_unc, wave_tot[4], running;
-  __shared__ float thr[2];
-  __shared__ int hist[256];
-  __shared__ unsigned sel[2];
+  __shared__ int hist[512];
+  __shared__ unsigned sel[4];
   const int p = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int b = p / a.hkv, h = p - b * a.hkv;
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
@@ -411,11 +418,11 @@ __global__ __launch_bounds__(256) void sqattn_resolve_kernel(SelArgs a) {
     const float* eb = a.ebound ? a.ebound + (size_t)p * a.max_blocks : nullptr;
     for (int j = tid; j < nblk; j += 256) se[j] = eb ? eb[j] : eps;
     __syncthreads();
-    // k-th largest lower bound and (k+1)-th largest upper bound by radix selection (4 passes of 8 bits
-    // over order-preserving integer keys), not by ranking every block against every other
-    thr[0] = radix_select_desc(sf, se, -1.0f, nblk, k, hist, sel);
-    thr[1] = radix_select_desc(sf, se, +1.0f, nblk, k + 1, hist, sel);
-    const float lk = thr[0], uk1 = thr[1];
+    // k-th largest lower bound and (k+1)-th largest upper bound by radix selection, both in the same
+    // four passes - not by ranking every block against every other
+    float both[2];
+    radix_select2_desc(sf, se, nblk, k, k + 1, hist, sel, both);
+    const float lk = both[0], uk1 = both[1];
     for (int j = tid; j < nblk; j += 256) {
       const float lj = sf[j] - se[j], uj = sf[j] + se[j];
       int stt = 2;
