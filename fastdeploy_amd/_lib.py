@@ -27,6 +27,15 @@ SIGNATURES = {
     "fdattn_append_attention_prefill_generic": (_i, [_vp] * 11 + [_i] * 10 + [_f, _vp]),
     "fdattn_append_attention_workspace_bytes": (_sz, [_i] * 6),
     "fdattn_append_attention": (_i, [_vp] * 14 + [_sz] + [_i] * 12 + [_f, _vp]),
+    "fdattn_pool_create": (_vp, [_i] * 4),
+    "fdattn_pool_destroy": (None, [_vp]),
+    "fdattn_pool_reserve": (_i, [_vp, _i, _i]),
+    "fdattn_pool_release": (_i, [_vp, _i]),
+    "fdattn_pool_fork": (_i, [_vp, _i, _i, _i]),
+    "fdattn_pool_free_blocks": (_i, [_vp]),
+    "fdattn_pool_seq_blocks": (_i, [_vp, _i]),
+    "fdattn_pool_refcount": (_i, [_vp, _i]),
+    "fdattn_pool_block_tables": (ctypes.POINTER(ctypes.c_int32), [_vp]),
 }
 
 _lib = None

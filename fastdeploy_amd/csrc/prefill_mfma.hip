@@ -42,6 +42,8 @@
 // LDS rows: K 272 B apart (the 32 rows a ds_read_b128 touches fall on distinct banks), V
 // 320 B apart (the 4 rows x 64 B a ds_read_b64_tr_b16 half-wave touches fall on distinct
 // banks); both tiles are written as whole 256 B rows by 16 consecutive lanes.
+#include <atomic>
+
 #include "prefill.h"
 
 namespace fdattn {
@@ -435,12 +437,16 @@ hipError_t launch_one(const PrefillArgs& a, int max_chunk, hipStream_t s) {
   constexpr int BM = 32 * NW;
   const dim3 grid((max_chunk + BM - 1) / BM, a.hq, a.batch), block(64 * NW);
   const size_t shm = (size_t)kSlots * BUF_ELEMS * sizeof(uint16_t);  // 151,552 B
-  static bool attr_set = false;  // one flag per instantiation
-  if (!attr_set) {
-    const hipError_t e = hipFuncSetAttribute((const void*)prefill_mfma_kernel<QUANT, NW>,
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm);
+  // the dynamic LDS limit is a per-device property of the kernel: raise it once on each device
+  static std::atomic<unsigned long long> raised{0};  // bit d: done on device d (one word per instantiation)
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev >= 64 || !(raised.load(std::memory_order_relaxed) >> dev & 1ull)) {
+    e = hipFuncSetAttribute((const void*)prefill_mfma_kernel<QUANT, NW>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)shm);
     if (e != hipSuccess) return e;
-    attr_set = true;
+    if (dev < 64) raised.fetch_or(1ull << dev, std::memory_order_relaxed);
   }
   hipLaunchKernelGGL((prefill_mfma_kernel<QUANT, NW>), grid, block, shm, s, a);
   return hipSuccess;

@@ -62,6 +62,7 @@ extern "C" {
 #define FDATTN_ERR_SHAPE -2       /* a shape the kernels do not support      */
 #define FDATTN_ERR_QUANT -3       /* unknown cache_quant_type / rope_style   */
 #define FDATTN_ERR_WORKSPACE -4   /* workspace too small                     */
+#define FDATTN_ERR_POOL -5        /* block pool exhausted / out of host memory */
 
 /* Library identification, "fdattn <major>.<minor> gfx950". */
 FDATTN_API const char* fdattn_version(void);
@@ -311,6 +312,34 @@ FDATTN_API int fdattn_append_attention(
     int num_tokens, int batch, int max_chunk, int hq, int hkv, int head_dim,
     int block_size, int max_blocks_per_seq, int num_blocks, int max_pos,
     int rope_style, int cache_quant_type, float softmax_scale, void* stream);
+
+/*
+ * Host-side block pool: the producer of block_tables (no counterpart in the reference,
+ * whose engines own their memory, fastdeploy/runtime/backends/paddle/paddle_backend.cc:425-427;
+ * handle-style C API after c_api/fastdeploy_capi/core/fd_type.h:104-155: create / destroy
+ * pairs, the caller owns the handle).  num_blocks cache blocks of block_size tokens,
+ * max_seqs sequence slots, each with a table row of max_blocks_per_seq entries (-1 = no
+ * block).  Blocks are reference counted; fdattn_pool_fork shares the whole blocks of a
+ * prefix between two slots.  Not thread-safe.  No GPU call is made: copy the table (int32
+ * [max_seqs, max_blocks_per_seq]) to the device where block_tables is needed.
+ */
+typedef struct fdattn_block_pool fdattn_block_pool;
+FDATTN_API fdattn_block_pool* fdattn_pool_create(int num_blocks, int block_size, int max_seqs,
+                                                 int max_blocks_per_seq);            /* NULL on error */
+FDATTN_API void fdattn_pool_destroy(fdattn_block_pool* pool);
+/* Grow slot seq so that it covers num_tokens tokens (never shrinks).  All or nothing:
+ * FDATTN_ERR_POOL if the free blocks do not suffice, and then nothing has changed. */
+FDATTN_API int fdattn_pool_reserve(fdattn_block_pool* pool, int seq, int num_tokens);
+/* Give every block of slot seq back (a shared block returns to the free list with its last owner). */
+FDATTN_API int fdattn_pool_release(fdattn_block_pool* pool, int seq);
+/* Let the empty slot dst_seq share the whole blocks that hold the first shared_tokens tokens of
+ * src_seq.  Returns the number of tokens now shared (a multiple of block_size), or < 0. */
+FDATTN_API int fdattn_pool_fork(fdattn_block_pool* pool, int src_seq, int dst_seq, int shared_tokens);
+FDATTN_API int fdattn_pool_free_blocks(const fdattn_block_pool* pool);
+FDATTN_API int fdattn_pool_seq_blocks(const fdattn_block_pool* pool, int seq);
+FDATTN_API int fdattn_pool_refcount(const fdattn_block_pool* pool, int block);
+/* The table, valid until the pool is destroyed; its contents change with reserve / release / fork. */
+FDATTN_API const int32_t* fdattn_pool_block_tables(const fdattn_block_pool* pool);
 
 #ifdef __cplusplus
 }

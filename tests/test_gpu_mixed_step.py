@@ -113,3 +113,65 @@ def test_mixed_step_other_shape_runs_on_the_generic_kernels(oracle):
     assert np.array_equal(np_of(dev["key_cache"]), kc) and np.array_equal(np_of(dev["value_cache"]), vc)
     ok, mx, bad = bf16_close(bits(out), want)
     assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
+
+
+def test_steps_over_block_pool_tables_with_a_shared_prefix(oracle):
+    """Two steps driven by the block pool's tables: a prompt is prefilled, a second sequence forks its
+    whole blocks and prefills only its own tail while the first decodes and a third arrives.  Every step is
+    checked against the oracle on the same tables; the fork's outputs must also be bit-identical to those
+    of a run whose prefix blocks are private copies."""
+    from fastdeploy_amd.block_pool import BlockPool
+    hq, hkv, d, bs, quant = 32, 8, 128, 64, CACHE_INT8
+    g = torch.Generator().manual_seed(21)
+    pool = BlockPool(num_blocks=24, block_size=bs, max_seqs=4, max_blocks_per_seq=6)
+    ks = ((torch.rand((hkv, d), generator=g) * 2 + 2.0) / 127.0).contiguous()
+    vs = ((torch.rand((hkv, d), generator=g) * 2 + 2.0) / 127.0).contiguous()
+    cos, sin = rope_table(1024, d, 500000.0, "cpu")
+    kc = torch.zeros((24, hkv, bs, d), dtype=torch.uint8)
+    vc = torch.zeros_like(kc)
+    kc_d, vc_d = kc.cuda(), vc.cuda()
+
+    def step(enc, dec, tables, kc_dev, vc_dev, qkv):
+        enc_t, dec_t = torch.tensor(enc, dtype=torch.int32), torch.tensor(dec, dtype=torch.int32)
+        this = seq_lens_this_time_of(enc_t, dec_t)
+        cu = cu_seqlens_of(this)
+        c = dict(qkv=qkv, key_cache=kc_dev.cpu(), value_cache=vc_dev.cpu(), cache_k_scale=ks, cache_v_scale=vs,
+                 block_tables=torch.from_numpy(np.array(tables)), seq_lens_encoder=enc_t, seq_lens_decoder=dec_t,
+                 seq_lens_this_time=this, cu_seqlens_q=cu, rope_cos=cos, rope_sin=sin, T=int(cu[-1]))
+        out = fd.append_attention(qkv.cuda(), kc_dev, vc_dev, enc_t.cuda(), dec_t.cuda(), this.cuda(),
+                                  c["block_tables"].cuda(), (cos.cuda(), sin.cuda()), ks.cuda(), vs.cuda(),
+                                  num_heads=hq, kv_num_heads=hkv, max_chunk=max(max(enc), 1), cache_quant_type=quant,
+                                  cu_seqlens_q=cu.cuda())
+        torch.cuda.synchronize()
+        want, kc_w, vc_w = oracle_step(oracle, c, quant)
+        assert np.array_equal(np_of(kc_dev), kc_w) and np.array_equal(np_of(vc_dev), vc_w)
+        ok, mx, bad = bf16_close(bits(out), want)
+        assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
+        return out, cu
+
+    width = (hq + 2 * hkv) * d
+    # step 1: sequence 0 prefills a 200-token prompt
+    pool.reserve(0, 200)
+    step([200, 0, 0, 0], [0, 0, 0, 0], pool.block_tables, kc_d, vc_d,
+         torch.randn((200, width), generator=g).to(torch.bfloat16))
+    # step 2: slot 1 shares the prompt's three whole blocks and prefills 38 tokens of its own from position 192,
+    # slot 0 decodes, slot 2 arrives with 70 tokens, slot 3 idles
+    assert pool.fork(0, 1, 200) == 192
+    pool.reserve(1, 192 + 38)
+    pool.reserve(0, 201)
+    pool.reserve(2, 70)
+    assert pool.block_tables[1, :3].tolist() == pool.block_tables[0, :3].tolist()
+    enc, dec = [0, 38, 70, 0], [200, 192, 0, 0]
+    qkv2 = torch.randn((1 + 38 + 70, width), generator=g).to(torch.bfloat16)
+    kc_p, vc_p = kc_d.clone(), vc_d.clone()                 # the state before step 2, for the private-copy run
+    out_shared, cu = step(enc, dec, pool.block_tables, kc_d, vc_d, qkv2)
+    # the same step with private copies of the prefix blocks (blocks 20..22 are unused by the pool so far)
+    private = np.array(pool.block_tables)
+    src = torch.from_numpy(private[0, :3].astype(np.int64)).cuda()
+    dst = torch.tensor([20, 21, 22]).cuda()
+    kc_p[dst], vc_p[dst] = kc_p[src], vc_p[src]
+    private[1, :3] = [20, 21, 22]
+    out_private, _ = step(enc, dec, private, kc_p, vc_p, qkv2)
+    assert torch.equal(out_shared.view(torch.int16), out_private.view(torch.int16))
+    pool.release(1)
+    assert pool.refcount(int(private[0, 0])) == 1 and pool.free_blocks == 24 - 4 - 2
