@@ -131,6 +131,23 @@ def other_workloads(args):
         ms = time_events(pf, max(args.steps // 10, 5), 3)
         line("configs[4] append attention (2 x 2048 new on 8192 cached)", ms, "mfma", 2 * syn.prefill_flops(8192, 2048),
              2500.0, "TFLOP/s")
+    if args.workload in ("kv_wire", "all"):
+        # the sequences of configs[1] leave the cache in wire form and enter another one: HBM copies (read + write)
+        from fastdeploy_amd import kv_wire
+        c = syn.decode_case(batch=64, ctx=(3584, 4608), pool_blocks=6000, seed=0, device=dev, direct_bytes=True)
+        plan = kv_wire.WirePlan(c["seq_lens_decoder"].tolist(), 8, 128, 64, dev)
+        wire = torch.empty(plan.total, dtype=torch.uint8, device=dev)
+        kc2, vc2 = torch.empty_like(c["key_cache"]), torch.empty_like(c["value_cache"])
+        status = torch.zeros(2, dtype=torch.int32, device=dev)
+        ex = lambda: kv_wire.kv_export(c["key_cache"], c["value_cache"], c["cache_k_scale"], c["cache_v_scale"],
+                                       c["block_tables"], plan, wire=wire)
+        im = lambda: kv_wire.kv_import(wire, kc2, vc2, c["block_tables"], plan, cache_k_scale=c["cache_k_scale"],
+                                       cache_v_scale=c["cache_v_scale"], status=status)
+        ms = time_events(ex, max(args.steps // 4, 5), 3)
+        line("KV export to wire form (64 sequences of configs[1])", ms, "hbm", 2 * plan.total, HBM_PEAK_GBPS, "GB/s")
+        ms = time_events(im, max(args.steps // 4, 5), 3)
+        line("KV import from wire form (64 sequences of configs[1])", ms, "hbm", 2 * plan.total, HBM_PEAK_GBPS, "GB/s",
+             {"status": status.tolist()})
     return res
 
 
@@ -141,7 +158,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--pools", type=int, default=2, help="distinct cache pools rotated between steps")
-    ap.add_argument("--workload", default="decode", choices=["decode", "write_decode", "sqattn", "prefill", "all"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "write_decode", "sqattn", "prefill", "kv_wire", "all"],
                     help="decode = the headline metric (default); the others print one line per kernel of that row")
     ap.add_argument("--calibrate", action="store_true",
                     help="kept for the profiling command line: the 1 GiB device copy (the yardstick the HBM byte "

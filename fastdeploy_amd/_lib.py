@@ -36,6 +36,9 @@ SIGNATURES = {
     "fdattn_pool_seq_blocks": (_i, [_vp, _i]),
     "fdattn_pool_refcount": (_i, [_vp, _i]),
     "fdattn_pool_block_tables": (ctypes.POINTER(ctypes.c_int32), [_vp]),
+    "fdattn_kv_wire_bytes": (_sz, [_i] * 4),
+    "fdattn_kv_export": (_i, [_vp] * 8 + [_i] * 8 + [_vp]),
+    "fdattn_kv_import": (_i, [_vp] * 9 + [_i] * 8 + [_vp]),
 }
 
 _lib = None

@@ -21,7 +21,8 @@ FLAGS = [
 ] + os.environ.get("FDATTN_EXTRA_FLAGS", "").split()
 
 SOURCES = ["api.hip", "cache_writer.hip", "decode_generic.hip", "decode_c8.hip", "decode_api.hip",
-           "sqattn.hip", "prefill.hip", "prefill_mfma.hip", "append_api.hip", "block_pool.hip"]
+           "sqattn.hip", "prefill.hip", "prefill_mfma.hip", "append_api.hip", "block_pool.hip",
+           "kv_wire.hip"]
 
 
 def _compile(src):

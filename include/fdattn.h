@@ -341,6 +341,43 @@ FDATTN_API int fdattn_pool_refcount(const fdattn_block_pool* pool, int block);
 /* The table, valid until the pool is destroyed; its contents change with reserve / release / fork. */
 FDATTN_API const int32_t* fdattn_pool_block_tables(const fdattn_block_pool* pool);
 
+/*
+ * KV pages of whole sequences to and from a contiguous, self-describing buffer: what a prefill
+ * instance hands to a decode instance, or a cache hands to host memory (no counterpart in the
+ * reference; device buffers in and out like every tensor of its runtime,
+ * fastdeploy/runtime/runtime.h:90-104 BindInputTensor / GetOutputTensor sharing memory with
+ * the caller).  Layout of one sequence, little-endian, every section 256-byte aligned:
+ *   header 256 B  u32 magic "FDKV" (0x564b4446), version 1, cache_quant_type, hkv, head_dim,
+ *                 block_size, num_tokens, num_pages; u64 scales_off, sums_off, pages_off,
+ *                 total_bytes; zero to the end
+ *   scales        f32 K [hkv, head_dim], f32 V [hkv, head_dim]
+ *   sums          u64 [num_pages][2][hkv]: sum of the 32-bit words of each (page, K|V, head) tile
+ *   pages         u8 [num_pages][2][hkv][block_size][head_dim]; rows past num_tokens are zero, so
+ *                 the bytes depend on the sequence's content only, not on stale cache rows
+ * fdattn_kv_wire_bytes = total_bytes of a sequence of num_tokens tokens (0 for a bad shape).
+ * Sequence b of a call lives at wire + wire_offsets[b] (device int64 [batch], multiples of 256);
+ * num_tokens (device int32 [batch]) must hold the values the host sized the offsets with, each
+ * <= max_tokens.  One launch per call, nothing synchronises.
+ */
+FDATTN_API size_t fdattn_kv_wire_bytes(int num_tokens, int hkv, int head_dim, int block_size);
+/* cache -> wire.  A table entry outside [0, num_blocks) exports as a page of zeros. */
+FDATTN_API int fdattn_kv_export(const void* key_cache, const void* value_cache, const float* k_scale,
+                                const float* v_scale, const int32_t* block_tables, const int32_t* num_tokens,
+                                const int64_t* wire_offsets, void* wire, int batch, int max_tokens, int hkv,
+                                int head_dim, int block_size, int max_blocks_per_seq, int num_blocks,
+                                int cache_quant_type, void* stream);
+/* wire -> cache, into the blocks block_tables names.  status (device int32[2], zeroed by the caller):
+ * [0] = OR of 1 (magic / version), 2 (header disagrees with the arguments), 4 (scales differ from
+ * k_scale / v_scale; both NULL = not compared), 8 (a tile's sum disagrees), 16 (a table entry
+ * outside the pool); [1] = number of tiles whose sum disagrees.  A sequence whose header fails
+ * writes nothing; a tile whose sum fails has been written - discard the sequence.  No offset is
+ * ever taken from the buffer: every access stays inside fdattn_kv_wire_bytes(num_tokens[b], ...). */
+FDATTN_API int fdattn_kv_import(const void* wire, const int64_t* wire_offsets, void* key_cache, void* value_cache,
+                                const float* k_scale, const float* v_scale, const int32_t* block_tables,
+                                const int32_t* num_tokens, int32_t* status, int batch, int max_tokens, int hkv,
+                                int head_dim, int block_size, int max_blocks_per_seq, int num_blocks,
+                                int cache_quant_type, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
