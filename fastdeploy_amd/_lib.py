@@ -27,6 +27,8 @@ SIGNATURES = {
     "fdattn_append_attention_prefill_generic": (_i, [_vp] * 11 + [_i] * 10 + [_f, _vp]),
     "fdattn_append_attention_workspace_bytes": (_sz, [_i] * 6),
     "fdattn_append_attention": (_i, [_vp] * 14 + [_sz] + [_i] * 12 + [_f, _vp]),
+    "fdattn_write_cache_kv_ex": (_i, [_vp] * 13 + [_i] * 11 + [_vp, _vp]),
+    "fdattn_append_attention_ex": (_i, [_vp] * 14 + [_sz] + [_i] * 12 + [_f, _vp, _vp]),
     "fdattn_pool_create": (_vp, [_i] * 4),
     "fdattn_pool_destroy": (None, [_vp]),
     "fdattn_pool_reserve": (_i, [_vp, _i, _i]),
@@ -40,6 +42,13 @@ SIGNATURES = {
     "fdattn_kv_export": (_i, [_vp] * 8 + [_i] * 8 + [_vp]),
     "fdattn_kv_import": (_i, [_vp] * 9 + [_i] * 8 + [_vp]),
 }
+
+
+
+class QkvEpilogue(ctypes.Structure):
+    """fdattn_qkv_epilogue of include/fdattn.h"""
+    _fields_ = [("qkv_bias", _vp), ("q_norm_weight", _vp), ("k_norm_weight", _vp), ("rms_norm_eps", _f)]
+
 
 _lib = None
 

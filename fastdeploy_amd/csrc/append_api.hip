@@ -39,6 +39,21 @@ extern "C" int fdattn_append_attention(
     void* workspace, size_t workspace_bytes, int num_tokens, int batch, int max_chunk, int hq, int hkv,
     int head_dim, int block_size, int max_blocks_per_seq, int num_blocks, int max_pos, int rope_style,
     int cache_quant_type, float softmax_scale, void* stream) {
+  return fdattn_append_attention_ex(qkv, key_cache, value_cache, cache_k_scale, cache_v_scale, rope_cos, rope_sin,
+                                    block_tables, seq_lens_encoder, seq_lens_decoder, seq_lens_this_time, cu_seqlens_q,
+                                    out, workspace, workspace_bytes, num_tokens, batch, max_chunk, hq, hkv, head_dim,
+                                    block_size, max_blocks_per_seq, num_blocks, max_pos, rope_style, cache_quant_type,
+                                    softmax_scale, nullptr, stream);
+}
+
+extern "C" int fdattn_append_attention_ex(
+    const void* qkv, void* key_cache, void* value_cache, const float* cache_k_scale, const float* cache_v_scale,
+    const float* rope_cos, const float* rope_sin, const int32_t* block_tables, const int32_t* seq_lens_encoder,
+    const int32_t* seq_lens_decoder, const int32_t* seq_lens_this_time, const int32_t* cu_seqlens_q, void* out,
+    void* workspace, size_t workspace_bytes, int num_tokens, int batch, int max_chunk, int hq, int hkv,
+    int head_dim, int block_size, int max_blocks_per_seq, int num_blocks, int max_pos, int rope_style,
+    int cache_quant_type, float softmax_scale,
+    const fdattn_qkv_epilogue* epilogue, void* stream) {
   if (!seq_lens_encoder || !seq_lens_this_time || !cu_seqlens_q || !out || !workspace)
     return fail(FDATTN_ERR_NULL, "fdattn_append_attention: a required pointer is NULL");
   if (num_tokens < 0 || batch <= 0 || max_chunk <= 0 || hq <= 0 || hkv <= 0 || head_dim <= 0 ||
@@ -56,10 +71,10 @@ extern "C" int fdattn_append_attention(
   void* k_new = any_prefill ? ws + w.k_new : nullptr;
   void* v_new = any_prefill ? ws + w.v_new : nullptr;
   // 1. every new token: rotate, quantise, store (argument checks of the shared kind happen here)
-  int rc = fdattn_write_cache_kv(qkv, q_rot, k_new, v_new, key_cache, value_cache, cache_k_scale, cache_v_scale,
-                                 rope_cos, rope_sin, block_tables, seq_lens_decoder, cu_seqlens_q, num_tokens, batch,
-                                 hq, hkv, head_dim, block_size, max_blocks_per_seq, num_blocks, max_pos, rope_style,
-                                 cache_quant_type, stream);
+  int rc = fdattn_write_cache_kv_ex(qkv, q_rot, k_new, v_new, key_cache, value_cache, cache_k_scale, cache_v_scale,
+                                    rope_cos, rope_sin, block_tables, seq_lens_decoder, cu_seqlens_q, num_tokens,
+                                    batch, hq, hkv, head_dim, block_size, max_blocks_per_seq, num_blocks, max_pos,
+                                    rope_style, cache_quant_type, epilogue, stream);
   if (rc) return rc;
   // 2. decode rows: one token, seq_lens_encoder == 0; they read their own token back from the cache
   const RowMap rows{cu_seqlens_q, seq_lens_encoder};

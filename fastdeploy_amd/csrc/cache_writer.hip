@@ -1,5 +1,6 @@
 // Cache writer: rotary embedding on Q/K + int8 / fp8-e4m3 quantisation of K/V into
-// block-tabled pages.  Memory-bound and tiny (launch-bound at decode sizes): one
+// block-tabled pages; optionally the QKV projection's epilogue in front of it (bias, per-head
+// RMS norm of Q and K).  Memory-bound and tiny (launch-bound at decode sizes): one
 // thread per 16 channels, 16-byte loads of qkv, 8/16-byte stores into the page.
 //
 // Bit-exactness contract (shared with the CPU oracle): every fp32 product, sum and
@@ -25,6 +26,11 @@ struct WriterArgs {
   const int32_t* seq_lens_decoder;
   const int32_t* cu_seqlens_q;
   int num_tokens, batch, hq, hkv, d, bs, max_blocks, num_blocks, max_pos, rope_style;
+  // the projection's epilogue, all optional
+  const uint16_t* qkv_bias;     // bf16 [(hq + 2 hkv) * d]
+  const float* q_norm_weight;   // [d]: RMS norm of every Q head before the rotation
+  const float* k_norm_weight;   // [d]: the same for K
+  float rms_norm_eps;
 };
 
 template <int QUANT>
@@ -93,6 +99,64 @@ __global__ __launch_bounds__(256) void write_cache_kv_kernel(WriterArgs a) {
     }
   }
 
+  bool changed = false;  // x no longer equals the loaded bf16 values
+  if (a.qkv_bias != nullptr) {
+    // x = bf16(x + bias): the sum an unfused bf16 add would have produced
+    const uint16_t* brow = a.qkv_bias + (size_t)head * a.d;
+    const uint4 b1 = *reinterpret_cast<const uint4*>(brow + c1);
+    const uint4 b2 = *reinterpret_cast<const uint4*>(brow + c2);
+    const u32 bs1[4] = {b1.x, b1.y, b1.z, b1.w}, bs2[4] = {b2.x, b2.y, b2.z, b2.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float a0 = bf16lo_to_f32(bs1[i]), a1 = bf16hi_to_f32(bs1[i]);
+      const float b0 = bf16lo_to_f32(bs2[i]), b1f = bf16hi_to_f32(bs2[i]);
+      if (is_v || neox) {
+        x1[2 * i] = __fadd_rn(x1[2 * i], a0); x1[2 * i + 1] = __fadd_rn(x1[2 * i + 1], a1);
+        x2[2 * i] = __fadd_rn(x2[2 * i], b0); x2[2 * i + 1] = __fadd_rn(x2[2 * i + 1], b1f);
+      } else {
+        x1[i] = __fadd_rn(x1[i], a0); x2[i] = __fadd_rn(x2[i], a1);
+        x1[4 + i] = __fadd_rn(x1[4 + i], b0); x2[4 + i] = __fadd_rn(x2[4 + i], b1f);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      x1[i] = bf16_to_f32(f32_to_bf16(x1[i]));
+      x2[i] = bf16_to_f32(f32_to_bf16(x2[i]));
+    }
+    changed = true;
+  }
+  const float* nw = is_v ? nullptr : (is_k ? a.k_norm_weight : a.q_norm_weight);
+  if (nw != nullptr) {
+    // RMS norm over the head.  The sum of squares has a fixed order (the oracle follows it): within
+    // a thread first members of its 8 pairs, then second members, each sequentially; across the
+    // d/16 threads of the head a butterfly (the host checked that d/16 is a power of two), whose
+    // additions are commutative, so every thread ends with the same bits.
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      s1 = __fadd_rn(s1, __fmul_rn(x1[i], x1[i]));
+      s2 = __fadd_rn(s2, __fmul_rn(x2[i], x2[i]));
+    }
+    float ss = __fadd_rn(s1, s2);
+    for (int o = 1; o < units_per_head; o <<= 1) ss = __fadd_rn(ss, __shfl_xor(ss, o, 64));
+    // sqrtf, not __fsqrt_rn: that intrinsic is the approximate square root here; sqrtf and the division
+    // are correctly rounded (hipcc's default), which is what the oracle's libm gives
+    const float r = __fdiv_rn(1.0f, sqrtf(__fadd_rn(__fdiv_rn(ss, (float)a.d), a.rms_norm_eps)));
+    // weights of this thread's channels, in the order of x1 / x2
+    const float4 wa = *reinterpret_cast<const float4*>(nw + c1), wb = *reinterpret_cast<const float4*>(nw + c1 + 4);
+    const float4 wc = *reinterpret_cast<const float4*>(nw + c2), wd = *reinterpret_cast<const float4*>(nw + c2 + 4);
+    const float g1w[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+    const float g2w[8] = {wc.x, wc.y, wc.z, wc.w, wd.x, wd.y, wd.z, wd.w};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float w1v, w2v;
+      if (neox) { w1v = g1w[i]; w2v = g2w[i]; }
+      else { w1v = i < 4 ? g1w[2 * i] : g2w[2 * (i - 4)]; w2v = i < 4 ? g1w[2 * i + 1] : g2w[2 * (i - 4) + 1]; }
+      x1[i] = __fmul_rn(__fmul_rn(x1[i], r), w1v);
+      x2[i] = __fmul_rn(__fmul_rn(x2[i], r), w2v);
+    }
+  }
+
   float y1[8], y2[8];
   if (!is_v && a.rope_cos != nullptr) {
     const float* cs = a.rope_cos + (size_t)pos * half + 8 * u;
@@ -140,7 +204,7 @@ __global__ __launch_bounds__(256) void write_cache_kv_kernel(WriterArgs a) {
   uint16_t* side = is_k ? a.k_out : a.v_out;
   if (side != nullptr) {
     uint16_t* o = side + ((size_t)tok * a.hkv + h) * a.d;
-    if (is_v) {
+    if (is_v && !changed) {
       *reinterpret_cast<uint4*>(o + c1) = w1;
       *reinterpret_cast<uint4*>(o + c2) = w2;
     } else {
@@ -186,6 +250,29 @@ extern "C" int fdattn_write_cache_kv(
     const int32_t* cu_seqlens_q, int num_tokens, int batch, int hq, int hkv, int head_dim,
     int block_size, int max_blocks_per_seq, int num_blocks, int max_pos, int rope_style,
     int cache_quant_type, void* stream) {
+  return fdattn_write_cache_kv_ex(qkv, q_out, k_out, v_out, key_cache, value_cache, cache_k_scale, cache_v_scale,
+                                  rope_cos, rope_sin, block_tables, seq_lens_decoder, cu_seqlens_q, num_tokens, batch,
+                                  hq, hkv, head_dim, block_size, max_blocks_per_seq, num_blocks, max_pos, rope_style,
+                                  cache_quant_type, nullptr, stream);
+}
+
+extern "C" int fdattn_write_cache_kv_ex(
+    const void* qkv, void* q_out, void* k_out, void* v_out, void* key_cache, void* value_cache,
+    const float* cache_k_scale, const float* cache_v_scale, const float* rope_cos,
+    const float* rope_sin, const int32_t* block_tables, const int32_t* seq_lens_decoder,
+    const int32_t* cu_seqlens_q, int num_tokens, int batch, int hq, int hkv, int head_dim,
+    int block_size, int max_blocks_per_seq, int num_blocks, int max_pos, int rope_style,
+    int cache_quant_type, const fdattn_qkv_epilogue* epilogue, void* stream) {
+  const fdattn_qkv_epilogue none = {nullptr, nullptr, nullptr, 0.f};
+  const fdattn_qkv_epilogue& ep = epilogue ? *epilogue : none;
+  if (ep.q_norm_weight || ep.k_norm_weight) {
+    const int u = head_dim / 16;
+    if (head_dim % 16 != 0 || u <= 0 || (u & (u - 1)) != 0 || u > 64)
+      return fail(FDATTN_ERR_SHAPE, "fdattn_write_cache_kv: the RMS norm needs head_dim = 16 * a power of two "
+                  "up to 1024, got %d", head_dim);
+    if (!(ep.rms_norm_eps >= 0.f))
+      return fail(FDATTN_ERR_SHAPE, "fdattn_write_cache_kv: rms_norm_eps must not be negative");
+  }
   if (!qkv || !q_out || !key_cache || !value_cache || !cache_k_scale || !cache_v_scale ||
       !block_tables || !seq_lens_decoder || !cu_seqlens_q)
     return fail(FDATTN_ERR_NULL, "fdattn_write_cache_kv: a required pointer is NULL");
@@ -207,7 +294,8 @@ extern "C" int fdattn_write_cache_kv(
   WriterArgs a{(const uint16_t*)qkv, (uint16_t*)q_out, (uint16_t*)k_out, (uint16_t*)v_out,
                (uint8_t*)key_cache, (uint8_t*)value_cache, cache_k_scale, cache_v_scale, rope_cos,
                rope_sin, block_tables, seq_lens_decoder, cu_seqlens_q, num_tokens, batch, hq, hkv,
-               head_dim, block_size, max_blocks_per_seq, num_blocks, max_pos, rope_style};
+               head_dim, block_size, max_blocks_per_seq, num_blocks, max_pos, rope_style,
+               (const uint16_t*)ep.qkv_bias, ep.q_norm_weight, ep.k_norm_weight, ep.rms_norm_eps};
   long long total = (long long)num_tokens * (hq + 2 * hkv) * (head_dim / 16);
   unsigned grid = (unsigned)((total + 255) / 256);
   hipStream_t s = (hipStream_t)stream;

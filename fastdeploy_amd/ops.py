@@ -11,6 +11,7 @@ custom operators do on their input's stream
 raise ValueError where the reference's operators PD_THROW
 (fastdeploy/runtime/backends/paddle/ops/voxelize_op.cc:172).
 """
+import ctypes
 import math
 
 import torch
@@ -70,6 +71,21 @@ def _scales(cache_k_scale, cache_v_scale, hkv, d):
     return pk, pv
 
 
+def _epilogue(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, width, d):
+    """fdattn_qkv_epilogue for the optional projection epilogue, or None"""
+    if qkv_bias is None and q_norm_weight is None and k_norm_weight is None:
+        return None
+    pb = _chk(qkv_bias, "qkv_bias", torch.bfloat16, 1, optional=True)
+    if qkv_bias is not None and qkv_bias.numel() != width:
+        raise ValueError("qkv_bias has %d entries, qkv %d columns" % (qkv_bias.numel(), width))
+    pq = _chk(q_norm_weight, "q_norm_weight", torch.float32, 1, optional=True)
+    pk = _chk(k_norm_weight, "k_norm_weight", torch.float32, 1, optional=True)
+    for name, t in (("q_norm_weight", q_norm_weight), ("k_norm_weight", k_norm_weight)):
+        if t is not None and t.numel() != d:
+            raise ValueError("%s has %d entries, head_dim is %d" % (name, t.numel(), d))
+    return _lib.QkvEpilogue(pb or None, pq or None, pk or None, float(rms_norm_eps))
+
+
 def seq_lens_this_time_of(seq_lens_encoder, seq_lens_decoder):
     """Tokens each sequence brings this step: its chunk length for a prefill row
     (seq_lens_encoder > 0), one for a decode row (seq_lens_decoder > 0), else none."""
@@ -86,10 +102,14 @@ def cu_seqlens_of(seq_lens_this_time):
 def write_cache_kv(qkv, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
                    seq_lens_encoder, seq_lens_decoder, seq_lens_this_time=None, cu_seqlens_q=None,
                    rotary_embs=None, *, num_heads, kv_num_heads, rope_style="neox",
-                   cache_quant_type="cache_int8", want_kv_out=False):
+                   cache_quant_type="cache_int8", want_kv_out=False, qkv_bias=None, q_norm_weight=None,
+                   k_norm_weight=None, rms_norm_eps=1e-6):
     """RoPE on Q/K, quantise K/V into their block-tabled cache slots (in place).
 
     rotary_embs = (cos, sin) float32 [max_pos, head_dim/2] from rope_table(), or None.
+    The projection's epilogue, all optional: qkv_bias bf16 [(num_heads+2*kv_num_heads)*head_dim]
+    (x = bf16(x + bias)), q_norm_weight / k_norm_weight float32 [head_dim] (RMS norm of every Q / K
+    head before the rotation, with rms_norm_eps).
     Returns (q_out, k_out, v_out); k_out / v_out are None unless want_kv_out.
     """
     nb, hkv, bs, d = _cache_dims(key_cache, value_cache)
@@ -133,11 +153,12 @@ def write_cache_kv(qkv, key_cache, value_cache, cache_k_scale, cache_v_scale, bl
     if want_kv_out:
         k_out = torch.empty((T, hkv * d), dtype=torch.bfloat16, device=qkv.device)
         v_out = torch.empty((T, hkv * d), dtype=torch.bfloat16, device=qkv.device)
-    rc = _lib.lib().fdattn_write_cache_kv(
+    ep = _epilogue(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, qkv.shape[1], d)
+    rc = _lib.lib().fdattn_write_cache_kv_ex(
         p_qkv, q_out.data_ptr(), k_out.data_ptr() if want_kv_out else 0,
         v_out.data_ptr() if want_kv_out else 0, p_kc, p_vc, p_ks, p_vs, p_cos, p_sin, p_bt, p_dec,
         p_cu, T, batch, num_heads, hkv, d, bs, mb, nb, max_pos, _ROPE[rope_style],
-        _quant(cache_quant_type), _stream())
+        _quant(cache_quant_type), ctypes.addressof(ep) if ep is not None else None, _stream())
     _lib.check(rc, "write_cache_kv")
     return q_out, k_out, v_out
 
@@ -319,12 +340,14 @@ def append_attention_workspace(num_tokens, batch, num_heads, kv_heads, head_dim,
 def append_attention(qkv, key_cache, value_cache, seq_lens_encoder, seq_lens_decoder, seq_lens_this_time,
                      block_tables, rotary_embs, cache_k_scale, cache_v_scale, *, num_heads, kv_num_heads,
                      max_chunk, rope_style="neox", cache_quant_type="cache_int8", softmax_scale=None,
-                     cu_seqlens_q=None, workspace=None, out=None):
+                     cu_seqlens_q=None, workspace=None, out=None, qkv_bias=None, q_norm_weight=None,
+                     k_norm_weight=None, rms_norm_eps=1e-6):
     """One attention step of a layer over a mixed batch (one call into the library):
     every new token is rotated and written to the cache, decode rows (one token,
     seq_lens_encoder == 0) attend to the cache, prefill rows (seq_lens_encoder > 0)
     to their cached prefix and causally to their own chunk; slots without a token
     are skipped.  max_chunk bounds the tokens of one sequence (1 = decode only).
+    qkv_bias / q_norm_weight / k_norm_weight / rms_norm_eps: the projection's epilogue, as in write_cache_kv.
     Returns bf16 [num_tokens, num_heads*head_dim]."""
     nb, hkv, bs, d = _cache_dims(key_cache, value_cache)
     if hkv != kv_num_heads:
@@ -370,10 +393,11 @@ def append_attention(qkv, key_cache, value_cache, seq_lens_encoder, seq_lens_dec
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=qkv.device)
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(d)
-    rc = _lib.lib().fdattn_append_attention(
+    ep = _epilogue(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, qkv.shape[1], d)
+    rc = _lib.lib().fdattn_append_attention_ex(
         p_qkv, p_kc, p_vc, p_ks, p_vs, p_cos, p_sin, p_bt, p_enc, p_dec, p_this, p_cu,
         _chk(out, "out", torch.bfloat16), workspace.data_ptr(), workspace.numel() * workspace.element_size(),
         T, batch, max_chunk, num_heads, hkv, d, bs, mb, nb, max_pos, _ROPE[rope_style], _quant(cache_quant_type),
-        scale, _stream())
+        scale, ctypes.addressof(ep) if ep is not None else None, _stream())
     _lib.check(rc, "append_attention")
     return out

@@ -96,6 +96,35 @@ FDATTN_API int fdattn_write_cache_kv(
     int rope_style, int cache_quant_type, void* stream);
 
 /*
+ * The QKV projection's epilogue, fused in front of the cache writer (every member optional;
+ * engine-side operators take optional inputs the same way,
+ * fastdeploy/runtime/backends/paddle/ops/voxelize_op.cc:194-204 lists inputs and attributes).
+ *   qkv_bias        bf16 [(hq + 2*hkv) * head_dim]: x = bf16(x + bias), the result of a bf16 add
+ *   q_norm_weight   f32 [head_dim]: every Q head x -> x / sqrt(mean(x^2) + eps) * weight, before
+ *   k_norm_weight   f32 [head_dim]  the rotation; the same for every K head (V is not normed)
+ * All arithmetic is fp32 with every operation rounded on its own; nothing is rounded to bf16
+ * between the norm and the rotation.  The norm needs head_dim = 16 * 2^n.
+ */
+typedef struct fdattn_qkv_epilogue {
+  const void* qkv_bias;
+  const float* q_norm_weight;
+  const float* k_norm_weight;
+  float rms_norm_eps;
+} fdattn_qkv_epilogue;
+
+/* fdattn_write_cache_kv with the epilogue (host pointer, read during the call; NULL = none). */
+FDATTN_API int fdattn_write_cache_kv_ex(
+    const void* qkv, void* q_out, void* k_out, void* v_out,
+    void* key_cache, void* value_cache,
+    const float* cache_k_scale, const float* cache_v_scale,
+    const float* rope_cos, const float* rope_sin,
+    const int32_t* block_tables, const int32_t* seq_lens_decoder,
+    const int32_t* cu_seqlens_q,
+    int num_tokens, int batch, int hq, int hkv, int head_dim, int block_size,
+    int max_blocks_per_seq, int num_blocks, int max_pos,
+    int rope_style, int cache_quant_type, const fdattn_qkv_epilogue* epilogue, void* stream);
+
+/*
  * Bytes of workspace fdattn_decode_attention / fdattn_decode_attention_sparse
  * need for these shapes (split-KV partial results).  Never 0.  The workspace needs
  * no initialisation; calls that overlap on the GPU must not share one.
@@ -312,6 +341,18 @@ FDATTN_API int fdattn_append_attention(
     int num_tokens, int batch, int max_chunk, int hq, int hkv, int head_dim,
     int block_size, int max_blocks_per_seq, int num_blocks, int max_pos,
     int rope_style, int cache_quant_type, float softmax_scale, void* stream);
+
+/* fdattn_append_attention with the QKV projection's epilogue in front of the cache write (NULL = none). */
+FDATTN_API int fdattn_append_attention_ex(
+    const void* qkv, void* key_cache, void* value_cache,
+    const float* cache_k_scale, const float* cache_v_scale,
+    const float* rope_cos, const float* rope_sin,
+    const int32_t* block_tables, const int32_t* seq_lens_encoder,
+    const int32_t* seq_lens_decoder, const int32_t* seq_lens_this_time,
+    const int32_t* cu_seqlens_q, void* out, void* workspace, size_t workspace_bytes,
+    int num_tokens, int batch, int max_chunk, int hq, int hkv, int head_dim,
+    int block_size, int max_blocks_per_seq, int num_blocks, int max_pos,
+    int rope_style, int cache_quant_type, float softmax_scale, const fdattn_qkv_epilogue* epilogue, void* stream);
 
 /*
  * Host-side block pool: the producer of block_tables (no counterpart in the reference,

@@ -14,6 +14,8 @@
  *     exhaustively over all 65,536 bf16 patterns (and all 256 fp8 codes);
  *   - fdo_write_cache_kv: closed forms (pos 0 = identity, pair norms kept,
  *     complex multiplication in fp64), |x - q*s| <= s/2, max-abs -> +-127;
+ *     its epilogue (bias, RMS norm of Q and K heads): torch's bf16 add and an
+ *     fp64 RMS norm, unit weights -> unit mean square, scale invariance;
  *   - fdo_decode_attention: torch CPU scaled_dot_product_attention in fp64 on
  *     the dequantised gathered cache, block-table permutation invariance,
  *     kv_len 1 = V row, constant K = mean of V; its softmax against the
@@ -119,13 +121,12 @@ static inline float dequant(uint8_t byte, int cache_type) {
  * to fp32 on its own.  Pair (j, j + d/2) for the NeoX style, (2j, 2j+1) for
  * the interleaved one.
  */
-static void rope_row(const uint16_t* x, float* y, int d, const float* cs, const float* sn,
-                     int style) {
+static void rope_row(const float* x, float* y, int d, const float* cs, const float* sn, int style) {
   int half = d / 2;
   for (int j = 0; j < half; ++j) {
     int i1 = style ? j : 2 * j;
     int i2 = style ? j + half : 2 * j + 1;
-    float x1 = fdo_bf16_to_f32(x[i1]), x2 = fdo_bf16_to_f32(x[i2]);
+    float x1 = x[i1], x2 = x[i2];
     if (cs) {
       float c = cs[j], s = sn[j];
       float a = x1 * c, b = x2 * s, e = x2 * c, f = x1 * s;
@@ -138,47 +139,96 @@ static void rope_row(const uint16_t* x, float* y, int d, const float* cs, const 
   }
 }
 
-int fdo_write_cache_kv(const uint16_t* qkv, uint16_t* q_out, uint16_t* k_out, uint16_t* v_out,
-                       uint8_t* key_cache, uint8_t* value_cache, const float* k_scale,
-                       const float* v_scale, const float* rope_cos, const float* rope_sin,
-                       const int32_t* block_tables, const int32_t* seq_lens_decoder,
-                       const int32_t* cu_seqlens_q, int num_tokens, int batch, int hq, int hkv,
-                       int d, int block_size, int max_blocks_per_seq, int num_blocks, int max_pos,
-                       int rope_style, int cache_type) {
+/*
+ * The QKV projection's epilogue on one head: x = bf16(x + bias) when a bias is given, then the
+ * RMS norm x / sqrt(mean(x^2) + eps) * w when a weight is given.  The sum of squares has a fixed
+ * order: the rotation pairs j = 0 .. d/2-1 are taken in groups of 8; a group's sum is (squares of
+ * its 8 first members, added one after the other from 0) + (the same over its 8 second members);
+ * the d/16 group sums are combined by a butterfly, t[u] <- t[u] + t[u ^ o] for o = 1, 2, 4, ...
+ * (d/16 must be a power of two).  mean = sum / d, then one add, one square root, one division,
+ * and two products per channel, each rounded to fp32.
+ */
+static void epilogue_row(const uint16_t* x, const uint16_t* bias, const float* w, float eps, int d, int style,
+                         float* out) {
+  for (int c = 0; c < d; ++c) {
+    float v = fdo_bf16_to_f32(x[c]);
+    if (bias) v = fdo_bf16_to_f32(fdo_f32_to_bf16(v + fdo_bf16_to_f32(bias[c])));
+    out[c] = v;
+  }
+  if (!w) return;
+  int half = d / 2, groups = d / 16;
+  float t[64], t2[64];
+  for (int u = 0; u < groups; ++u) {
+    float s1 = 0.f, s2 = 0.f;
+    for (int i = 0; i < 8; ++i) {
+      int j = 8 * u + i;
+      float a = out[style ? j : 2 * j], b = out[style ? j + half : 2 * j + 1];
+      float aa = a * a, bb = b * b;
+      s1 = s1 + aa;
+      s2 = s2 + bb;
+    }
+    t[u] = s1 + s2;
+  }
+  for (int o = 1; o < groups; o <<= 1) {
+    for (int u = 0; u < groups; ++u) t2[u] = t[u] + t[u ^ o];
+    memcpy(t, t2, sizeof(float) * groups);
+  }
+  float ms = t[0] / (float)d;
+  float r = 1.0f / sqrtf(ms + eps);
+  for (int c = 0; c < d; ++c) {
+    float v = out[c] * r;
+    out[c] = v * w[c];
+  }
+}
+
+int fdo_write_cache_kv_ex(const uint16_t* qkv, uint16_t* q_out, uint16_t* k_out, uint16_t* v_out,
+                          uint8_t* key_cache, uint8_t* value_cache, const float* k_scale,
+                          const float* v_scale, const float* rope_cos, const float* rope_sin,
+                          const int32_t* block_tables, const int32_t* seq_lens_decoder,
+                          const int32_t* cu_seqlens_q, int num_tokens, int batch, int hq, int hkv,
+                          int d, int block_size, int max_blocks_per_seq, int num_blocks, int max_pos,
+                          int rope_style, int cache_type, const uint16_t* qkv_bias, const float* q_norm_w,
+                          const float* k_norm_w, float eps) {
   int row = (hq + 2 * hkv) * d;
-  float* y = (float*)malloc(sizeof(float) * d);
+  if ((q_norm_w || k_norm_w) && (d % 16 != 0 || d / 16 > 64 || ((d / 16) & (d / 16 - 1)) != 0)) return -2;
+  float* x = (float*)malloc(sizeof(float) * d * 3);
+  float* y = x + d;
+  float* vx = x + 2 * d;
   int b = 0;
   for (int i = 0; i < num_tokens; ++i) {
     while (b < batch && i >= cu_seqlens_q[b + 1]) ++b;
     if (b >= batch) break;
     int pos = seq_lens_decoder[b] + (i - cu_seqlens_q[b]);
     if (pos < 0 || (rope_cos && pos >= max_pos)) {
-      free(y);
+      free(x);
       return -2;
     }
     const float* cs = rope_cos ? rope_cos + (size_t)pos * (d / 2) : NULL;
     const float* sn = rope_cos ? rope_sin + (size_t)pos * (d / 2) : NULL;
     const uint16_t* r = qkv + (size_t)i * row;
     for (int h = 0; h < hq; ++h) {
-      rope_row(r + h * d, y, d, cs, sn, rope_style);
+      epilogue_row(r + h * d, qkv_bias ? qkv_bias + h * d : NULL, q_norm_w, eps, d, rope_style, x);
+      rope_row(x, y, d, cs, sn, rope_style);
       for (int c = 0; c < d; ++c) q_out[((size_t)i * hq + h) * d + c] = fdo_f32_to_bf16(y[c]);
     }
     int lb = pos / block_size, slot = pos % block_size;
     int pb = lb < max_blocks_per_seq ? block_tables[(size_t)b * max_blocks_per_seq + lb] : -1;
     if (pb >= num_blocks) {
-      free(y);
+      free(x);
       return -2;
     }
     for (int h = 0; h < hkv; ++h) {
       const uint16_t* kr = r + (size_t)(hq + h) * d;
       const uint16_t* vr = r + (size_t)(hq + hkv + h) * d;
-      rope_row(kr, y, d, cs, sn, rope_style);
+      epilogue_row(kr, qkv_bias ? qkv_bias + (size_t)(hq + h) * d : NULL, k_norm_w, eps, d, rope_style, x);
+      rope_row(x, y, d, cs, sn, rope_style);
+      epilogue_row(vr, qkv_bias ? qkv_bias + (size_t)(hq + hkv + h) * d : NULL, NULL, 0.f, d, rope_style, vx);
       size_t base = (((size_t)pb * hkv + h) * block_size + slot) * d;
       for (int c = 0; c < d; ++c) {
         float sk = k_scale[h * d + c], sv = v_scale[h * d + c];
-        float v = fdo_bf16_to_f32(vr[c]);
+        float v = vx[c];
         if (k_out) k_out[((size_t)i * hkv + h) * d + c] = fdo_f32_to_bf16(y[c]);
-        if (v_out) v_out[((size_t)i * hkv + h) * d + c] = vr[c];
+        if (v_out) v_out[((size_t)i * hkv + h) * d + c] = fdo_f32_to_bf16(v); /* exact: v is a bf16 value */
         if (pb < 0) continue;
         if (cache_type == FDO_CACHE_INT8) {
           key_cache[base + c] = (uint8_t)fdo_quant_int8(y[c], sk);
@@ -190,8 +240,21 @@ int fdo_write_cache_kv(const uint16_t* qkv, uint16_t* q_out, uint16_t* k_out, ui
       }
     }
   }
-  free(y);
+  free(x);
   return 0;
+}
+
+int fdo_write_cache_kv(const uint16_t* qkv, uint16_t* q_out, uint16_t* k_out, uint16_t* v_out,
+                       uint8_t* key_cache, uint8_t* value_cache, const float* k_scale,
+                       const float* v_scale, const float* rope_cos, const float* rope_sin,
+                       const int32_t* block_tables, const int32_t* seq_lens_decoder,
+                       const int32_t* cu_seqlens_q, int num_tokens, int batch, int hq, int hkv,
+                       int d, int block_size, int max_blocks_per_seq, int num_blocks, int max_pos,
+                       int rope_style, int cache_type) {
+  return fdo_write_cache_kv_ex(qkv, q_out, k_out, v_out, key_cache, value_cache, k_scale, v_scale, rope_cos,
+                               rope_sin, block_tables, seq_lens_decoder, cu_seqlens_q, num_tokens, batch, hq,
+                               hkv, d, block_size, max_blocks_per_seq, num_blocks, max_pos, rope_style,
+                               cache_type, NULL, NULL, NULL, 0.f);
 }
 
 /* ------------------------------------------------------- decode attention */

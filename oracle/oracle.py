@@ -105,9 +105,11 @@ def softmax_row(x):
 
 def write_cache_kv(qkv, key_cache, value_cache, k_scale, v_scale, rope_cos, rope_sin,
                    block_tables, seq_lens_decoder, cu_seqlens_q, hq, hkv, d, rope_style,
-                   cache_type, want_kv_out=True):
+                   cache_type, want_kv_out=True, qkv_bias=None, q_norm_weight=None, k_norm_weight=None,
+                   rms_norm_eps=0.0):
     """Mutates key_cache / value_cache (uint8 [num_blocks,hkv,bs,d]) in place.
 
+    qkv_bias: uint16 bf16 patterns [(hq+2hkv)*d]; q_norm_weight / k_norm_weight: float32 [d].
     Returns (q_out, k_out, v_out) as uint16 bf16 patterns.
     """
     qkv = _c(qkv, np.uint16)
@@ -125,10 +127,14 @@ def write_cache_kv(qkv, key_cache, value_cache, k_scale, v_scale, rope_cos, rope
     k_out = np.zeros((T, hkv * d), np.uint16) if want_kv_out else None
     v_out = np.zeros((T, hkv * d), np.uint16) if want_kv_out else None
     max_pos = rope_cos.shape[0] if rope_cos is not None else 0
-    rc = lib().fdo_write_cache_kv(
+    bias = _c(qkv_bias, np.uint16) if qkv_bias is not None else None
+    qw = _c(q_norm_weight, np.float32) if q_norm_weight is not None else None
+    kw = _c(k_norm_weight, np.float32) if k_norm_weight is not None else None
+    rc = lib().fdo_write_cache_kv_ex(
         _p(qkv), _p(q_out), _p(k_out), _p(v_out), _p(key_cache), _p(value_cache), _p(k_scale),
         _p(v_scale), _p(rope_cos), _p(rope_sin), _p(bt), _p(dec), _p(cu), T, batch, hq, hkv, d,
-        bs, mb, num_blocks, max_pos, rope_style, cache_type)
+        bs, mb, num_blocks, max_pos, rope_style, cache_type, _p(bias), _p(qw), _p(kw),
+        ctypes.c_float(rms_norm_eps))
     if rc != 0:
         raise ValueError("fdo_write_cache_kv: bad position or block id (%d)" % rc)
     return q_out, k_out, v_out

@@ -63,6 +63,48 @@ def test_writer_chunks_ragged_and_no_rope(oracle, quant):
     _run_both(oracle, case)
 
 
+@pytest.mark.parametrize("style", ["neox", "interleaved"])
+@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+def test_writer_epilogue_bit_exact(oracle, quant, style):
+    """bias, RMS norm of Q and K heads, both, and each norm alone - in front of the rotation; every output
+    bit for bit as the oracle's."""
+    g = torch.Generator().manual_seed(8)
+    for d, hq, hkv in ((128, 32, 8), (64, 4, 2), (32, 2, 1)):
+        case = syn.write_case(num_seqs=11, max_pos=500, quant=quant, seed=d, rope_style=style, hq=hq, hkv=hkv, d=d,
+                              chunk=3)
+        dev = syn.to_device(case, "cuda")
+        bias = (torch.randn(((hq + 2 * hkv) * d,), generator=g) * 0.5).to(torch.bfloat16)
+        qw = torch.rand((d,), generator=g) + 0.5
+        kw = torch.rand((d,), generator=g) + 0.5
+        for use_bias, use_q, use_k, eps in ((1, 0, 0, 0.0), (0, 1, 1, 1e-6), (1, 1, 1, 1e-5), (0, 1, 0, 0.0), (1, 0, 1, 1e-6)):
+            kc_d, vc_d = dev["key_cache"].clone(), dev["value_cache"].clone()
+            q, k, v = fd.write_cache_kv(
+                dev["qkv"], kc_d, vc_d, dev["cache_k_scale"], dev["cache_v_scale"], dev["block_tables"],
+                dev["seq_lens_encoder"], dev["seq_lens_decoder"], dev["seq_lens_this_time"], dev["cu_seqlens_q"],
+                (dev["rope_cos"], dev["rope_sin"]), num_heads=hq, kv_num_heads=hkv, rope_style=style,
+                cache_quant_type=quant, want_kv_out=True, qkv_bias=bias.cuda() if use_bias else None,
+                q_norm_weight=qw.cuda() if use_q else None, k_norm_weight=kw.cuda() if use_k else None, rms_norm_eps=eps)
+            torch.cuda.synchronize()
+            kc, vc = np_of(case["key_cache"]).copy(), np_of(case["value_cache"]).copy()
+            oq, ok, ov = oracle.write_cache_kv(
+                bits(case["qkv"]), kc, vc, np_of(case["cache_k_scale"]), np_of(case["cache_v_scale"]),
+                np_of(case["rope_cos"]), np_of(case["rope_sin"]), np_of(case["block_tables"]),
+                np_of(case["seq_lens_decoder"]), np_of(case["cu_seqlens_q"]), hq, hkv, d, 1 if style == "neox" else 0,
+                quant, True, qkv_bias=bits(bias) if use_bias else None, q_norm_weight=np_of(qw) if use_q else None,
+                k_norm_weight=np_of(kw) if use_k else None, rms_norm_eps=eps)
+            what = "d=%d bias=%d qnorm=%d knorm=%d" % (d, use_bias, use_q, use_k)
+            assert np.array_equal(bits(q), oq), what + ": Q"
+            assert np.array_equal(bits(k), ok), what + ": K"
+            assert np.array_equal(bits(v), ov), what + ": V"
+            assert np.array_equal(np_of(kc_d), kc) and np.array_equal(np_of(vc_d), vc), what + ": cache bytes"
+    with pytest.raises(ValueError):      # head_dim 96: six threads per head, no butterfly
+        c96 = syn.to_device(syn.write_case(num_seqs=2, max_pos=64, hq=2, hkv=1, d=96), "cuda")
+        fd.write_cache_kv(c96["qkv"], c96["key_cache"], c96["value_cache"], c96["cache_k_scale"], c96["cache_v_scale"],
+                          c96["block_tables"], c96["seq_lens_encoder"], c96["seq_lens_decoder"], c96["seq_lens_this_time"],
+                          c96["cu_seqlens_q"], None, num_heads=2, kv_num_heads=1,
+                          q_norm_weight=torch.ones(96, device="cuda"))
+
+
 def test_quantisers_exhaustive_over_bf16(oracle):
     """Every finite bf16 value through the int8 and fp8 quantisers at several scales, via V (no rotation)."""
     allbits = np.arange(65536, dtype=np.uint16)

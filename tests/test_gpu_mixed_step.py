@@ -40,7 +40,7 @@ def mixed_case(enc, dec, quant, seed, hq=32, hkv=8, d=128, bs=64, max_pos=4096):
                 rope_cos=cos, rope_sin=sin, T=T)
 
 
-def oracle_step(oracle, c, quant, hq=32, hkv=8, d=128):
+def oracle_step(oracle, c, quant, hq=32, hkv=8, d=128, **epilogue):
     """The step composed from the oracle's pieces; returns (out bf16 bits [T, hq*d] with NaN-free rows only where
     a token exists, key cache, value cache)."""
     kc, vc = np_of(c["key_cache"]).copy(), np_of(c["value_cache"]).copy()
@@ -48,7 +48,7 @@ def oracle_step(oracle, c, quant, hq=32, hkv=8, d=128):
     bt, dec, cu = np_of(c["block_tables"]), np_of(c["seq_lens_decoder"]), np_of(c["cu_seqlens_q"])
     enc, this = np_of(c["seq_lens_encoder"]), np_of(c["seq_lens_this_time"])
     q, k_new, v_new = oracle.write_cache_kv(bits(c["qkv"]), kc, vc, ks, vs, np_of(c["rope_cos"]), np_of(c["rope_sin"]),
-                                            bt, dec, cu, hq, hkv, d, 1, quant, want_kv_out=True)
+                                            bt, dec, cu, hq, hkv, d, 1, quant, want_kv_out=True, **epilogue)
     out = np.zeros((c["T"], hq * d), np.uint16)
     drows = [b for b in range(len(enc)) if enc[b] == 0 and this[b] == 1]
     if drows:
@@ -78,6 +78,27 @@ def test_mixed_batch_step(oracle, quant):
                               cu_seqlens_q=dev["cu_seqlens_q"])
     torch.cuda.synchronize()
     want, kc, vc = oracle_step(oracle, c, quant)
+    assert np.array_equal(np_of(dev["key_cache"]), kc) and np.array_equal(np_of(dev["value_cache"]), vc)
+    ok, mx, bad = bf16_close(bits(out), want)
+    assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
+
+
+def test_mixed_batch_step_with_projection_epilogue(oracle):
+    """qkv bias and the RMS norm of Q and K heads in front of the cache write, inside the one-call step."""
+    enc, dec = [0, 90, 0, 33], [130, 64, 7, 0]
+    c = mixed_case(enc, dec, CACHE_INT8, seed=12)
+    g = torch.Generator().manual_seed(3)
+    bias = (torch.randn((48 * 128,), generator=g) * 0.25).to(torch.bfloat16)
+    qw, kw = torch.rand((128,), generator=g) + 0.5, torch.rand((128,), generator=g) + 0.5
+    dev = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
+    out = fd.append_attention(dev["qkv"], dev["key_cache"], dev["value_cache"], dev["seq_lens_encoder"],
+                              dev["seq_lens_decoder"], dev["seq_lens_this_time"], dev["block_tables"],
+                              (dev["rope_cos"], dev["rope_sin"]), dev["cache_k_scale"], dev["cache_v_scale"],
+                              num_heads=32, kv_num_heads=8, max_chunk=90, cu_seqlens_q=dev["cu_seqlens_q"],
+                              qkv_bias=bias.cuda(), q_norm_weight=qw.cuda(), k_norm_weight=kw.cuda(), rms_norm_eps=1e-6)
+    torch.cuda.synchronize()
+    want, kc, vc = oracle_step(oracle, c, CACHE_INT8, qkv_bias=bits(bias), q_norm_weight=np_of(qw),
+                               k_norm_weight=np_of(kw), rms_norm_eps=1e-6)
     assert np.array_equal(np_of(dev["key_cache"]), kc) and np.array_equal(np_of(dev["value_cache"]), vc)
     ok, mx, bad = bf16_close(bits(out), want)
     assert ok, "%d out of tolerance, max %.4g" % (bad, mx)

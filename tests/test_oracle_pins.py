@@ -161,6 +161,83 @@ def test_writer_rope_against_complex_multiplication(oracle, style):
         assert (got - torch.clamp(ideal, -127, 127)).abs().max() <= 0.5 + 1e-3
 
 
+def _write_ep(oracle, case, bias=None, qw=None, kw=None, eps=0.0, rope=True):
+    kc, vc = np_of(case["key_cache"]).copy(), np_of(case["value_cache"]).copy()
+    q, k, v = oracle.write_cache_kv(
+        bits(case["qkv"]), kc, vc, np_of(case["cache_k_scale"]), np_of(case["cache_v_scale"]),
+        np_of(case["rope_cos"]) if rope else None, np_of(case["rope_sin"]) if rope else None,
+        np_of(case["block_tables"]), np_of(case["seq_lens_decoder"]), np_of(case["cu_seqlens_q"]), case["hq"],
+        case["hkv"], case["d"], 1 if case["rope_style"] == "neox" else 0, case["quant"], True,
+        qkv_bias=None if bias is None else bits(bias), q_norm_weight=qw, k_norm_weight=kw, rms_norm_eps=eps)
+    return q, k, v, kc, vc
+
+
+@pytest.mark.parametrize("style", ["neox", "interleaved"])
+def test_writer_epilogue_bias_and_rms_norm(oracle, style):
+    """The projection epilogue of the writer: the bias add is torch's bf16 add; the RMS norm agrees with
+    an fp64 one; unit weights give heads of unit mean square; the norm forgets the input's scale; and the
+    epilogue composes with the rotation (norm in front of the complex multiplication)."""
+    case = syn.write_case(num_seqs=16, max_pos=300, seed=11, rope_style=style)
+    hq, hkv, d = case["hq"], case["hkv"], case["d"]
+    g = torch.Generator().manual_seed(1)
+    bias = (torch.randn(((hq + 2 * hkv) * d,), generator=g) * 0.5).to(torch.bfloat16)
+    # bias alone, no rotation: every output is torch's bf16 sum, V included
+    q, k, v, kc, vc = _write_ep(oracle, case, bias=bias, rope=False)
+    want = (case["qkv"] + bias[None]).view(16, hq + 2 * hkv, d)                        # bf16 + bf16 -> bf16 (RNE of the exact sum)
+    assert np.array_equal(q.reshape(16, hq, d), bits(want[:, :hq]))
+    assert np.array_equal(k.reshape(16, hkv, d), bits(want[:, hq:hq + hkv]))
+    assert np.array_equal(v.reshape(16, hkv, d), bits(want[:, hq + hkv:]))
+    # the V bytes are the quantised biased values
+    pos = case["seq_lens_decoder"].long()
+    bt = case["block_tables"]
+    for b in range(16):
+        blk, slot = int(bt[b, int(pos[b]) // 64]), int(pos[b]) % 64
+        ideal = want[b, hq + hkv:].double() / case["cache_v_scale"].double()
+        got = torch.from_numpy(vc[blk, :, slot, :].view(np.int8).astype(np.float64))
+        assert (got - torch.clamp(ideal, -127, 127)).abs().max() <= 0.5 + 1e-6
+    # norm (with bias), no rotation, against fp64
+    qw = (torch.rand((d,), generator=g) + 0.5).numpy()
+    kw = (torch.rand((d,), generator=g) + 0.5).numpy()
+    eps = 1e-6
+    q, k, v, _, _ = _write_ep(oracle, case, bias=bias, qw=qw, kw=kw, eps=eps, rope=False)
+    x = want.double()
+    rms = torch.rsqrt((x * x).mean(-1, keepdim=True) + eps)
+    nq = x[:, :hq] * rms[:, :hq] * torch.from_numpy(qw).double()
+    nk = x[:, hq:hq + hkv] * rms[:, hq:hq + hkv] * torch.from_numpy(kw).double()
+    gq = torch.from_numpy(oracle.bf16_to_f32(q)).double().view(16, hq, d)
+    gk = torch.from_numpy(oracle.bf16_to_f32(k)).double().view(16, hkv, d)
+    assert torch.allclose(gq, nq, atol=1e-6, rtol=2.0 ** -8) and torch.allclose(gk, nk, atol=1e-6, rtol=2.0 ** -8)
+    assert np.array_equal(v.reshape(16, hkv, d), bits(want[:, hq + hkv:]))             # V is never normed
+    # only K normed: Q stays the biased input
+    q2, k2, _, _, _ = _write_ep(oracle, case, bias=bias, kw=kw, eps=eps, rope=False)
+    assert np.array_equal(q2.reshape(16, hq, d), bits(want[:, :hq])) and np.array_equal(k2, k)
+    # unit weights, eps 0: mean square 1 (up to bf16 rounding of the outputs); input scale is forgotten
+    one = np.ones(d, np.float32)
+    q3, _, _, _, _ = _write_ep(oracle, case, qw=one, kw=one, rope=False)
+    ms = (torch.from_numpy(oracle.bf16_to_f32(q3)).double().view(16, hq, d) ** 2).mean(-1)
+    assert (ms - 1).abs().max() < 5e-3
+    scaled = dict(case)
+    scaled["qkv"] = (case["qkv"].float() * 4.0).to(torch.bfloat16)                      # exact in bf16
+    q4, k4, _, kc4, _ = _write_ep(oracle, scaled, qw=qw, kw=kw, eps=0.0)
+    q5, k5, _, kc5, _ = _write_ep(oracle, case, qw=qw, kw=kw, eps=0.0)
+    assert np.array_equal(q4, q5) and np.array_equal(k4, k5) and np.array_equal(kc4, kc5)   # x4 is exact at every step
+    # with the rotation: the norm comes first (rotation keeps pair norms, so rotating the fp64 norm matches)
+    ang = torch.arange(300, dtype=torch.float64)[:, None] * (500000.0 ** (-2.0 * torch.arange(d // 2, dtype=torch.float64) / d))[None]
+    rot = torch.polar(torch.ones_like(ang), ang)[pos][:, None, :]
+    xq = case["qkv"].double().view(16, hq + 2 * hkv, d)[:, :hq]
+    nq = xq * torch.rsqrt((xq * xq).mean(-1, keepdim=True) + eps) * torch.from_numpy(qw).double()
+    z = torch.complex(nq[..., : d // 2], nq[..., d // 2:]) if style == "neox" else torch.complex(nq[..., 0::2], nq[..., 1::2])
+    zr = z * rot
+    wq = torch.empty_like(nq)
+    if style == "neox":
+        wq[..., : d // 2], wq[..., d // 2:] = zr.real, zr.imag
+    else:
+        wq[..., 0::2], wq[..., 1::2] = zr.real, zr.imag
+    q6, _, _, _, _ = _write_ep(oracle, case, qw=qw, kw=kw, eps=eps)
+    g6 = torch.from_numpy(oracle.bf16_to_f32(q6)).double().view(16, hq, d)
+    assert torch.allclose(g6, wq, atol=2e-2, rtol=8e-3)
+
+
 def test_writer_position_zero_is_identity_and_untouched_slots_stay(oracle):
     case = syn.write_case(num_seqs=8, max_pos=256, seed=5)
     case["seq_lens_decoder"][:] = 0
