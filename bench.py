@@ -92,7 +92,7 @@ def other_workloads(args):
         def fused():
             fd.append_attention(c["qkv"], c["key_cache"], c["value_cache"], c["seq_lens_encoder"], c["seq_lens_decoder"],
                                 c["seq_lens_this_time"], c["block_tables"], rot, c["cache_k_scale"], c["cache_v_scale"],
-                                num_heads=32, kv_num_heads=8, max_chunk=1, cu_seqlens_q=c["cu_seqlens_q"], workspace=sws,
+                                num_heads=32, kv_num_heads=8, max_chunk=0, cu_seqlens_q=c["cu_seqlens_q"], workspace=sws,
                                 out=sout)
         ms = time_events(fused, args.steps, args.warmup)
         line("configs[2] fused step: cache write + decode in one call", ms, "hbm",

@@ -16,6 +16,7 @@ from .ops import (  # noqa: F401
     sqattn_select,
     write_cache_kv,
 )
+from .backend import AppendAttentionBackend, AttentionLayer, ForwardMeta, SequenceBook  # noqa: F401
 from .block_pool import BlockPool  # noqa: F401
 from .rope import rope_table  # noqa: F401
 

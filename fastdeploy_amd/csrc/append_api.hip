@@ -56,7 +56,7 @@ extern "C" int fdattn_append_attention_ex(
     const fdattn_qkv_epilogue* epilogue, void* stream) {
   if (!seq_lens_encoder || !seq_lens_this_time || !cu_seqlens_q || !out || !workspace)
     return fail(FDATTN_ERR_NULL, "fdattn_append_attention: a required pointer is NULL");
-  if (num_tokens < 0 || batch <= 0 || max_chunk <= 0 || hq <= 0 || hkv <= 0 || head_dim <= 0 ||
+  if (num_tokens < 0 || batch <= 0 || max_chunk < 0 || hq <= 0 || hkv <= 0 || head_dim <= 0 ||
       max_blocks_per_seq <= 0)
     return fail(FDATTN_ERR_SHAPE, "fdattn_append_attention: bad shape tokens=%d batch=%d max_chunk=%d hq=%d hkv=%d "
                 "head_dim=%d max_blocks=%d", num_tokens, batch, max_chunk, hq, hkv, head_dim, max_blocks_per_seq);
@@ -67,7 +67,7 @@ extern "C" int fdattn_append_attention_ex(
                 w.total);
   char* ws = (char*)workspace;
   void* q_rot = ws + w.q_rot;
-  const bool any_prefill = max_chunk > 1;
+  const bool any_prefill = max_chunk > 0;  // the caller's word: 0 = no sequence has seq_lens_encoder > 0
   void* k_new = any_prefill ? ws + w.k_new : nullptr;
   void* v_new = any_prefill ? ws + w.v_new : nullptr;
   // 1. every new token: rotate, quantise, store (argument checks of the shared kind happen here)

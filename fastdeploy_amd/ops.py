@@ -330,10 +330,14 @@ def append_attention_prefill(q, k_new, v_new, key_cache, value_cache, cache_k_sc
     return out
 
 
+def append_attention_workspace_bytes(num_tokens, batch, num_heads, kv_heads, head_dim, max_blocks_per_seq):
+    return _lib.lib().fdattn_append_attention_workspace_bytes(num_tokens, batch, num_heads, kv_heads, head_dim,
+                                                             max_blocks_per_seq)
+
+
 def append_attention_workspace(num_tokens, batch, num_heads, kv_heads, head_dim, max_blocks_per_seq, device="cuda"):
     """A workspace tensor large enough for append_attention at these shapes."""
-    n = _lib.lib().fdattn_append_attention_workspace_bytes(num_tokens, batch, num_heads, kv_heads, head_dim,
-                                                          max_blocks_per_seq)
+    n = append_attention_workspace_bytes(num_tokens, batch, num_heads, kv_heads, head_dim, max_blocks_per_seq)
     return torch.empty(n, dtype=torch.uint8, device=device)
 
 
@@ -346,7 +350,7 @@ def append_attention(qkv, key_cache, value_cache, seq_lens_encoder, seq_lens_dec
     every new token is rotated and written to the cache, decode rows (one token,
     seq_lens_encoder == 0) attend to the cache, prefill rows (seq_lens_encoder > 0)
     to their cached prefix and causally to their own chunk; slots without a token
-    are skipped.  max_chunk bounds the tokens of one sequence (1 = decode only).
+    are skipped.  max_chunk bounds the tokens of a prefill row (0: the step has none, decode only).
     qkv_bias / q_norm_weight / k_norm_weight / rms_norm_eps: the projection's epilogue, as in write_cache_kv.
     Returns bf16 [num_tokens, num_heads*head_dim]."""
     nb, hkv, bs, d = _cache_dims(key_cache, value_cache)
@@ -385,8 +389,8 @@ def append_attention(qkv, key_cache, value_cache, seq_lens_encoder, seq_lens_dec
         max_pos = cos.shape[0]
     if rope_style not in _ROPE:
         raise ValueError("unknown rope_style %r (neox | interleaved)" % (rope_style,))
-    if max_chunk < 1:
-        raise ValueError("max_chunk must be >= 1")
+    if max_chunk < 0:
+        raise ValueError("max_chunk must be >= 0")
     if out is None:
         out = torch.empty((T, num_heads * d), dtype=torch.bfloat16, device=qkv.device)
     need = _lib.lib().fdattn_append_attention_workspace_bytes(T, batch, num_heads, hkv, d, mb)

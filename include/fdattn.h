@@ -328,7 +328,8 @@ FDATTN_API size_t fdattn_append_attention_workspace_bytes(int num_tokens, int ba
  *                  (fdattn_decode_attention),
  *   idle           otherwise (no token: nothing is read or written for it).
  * Every new token is first rotated and written to the cache (fdattn_write_cache_kv).
- * max_chunk bounds the tokens of one sequence in this step (1 = no prefill row).
+ * max_chunk bounds the tokens of a prefill row in this step; 0 says that the step has no
+ * prefill row (the prefill pass is then not launched at all).
  * Nothing is gathered or synchronised on the host; out rows of idle slots do not exist.
  */
 FDATTN_API int fdattn_append_attention(

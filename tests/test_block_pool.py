@@ -155,3 +155,34 @@ def test_random_workload_against_a_dictionary_model():
         assert t[s, :len(model[s])].tolist() == model[s]
     assert p.free_blocks == len(free) and [p.refcount(b) for b in range(N)] == rc
     check_invariants(p)
+
+
+def test_sequence_book_builds_the_step_description():
+    """Host bookkeeping between steps: which slots are prefill rows, decode rows or idle, the lengths the
+    kernels are given, blocks reserved before the step and lengths advanced after it."""
+    from fastdeploy_amd.backend import SequenceBook
+    pool = BlockPool(num_blocks=8, block_size=16, max_seqs=4, max_blocks_per_seq=4)
+    book = SequenceBook(pool, device="cpu")
+    m = book.schedule({0: 20, 2: 1})                       # a prompt, and a one-token prompt: both prefill rows
+    assert m.seq_lens_encoder.tolist() == [20, 0, 1, 0] and m.seq_lens_decoder.tolist() == [0, 0, 0, 0]
+    assert m.seq_lens_this_time.tolist() == [20, 0, 1, 0] and (m.num_tokens, m.max_enc_len_this_time) == (21, 20)
+    assert m.block_tables.tolist() == [[0, 1, -1, -1], [-1] * 4, [2, -1, -1, -1], [-1] * 4]
+    assert book.lengths == [0, 0, 0, 0]                    # nothing advances before commit
+    book.commit()
+    assert book.lengths == [20, 0, 1, 0]
+    m = book.schedule({0: 1, 2: 1, 3: 0})                  # two decode rows; a zero count is an idle slot
+    assert m.seq_lens_encoder.tolist() == [0, 0, 0, 0] and m.seq_lens_decoder.tolist() == [20, 0, 1, 0]
+    assert m.seq_lens_this_time.tolist() == [1, 0, 1, 0] and m.max_enc_len_this_time == 0
+    book.commit()
+    m = book.schedule({0: 12})                             # a later chunk of several tokens: prefill row on a prefix
+    assert m.seq_lens_encoder.tolist() == [12, 0, 0, 0] and m.seq_lens_decoder.tolist() == [21, 0, 2, 0]
+    assert pool.seq_blocks(0) == 3                         # 33 tokens
+    book.commit()
+    assert book.fork(0, 1) == 32 and book.lengths[1] == 32 and pool.refcount(0) == 2
+    with pytest.raises(ValueError):
+        book.schedule({3: 16 * 4 + 1})                     # more than a table row holds
+    with pytest.raises(ValueError):
+        book.schedule({3: 16 * 4, 2: 60})                  # slot 3 takes the last four blocks, slot 2 finds none
+    book.finish(3)
+    book.finish(0)
+    assert book.lengths[0] == 0 and pool.refcount(0) == 1 and pool.refcount(3) == 0 and pool.free_blocks == 5

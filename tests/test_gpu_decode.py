@@ -188,7 +188,7 @@ def test_write_then_decode_config3_full_size(oracle):
     out = fd.append_attention(dev["qkv"], dev["key_cache"], dev["value_cache"], dev["seq_lens_encoder"],
                               dev["seq_lens_decoder"], dev["seq_lens_this_time"], dev["block_tables"],
                               (dev["rope_cos"], dev["rope_sin"]), dev["cache_k_scale"], dev["cache_v_scale"],
-                              num_heads=32, kv_num_heads=8, max_chunk=1)
+                              num_heads=32, kv_num_heads=8, max_chunk=0)
     torch.cuda.synchronize()
     kc, vc = np_of(case["key_cache"]).copy(), np_of(case["value_cache"]).copy()
     q, _, _ = oracle.write_cache_kv(bits(case["qkv"]), kc, vc, np_of(case["cache_k_scale"]), np_of(case["cache_v_scale"]),
@@ -216,7 +216,7 @@ def test_decode_step_replays_from_a_hip_graph():
     def step(c, rot, ws):
         out = fd.append_attention(c["qkv"], c["key_cache"], c["value_cache"], c["seq_lens_encoder"],
                                   c["seq_lens_decoder"], c["seq_lens_this_time"], c["block_tables"], rot,
-                                  c["cache_k_scale"], c["cache_v_scale"], num_heads=32, kv_num_heads=8, max_chunk=1,
+                                  c["cache_k_scale"], c["cache_v_scale"], num_heads=32, kv_num_heads=8, max_chunk=0,
                                   workspace=ws)
         c["seq_lens_decoder"].add_(1)
         return out

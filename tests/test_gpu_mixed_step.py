@@ -105,7 +105,7 @@ def test_mixed_batch_step_with_projection_epilogue(oracle):
 
 
 def test_decode_only_and_prefill_only_steps_through_the_same_entry(oracle):
-    for enc, dec, mc in (([0, 0, 0, 0], [5, 64, 1000, 0], 1), ([64, 1, 257, 0], [0, 0, 100, 0], 257)):
+    for enc, dec, mc in (([0, 0, 0, 0], [5, 64, 1000, 0], 0), ([64, 1, 257, 0], [0, 0, 100, 0], 257)):
         c = mixed_case(enc, dec, CACHE_INT8, seed=9)
         dev = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
         ws = fd.append_attention_workspace(c["T"], len(enc), 32, 8, 128, dev["block_tables"].shape[1])
@@ -161,7 +161,7 @@ def test_steps_over_block_pool_tables_with_a_shared_prefix(oracle):
                  seq_lens_this_time=this, cu_seqlens_q=cu, rope_cos=cos, rope_sin=sin, T=int(cu[-1]))
         out = fd.append_attention(qkv.cuda(), kc_dev, vc_dev, enc_t.cuda(), dec_t.cuda(), this.cuda(),
                                   c["block_tables"].cuda(), (cos.cuda(), sin.cuda()), ks.cuda(), vs.cuda(),
-                                  num_heads=hq, kv_num_heads=hkv, max_chunk=max(max(enc), 1), cache_quant_type=quant,
+                                  num_heads=hq, kv_num_heads=hkv, max_chunk=max(enc), cache_quant_type=quant,
                                   cu_seqlens_q=cu.cuda())
         torch.cuda.synchronize()
         want, kc_w, vc_w = oracle_step(oracle, c, quant)
