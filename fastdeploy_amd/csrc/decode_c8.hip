@@ -75,11 +75,22 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
   const int ticket = blockIdx.x;
   const int p = ticket / a.chunks_per_pair, ck = ticket - p * a.chunks_per_pair;
   const int b = p / a.hkv, h = p - b * a.hkv;
+  const int first = ck * a.chunk;
+  // ---- unit table, requested before anything else: lane j asks for the physical block of unit
+  // first + j.  The request depends on the block index alone, so it travels together with the
+  // loads of the sequence's length below instead of behind them - under load every dependent
+  // round trip to memory at the start of a workgroup costs microseconds in which its LDS slots
+  // carry nothing.
+  int lb = -1, pb_raw = -1;
+  if (lane < a.chunk) {
+    lb = first + lane;
+    if (SPARSE) lb = lb < a.max_kept ? a.kept_blocks[(size_t)p * a.max_kept + lb] : -1;
+    if (lb >= 0 && lb < a.max_blocks) pb_raw = a.block_tables[(size_t)b * a.max_blocks + lb];
+  }
   int row;
   if (!decode_row(a.rows, b, row)) return;
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
   const int n_p = pair_units<SPARSE>(a, p, kv_len);
-  const int first = ck * a.chunk;
   const int cnt = min(a.chunk, n_p - first);  // <= 0: past the end of this pair's list
   const bool single = n_p <= a.chunk;
   if (cnt <= 0) {
@@ -97,20 +108,14 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
   const DmaOffsets offK = dma_offsets<kShiftK>(lane), offV = dma_offsets<kShiftV>(lane);
   const int n16 = lane & 15, g4 = lane >> 4;
 
-  // ---- unit table: lane j describes unit first + j (physical block, valid tokens)
+  // lane j describes unit first + j (physical block, valid tokens)
   int my_pb = 0, my_valid = 0;
   {
-    int lb = -1, pb = -1;
-    if (lane < cnt) {
-      lb = first + lane;
-      if (SPARSE) lb = a.kept_blocks[(size_t)p * a.max_kept + lb];
-      if (lb >= 0 && lb < a.max_blocks) pb = a.block_tables[(size_t)b * a.max_blocks + lb];
-    }
-    // both loads are consumed here on every path: nothing of the table build stays in
+    // the table loads are consumed here on every path: nothing of the table build stays in
     // flight when the streaming loop starts
-    asm volatile("" ::"v"(lb), "v"(pb));
-    if (pb >= 0 && pb < a.num_blocks) {
-      my_pb = pb;
+    asm volatile("" ::"v"(lb), "v"(pb_raw));
+    if (lane < cnt && pb_raw >= 0 && pb_raw < a.num_blocks) {
+      my_pb = pb_raw;
       my_valid = min(max(kv_len - lb * kBS, 0), kBS);
     }
   }
