@@ -112,28 +112,53 @@ struct PairState {
   float o[8];  // channel 16*ct + lane%16 of head lane/16
 };
 
-// A operand rows: row = head*4 + limb; lane (m = lane%16, g = lane/16) holds channels
-// 16*(g + 4s) .. +15 of k-step s.
-template <int QUANT>
-__device__ __forceinline__ void load_pair(const uint16_t* q, const float* k_scale, int hkv, float sm_scale_log2, int p, int row,
-                                          int lane, PairState& st) {
+// The q and k_scale values a lane needs for its A operand rows, as loaded: requested early (they depend
+// on the pair alone), turned into limbs later, when the first tiles are already on their way.
+struct PairRaw {
+  uint4 w[2][2];    // k-step s: 16 bf16 channels 16*(g + 4s) .. +15 of head (lane%16)/4
+  float4 ks[2][4];  // their K scales
+};
+
+__device__ __forceinline__ PairRaw load_pair_issue(const uint16_t* q, const float* k_scale, int hkv, int p, int row, int lane) {
   const int h = p % hkv;  // row: the sequence's row of q
-  const int m = lane & 15, g = lane >> 4, head = m >> 2, limb = m & 3;
+  const int m = lane & 15, g = lane >> 4, head = m >> 2;
   const uint16_t* qrow = q + ((size_t)row * hkv * kG + h * kG + head) * kD;
   const float* ks = k_scale + (size_t)h * kD;
+  PairRaw r;
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    const int c0 = 16 * (g + 4 * s);
+    r.w[s][0] = *reinterpret_cast<const uint4*>(qrow + c0);
+    r.w[s][1] = *reinterpret_cast<const uint4*>(qrow + c0 + 8);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r.ks[s][i] = *reinterpret_cast<const float4*>(ks + c0 + 4 * i);
+  }
+  return r;
+}
+
+// A operand rows: row = head*4 + limb; lane (m = lane%16, g = lane/16) holds channels
+// 16*(g + 4s) .. +15 of k-step s.  qs_out (optional): the lane's 32 products q * k_scale.
+template <int QUANT>
+__device__ __forceinline__ void load_pair_finish(const PairRaw& r, float sm_scale_log2, int lane, PairState& st,
+                                                 float (*qs_out)[16] = nullptr) {
+  const int m = lane & 15, limb = m & 3;
   float qs[2][16];
   float amax = 0.f;
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
-    const int c0 = 16 * (g + 4 * s);
-    const uint4 w0 = *reinterpret_cast<const uint4*>(qrow + c0);
-    const uint4 w1 = *reinterpret_cast<const uint4*>(qrow + c0 + 8);
-    const u32 w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+    const u32 w[8] = {r.w[s][0].x, r.w[s][0].y, r.w[s][0].z, r.w[s][0].w, r.w[s][1].x, r.w[s][1].y, r.w[s][1].z, r.w[s][1].w};
+    const float k[16] = {r.ks[s][0].x, r.ks[s][0].y, r.ks[s][0].z, r.ks[s][0].w, r.ks[s][1].x, r.ks[s][1].y,
+                         r.ks[s][1].z, r.ks[s][1].w, r.ks[s][2].x, r.ks[s][2].y, r.ks[s][2].z, r.ks[s][2].w,
+                         r.ks[s][3].x, r.ks[s][3].y, r.ks[s][3].z, r.ks[s][3].w};
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      qs[s][2 * j] = bf16lo_to_f32(w[j]) * ks[c0 + 2 * j];
-      qs[s][2 * j + 1] = bf16hi_to_f32(w[j]) * ks[c0 + 2 * j + 1];
+      qs[s][2 * j] = bf16lo_to_f32(w[j]) * k[2 * j];
+      qs[s][2 * j + 1] = bf16hi_to_f32(w[j]) * k[2 * j + 1];
       amax = fmaxf(amax, fmaxf(fabsf(qs[s][2 * j]), fabsf(qs[s][2 * j + 1])));
+    }
+    if (qs_out) {
+#pragma unroll
+      for (int j = 0; j < 16; ++j) qs_out[s][j] = qs[s][j];
     }
   }
   amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
@@ -185,6 +210,12 @@ __device__ __forceinline__ void load_pair(const uint16_t* q, const float* k_scal
   st.l = 0.f;
 #pragma unroll
   for (int i = 0; i < 8; ++i) st.o[i] = 0.f;
+}
+
+template <int QUANT>
+__device__ __forceinline__ void load_pair(const uint16_t* q, const float* k_scale, int hkv, float sm_scale_log2, int p, int row,
+                                          int lane, PairState& st) {
+  load_pair_finish<QUANT>(load_pair_issue(q, k_scale, hkv, p, row, lane), sm_scale_log2, lane, st);
 }
 
 }  // namespace fdattn

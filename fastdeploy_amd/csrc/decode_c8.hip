@@ -89,6 +89,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
   }
   int row;
   if (!decode_row(a.rows, b, row)) return;
+  const PairRaw raw = load_pair_issue(a.q, a.k_scale, a.hkv, p, row, lane);  // in flight with the table entries
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
   const int n_p = pair_units<SPARSE>(a, p, kv_len);
   const int cnt = min(a.chunk, n_p - first);  // <= 0: past the end of this pair's list
@@ -136,7 +137,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
     int valid = __builtin_amdgcn_readlane(my_valid, wv);
     dma_tile(kbase + (size_t)pb * blk_stride, kaddr, offK);
     dma_tile(vbase + (size_t)pb * blk_stride, vaddr, offV);
-    load_pair<QUANT>(a.q, a.k_scale, a.hkv, a.sm_scale_log2, p, row, lane, st);
+    load_pair_finish<QUANT>(raw, a.sm_scale_log2, lane, st);
 
     for (int j = wv; j < cnt; j += kWaves) {
       const bool has_next = j + kWaves < cnt;

@@ -174,9 +174,15 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
   const int wv = uni(threadIdx.x >> 6);
   const int p = blockIdx.x / a.chunks_per_pair, ck = blockIdx.x - p * a.chunks_per_pair;
   const int b = p / a.hkv, h = p - b * a.hkv;
+  const int first = ck * a.chunk;
+  // Everything that depends on the block index alone is requested first and together - the table
+  // entries of this chunk, q and the K scales - so that the start of a workgroup costs two round
+  // trips to memory (these, then the first tiles), not one per step of a chain.
+  int pb_raw = -1;
+  if (lane < a.chunk && first + lane < a.max_blocks) pb_raw = a.block_tables[(size_t)b * a.max_blocks + first + lane];
+  const PairRaw raw = load_pair_issue(a.q, a.k_scale, a.hkv, p, b, lane);
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
   const int n_p = min((max(kv_len, 0) + kBS - 1) / kBS, a.max_blocks);
-  const int first = ck * a.chunk;
   const int cnt = min(a.chunk, n_p - first);
   float* const srow = a.approx + (size_t)p * a.max_blocks;
   // blocks of this chunk past the sequence: -inf
@@ -185,6 +191,26 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
     if (a.scores_out) a.scores_out[(size_t)p * a.max_blocks + j] = -INFINITY;
   }
   if (cnt <= 0) return;
+
+  const u32 saddr0 = (u32)uni((int)lds_addr_of(ldsK[wv][0]));
+  const DmaOffsets offK = dma_offsets<kShiftK>(lane);
+  const int n16 = lane & 15, g4 = lane >> 4;
+
+  int my_pb = 0, my_valid = 0;
+  {
+    asm volatile("" ::"v"(pb_raw));
+    if (lane < cnt && pb_raw >= 0 && pb_raw < a.num_blocks) {
+      my_pb = pb_raw;
+      my_valid = min(max(kv_len - (first + lane) * kBS, 0), kBS);
+    }
+  }
+  const size_t tile_stride = (size_t)kBS * kD;
+  const uint8_t* const kbase = a.key_cache + (size_t)h * tile_stride;
+  const size_t blk_stride = (size_t)a.hkv * tile_stride;
+
+  if (wv < cnt) dma_tile(kbase + (size_t)__builtin_amdgcn_readlane(my_pb, wv) * blk_stride, saddr0, offK);
+  if (wv + kWaves < cnt)
+    dma_tile(kbase + (size_t)__builtin_amdgcn_readlane(my_pb, wv + kWaves) * blk_stride, saddr0 + kTileB, offK);
 
   if (ck == 0 && wv == 0) {
     // error bound of the MFMA scores of this pair (see the top of the file): q*scale is cut to
@@ -212,47 +238,25 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
     if (lane == 0) a.eps[p] = e * 1.0001f;
   }
 
-  const u32 saddr0 = (u32)uni((int)lds_addr_of(ldsK[wv][0]));
-  const DmaOffsets offK = dma_offsets<kShiftK>(lane);
-  const int n16 = lane & 15, g4 = lane >> 4;
-
-  int my_pb = 0, my_valid = 0;
-  {
-    int pb = -1;
-    if (lane < cnt) pb = a.block_tables[(size_t)b * a.max_blocks + first + lane];
-    asm volatile("" ::"v"(pb));
-    if (pb >= 0 && pb < a.num_blocks) {
-      my_pb = pb;
-      my_valid = min(max(kv_len - (first + lane) * kBS, 0), kBS);
-    }
-  }
   if (wv >= cnt) return;
-  const size_t tile_stride = (size_t)kBS * kD;
-  const uint8_t* const kbase = a.key_cache + (size_t)h * tile_stride;
-  const size_t blk_stride = (size_t)a.hkv * tile_stride;
-
-  dma_tile(kbase + (size_t)__builtin_amdgcn_readlane(my_pb, wv) * blk_stride, saddr0, offK);
-  if (wv + kWaves < cnt)
-    dma_tile(kbase + (size_t)__builtin_amdgcn_readlane(my_pb, wv + kWaves) * blk_stride, saddr0 + kTileB, offK);
   PairState st;
-  load_pair<QUANT>(a.q, a.k_scale, a.hkv, 1.0f, p, p / a.hkv, lane, st);  // scores in natural units
+  float qs[2][16];
+  load_pair_finish<QUANT>(raw, 1.0f, lane, st, qs);  // scores in natural units
   // fp8: a second operand, |q*scale| in one e4m3 limb, gives sum_c |q*scale||k| per token next to the score;
   // the error of a block's score is a small multiple of that sum (see the bound below)
   v4i aabs[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
   float amax_pair = 0.f;
   if (QUANT != FDATTN_CACHE_INT8) {
-    const int m = lane & 15, g = lane >> 4, head = m >> 2, limb = m & 3;
-    const uint16_t* qrow = a.q + ((size_t)b * a.hkv * kG + h * kG + head) * kD;
+    const int m = lane & 15, head = m >> 2, limb = m & 3;
     // st.rs = amax / 256 of this lane's S-layout head; the A layout wants the head of row m
     const float rs_row = __shfl(st.rs, 16 * head, 64);
     const float inv = rs_row > 0.f ? 1.0f / rs_row : 0.f;
 #pragma unroll
     for (int k2 = 0; k2 < 2; ++k2) {
-      const int c0 = 16 * (g + 4 * k2);
       u32 pk[4] = {0, 0, 0, 0};
 #pragma unroll
       for (int jj = 0; jj < 16; ++jj) {
-        const float x = fabsf(bf16_to_f32(qrow[c0 + jj]) * a.k_scale[h * kD + c0 + jj]) * inv;
+        const float x = fabsf(qs[k2][jj]) * inv;
         const u32 code = limb == 0 ? ((u32)__builtin_amdgcn_cvt_pk_fp8_f32(x, x, 0, false) & 0xffu) : 0u;
         pk[jj >> 2] |= code << (8 * (jj & 3));
       }
