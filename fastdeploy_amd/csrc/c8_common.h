@@ -10,7 +10,7 @@ constexpr int kWaves = 4;      // wavefronts per workgroup
 constexpr int kTileB = 8192;   // bytes of one K or V tile (64 tokens x 128 channels)
 constexpr int kD = 128, kG = 4, kBS = 64;
 constexpr int kSlotFloats = kG * kD;  // partial o per slot
-constexpr int kMaxChunk = 64;         // units per chunk: one unit-table entry per lane
+constexpr int kMaxChunk = 128;        // units per chunk: two unit-table entries per lane
 
 __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
 

@@ -57,6 +57,12 @@ extern "C" int fdattn_decode_uses_mfma(int hq, int hkv, int head_dim, int block_
   return c8_supported(hq, hkv, head_dim, block_size, cache_quant_type) ? 1 : 0;
 }
 
+extern "C" int fdattn_decode_chunks_per_sequence(int batch, int hkv, int max_blocks_per_seq) {
+  if (batch <= 0 || hkv <= 0 || max_blocks_per_seq <= 0) return 0;
+  const int chunk = c8_pick_chunk(batch * hkv, max_blocks_per_seq);
+  return (max_blocks_per_seq + chunk - 1) / chunk;
+}
+
 extern "C" int fdattn_decode_attention_stages(
     const void* q, const void* key_cache, const void* value_cache, const float* cache_k_scale,
     const float* cache_v_scale, const int32_t* block_tables, const int32_t* seq_lens_decoder,

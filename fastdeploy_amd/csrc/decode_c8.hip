@@ -73,7 +73,12 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
   const int lane = threadIdx.x & 63;
   const int wv = uni(threadIdx.x >> 6);
   const int ticket = blockIdx.x;
-  const int p = ticket / a.chunks_per_pair, ck = ticket - p * a.chunks_per_pair;
+  // Chunk-major: workgroups are dealt to the 8 XCDs in turn, so with the pair running fastest every
+  // XCD sees every chunk position (pair-major, a chunk count that shares a factor with 8 sends the
+  // often-empty late chunks of short sequences to the same XCDs); and the launch ends with the
+  // late chunks, the ones most often short or empty.
+  const int pairs = a.batch * a.hkv;
+  const int ck = ticket / pairs, p = ticket - ck * pairs;
   const int b = p / a.hkv, h = p - b * a.hkv;
   const int first = ck * a.chunk;
   // ---- unit table, requested before anything else: lane j asks for the physical block of unit
@@ -81,11 +86,16 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
   // loads of the sequence's length below instead of behind them - under load every dependent
   // round trip to memory at the start of a workgroup costs microseconds in which its LDS slots
   // carry nothing.
-  int lb = -1, pb_raw = -1;
-  if (lane < a.chunk) {
-    lb = first + lane;
-    if (SPARSE) lb = lb < a.max_kept ? a.kept_blocks[(size_t)p * a.max_kept + lb] : -1;
-    if (lb >= 0 && lb < a.max_blocks) pb_raw = a.block_tables[(size_t)b * a.max_blocks + lb];
+  int lb[2] = {-1, -1}, pb_raw[2] = {-1, -1};
+#pragma unroll
+  for (int e = 0; e < 2; ++e) {
+    const int u = lane + 64 * e;
+    if (u < a.chunk) {
+      int l = first + u;
+      if (SPARSE) l = l < a.max_kept ? a.kept_blocks[(size_t)p * a.max_kept + l] : -1;
+      if (l >= 0 && l < a.max_blocks) pb_raw[e] = a.block_tables[(size_t)b * a.max_blocks + l];
+      lb[e] = l;
+    }
   }
   int row;
   if (!decode_row(a.rows, b, row)) return;
@@ -109,17 +119,22 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
   const DmaOffsets offK = dma_offsets<kShiftK>(lane), offV = dma_offsets<kShiftV>(lane);
   const int n16 = lane & 15, g4 = lane >> 4;
 
-  // lane j describes unit first + j (physical block, valid tokens)
-  int my_pb = 0, my_valid = 0;
+  // lane j describes units first + j and first + j + 64 (physical block, valid tokens)
+  int my_pb[2] = {0, 0}, my_valid[2] = {0, 0};
   {
     // the table loads are consumed here on every path: nothing of the table build stays in
     // flight when the streaming loop starts
-    asm volatile("" ::"v"(lb), "v"(pb_raw));
-    if (lane < cnt && pb_raw >= 0 && pb_raw < a.num_blocks) {
-      my_pb = pb_raw;
-      my_valid = min(max(kv_len - lb * kBS, 0), kBS);
-    }
+    asm volatile("" ::"v"(lb[0]), "v"(pb_raw[0]), "v"(lb[1]), "v"(pb_raw[1]));
+#pragma unroll
+    for (int e = 0; e < 2; ++e)
+      if (lane + 64 * e < cnt && pb_raw[e] >= 0 && pb_raw[e] < a.num_blocks) {
+        my_pb[e] = pb_raw[e];
+        my_valid[e] = min(max(kv_len - lb[e] * kBS, 0), kBS);
+      }
   }
+  // entry of unit j (uniform)
+  auto unit_pb = [&](int j) { return j < 64 ? __builtin_amdgcn_readlane(my_pb[0], j) : __builtin_amdgcn_readlane(my_pb[1], j - 64); };
+  auto unit_valid = [&](int j) { return j < 64 ? __builtin_amdgcn_readlane(my_valid[0], j) : __builtin_amdgcn_readlane(my_valid[1], j - 64); };
 
   const size_t tile_stride = (size_t)kBS * kD;  // bytes of one (block, head) tile
   const uint8_t* const kbase = a.key_cache + (size_t)h * tile_stride;
@@ -133,8 +148,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
   for (int i = 0; i < 8; ++i) st.o[i] = 0.f;
 
   if (wv < cnt) {  // this wavefront has units wv, wv + 4, ...
-    int pb = __builtin_amdgcn_readlane(my_pb, wv);
-    int valid = __builtin_amdgcn_readlane(my_valid, wv);
+    int pb = unit_pb(wv);
+    int valid = unit_valid(wv);
     dma_tile(kbase + (size_t)pb * blk_stride, kaddr, offK);
     dma_tile(vbase + (size_t)pb * blk_stride, vaddr, offV);
     load_pair_finish<QUANT>(raw, a.sm_scale_log2, lane, st);
@@ -143,8 +158,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
       const bool has_next = j + kWaves < cnt;
       int pbn = 0, validn = 0;
       if (has_next) {
-        pbn = __builtin_amdgcn_readlane(my_pb, j + kWaves);
-        validn = __builtin_amdgcn_readlane(my_valid, j + kWaves);
+        pbn = unit_pb(j + kWaves);
+        validn = unit_valid(j + kWaves);
       }
 
       // ---------------- S = Q K^T : rows = head*4 + limb, columns = token slots
@@ -359,16 +374,30 @@ __global__ __launch_bounds__(256) void decode_c8_combine_kernel(C8Args a) {
   *reinterpret_cast<u32*>(o) = (u32)f32_to_bf16(r0) | ((u32)f32_to_bf16(r1) << 16);
 }
 
-#ifndef FDATTN_CHUNK
-#define FDATTN_CHUNK 24
-#endif
+// Units per workgroup.  The aim is one workgroup per LDS slot of the GPU (two per CU): every pair's
+// block list is cut into as few chunks as fill the slots once, so that workgroups start once, stream
+// for as long as possible and - when one chunk covers the pair - finish it without a partial or a
+// merge.  Lists too long for the unit table (kMaxChunk entries) get more chunks; short lists keep at
+// least one unit per wavefront.
+static int gpu_slots() {
+  static int slots = 0;  // benign race: every thread computes the same value
+  if (slots == 0) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    slots = 2 * cus;
+  }
+  return slots;
+}
 
-// Units per workgroup: 24 (384 KiB of cache) keeps workgroups short enough for the
-// dispatcher to balance and long enough to amortise their start; small launches get
-// smaller chunks so that the grid still covers the GPU.
-static int pick_chunk(int pairs, int max_units) {
-  int chunk = FDATTN_CHUNK;  // at most kMaxChunk
-  while (chunk > 4 && (long long)pairs * ((max_units + chunk - 1) / chunk) < 1024) chunk /= 2;
+int c8_pick_chunk(int pairs, int max_units) {
+#ifdef FDATTN_FORCE_CHUNK
+  return FDATTN_FORCE_CHUNK;
+#endif
+  const int cpp = (gpu_slots() + pairs - 1) / pairs;
+  int chunk = (max_units + cpp - 1) / cpp;
+  if (chunk < kWaves) chunk = kWaves;
+  if (chunk > kMaxChunk) chunk = kMaxChunk;
   return chunk;
 }
 
@@ -376,7 +405,7 @@ constexpr int kMaxPairs = 1 << 20;
 
 size_t c8_workspace_bytes(int batch, int hkv, int max_units) {
   const int pairs = batch * hkv;
-  const int chunk = pick_chunk(pairs, max_units);
+  const int chunk = c8_pick_chunk(pairs, max_units);
   const size_t slots = (size_t)pairs * ((max_units + chunk - 1) / chunk);
   return slots * (kSlotFloats + 8) * sizeof(float);
 }
@@ -396,7 +425,7 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
   const bool sparse = kept_blocks != nullptr;
   const int pairs = batch * hkv;
   const int max_units = sparse ? (max_kept < max_blocks ? max_kept : max_blocks) : max_blocks;
-  const int chunk = pick_chunk(pairs, max_units);
+  const int chunk = c8_pick_chunk(pairs, max_units);
   const int cpp = ((max_units + chunk - 1) / chunk);
   if (pairs > kMaxPairs)
     return fail(FDATTN_ERR_SHAPE, "fdattn_decode_attention: batch*kv_heads = %d exceeds %d", pairs, kMaxPairs);
@@ -423,6 +452,7 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
   }
   int rc = check_launch("fdattn_decode_attention (mfma)");
   if (rc || !(stages & 2)) return rc;
+  if (cpp == 1) return 0;  // every pair was one chunk and has been finished by the main kernel
   if (sparse) hipLaunchKernelGGL(decode_c8_combine_kernel<true>, dim3(pairs), dim3(256), 0, s, a);
   else hipLaunchKernelGGL(decode_c8_combine_kernel<false>, dim3(pairs), dim3(256), 0, s, a);
   return check_launch("fdattn_decode_attention (merge)");

@@ -16,6 +16,7 @@
 //    beat it whatever the errors are) or undecided; only the undecided blocks - those
 //    within 2*eps of the k-th score, a handful - are re-scored in fp64 and ranked exactly.
 #include "c8_common.h"
+#include "launch.h"
 
 namespace fdattn {
 
@@ -172,14 +173,20 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
   __shared__ __attribute__((aligned(16))) uint8_t ldsK[kWaves][2][kTileB];  // two K slots per wavefront
   const int lane = threadIdx.x & 63;
   const int wv = uni(threadIdx.x >> 6);
-  const int p = blockIdx.x / a.chunks_per_pair, ck = blockIdx.x - p * a.chunks_per_pair;
+  // chunk-major: every XCD (workgroups are dealt to them in turn) sees every chunk position
+  const int pairs = a.batch * a.hkv;
+  const int ck = blockIdx.x / pairs, p = blockIdx.x - ck * pairs;
   const int b = p / a.hkv, h = p - b * a.hkv;
   const int first = ck * a.chunk;
   // Everything that depends on the block index alone is requested first and together - the table
-  // entries of this chunk, q and the K scales - so that the start of a workgroup costs two round
-  // trips to memory (these, then the first tiles), not one per step of a chain.
-  int pb_raw = -1;
-  if (lane < a.chunk && first + lane < a.max_blocks) pb_raw = a.block_tables[(size_t)b * a.max_blocks + first + lane];
+  // entries of this chunk (two per lane), q and the K scales - so that the start of a workgroup
+  // costs two round trips to memory (these, then the first tiles), not one per step of a chain.
+  int pb_raw[2] = {-1, -1};
+#pragma unroll
+  for (int e = 0; e < 2; ++e) {
+    const int u = lane + 64 * e;
+    if (u < a.chunk && first + u < a.max_blocks) pb_raw[e] = a.block_tables[(size_t)b * a.max_blocks + first + u];
+  }
   const PairRaw raw = load_pair_issue(a.q, a.k_scale, a.hkv, p, b, lane);
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
   const int n_p = min((max(kv_len, 0) + kBS - 1) / kBS, a.max_blocks);
@@ -196,21 +203,25 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
   const DmaOffsets offK = dma_offsets<kShiftK>(lane);
   const int n16 = lane & 15, g4 = lane >> 4;
 
-  int my_pb = 0, my_valid = 0;
+  int my_pb[2] = {0, 0}, my_valid[2] = {0, 0};
   {
-    asm volatile("" ::"v"(pb_raw));
-    if (lane < cnt && pb_raw >= 0 && pb_raw < a.num_blocks) {
-      my_pb = pb_raw;
-      my_valid = min(max(kv_len - (first + lane) * kBS, 0), kBS);
-    }
+    asm volatile("" ::"v"(pb_raw[0]), "v"(pb_raw[1]));
+#pragma unroll
+    for (int e = 0; e < 2; ++e)
+      if (lane + 64 * e < cnt && pb_raw[e] >= 0 && pb_raw[e] < a.num_blocks) {
+        my_pb[e] = pb_raw[e];
+        my_valid[e] = min(max(kv_len - (first + lane + 64 * e) * kBS, 0), kBS);
+      }
   }
+  auto unit_pb = [&](int j) { return j < 64 ? __builtin_amdgcn_readlane(my_pb[0], j) : __builtin_amdgcn_readlane(my_pb[1], j - 64); };
+  auto unit_valid = [&](int j) { return j < 64 ? __builtin_amdgcn_readlane(my_valid[0], j) : __builtin_amdgcn_readlane(my_valid[1], j - 64); };
   const size_t tile_stride = (size_t)kBS * kD;
   const uint8_t* const kbase = a.key_cache + (size_t)h * tile_stride;
   const size_t blk_stride = (size_t)a.hkv * tile_stride;
 
-  if (wv < cnt) dma_tile(kbase + (size_t)__builtin_amdgcn_readlane(my_pb, wv) * blk_stride, saddr0, offK);
+  if (wv < cnt) dma_tile(kbase + (size_t)unit_pb(wv) * blk_stride, saddr0, offK);
   if (wv + kWaves < cnt)
-    dma_tile(kbase + (size_t)__builtin_amdgcn_readlane(my_pb, wv + kWaves) * blk_stride, saddr0 + kTileB, offK);
+    dma_tile(kbase + (size_t)unit_pb(wv + kWaves) * blk_stride, saddr0 + kTileB, offK);
 
   if (ck == 0 && wv == 0) {
     // error bound of the MFMA scores of this pair (see the top of the file): q*scale is cut to
@@ -267,7 +278,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
 
   int it = 0;
   for (int j = wv; j < cnt; j += kWaves, ++it) {
-    const int valid = __builtin_amdgcn_readlane(my_valid, j);
+    const int valid = unit_valid(j);
     const uint8_t* kbuf = ldsK[wv][it & 1];  // indexed, not picked from a pointer array: stays an LDS address
     if (j + kWaves < cnt) wait_vm8(); else wait_vm0();
     float sv = -INFINITY, bv = 0.f;
@@ -308,7 +319,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
     }
     wait_lgkm0();  // tile consumed: refill its slot with the block two steps ahead
     if (j + 2 * kWaves < cnt)
-      dma_tile(kbase + (size_t)__builtin_amdgcn_readlane(my_pb, j + 2 * kWaves) * blk_stride, saddr0 + (u32)(it & 1) * kTileB, offK);
+      dma_tile(kbase + (size_t)unit_pb(j + 2 * kWaves) * blk_stride, saddr0 + (u32)(it & 1) * kTileB, offK);
     sv = row_max16(sv);                          // over the tokens of this head
     sv = fmaxf(sv, __shfl_xor(sv, 16, 64));      // over the 4 heads of the group
     sv = fmaxf(sv, __shfl_xor(sv, 32, 64));
@@ -337,56 +348,55 @@ __device__ __forceinline__ float key_to_float(unsigned k) {
   return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
 }
 
-// Two order statistics in one sweep, by a whole 256-thread workgroup: out[0] = the r0-th largest
+constexpr int kResolveThreads = 1024;  // 16 wavefronts: the undecided blocks are re-scored one per wavefront
+
+// Two order statistics in one sweep, by the whole workgroup (kResolveThreads threads): out[0] = the r0-th largest
 // (r = 1 is the maximum) of v[j] - e[j] and out[1] = the r1-th largest of v[j] + e[j], j < n.  Radix
-// selection over order-preserving integer keys, 4 passes of 8 bits; wavefront w < 2 scans the
-// histogram of selection w.  hist: 2 x 256 ints, sel: 2 x 2 unsigneds of shared memory.
+// selection over order-preserving integer keys, 4 passes of 8 bits.  Every pass has its own pair of
+// histograms (hist: 4 x 2 x 256 ints, zeroed by the caller before its last barrier) and its own result
+// slots (sel: 4 x 4 unsigneds), so a pass costs two barriers: count, then wavefront w < 2 scans histogram w
+// - 4 bins per lane, one 64-lane prefix sum - for the bin where the count from the top reaches the rank.
 __device__ void radix_select2_desc(const float* v, const float* e, int n, int r0, int r1, int* hist, unsigned* sel,
                                    float* out) {
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   unsigned prefix[2] = {0u, 0u}, mask = 0;
   int remaining[2] = {r0, r1};
-  for (int shift = 24; shift >= 0; shift -= 8) {
-    hist[tid] = 0;
-    hist[256 + tid] = 0;
-    __syncthreads();
-    for (int j = tid; j < n; j += 256) {
+  for (int pass = 0; pass < 4; ++pass) {
+    const int shift = 24 - 8 * pass;
+    int* hp = hist + 512 * pass;
+    for (int j = tid; j < n; j += kResolveThreads) {
       const unsigned k0 = order_key(v[j] - e[j]), k1 = order_key(v[j] + e[j]);
-      if ((k0 & mask) == prefix[0]) atomicAdd(&hist[(k0 >> shift) & 255u], 1);
-      if ((k1 & mask) == prefix[1]) atomicAdd(&hist[256 + ((k1 >> shift) & 255u)], 1);
+      if ((k0 & mask) == prefix[0]) atomicAdd(&hp[(k0 >> shift) & 255u], 1);
+      if ((k1 & mask) == prefix[1]) atomicAdd(&hp[256 + ((k1 >> shift) & 255u)], 1);
     }
     __syncthreads();
     if (wv < 2) {
-      // bins 255 .. 0 in 4 groups of 64: find the bin where the count from the top reaches `remaining`
-      const int* hs = hist + 256 * wv;
-      int rem = remaining[wv], found = -1;
-      for (int grp = 3; grp >= 0 && found < 0; --grp) {
-        const int bin = grp * 64 + (63 - lane);  // lane 0 holds the highest bin of the group
-        const int c = hs[bin];
-        int incl = c;
+      // lane l owns bins 255-4l .. 252-4l (descending); c[i] = their counts
+      const int4 c4 = *reinterpret_cast<const int4*>(hp + 256 * wv + 252 - 4 * lane);  // bins 252-4l .. 255-4l
+      const int c[4] = {c4.w, c4.z, c4.y, c4.x};
+      const int mine = (c[0] + c[1]) + (c[2] + c[3]);
+      int incl = mine;
 #pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-          const int t = __shfl_up(incl, o, 64);
-          if (lane >= o) incl += t;
-        }
-        const unsigned long long hit = __ballot(incl >= rem);
-        if (hit) {
-          const int l = __ffsll((long long)hit) - 1;
-          found = grp * 64 + (63 - l);
-          rem -= __shfl(incl - c, l, 64);
-        } else {
-          rem -= __shfl(incl, 63, 64);
-        }
+      for (int o = 1; o < 64; o <<= 1) {
+        const int t = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += t;
       }
-      if (lane == 0) { sel[2 * wv] = (unsigned)found; sel[2 * wv + 1] = (unsigned)rem; }
+      const int rem = remaining[wv];
+      const unsigned long long hit = __ballot(incl >= rem);  // never empty: the candidates number at least rem
+      const int l = __ffsll((long long)hit) - 1;
+      if (lane == l) {
+        int before = incl - mine, i = 0;
+        while (i < 3 && before + c[i] < rem) before += c[i++];
+        sel[4 * pass + 2 * wv] = (unsigned)(255 - 4 * l - i);
+        sel[4 * pass + 2 * wv + 1] = (unsigned)(rem - before);
+      }
     }
     __syncthreads();
-    prefix[0] |= sel[0] << shift;
-    prefix[1] |= sel[2] << shift;
+    prefix[0] |= sel[4 * pass] << shift;
+    prefix[1] |= sel[4 * pass + 2] << shift;
     mask |= 255u << shift;
-    remaining[0] = (int)sel[1];
-    remaining[1] = (int)sel[3];
-    __syncthreads();
+    remaining[0] = (int)sel[4 * pass + 1];
+    remaining[1] = (int)sel[4 * pass + 3];
   }
   out[0] = key_to_float(prefix[0]);
   out[1] = key_to_float(prefix[1]);
@@ -394,40 +404,51 @@ __device__ void radix_select2_desc(const float* v, const float* e, int n, int r0
 
 // One workgroup per (sequence, KV head): classify, re-score the undecided blocks in fp64, emit.
 template <int QUANT>
-__global__ __launch_bounds__(256) void sqattn_resolve_kernel(SelArgs a) {
+__global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs a) {
   extern __shared__ double smd[];                  // exact scores of undecided blocks [max_blocks]
   float* sf = reinterpret_cast<float*>(smd + a.max_blocks);      // approx scores [max_blocks]
   float* se = sf + a.max_blocks;                                  // error bounds [max_blocks]
   int* state = reinterpret_cast<int*>(se + a.max_blocks);         // 0 dropped, 1 kept, 2 undecided
   int* ulist = state + a.max_blocks;                              // undecided block ids
+  int* tbl = ulist + a.max_blocks;                                // this sequence's block table row
   __shared__ float qs[kG][kD];
-  __shared__ int n_in, n_unc, wave_tot[4], running;
-  __shared__ int hist[512];
-  __shared__ unsigned sel[4];
+  __shared__ int n_in, n_unc, wave_tot[kResolveThreads / 64], running;
+  __shared__ __attribute__((aligned(16))) int hist[4 * 512];
+  __shared__ unsigned sel[16];
   const int p = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int b = p / a.hkv, h = p - b * a.hkv;
+  // Everything the kernel will need from memory is requested here, in one round trip: the scores and
+  // their bounds, the table row and q * k_scale of the re-scoring step (needed only if a block stays
+  // undecided, but a second and third trip would cost more than these few KB).
+  const float* s = a.approx + (size_t)p * a.max_blocks;
+  const float* eb = a.ebound ? a.ebound + (size_t)p * a.max_blocks : nullptr;
+  const float eps = a.eps[p];
+  for (int j = tid; j < a.max_blocks; j += kResolveThreads) {
+    sf[j] = s[j];
+    se[j] = eb ? eb[j] : eps;
+    tbl[j] = a.block_tables[(size_t)b * a.max_blocks + j];
+  }
+  for (int i = tid; i < kG * kD; i += kResolveThreads) {
+    const int g = i / kD, c = i % kD;
+    qs[g][c] = __fmul_rn(bf16_to_f32(a.q[((size_t)b * a.hkv * kG + h * kG + g) * kD + c]), a.k_scale[h * kD + c]);
+  }
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
   const int nblk = min((max(kv_len, 0) + kBS - 1) / kBS, a.max_blocks);
   const int k = min(a.top_k, nblk);
   int32_t* out = a.kept_blocks + (size_t)p * a.top_k;
   if (tid == 0) { n_in = 0; n_unc = 0; running = 0; }
-  const float* s = a.approx + (size_t)p * a.max_blocks;
-  for (int j = tid; j < nblk; j += 256) sf[j] = s[j];
+  for (int i = tid; i < 4 * 512; i += kResolveThreads) hist[i] = 0;
   __syncthreads();
   if (k < nblk) {
     // With score i known to within e_i (L_i = s_i - e_i, U_i = s_i + e_i): block j is surely kept if
     // L_j > the (k+1)-th largest U (then at most k blocks, itself included, can reach it) and surely
     // dropped if U_j < the k-th largest L (then k blocks beat it for certain); the rest is undecided.
-    const float eps = a.eps[p];
-    const float* eb = a.ebound ? a.ebound + (size_t)p * a.max_blocks : nullptr;
-    for (int j = tid; j < nblk; j += 256) se[j] = eb ? eb[j] : eps;
-    __syncthreads();
     // k-th largest lower bound and (k+1)-th largest upper bound by radix selection, both in the same
     // four passes - not by ranking every block against every other
     float both[2];
     radix_select2_desc(sf, se, nblk, k, k + 1, hist, sel, both);
     const float lk = both[0], uk1 = both[1];
-    for (int j = tid; j < nblk; j += 256) {
+    for (int j = tid; j < nblk; j += kResolveThreads) {
       const float lj = sf[j] - se[j], uj = sf[j] + se[j];
       int stt = 2;
       if (lj > uk1) stt = 1;
@@ -439,15 +460,10 @@ __global__ __launch_bounds__(256) void sqattn_resolve_kernel(SelArgs a) {
     __syncthreads();
     const int nu = n_unc, need = k - n_in;
     if (nu > 0) {
-      for (int i = tid; i < kG * kD; i += 256) {
-        const int g = i / kD, c = i % kD;
-        qs[g][c] = __fmul_rn(bf16_to_f32(a.q[((size_t)b * a.hkv * kG + h * kG + g) * kD + c]), a.k_scale[h * kD + c]);
-      }
-      __syncthreads();
       // exact score of each undecided block: fp64, channels in ascending order, lane = token
-      for (int u = wv; u < nu; u += 4) {
+      for (int u = wv; u < nu; u += kResolveThreads / 64) {
         const int j = ulist[u];
-        const int pb = a.block_tables[(size_t)b * a.max_blocks + j];
+        const int pb = tbl[j];
         double best = -INFINITY;
         if (pb >= 0 && pb < a.num_blocks && j * kBS + lane < kv_len) {
           const uint8_t* kr = a.key_cache + (((size_t)pb * a.hkv + h) * kBS + lane) * kD;
@@ -471,7 +487,7 @@ __global__ __launch_bounds__(256) void sqattn_resolve_kernel(SelArgs a) {
       }
       __syncthreads();
       // the `need` best undecided blocks: exact score descending, block index ascending
-      for (int u = tid; u < nu; u += 256) {
+      for (int u = tid; u < nu; u += kResolveThreads) {
         const double su = smd[u];
         const int ju = ulist[u];
         int rank = 0;
@@ -484,11 +500,11 @@ __global__ __launch_bounds__(256) void sqattn_resolve_kernel(SelArgs a) {
       __syncthreads();
     }
   } else {
-    for (int j = tid; j < nblk; j += 256) state[j] = 1;
+    for (int j = tid; j < nblk; j += kResolveThreads) state[j] = 1;
     __syncthreads();
   }
   // ordered compaction of the kept blocks
-  for (int base = 0; base < nblk; base += 256) {
+  for (int base = 0; base < nblk; base += kResolveThreads) {
     const int j = base + tid;
     const int f = j < nblk ? (state[j] == 1) : 0;
     const unsigned long long bal = __ballot(f);
@@ -499,15 +515,19 @@ __global__ __launch_bounds__(256) void sqattn_resolve_kernel(SelArgs a) {
     for (int ww = 0; ww < wv; ++ww) off += wave_tot[ww];
     if (f && off + before < a.top_k) out[off + before] = j;
     __syncthreads();
-    if (tid == 0) running += wave_tot[0] + wave_tot[1] + wave_tot[2] + wave_tot[3];
+    if (tid == 0) {
+      int tot = 0;
+      for (int ww = 0; ww < kResolveThreads / 64; ++ww) tot += wave_tot[ww];
+      running += tot;
+    }
     __syncthreads();
   }
-  for (int j = k + tid; j < a.top_k; j += 256) out[j] = -1;
+  for (int j = k + tid; j < a.top_k; j += kResolveThreads) out[j] = -1;
   if (tid == 0) a.kept_counts[p] = k;
 }
 
 static bool sel_fast_supported(int hq, int hkv, int d, int bs, int max_blocks) {
-  return d == kD && hq == kG * hkv && bs == kBS && max_blocks <= 2048;  // 24 B of LDS per block in the top-k kernel
+  return d == kD && hq == kG * hkv && bs == kBS && max_blocks <= 2048;  // 28 B of LDS per block in the resolve kernel
 }
 
 }  // namespace fdattn
@@ -544,8 +564,7 @@ static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_ca
   hipStream_t s = (hipStream_t)stream;
   if (allow_fast && sel_fast_supported(hq, hkv, head_dim, block_size, max_blocks_per_seq)) {
     const int pairs = batch * hkv;
-    int chunk = 64;
-    while (chunk > 4 && (long long)pairs * ((max_blocks_per_seq + chunk - 1) / chunk) < 1024) chunk /= 2;
+    const int chunk = c8_pick_chunk(pairs, max_blocks_per_seq);
     const int cpp = (max_blocks_per_seq + chunk - 1) / chunk;
     float* approx = (float*)workspace;
     float* ebound = approx + (size_t)pairs * max_blocks_per_seq;
@@ -553,13 +572,13 @@ static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_ca
     SelArgs sa{(const uint16_t*)q, (const uint8_t*)key_cache, cache_k_scale, block_tables, seq_lens_decoder,
                seq_lens_this_time, approx, eps, cache_quant_type == FDATTN_CACHE_INT8 ? nullptr : ebound, scores, kept_blocks, kept_counts, batch, hkv,
                max_blocks_per_seq, num_blocks, chunk, cpp, top_k};
-    const size_t shm2 = (size_t)max_blocks_per_seq * (sizeof(double) + 2 * sizeof(float) + 2 * sizeof(int));
+    const size_t shm2 = (size_t)max_blocks_per_seq * (sizeof(double) + 2 * sizeof(float) + 3 * sizeof(int));
     if (cache_quant_type == FDATTN_CACHE_INT8) {
       hipLaunchKernelGGL(sqattn_scores_mfma_kernel<FDATTN_CACHE_INT8>, dim3(pairs * cpp), dim3(256), 0, s, sa);
-      hipLaunchKernelGGL(sqattn_resolve_kernel<FDATTN_CACHE_INT8>, dim3(pairs), dim3(256), shm2, s, sa);
+      hipLaunchKernelGGL(sqattn_resolve_kernel<FDATTN_CACHE_INT8>, dim3(pairs), dim3(kResolveThreads), shm2, s, sa);
     } else {
       hipLaunchKernelGGL(sqattn_scores_mfma_kernel<FDATTN_CACHE_FP8_E4M3>, dim3(pairs * cpp), dim3(256), 0, s, sa);
-      hipLaunchKernelGGL(sqattn_resolve_kernel<FDATTN_CACHE_FP8_E4M3>, dim3(pairs), dim3(256), shm2, s, sa);
+      hipLaunchKernelGGL(sqattn_resolve_kernel<FDATTN_CACHE_FP8_E4M3>, dim3(pairs), dim3(kResolveThreads), shm2, s, sa);
     }
     return check_launch("fdattn_sqattn_select (mfma)");
   }

@@ -160,6 +160,13 @@ FDATTN_API int fdattn_decode_attention(
 FDATTN_API int fdattn_decode_uses_mfma(int hq, int hkv, int head_dim, int block_size, int cache_quant_type);
 
 /*
+ * Into how many chunks the MFMA decode kernel cuts the block list of one (sequence, KV head)
+ * for a launch of this size: as few as give every workgroup slot of the GPU one chunk.  1 means
+ * that every list is finished by the main kernel and no merge kernel is launched.
+ */
+FDATTN_API int fdattn_decode_chunks_per_sequence(int batch, int hkv, int max_blocks_per_seq);
+
+/*
  * fdattn_decode_attention split into its two kernels, for profiling and for callers
  * that overlap other work with the merge: stages = 1 runs only the split-KV kernel
  * (partials into `workspace`; sequences that fit one chunk are finished by it), 2 only
