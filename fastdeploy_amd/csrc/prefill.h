@@ -19,6 +19,7 @@ struct PrefillArgs {
   uint16_t* out;
   int num_tokens, batch, hq, hkv, d, bs, max_blocks, num_blocks;
   float sm_scale;
+  int q_tiles;  // MFMA kernel: workgroups per (sequence, query head), set by its launcher
 };
 
 bool prefill_mfma_supported(int hq, int hkv, int d, int bs, int quant);

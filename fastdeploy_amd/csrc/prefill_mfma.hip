@@ -133,9 +133,28 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];  // [kSlots][K tile | V tile]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // in a scalar register: what depends on it stays uniform
-  const int b = blockIdx.z, qh = blockIdx.y, h = qh / (a.hq / a.hkv);
+  // Workgroup -> (sequence, query head, query tile).  The hardware deals workgroups to the 8 XCDs in
+  // turn (workgroup i to XCD i % 8), each with its own L2.  So: the XCD index picks the (sequence, KV
+  // head) pair - every workgroup that reads one pair's K and V shares one L2 - and inside an XCD the
+  // query tiles come longest first (the causal rows of late tokens walk more keys), so every XCD gets
+  // the same mix of long and short workgroups and the short ones fill the end of the launch.
+  const int G = a.hq / a.hkv, pairs = a.batch * a.hkv, units = a.batch * a.hq;
+  int qt, b, qh;
+  if ((pairs & 7) == 0) {
+    const int ppx = pairs >> 3;  // pairs per XCD
+    const int x = blockIdx.x & 7, jx = blockIdx.x >> 3;
+    const int r = jx % (ppx * G), pk = (r / G) * 8 + x;
+    qt = a.q_tiles - 1 - jx / (ppx * G);
+    b = pk / a.hkv;
+    qh = (pk - b * a.hkv) * G + r % G;
+  } else {  // no whole number of pairs per XCD: query heads in turn, still longest tiles first
+    const int u = blockIdx.x % units;
+    qt = a.q_tiles - 1 - blockIdx.x / units;
+    b = u / a.hq;
+    qh = u - b * a.hq;
+  }
+  const int h = qh / G;
   const int tok0 = a.cu_seqlens_q[b], n_b = a.cu_seqlens_q[b + 1] - tok0, p = a.seq_lens_decoder[b];
-  const int qt = (int)gridDim.x - 1 - (int)blockIdx.x;  // long rows (late tokens) first
   const int q0 = qt * BM;
   if (q0 >= n_b) return;
   if (a.seq_lens_encoder && a.seq_lens_encoder[b] <= 0) return;  // a decode row or an idle slot of a mixed batch
@@ -435,7 +454,9 @@ namespace {
 template <int QUANT, int NW>
 hipError_t launch_one(const PrefillArgs& a, int max_chunk, hipStream_t s) {
   constexpr int BM = 32 * NW;
-  const dim3 grid((max_chunk + BM - 1) / BM, a.hq, a.batch), block(64 * NW);
+  PrefillArgs args = a;
+  args.q_tiles = (max_chunk + BM - 1) / BM;
+  const dim3 grid((unsigned)a.batch * a.hq * args.q_tiles), block(64 * NW);
   const size_t shm = (size_t)kSlots * BUF_ELEMS * sizeof(uint16_t);  // 151,552 B
   // the dynamic LDS limit is a per-device property of the kernel: raise it once on each device
   static std::atomic<unsigned long long> raised{0};  // bit d: done on device d (one word per instantiation)
@@ -448,15 +469,15 @@ hipError_t launch_one(const PrefillArgs& a, int max_chunk, hipStream_t s) {
     if (e != hipSuccess) return e;
     if (dev < 64) raised.fetch_or(1ull << dev, std::memory_order_relaxed);
   }
-  hipLaunchKernelGGL((prefill_mfma_kernel<QUANT, NW>), grid, block, shm, s, a);
+  hipLaunchKernelGGL((prefill_mfma_kernel<QUANT, NW>), grid, block, shm, s, args);
   return hipSuccess;
 }
 
 }  // namespace
 
 int prefill_mfma_launch(const PrefillArgs& a, int max_chunk, int quant, hipStream_t s) {
-  if (a.batch > 65535 || a.hq > 65535)
-    return fail(FDATTN_ERR_SHAPE, "fdattn_append_attention_prefill: batch or head count exceeds the grid limit");
+  if ((long long)a.batch * a.hq * ((max_chunk + 127) / 128) > 0x7fffffffLL)
+    return fail(FDATTN_ERR_SHAPE, "fdattn_append_attention_prefill: too many workgroups for one launch");
   // 256-token workgroups share each staged tile among 8 wavefronts; short chunks keep 128
   const bool wide = max_chunk > 128;
   hipError_t e;
