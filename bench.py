@@ -27,7 +27,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes of one decode_c8_kernel launch on this workload, from the TCC counters
 # (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB copy: summary in
 # profiles/decode_c8_kernel_configs1_b64_ctx4k.md); it cannot be measured from inside this script.
-MEASURED_TRAFFIC_BYTES = 527_798_000 + 3_195_000
+MEASURED_TRAFFIC_BYTES = 526_724_000 + 524_000
 
 
 def time_events(fn, steps, warmup):
