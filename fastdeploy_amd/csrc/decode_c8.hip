@@ -379,13 +379,13 @@ __global__ __launch_bounds__(256) void decode_c8_combine_kernel(C8Args a) {
 // for as long as possible and - when one chunk covers the pair - finish it without a partial or a
 // merge.  Lists too long for the unit table (kMaxChunk entries) get more chunks; short lists keep at
 // least one unit per wavefront.
-static int gpu_slots() {
-  static int slots = 0;  // benign race: every thread computes the same value
+int gpu_cu_count() {
+  static int slots = 0;  // CUs of the current device; benign race: every thread computes the same value
   if (slots == 0) {
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
       cus = 256;
-    slots = 2 * cus;
+    slots = cus;
   }
   return slots;
 }
@@ -394,7 +394,7 @@ int c8_pick_chunk(int pairs, int max_units) {
 #ifdef FDATTN_FORCE_CHUNK
   return FDATTN_FORCE_CHUNK;
 #endif
-  const int cpp = (gpu_slots() + pairs - 1) / pairs;
+  const int cpp = (2 * gpu_cu_count() + pairs - 1) / pairs;  // two workgroups of this kernel fit a CU
   int chunk = (max_units + cpp - 1) / cpp;
   if (chunk < kWaves) chunk = kWaves;
   if (chunk > kMaxChunk) chunk = kMaxChunk;

@@ -12,6 +12,8 @@ int decode_generic_launch(const void* q, const void* key_cache, const void* valu
                           void* out, void* workspace, size_t workspace_bytes, int batch, int hq,
                           int hkv, int d, int bs, int max_blocks, int num_blocks, int quant,
                           float sm_scale, hipStream_t s, RowMap rows = RowMap{nullptr, nullptr});
+// compute units of the current device (256 on MI355X; that value if the query fails)
+int gpu_cu_count();
 // units (cache blocks) per workgroup for `pairs` block lists of at most max_units blocks: as few chunks per
 // list as fill the GPU's workgroup slots once, at most kMaxChunk units each
 int c8_pick_chunk(int pairs, int max_units);

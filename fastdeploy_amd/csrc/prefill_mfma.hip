@@ -45,6 +45,7 @@
 #include <atomic>
 
 #include "prefill.h"
+#include "launch.h"
 
 namespace fdattn {
 
@@ -478,8 +479,11 @@ hipError_t launch_one(const PrefillArgs& a, int max_chunk, hipStream_t s) {
 int prefill_mfma_launch(const PrefillArgs& a, int max_chunk, int quant, hipStream_t s) {
   if ((long long)a.batch * a.hq * ((max_chunk + 127) / 128) > 0x7fffffffLL)
     return fail(FDATTN_ERR_SHAPE, "fdattn_append_attention_prefill: too many workgroups for one launch");
-  // 256-token workgroups share each staged tile among 8 wavefronts; short chunks keep 128
-  const bool wide = max_chunk > 128;
+  // 256-token workgroups share each staged tile among 8 wavefronts (their two groups alternate between the MFMA
+  // units and the vector ALU); short chunks keep 128
+  // when they would still leave CUs without a workgroup (one fits a CU), 128-token workgroups cover twice as
+  // many CUs: 10-14 % faster at e.g. 2 x 512 tokens, although a 4-wavefront workgroup overlaps nothing
+  const bool wide = max_chunk > 128 && (long long)a.batch * a.hq * ((max_chunk + 255) / 256) >= gpu_cu_count();
   hipError_t e;
   if (quant == FDATTN_CACHE_INT8)
     e = wide ? launch_one<FDATTN_CACHE_INT8, 8>(a, max_chunk, s) : launch_one<FDATTN_CACHE_INT8, 4>(a, max_chunk, s);
