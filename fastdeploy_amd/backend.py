@@ -112,7 +112,9 @@ class SequenceBook:
     """Host-side bookkeeping of the sequence slots between steps: lengths, the block pool, and the
     ForwardMeta of the next step.  `schedule` takes the new tokens per slot ({slot: count}) - a count
     above one, or any count for an empty slot, makes a prefill row - reserves blocks and returns the meta;
-    `commit` advances the lengths after the step has been enqueued."""
+    `commit` advances the lengths after the step has been enqueued.  A reservation that fails (ValueError: the
+    pool is exhausted or a table row is full) leaves the slots reserved earlier in the same call with their
+    blocks: finish a sequence or retry with fewer tokens."""
 
     def __init__(self, pool: BlockPool, device="cuda"):
         self.pool, self.device = pool, device

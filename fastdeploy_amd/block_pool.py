@@ -68,7 +68,13 @@ class BlockPool:
 
     @property
     def block_tables(self):
-        """The live table (numpy int32, read-only view); copy before the pool changes or closes."""
+        """A copy of the table as it is now (numpy int32 [max_seqs, max_blocks_per_seq], -1 = no block)."""
+        self._handle()
+        return np.array(self._table)
+
+    def block_tables_view(self):
+        """The pool's own table, read-only and live: it changes with reserve / release / fork and must not
+        be touched after close()."""
         self._handle()
         return self._table
 

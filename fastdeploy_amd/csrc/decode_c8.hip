@@ -31,6 +31,8 @@
 // (the last workgroup to arrive at a pair combines it: the device-scope stores, the atomic
 // and the barrier sit at the end of every workgroup, where nothing hides their latency),
 // and handing chunks out through an atomic ticket counter instead of the block index.
+#include <atomic>
+
 #include "c8_common.h"
 
 
@@ -380,14 +382,15 @@ __global__ __launch_bounds__(256) void decode_c8_combine_kernel(C8Args a) {
 // merge.  Lists too long for the unit table (kMaxChunk entries) get more chunks; short lists keep at
 // least one unit per wavefront.
 int gpu_cu_count() {
-  static int slots = 0;  // CUs of the current device; benign race: every thread computes the same value
-  if (slots == 0) {
-    int dev = 0, cus = 0;
+  static std::atomic<int> cached{0};  // CUs of the current device (the devices of one machine are alike)
+  int cus = cached.load(std::memory_order_relaxed);
+  if (cus == 0) {
+    int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
       cus = 256;
-    slots = cus;
+    cached.store(cus, std::memory_order_relaxed);
   }
-  return slots;
+  return cus;
 }
 
 int c8_pick_chunk(int pairs, int max_units) {
