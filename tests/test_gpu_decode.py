@@ -179,6 +179,24 @@ def test_decode_config2_full_size(oracle):
     check(bits(out3), bits(out), "dense vs keep-all sparse")
 
 
+@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+def test_decode_launch_shapes(oracle, quant):
+    """The chunking follows the launch size (as few chunks per block list as fill the GPU's workgroup slots):
+    long lists in a small batch are cut into several chunks of more than 64 units (second unit-table entry
+    of a lane, partials, merge kernel), a single sequence into many short chunks, a large batch into one
+    chunk per list.  Every shape against the oracle."""
+    from fastdeploy_amd import _lib
+    for batch, ctx, cpp in ((16, [20000 - 37 * i for i in range(16)], 4), (1, 64 * 300 - 11, 60), (70, 64 * 9 + 1, 1)):
+        mb = (max(ctx) if isinstance(ctx, list) else ctx) // 64 + 1
+        assert _lib.lib().fdattn_decode_chunks_per_sequence(batch, 8, mb) == cpp
+        case = syn.decode_case(batch=batch, ctx=ctx, quant=quant, seed=batch, device="cuda", max_blocks=mb)
+        out = fd.decode_attention(case["q"], case["key_cache"], case["value_cache"], case["cache_k_scale"],
+                                  case["cache_v_scale"], case["block_tables"], case["seq_lens_decoder"], num_heads=32,
+                                  cache_quant_type=quant)
+        torch.cuda.synchronize()
+        check(bits(out), oracle_decode(oracle, syn.to_device(case, "cpu")), "batch %d" % batch)
+
+
 def test_write_then_decode_config3_full_size(oracle):
     """256 new tokens (bf16 qkv ~ N(0,1)), RoPE theta 500000 at positions U{0..8191}, int8 write into the
     block-tabled slots, then decode over ctx = pos + 1: cache bytes bit-exact, outputs within tolerance."""
