@@ -77,6 +77,21 @@ def other_workloads(args):
         ms = time_events(wr, args.steps, args.warmup)
         line("configs[2] cache write (256 tokens, RoPE + int8)", ms, "hbm", 256 * (48 * 128 * 2 + 2 * 8 * 128 + 32 * 128 * 2),
              HBM_PEAK_GBPS, "GB/s", {"note": "5.8 MB of traffic: launch-bound"})
+        # the same kernel at prefill size: 2 sequences x 2048 new tokens behind 8192 cached ones (configs[4]'s write),
+        # with the rotated K and the V handed on for the append attention - large enough to be HBM-bound
+        cw = syn.write_case(num_seqs=2, max_pos=8192 + 2048, seed=1, device=dev, chunk=2048, blocks_per_seq=160)
+        cw["seq_lens_decoder"].fill_(8192)
+        rotw = (cw["rope_cos"], cw["rope_sin"])
+
+        def wr_big():
+            return fd.write_cache_kv(cw["qkv"], cw["key_cache"], cw["value_cache"], cw["cache_k_scale"], cw["cache_v_scale"],
+                                     cw["block_tables"], cw["seq_lens_encoder"], cw["seq_lens_decoder"], cw["seq_lens_this_time"],
+                                     cw["cu_seqlens_q"], rotw, num_heads=32, kv_num_heads=8, want_kv_out=True)
+        ms = time_events(wr_big, args.steps, args.warmup)
+        # per token: qkv read 48*128*2, q/k/v out (32+8+8)*128*2, cache bytes 2*8*128, cos/sin 2*64*4
+        line("configs[4] cache write (4096 tokens, RoPE + int8, q/k/v handed on)", ms, "hbm",
+             4096 * (48 * 128 * 2 * 2 + 2 * 8 * 128 + 2 * 64 * 4), HBM_PEAK_GBPS, "GB/s")
+        del cw
         lens = (c["seq_lens_decoder"] + 1).tolist()
 
         def dec():
