@@ -31,6 +31,7 @@ struct WriterArgs {
   const float* q_norm_weight;   // [d]: RMS norm of every Q head before the rotation
   const float* k_norm_weight;   // [d]: the same for K
   float rms_norm_eps;
+  int tok0;  // first token of this launch (the grid's y dimension holds 65,535)
 };
 
 template <int QUANT>
@@ -52,14 +53,14 @@ __device__ __forceinline__ u32 quant1(float x, float s) {
 //   heads [hq+hkv, hq+2hkv)  V   : (copy -> v_out), quantise, store to value_cache
 template <int QUANT>
 __global__ __launch_bounds__(256) void write_cache_kv_kernel(WriterArgs a) {
+  // grid (units of a token / 256, tokens): the token - and with it the sequence, the position and the
+  // cache slot - is uniform over the workgroup and is worked out in scalar registers
   const int units_per_head = a.d / 16;
   const int heads = a.hq + 2 * a.hkv;
-  const long long total = (long long)a.num_tokens * heads * units_per_head;
-  long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (gid >= total) return;
-  const int u = (int)(gid % units_per_head);
-  const int head = (int)((gid / units_per_head) % heads);
-  const int tok = (int)(gid / ((long long)units_per_head * heads));
+  const int unit = blockIdx.x * blockDim.x + threadIdx.x;
+  if (unit >= heads * units_per_head) return;
+  const int head = unit / units_per_head, u = unit - head * units_per_head;
+  const int tok = a.tok0 + blockIdx.y;
 
   // sequence of this token: last b with cu_seqlens_q[b] <= tok
   int lo = 0, hi = a.batch;
@@ -295,13 +296,17 @@ extern "C" int fdattn_write_cache_kv_ex(
                (uint8_t*)key_cache, (uint8_t*)value_cache, cache_k_scale, cache_v_scale, rope_cos,
                rope_sin, block_tables, seq_lens_decoder, cu_seqlens_q, num_tokens, batch, hq, hkv,
                head_dim, block_size, max_blocks_per_seq, num_blocks, max_pos, rope_style,
-               (const uint16_t*)ep.qkv_bias, ep.q_norm_weight, ep.k_norm_weight, ep.rms_norm_eps};
-  long long total = (long long)num_tokens * (hq + 2 * hkv) * (head_dim / 16);
-  unsigned grid = (unsigned)((total + 255) / 256);
+               (const uint16_t*)ep.qkv_bias, ep.q_norm_weight, ep.k_norm_weight, ep.rms_norm_eps, 0};
+  const int units = (hq + 2 * hkv) * (head_dim / 16);
   hipStream_t s = (hipStream_t)stream;
-  if (cache_quant_type == FDATTN_CACHE_INT8)
-    hipLaunchKernelGGL(write_cache_kv_kernel<FDATTN_CACHE_INT8>, dim3(grid), dim3(256), 0, s, a);
-  else
-    hipLaunchKernelGGL(write_cache_kv_kernel<FDATTN_CACHE_FP8_E4M3>, dim3(grid), dim3(256), 0, s, a);
+  // the y dimension of a grid holds 65,535 workgroups: more tokens go in slices
+  for (int t0 = 0; t0 < num_tokens; t0 += 65535) {
+    a.tok0 = t0;
+    const dim3 grid((units + 255) / 256, num_tokens - t0 < 65535 ? num_tokens - t0 : 65535);
+    if (cache_quant_type == FDATTN_CACHE_INT8)
+      hipLaunchKernelGGL(write_cache_kv_kernel<FDATTN_CACHE_INT8>, grid, dim3(256), 0, s, a);
+    else
+      hipLaunchKernelGGL(write_cache_kv_kernel<FDATTN_CACHE_FP8_E4M3>, grid, dim3(256), 0, s, a);
+  }
   return check_launch("fdattn_write_cache_kv");
 }
