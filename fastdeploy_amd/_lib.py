@@ -28,6 +28,10 @@ SIGNATURES = {
     "fdattn_append_attention_prefill_generic": (_i, [_vp] * 11 + [_i] * 10 + [_f, _vp]),
     "fdattn_append_attention_workspace_bytes": (_sz, [_i] * 6),
     "fdattn_append_attention": (_i, [_vp] * 14 + [_sz] + [_i] * 12 + [_f, _vp]),
+    "fdattn_prefill_auto_splits": (_i, [_i] * 3),
+    "fdattn_append_attention_prefill_split_workspace_bytes": (_sz, [_i] * 3),
+    "fdattn_append_attention_prefill_split": (_i, [_vp] * 12 + [_sz] + [_i] * 11 + [_f, _vp]),
+    "fdattn_append_attention_workspace_bytes_ex": (_sz, [_i] * 7),
     "fdattn_write_cache_kv_ex": (_i, [_vp] * 13 + [_i] * 11 + [_vp, _vp]),
     "fdattn_append_attention_ex": (_i, [_vp] * 14 + [_sz] + [_i] * 12 + [_f, _vp, _vp]),
     "fdattn_pool_create": (_vp, [_i] * 4),
@@ -46,9 +50,10 @@ SIGNATURES = {
 
 
 
-class QkvEpilogue(ctypes.Structure):
-    """fdattn_qkv_epilogue of include/fdattn.h"""
-    _fields_ = [("qkv_bias", _vp), ("q_norm_weight", _vp), ("k_norm_weight", _vp), ("rms_norm_eps", _f)]
+class StepExtras(ctypes.Structure):
+    """fdattn_step_extras of include/fdattn.h"""
+    _fields_ = [("qkv_bias", _vp), ("q_norm_weight", _vp), ("k_norm_weight", _vp), ("rms_norm_eps", _f),
+                ("prefill_rows", _i)]
 
 
 _lib = None

@@ -38,6 +38,8 @@ class ForwardMeta:
     max_enc_len_this_time: Optional[int] = None  # host-side bound on seq_lens_encoder (0: no prefill row); found with one sync if None
     cu_seqlens_q: Optional[torch.Tensor] = None  # filled by init_attention_metadata
     num_tokens: int = 0                          # filled by init_attention_metadata
+    prefill_rows: Optional[int] = None           # host-side count of prefill rows (None: unknown, no key splits)
+    prefill_splits: int = 1                      # filled by init_attention_metadata
     extra: dict = field(default_factory=dict)
 
 
@@ -86,8 +88,12 @@ class AppendAttentionBackend:
             meta.num_tokens, meta.max_enc_len_this_time = int(both[0]), max(int(both[1]), 0)
         elif meta.num_tokens <= 0:
             meta.num_tokens = int(meta.cu_seqlens_q[-1])
+        # a step whose few prefill rows would leave CUs idle shares every query tile's keys among several workgroups
+        meta.prefill_splits = 1
+        if meta.prefill_rows and meta.max_enc_len_this_time > 0:
+            meta.prefill_splits = ops.prefill_auto_splits(meta.prefill_rows, self.num_heads, meta.max_enc_len_this_time)
         need = ops.append_attention_workspace_bytes(meta.num_tokens, slots, self.num_heads, self.kv_num_heads,
-                                                    self.head_dim, meta.block_tables.shape[1])
+                                                    self.head_dim, meta.block_tables.shape[1], meta.prefill_splits)
         if self._workspace is None or self._workspace.numel() < need:
             self._workspace = torch.empty(need, dtype=torch.uint8, device=self.device)
         return meta
@@ -105,7 +111,8 @@ class AppendAttentionBackend:
             num_heads=self.num_heads, kv_num_heads=self.kv_num_heads, max_chunk=meta.max_enc_len_this_time,
             rope_style=self.rope_style, cache_quant_type=self.cache_quant_type, softmax_scale=self.softmax_scale,
             cu_seqlens_q=meta.cu_seqlens_q, workspace=self._workspace, out=out, qkv_bias=layer.qkv_bias,
-            q_norm_weight=layer.q_norm_weight, k_norm_weight=layer.k_norm_weight, rms_norm_eps=layer.rms_norm_eps)
+            q_norm_weight=layer.q_norm_weight, k_norm_weight=layer.k_norm_weight, rms_norm_eps=layer.rms_norm_eps,
+            prefill_rows=meta.prefill_rows)
 
 
 class SequenceBook:
@@ -134,7 +141,8 @@ class SequenceBook:
         i32 = lambda v: torch.tensor(v, dtype=torch.int32).to(self.device)
         self._pending = this
         return ForwardMeta(i32(enc), i32(dec), i32(this), self.pool.block_tables_tensor(self.device),
-                           max_enc_len_this_time=max(enc), num_tokens=sum(this))
+                           max_enc_len_this_time=max(enc), num_tokens=sum(this),
+                           prefill_rows=sum(1 for n in enc if n > 0))
 
     def commit(self):
         for s, n in enumerate(self._pending or []):

@@ -9,16 +9,17 @@ namespace fdattn {
 static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 
 struct StepWorkspace {
-  size_t q_rot, k_new, v_new, decode, total;  // byte offsets of the parts, and the sum
+  size_t q_rot, k_new, v_new, decode, split, total;  // byte offsets of the parts, and the sum
 };
 
-static StepWorkspace step_workspace(int num_tokens, int batch, int hq, int hkv, int d, int max_blocks) {
+static StepWorkspace step_workspace(int num_tokens, int batch, int hq, int hkv, int d, int max_blocks, int prefill_splits) {
   StepWorkspace w;
   w.q_rot = 0;
   w.k_new = w.q_rot + align256((size_t)num_tokens * hq * d * 2);
   w.v_new = w.k_new + align256((size_t)num_tokens * hkv * d * 2);
   w.decode = w.v_new + align256((size_t)num_tokens * hkv * d * 2);
-  w.total = w.decode + fdattn_decode_workspace_bytes(batch, hq, hkv, d, max_blocks);
+  w.split = w.decode + align256(fdattn_decode_workspace_bytes(batch, hq, hkv, d, max_blocks));
+  w.total = w.split + align256(prefill_split_workspace_bytes(num_tokens, hq, prefill_splits));
   return w;
 }
 
@@ -28,8 +29,13 @@ using namespace fdattn;
 
 extern "C" size_t fdattn_append_attention_workspace_bytes(int num_tokens, int batch, int hq, int hkv, int head_dim,
                                                           int max_blocks_per_seq) {
+  return fdattn_append_attention_workspace_bytes_ex(num_tokens, batch, hq, hkv, head_dim, max_blocks_per_seq, 1);
+}
+
+extern "C" size_t fdattn_append_attention_workspace_bytes_ex(int num_tokens, int batch, int hq, int hkv, int head_dim,
+                                                             int max_blocks_per_seq, int prefill_splits) {
   if (num_tokens < 0 || batch <= 0 || hq <= 0 || hkv <= 0 || head_dim <= 0 || max_blocks_per_seq <= 0) return 256;
-  return step_workspace(num_tokens, batch, hq, hkv, head_dim, max_blocks_per_seq).total;
+  return step_workspace(num_tokens, batch, hq, hkv, head_dim, max_blocks_per_seq, prefill_splits).total;
 }
 
 extern "C" int fdattn_append_attention(
@@ -53,7 +59,7 @@ extern "C" int fdattn_append_attention_ex(
     void* workspace, size_t workspace_bytes, int num_tokens, int batch, int max_chunk, int hq, int hkv,
     int head_dim, int block_size, int max_blocks_per_seq, int num_blocks, int max_pos, int rope_style,
     int cache_quant_type, float softmax_scale,
-    const fdattn_qkv_epilogue* epilogue, void* stream) {
+    const fdattn_step_extras* extras, void* stream) {
   if (!seq_lens_encoder || !seq_lens_this_time || !cu_seqlens_q || !out || !workspace)
     return fail(FDATTN_ERR_NULL, "fdattn_append_attention: a required pointer is NULL");
   if (num_tokens < 0 || batch <= 0 || max_chunk < 0 || hq <= 0 || hkv <= 0 || head_dim <= 0 ||
@@ -61,7 +67,12 @@ extern "C" int fdattn_append_attention_ex(
     return fail(FDATTN_ERR_SHAPE, "fdattn_append_attention: bad shape tokens=%d batch=%d max_chunk=%d hq=%d hkv=%d "
                 "head_dim=%d max_blocks=%d", num_tokens, batch, max_chunk, hq, hkv, head_dim, max_blocks_per_seq);
   if (num_tokens == 0) return 0;
-  const StepWorkspace w = step_workspace(num_tokens, batch, hq, hkv, head_dim, max_blocks_per_seq);
+  // key splits for the prefill rows: only when the host says how few they are
+  const int prefill_rows = extras && extras->prefill_rows > 0 ? extras->prefill_rows : 0;
+  int splits = prefill_rows > 0 && max_chunk > 0 ? prefill_auto_splits(prefill_rows, hq, max_chunk) : 1;
+  StepWorkspace w = step_workspace(num_tokens, batch, hq, hkv, head_dim, max_blocks_per_seq, splits);
+  while (splits > 1 && workspace_bytes < w.total)  // a workspace sized for fewer splits: use as many as it holds
+    w = step_workspace(num_tokens, batch, hq, hkv, head_dim, max_blocks_per_seq, --splits);
   if (workspace_bytes < w.total)
     return fail(FDATTN_ERR_WORKSPACE, "fdattn_append_attention: workspace %zu B < required %zu B", workspace_bytes,
                 w.total);
@@ -74,11 +85,11 @@ extern "C" int fdattn_append_attention_ex(
   int rc = fdattn_write_cache_kv_ex(qkv, q_rot, k_new, v_new, key_cache, value_cache, cache_k_scale, cache_v_scale,
                                     rope_cos, rope_sin, block_tables, seq_lens_decoder, cu_seqlens_q, num_tokens,
                                     batch, hq, hkv, head_dim, block_size, max_blocks_per_seq, num_blocks, max_pos,
-                                    rope_style, cache_quant_type, epilogue, stream);
+                                    rope_style, cache_quant_type, extras, stream);
   if (rc) return rc;
   // 2. decode rows: one token, seq_lens_encoder == 0; they read their own token back from the cache
   const RowMap rows{cu_seqlens_q, seq_lens_encoder};
-  const size_t dws = w.total - w.decode;
+  const size_t dws = w.split - w.decode;
   hipStream_t s = (hipStream_t)stream;
   if (c8_supported(hq, hkv, head_dim, block_size, cache_quant_type))
     rc = decode_c8_launch(q_rot, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
@@ -96,6 +107,6 @@ extern "C" int fdattn_append_attention_ex(
     rc = prefill_launch(q_rot, k_new, v_new, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
                         seq_lens_decoder, cu_seqlens_q, seq_lens_encoder, out, num_tokens, batch, max_chunk, hq, hkv,
                         head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type, softmax_scale, s,
-                        false);
+                        false, ws + w.split, w.total - w.split, splits, prefill_rows);
   return rc;
 }

@@ -263,9 +263,9 @@ extern "C" int fdattn_write_cache_kv_ex(
     const float* rope_sin, const int32_t* block_tables, const int32_t* seq_lens_decoder,
     const int32_t* cu_seqlens_q, int num_tokens, int batch, int hq, int hkv, int head_dim,
     int block_size, int max_blocks_per_seq, int num_blocks, int max_pos, int rope_style,
-    int cache_quant_type, const fdattn_qkv_epilogue* epilogue, void* stream) {
-  const fdattn_qkv_epilogue none = {nullptr, nullptr, nullptr, 0.f};
-  const fdattn_qkv_epilogue& ep = epilogue ? *epilogue : none;
+    int cache_quant_type, const fdattn_step_extras* extras, void* stream) {
+  const fdattn_step_extras none = {nullptr, nullptr, nullptr, 0.f, 0};
+  const fdattn_step_extras& ep = extras ? *extras : none;
   if (ep.q_norm_weight || ep.k_norm_weight) {
     const int u = head_dim / 16;
     if (head_dim % 16 != 0 || u <= 0 || (u & (u - 1)) != 0 || u > 64)

@@ -1,6 +1,7 @@
 // Launchers shared by the entry-point files of libfdattn.so.
 #pragma once
 #include "fdattn_common.h"
+#include "prefill.h"
 
 namespace fdattn {
 
@@ -28,11 +29,14 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
                      int hkv, int d, int bs, int max_blocks, int num_blocks, int quant,
                      float sm_scale, hipStream_t s, int stages, RowMap rows = RowMap{nullptr, nullptr});
 // append (prefill) attention; seq_lens_encoder may be NULL (every sequence is a prefill row)
+// workspace / n_splits: the MFMA kernel may split every query tile's keys over n_splits workgroups (partials in
+// workspace); rows_hint: how many of the batch's rows are prefill rows, if known (0: all of them)
 int prefill_launch(const void* q, const void* k_new, const void* v_new, const void* key_cache,
                    const void* value_cache, const float* cache_k_scale, const float* cache_v_scale,
                    const int32_t* block_tables, const int32_t* seq_lens_decoder, const int32_t* cu_seqlens_q,
                    const int32_t* seq_lens_encoder, void* out, int num_tokens, int batch, int max_chunk, int hq,
                    int hkv, int head_dim, int block_size, int max_blocks, int num_blocks, int cache_quant_type,
-                   float softmax_scale, hipStream_t s, bool force_generic);
+                   float softmax_scale, hipStream_t s, bool force_generic, void* workspace = nullptr,
+                   size_t workspace_bytes = 0, int n_splits = 1, int rows_hint = 0);
 
 }  // namespace fdattn

@@ -20,9 +20,20 @@ struct PrefillArgs {
   int num_tokens, batch, hq, hkv, d, bs, max_blocks, num_blocks;
   float sm_scale;
   int q_tiles;  // MFMA kernel: workgroups per (sequence, query head), set by its launcher
+  // MFMA kernel, split along the keys: n_splits > 1 workgroups share a query tile, each walks 1/n_splits of its
+  // key tiles and leaves a partial (unnormalised o in fp32, exponent reference m, weight sum l) for the merge
+  int n_splits;
+  int tile_tokens;  // queries per workgroup of this launch (128 or 256), for the merge kernel
+  float* part_o;   // [n_splits][num_tokens][hq][128]
+  float* part_ml;  // [n_splits][num_tokens][hq][2]
 };
 
 bool prefill_mfma_supported(int hq, int hkv, int d, int bs, int quant);
-int prefill_mfma_launch(const PrefillArgs& a, int max_chunk, int quant, hipStream_t s);
+// workspace may be NULL (no split); n_splits is clamped to what the workspace holds
+int prefill_mfma_launch(const PrefillArgs& a, int max_chunk, int quant, hipStream_t s, void* workspace = nullptr,
+                        size_t workspace_bytes = 0, int n_splits = 1, int rows_hint = 0);
+size_t prefill_split_workspace_bytes(int num_tokens, int hq, int n_splits);
+// splits that fill the GPU when `rows` sequences bring at most max_chunk new tokens each (1 = none needed)
+int prefill_auto_splits(int rows, int hq, int max_chunk);
 
 }  // namespace fdattn

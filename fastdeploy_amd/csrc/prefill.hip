@@ -102,7 +102,8 @@ int prefill_launch(const void* q, const void* k_new, const void* v_new, const vo
                    const int32_t* block_tables, const int32_t* seq_lens_decoder, const int32_t* cu_seqlens_q,
                    const int32_t* seq_lens_encoder, void* out, int num_tokens, int batch, int max_chunk, int hq,
                    int hkv, int head_dim, int block_size, int max_blocks_per_seq, int num_blocks,
-                   int cache_quant_type, float softmax_scale, hipStream_t s, bool force_generic) {
+                   int cache_quant_type, float softmax_scale, hipStream_t s, bool force_generic, void* workspace,
+                   size_t workspace_bytes, int n_splits, int rows_hint) {
   if (!q || !k_new || !v_new || !key_cache || !value_cache || !cache_k_scale || !cache_v_scale ||
       !block_tables || !seq_lens_decoder || !cu_seqlens_q || !out)
     return fail(FDATTN_ERR_NULL, "fdattn_append_attention_prefill: a required pointer is NULL");
@@ -120,7 +121,7 @@ int prefill_launch(const void* q, const void* k_new, const void* v_new, const vo
                 cu_seqlens_q, seq_lens_encoder, (uint16_t*)out, num_tokens, batch, hq, hkv, head_dim, block_size,
                 max_blocks_per_seq, num_blocks, softmax_scale};
   if (!force_generic && prefill_mfma_supported(hq, hkv, head_dim, block_size, cache_quant_type))
-    return prefill_mfma_launch(a, max_chunk, cache_quant_type, s);
+    return prefill_mfma_launch(a, max_chunk, cache_quant_type, s, workspace, workspace_bytes, n_splits, rows_hint);
   if (cache_quant_type == FDATTN_CACHE_INT8)
     hipLaunchKernelGGL(prefill_generic_kernel<FDATTN_CACHE_INT8>, dim3(num_tokens, hq), dim3(64), 0, s, a);
   else
@@ -141,7 +142,29 @@ extern "C" int fdattn_append_attention_prefill(
   return prefill_launch(q, k_new, v_new, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
                         seq_lens_decoder, cu_seqlens_q, nullptr, out, num_tokens, batch, max_chunk, hq, hkv,
                         head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type, softmax_scale,
-                        (hipStream_t)stream, false);
+                        (hipStream_t)stream, false, nullptr, 0, 1);
+}
+
+extern "C" int fdattn_prefill_auto_splits(int rows, int hq, int max_chunk) { return prefill_auto_splits(rows, hq, max_chunk); }
+
+extern "C" size_t fdattn_append_attention_prefill_split_workspace_bytes(int num_tokens, int hq, int num_splits) {
+  return prefill_split_workspace_bytes(num_tokens, hq, num_splits);
+}
+
+extern "C" int fdattn_append_attention_prefill_split(
+    const void* q, const void* k_new, const void* v_new, const void* key_cache, const void* value_cache,
+    const float* cache_k_scale, const float* cache_v_scale, const int32_t* block_tables,
+    const int32_t* seq_lens_decoder, const int32_t* cu_seqlens_q, void* out, void* workspace, size_t workspace_bytes,
+    int num_splits, int num_tokens, int batch, int max_chunk, int hq, int hkv, int head_dim, int block_size,
+    int max_blocks_per_seq, int num_blocks, int cache_quant_type, float softmax_scale, void* stream) {
+  if (num_splits < 1) return fail(FDATTN_ERR_SHAPE, "fdattn_append_attention_prefill_split: num_splits %d < 1", num_splits);
+  if (num_splits > 1 && (!workspace || workspace_bytes < prefill_split_workspace_bytes(num_tokens, hq, num_splits)))
+    return fail(FDATTN_ERR_WORKSPACE, "fdattn_append_attention_prefill_split: workspace %zu B < required %zu B",
+                workspace_bytes, prefill_split_workspace_bytes(num_tokens, hq, num_splits));
+  return prefill_launch(q, k_new, v_new, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
+                        seq_lens_decoder, cu_seqlens_q, nullptr, out, num_tokens, batch, max_chunk, hq, hkv,
+                        head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type, softmax_scale,
+                        (hipStream_t)stream, false, workspace, workspace_bytes, num_splits);
 }
 
 extern "C" int fdattn_append_attention_prefill_generic(
@@ -153,5 +176,5 @@ extern "C" int fdattn_append_attention_prefill_generic(
   return prefill_launch(q, k_new, v_new, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
                         seq_lens_decoder, cu_seqlens_q, nullptr, out, num_tokens, batch, max_chunk, hq, hkv,
                         head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type, softmax_scale,
-                        (hipStream_t)stream, true);
+                        (hipStream_t)stream, true, nullptr, 0, 1);
 }

@@ -126,6 +126,9 @@ __device__ __forceinline__ u32 lds_addr(const void* p) {
 
 }  // namespace
 
+// how many of the launch's max_splits key splits a walk of n_tiles tiles uses
+__device__ __forceinline__ int splits_of(int n_tiles, int max_splits) { return min(max(n_tiles / 32, 1), max_splits); }
+
 template <int QUANT, int NW>
 __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   constexpr int BM = 32 * NW;       // queries per workgroup
@@ -170,6 +173,22 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   const int n_pre = (p + BN - 1) / BN;
   const int n_chk = (min(n_b, q0 + BM) + BN - 1) / BN;
   const int n_tiles = n_pre + n_chk;
+  // this workgroup's share of the key tiles: [t0, t1).  A share is worth its fixed costs (prologue, partial,
+  // merge) from about 32 tiles on: shorter walks are split less, or not at all - then split 0 walks everything
+  // and writes the final rows itself.
+  const int n_splits = splits_of(n_tiles, a.n_splits);
+  if ((int)blockIdx.y >= n_splits) return;
+  const int per = (n_tiles + n_splits - 1) / n_splits;
+  const int t0 = (int)blockIdx.y * per, t1 = min(t0 + per, n_tiles);
+  if (t0 >= t1) {  // nothing to walk (only with splits): an empty partial for each of the tile's queries
+    for (int i = tid; i < BM; i += 64 * NW)
+      if (q0 + i < n_b) {
+        float* ml = a.part_ml + (((size_t)blockIdx.y * a.num_tokens + tok0 + q0 + i) * a.hq + qh) * 2;
+        ml[0] = -INFINITY;
+        ml[1] = 0.f;
+      }
+    return;
+  }
   const int32_t* table = a.block_tables + (size_t)b * a.max_blocks;
   const float sc = a.sm_scale * 1.4426950408889634f;  // logits go to the log2 domain
 
@@ -222,9 +241,9 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   // straight away).
   int vzero;
   asm("v_mov_b32 %0, 0" : "=v"(vzero));
-  int pb_next = n_pre > 0 ? table[vzero] : 0;
+  int pb_next = t0 < n_pre ? table[t0 + vzero] : 0;
   auto fetch = [&](int t) {
-    if (t >= n_tiles) return;
+    if (t >= t1) return;
     if (t < n_pre) {
       // the block id was requested one fetch earlier: its scalar load has long returned
       const int pb_u = __builtin_amdgcn_readfirstlane(pb_next);
@@ -253,7 +272,7 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   // this thread's fetched chunks of tile t into its LDS slot: fp16 for cache bytes and for the
   // chunk's V, the chunk's bf16 K as it is
   auto commit = [&](int t) {
-    if (t >= n_tiles) return;
+    if (t >= t1) return;
     const u32 slot_off = (u32)(t & (kSlots - 1)) * (u32)(BUF_ELEMS * sizeof(uint16_t));
     const u32 kd = kw0 + slot_off, vd = vw0 + slot_off;
     if (t < n_pre) {
@@ -292,33 +311,49 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
 
   // tiles this wavefront computes on; chunk tiles wholly above its diagonal contribute
   // nothing and it only helps staging them
-  const int my_tiles = wave_active ? n_pre + ci_wave_max / BN + 1 : 0;
+  const int my_tiles = wave_active ? min(n_pre + ci_wave_max / BN + 1, t1) : 0;
   const int q16 = lane >> 4, i16 = lane & 15;
 
-  load_q(n_pre > 0);
+  load_q(t0 < n_pre);
   // log2-domain constant that removes the byte offset from the prefix scores
   const float qbias = -ByteFmt<QUANT>::kOff * sc * (qsum + __shfl_xor(qsum, 32, 64));
 
-  // prologue: tile 0 (and group 1's rows of tile 1) into LDS
-  fetch(0);
-  commit(0);
+  // prologue: the first tile (and group 1's rows of the second) into LDS
+  fetch(t0);
+  commit(t0);
   if (grp == 1) {
-    fetch(1);
-    commit(1);
+    fetch(t0 + 1);
+    commit(t0 + 1);
   }
   __syncthreads();
   if (grp == 1) __syncthreads();  // group 1 trails by one phase
 
+  // leaving the quantised prefix: o holds sums over offset bytes; remove the offset and give the channels
+  // their scale
+  auto leave_prefix = [&]() {
+    const float l_off = -ByteFmt<QUANT>::kOff * (l_run + __shfl_xor(l_run, 32, 64));
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+      for (int rb = 0; rb < 4; ++rb) {
+        const float4 vs = *reinterpret_cast<const float4*>(a.v_scale + h * HD + 32 * ct + 8 * rb + 4 * hf);
+        o[ct][4 * rb + 0] = (o[ct][4 * rb + 0] * ByteFmt<QUANT>::kMul + l_off) * vs.x;
+        o[ct][4 * rb + 1] = (o[ct][4 * rb + 1] * ByteFmt<QUANT>::kMul + l_off) * vs.y;
+        o[ct][4 * rb + 2] = (o[ct][4 * rb + 2] * ByteFmt<QUANT>::kMul + l_off) * vs.z;
+        o[ct][4 * rb + 3] = (o[ct][4 * rb + 3] * ByteFmt<QUANT>::kMul + l_off) * vs.w;
+      }
+  };
+
   v16f st[2];
   v8h pf[2][2];
-  for (int t = 0; t <= n_tiles; ++t) {
+  for (int t = t0; t <= t1; ++t) {
     // ================= matrix phase =================
     if (t == n_pre && n_pre > 0 && t < my_tiles) load_q(false);  // the chunk's scores meet the bf16 q
     fetch(t + lead);  // converted and written to LDS in the vector phase that follows
     // ---- O^T += V^T P^T, tile t-1, then S^T = K Q^T, tile t.  In the first product k-slot e of
     // lane group hf is key 32kb + 16ss + 8(e/4) + 4hf + e%4 (the P^T layout); lane i16 supplies
     // the row (key kbase + i16/4, channels cbase + 4(i16%4)..+3)
-    const bool do_pv = t >= 1 && t <= my_tiles, do_qk = t < my_tiles;
+    const bool do_pv = t > t0 && t <= my_tiles, do_qk = t < my_tiles;
     const u32 va = lds_addr(lds + (size_t)((t + kSlots - 1) & (kSlots - 1)) * BUF_ELEMS + K_ELEMS + (4 * hf + (i16 >> 2)) * LDV +
                             16 * (q16 & 1) + 4 * (i16 & 3));
     const u32 ka = lds_addr(lds + (size_t)(t & (kSlots - 1)) * BUF_ELEMS + j32 * LDK + 8 * hf);
@@ -334,21 +369,7 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
     // staging first: its LDS writes and global loads then run under the softmax arithmetic
     commit(t + lead);
     if (t < my_tiles) {
-      if (t == n_pre && n_pre > 0) {
-        // leaving the quantised prefix: o holds sums over offset bytes; remove the offset
-        // and give the channels their scale
-        const float l_off = -ByteFmt<QUANT>::kOff * (l_run + __shfl_xor(l_run, 32, 64));
-#pragma unroll
-        for (int ct = 0; ct < 4; ++ct)
-#pragma unroll
-          for (int rb = 0; rb < 4; ++rb) {
-            const float4 vs = *reinterpret_cast<const float4*>(a.v_scale + h * HD + 32 * ct + 8 * rb + 4 * hf);
-            o[ct][4 * rb + 0] = (o[ct][4 * rb + 0] * ByteFmt<QUANT>::kMul + l_off) * vs.x;
-            o[ct][4 * rb + 1] = (o[ct][4 * rb + 1] * ByteFmt<QUANT>::kMul + l_off) * vs.y;
-            o[ct][4 * rb + 2] = (o[ct][4 * rb + 2] * ByteFmt<QUANT>::kMul + l_off) * vs.z;
-            o[ct][4 * rb + 3] = (o[ct][4 * rb + 3] * ByteFmt<QUANT>::kMul + l_off) * vs.w;
-          }
-      }
+      if (t == n_pre && n_pre > 0) leave_prefix();
       // ---- mask + online softmax; this lane: one query, keys 32kb + (r%4) + 8(r/4) + 4hf
       const bool pre = t < n_pre;
       const int key0 = pre ? t * BN : (t - n_pre) * BN;  // index of the tile's first key in its segment
@@ -429,9 +450,27 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   }
   if (grp == 0) __syncthreads();  // the barrier group 1 took before its first phase
 
-  // ---- epilogue: normalise and store bf16 (every query saw at least its own chunk tile)
-  if (!wave_active || ci_raw >= n_b) return;
+  if (!wave_active) return;
+  if (t1 <= n_pre) leave_prefix();  // a share that ends inside the prefix (only with splits)
+  if (ci_raw >= n_b) return;
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  if (n_splits > 1) {
+    // ---- a partial for the merge: o unnormalised in fp32, the exponent reference and the weight sum
+    const size_t row = ((size_t)blockIdx.y * a.num_tokens + tok0 + ci) * a.hq + qh;
+    float* po = a.part_o + row * HD;
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+      for (int rb = 0; rb < 4; ++rb)
+        *reinterpret_cast<float4*>(po + 32 * ct + 8 * rb + 4 * hf) =
+            make_float4(o[ct][4 * rb], o[ct][4 * rb + 1], o[ct][4 * rb + 2], o[ct][4 * rb + 3]);
+    if (hf == 0) {
+      a.part_ml[row * 2] = m_ref;
+      a.part_ml[row * 2 + 1] = l_tot;
+    }
+    return;
+  }
+  // ---- epilogue: normalise and store bf16 (every query saw at least its own chunk tile)
   const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
   uint16_t* orow = a.out + ((size_t)(tok0 + ci) * a.hq + qh) * HD;
 #pragma unroll
@@ -445,6 +484,40 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
     }
 }
 
+// Merge of the split partials: one wavefront per new token of a prefill row, looping over the query heads;
+// lane = two channels.  grid (ceil(max_chunk / 4), batch), 256 threads.
+__global__ __launch_bounds__(256) void prefill_merge_kernel(PrefillArgs a) {
+  const int b = blockIdx.y, lane = threadIdx.x & 63;
+  if (a.seq_lens_encoder && a.seq_lens_encoder[b] <= 0) return;
+  const int tok0 = a.cu_seqlens_q[b], n_b = a.cu_seqlens_q[b + 1] - tok0;
+  const int i = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (i >= n_b) return;
+  // the split count of this token's query tile, as the main kernel worked it out
+  const int q0 = i / a.tile_tokens * a.tile_tokens;
+  const int n_tiles = (a.seq_lens_decoder[b] + BN - 1) / BN + (min(n_b, q0 + a.tile_tokens) + BN - 1) / BN;
+  const int n_splits = splits_of(n_tiles, a.n_splits);
+  if (n_splits <= 1) return;  // the row is final already
+  for (int qh = 0; qh < a.hq; ++qh) {
+    const size_t row0 = ((size_t)(tok0 + i)) * a.hq + qh, stride = (size_t)a.num_tokens * a.hq;
+    float M = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) M = fmaxf(M, a.part_ml[(row0 + s * stride) * 2]);
+    float L = 0.f, o0 = 0.f, o1 = 0.f;
+    if (M > -INFINITY) {
+      for (int s = 0; s < n_splits; ++s) {
+        const float ms = a.part_ml[(row0 + s * stride) * 2];
+        if (ms == -INFINITY) continue;
+        const float f = __builtin_amdgcn_exp2f(ms - M);
+        L += a.part_ml[(row0 + s * stride) * 2 + 1] * f;
+        const float2 v = *reinterpret_cast<const float2*>(a.part_o + (row0 + s * stride) * HD + 2 * lane);
+        o0 += v.x * f;
+        o1 += v.y * f;
+      }
+    }
+    const float inv = L > 0.f ? 1.0f / L : 0.f;
+    *reinterpret_cast<u32*>(a.out + row0 * HD + 2 * lane) = pack_bf16(o0 * inv, o1 * inv);
+  }
+}
+
 bool prefill_mfma_supported(int hq, int hkv, int d, int bs, int quant) {
   return d == HD && bs == BN && hq % hkv == 0 &&
          (quant == FDATTN_CACHE_INT8 || quant == FDATTN_CACHE_FP8_E4M3);
@@ -452,12 +525,15 @@ bool prefill_mfma_supported(int hq, int hkv, int d, int bs, int quant) {
 
 namespace {
 
+constexpr int kMaxSplits = 8;
+
 template <int QUANT, int NW>
 hipError_t launch_one(const PrefillArgs& a, int max_chunk, hipStream_t s) {
   constexpr int BM = 32 * NW;
   PrefillArgs args = a;
   args.q_tiles = (max_chunk + BM - 1) / BM;
-  const dim3 grid((unsigned)a.batch * a.hq * args.q_tiles), block(64 * NW);
+  args.tile_tokens = BM;
+  const dim3 grid((unsigned)a.batch * a.hq * args.q_tiles, a.n_splits), block(64 * NW);
   const size_t shm = (size_t)kSlots * BUF_ELEMS * sizeof(uint16_t);  // 151,552 B
   // the dynamic LDS limit is a per-device property of the kernel: raise it once on each device
   static std::atomic<unsigned long long> raised{0};  // bit d: done on device d (one word per instantiation)
@@ -476,14 +552,48 @@ hipError_t launch_one(const PrefillArgs& a, int max_chunk, hipStream_t s) {
 
 }  // namespace
 
-int prefill_mfma_launch(const PrefillArgs& a, int max_chunk, int quant, hipStream_t s) {
+size_t prefill_split_workspace_bytes(int num_tokens, int hq, int n_splits) {
+  if (n_splits <= 1 || num_tokens <= 0 || hq <= 0) return 0;
+  if (n_splits > kMaxSplits) n_splits = kMaxSplits;
+  return (size_t)n_splits * num_tokens * hq * (HD + 2) * sizeof(float);
+}
+
+// 256-token workgroups (8 wavefronts, the two groups overlapping MFMA and vector work) whenever they - times the
+// key splits - cover the CUs (one workgroup fits a CU); 128-token ones otherwise
+static bool wide_workgroups(int rows, int hq, int max_chunk, int n_splits) {
+  return max_chunk > 128 && (long long)rows * hq * ((max_chunk + 255) / 256) * n_splits >= gpu_cu_count();
+}
+
+int prefill_auto_splits(int rows, int hq, int max_chunk) {
+  if (rows <= 0 || hq <= 0 || max_chunk <= 0) return 1;
+  const int cus = gpu_cu_count();
+  auto splits_for = [&](int bm) {
+    const long long wgs = (long long)rows * hq * ((max_chunk + bm - 1) / bm);
+    const long long s = (cus + wgs - 1) / wgs;  // enough to give every CU a workgroup
+    return (int)(s < 1 ? 1 : (s > kMaxSplits ? kMaxSplits : s));
+  };
+  if (max_chunk > 128) {
+    const int s = splits_for(256);
+    if (wide_workgroups(rows, hq, max_chunk, s)) return s;
+  }
+  return splits_for(128);
+}
+
+int prefill_mfma_launch(const PrefillArgs& a_in, int max_chunk, int quant, hipStream_t s, void* workspace,
+                        size_t workspace_bytes, int n_splits, int rows_hint) {
+  PrefillArgs a = a_in;
+  if (n_splits > kMaxSplits) n_splits = kMaxSplits;
+  while (n_splits > 1 && (!workspace || workspace_bytes < prefill_split_workspace_bytes(a.num_tokens, a.hq, n_splits))) --n_splits;
+  a.n_splits = n_splits < 1 ? 1 : n_splits;
+  a.part_o = (float*)workspace;
+  a.part_ml = a.part_o + (size_t)a.n_splits * a.num_tokens * a.hq * HD;
   if ((long long)a.batch * a.hq * ((max_chunk + 127) / 128) > 0x7fffffffLL)
     return fail(FDATTN_ERR_SHAPE, "fdattn_append_attention_prefill: too many workgroups for one launch");
   // 256-token workgroups share each staged tile among 8 wavefronts (their two groups alternate between the MFMA
   // units and the vector ALU); short chunks keep 128
   // when they would still leave CUs without a workgroup (one fits a CU), 128-token workgroups cover twice as
   // many CUs: 10-14 % faster at e.g. 2 x 512 tokens, although a 4-wavefront workgroup overlaps nothing
-  const bool wide = max_chunk > 128 && (long long)a.batch * a.hq * ((max_chunk + 255) / 256) >= gpu_cu_count();
+  const bool wide = wide_workgroups(rows_hint > 0 ? rows_hint : a.batch, a.hq, max_chunk, a.n_splits);
   hipError_t e;
   if (quant == FDATTN_CACHE_INT8)
     e = wide ? launch_one<FDATTN_CACHE_INT8, 8>(a, max_chunk, s) : launch_one<FDATTN_CACHE_INT8, 4>(a, max_chunk, s);
@@ -491,7 +601,11 @@ int prefill_mfma_launch(const PrefillArgs& a, int max_chunk, int quant, hipStrea
     e = wide ? launch_one<FDATTN_CACHE_FP8_E4M3, 8>(a, max_chunk, s)
              : launch_one<FDATTN_CACHE_FP8_E4M3, 4>(a, max_chunk, s);
   if (e != hipSuccess) return fail((int)e, "fdattn_append_attention_prefill: %s", hipGetErrorString(e));
-  return check_launch("fdattn_append_attention_prefill (mfma)");
+  int rc = check_launch("fdattn_append_attention_prefill (mfma)");
+  if (rc || a.n_splits <= 1) return rc;
+  a.tile_tokens = wide ? 256 : 128;
+  hipLaunchKernelGGL(prefill_merge_kernel, dim3((max_chunk + 3) / 4, a.batch), dim3(256), 0, s, a);
+  return check_launch("fdattn_append_attention_prefill (merge)");
 }
 
 }  // namespace fdattn

@@ -71,9 +71,9 @@ def _scales(cache_k_scale, cache_v_scale, hkv, d):
     return pk, pv
 
 
-def _epilogue(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, width, d):
-    """fdattn_qkv_epilogue for the optional projection epilogue, or None"""
-    if qkv_bias is None and q_norm_weight is None and k_norm_weight is None:
+def _extras(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, width, d, prefill_rows=0):
+    """fdattn_step_extras for the optional projection epilogue / prefill splits, or None"""
+    if qkv_bias is None and q_norm_weight is None and k_norm_weight is None and prefill_rows <= 0:
         return None
     pb = _chk(qkv_bias, "qkv_bias", torch.bfloat16, 1, optional=True)
     if qkv_bias is not None and qkv_bias.numel() != width:
@@ -83,7 +83,12 @@ def _epilogue(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, width, d):
     for name, t in (("q_norm_weight", q_norm_weight), ("k_norm_weight", k_norm_weight)):
         if t is not None and t.numel() != d:
             raise ValueError("%s has %d entries, head_dim is %d" % (name, t.numel(), d))
-    return _lib.QkvEpilogue(pb or None, pq or None, pk or None, float(rms_norm_eps))
+    return _lib.StepExtras(pb or None, pq or None, pk or None, float(rms_norm_eps), int(prefill_rows))
+
+
+def prefill_auto_splits(rows, num_heads, max_chunk):
+    """How many key splits fill the GPU when `rows` sequences bring at most max_chunk new tokens each (1..8)."""
+    return _lib.lib().fdattn_prefill_auto_splits(int(rows), int(num_heads), int(max_chunk))
 
 
 def seq_lens_this_time_of(seq_lens_encoder, seq_lens_decoder):
@@ -153,7 +158,7 @@ def write_cache_kv(qkv, key_cache, value_cache, cache_k_scale, cache_v_scale, bl
     if want_kv_out:
         k_out = torch.empty((T, hkv * d), dtype=torch.bfloat16, device=qkv.device)
         v_out = torch.empty((T, hkv * d), dtype=torch.bfloat16, device=qkv.device)
-    ep = _epilogue(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, qkv.shape[1], d)
+    ep = _extras(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, qkv.shape[1], d)
     rc = _lib.lib().fdattn_write_cache_kv_ex(
         p_qkv, q_out.data_ptr(), k_out.data_ptr() if want_kv_out else 0,
         v_out.data_ptr() if want_kv_out else 0, p_kc, p_vc, p_ks, p_vs, p_cos, p_sin, p_bt, p_dec,
@@ -299,9 +304,12 @@ def sqattn_select(q, key_cache, cache_k_scale, block_tables, seq_lens_decoder, s
 
 def append_attention_prefill(q, k_new, v_new, key_cache, value_cache, cache_k_scale, cache_v_scale,
                              block_tables, seq_lens_decoder, cu_seqlens_q, *, num_heads, max_chunk,
-                             cache_quant_type="cache_int8", softmax_scale=None, out=None, impl="auto"):
+                             cache_quant_type="cache_int8", softmax_scale=None, out=None, impl="auto",
+                             num_splits=None, workspace=None):
     """Chunked prefill: the chunk's tokens attend to the cached prefix (quantised pages)
-    and causally to the chunk itself (bf16 k_new / v_new)."""
+    and causally to the chunk itself (bf16 k_new / v_new).
+    num_splits: workgroups that share one query tile's keys (None: as many as fill the GPU when the
+    batch's query tiles alone would not, 1: none); partials go to `workspace` (allocated if None)."""
     nb, hkv, bs, d = _cache_dims(key_cache, value_cache)
     p_q = _chk(q, "q", torch.bfloat16, 2)
     p_k = _chk(k_new, "k_new", torch.bfloat16, 2)
@@ -321,23 +329,38 @@ def append_attention_prefill(q, k_new, v_new, key_cache, value_cache, cache_k_sc
     if out is None:
         out = torch.empty((T, num_heads * d), dtype=torch.bfloat16, device=q.device)
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(d)
-    fn = _lib.lib().fdattn_append_attention_prefill if impl == "auto" else \
-        _lib.lib().fdattn_append_attention_prefill_generic
-    rc = fn(
-        p_q, p_k, p_v, p_kc, p_vc, p_ks, p_vs, p_bt, p_dec, p_cu, _chk(out, "out", torch.bfloat16), T, batch,
-        max_chunk, num_heads, hkv, d, bs, mb, nb, _quant(cache_quant_type), scale, _stream())
+    if impl == "auto":
+        if num_splits is None:
+            num_splits = prefill_auto_splits(batch, num_heads, max_chunk)
+        p_ws = n_ws = 0
+        if num_splits > 1:
+            need = _lib.lib().fdattn_append_attention_prefill_split_workspace_bytes(T, num_heads, num_splits)
+            if workspace is None:
+                workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+            p_ws, n_ws = _chk(workspace, "workspace", torch.uint8), workspace.numel()
+        rc = _lib.lib().fdattn_append_attention_prefill_split(
+            p_q, p_k, p_v, p_kc, p_vc, p_ks, p_vs, p_bt, p_dec, p_cu, _chk(out, "out", torch.bfloat16), p_ws or None,
+            n_ws, num_splits, T, batch, max_chunk, num_heads, hkv, d, bs, mb, nb, _quant(cache_quant_type), scale,
+            _stream())
+    else:
+        rc = _lib.lib().fdattn_append_attention_prefill_generic(
+            p_q, p_k, p_v, p_kc, p_vc, p_ks, p_vs, p_bt, p_dec, p_cu, _chk(out, "out", torch.bfloat16), T, batch,
+            max_chunk, num_heads, hkv, d, bs, mb, nb, _quant(cache_quant_type), scale, _stream())
     _lib.check(rc, "append_attention_prefill")
     return out
 
 
-def append_attention_workspace_bytes(num_tokens, batch, num_heads, kv_heads, head_dim, max_blocks_per_seq):
-    return _lib.lib().fdattn_append_attention_workspace_bytes(num_tokens, batch, num_heads, kv_heads, head_dim,
-                                                             max_blocks_per_seq)
+def append_attention_workspace_bytes(num_tokens, batch, num_heads, kv_heads, head_dim, max_blocks_per_seq,
+                                     prefill_splits=1):
+    return _lib.lib().fdattn_append_attention_workspace_bytes_ex(num_tokens, batch, num_heads, kv_heads, head_dim,
+                                                                max_blocks_per_seq, prefill_splits)
 
 
-def append_attention_workspace(num_tokens, batch, num_heads, kv_heads, head_dim, max_blocks_per_seq, device="cuda"):
+def append_attention_workspace(num_tokens, batch, num_heads, kv_heads, head_dim, max_blocks_per_seq, device="cuda",
+                               prefill_splits=1):
     """A workspace tensor large enough for append_attention at these shapes."""
-    n = append_attention_workspace_bytes(num_tokens, batch, num_heads, kv_heads, head_dim, max_blocks_per_seq)
+    n = append_attention_workspace_bytes(num_tokens, batch, num_heads, kv_heads, head_dim, max_blocks_per_seq,
+                                         prefill_splits)
     return torch.empty(n, dtype=torch.uint8, device=device)
 
 
@@ -345,13 +368,16 @@ def append_attention(qkv, key_cache, value_cache, seq_lens_encoder, seq_lens_dec
                      block_tables, rotary_embs, cache_k_scale, cache_v_scale, *, num_heads, kv_num_heads,
                      max_chunk, rope_style="neox", cache_quant_type="cache_int8", softmax_scale=None,
                      cu_seqlens_q=None, workspace=None, out=None, qkv_bias=None, q_norm_weight=None,
-                     k_norm_weight=None, rms_norm_eps=1e-6):
+                     k_norm_weight=None, rms_norm_eps=1e-6, prefill_rows=None):
     """One attention step of a layer over a mixed batch (one call into the library):
     every new token is rotated and written to the cache, decode rows (one token,
     seq_lens_encoder == 0) attend to the cache, prefill rows (seq_lens_encoder > 0)
     to their cached prefix and causally to their own chunk; slots without a token
     are skipped.  max_chunk bounds the tokens of a prefill row (0: the step has none, decode only).
     qkv_bias / q_norm_weight / k_norm_weight / rms_norm_eps: the projection's epilogue, as in write_cache_kv.
+    prefill_rows: how many rows of the step are prefill rows, if the host knows (None: unknown).  When those rows
+    alone would leave CUs idle, every query tile is shared by prefill_auto_splits(prefill_rows, num_heads,
+    max_chunk) workgroups; a workspace passed in must have been sized with that number of splits.
     Returns bf16 [num_tokens, num_heads*head_dim]."""
     nb, hkv, bs, d = _cache_dims(key_cache, value_cache)
     if hkv != kv_num_heads:
@@ -393,11 +419,12 @@ def append_attention(qkv, key_cache, value_cache, seq_lens_encoder, seq_lens_dec
         raise ValueError("max_chunk must be >= 0")
     if out is None:
         out = torch.empty((T, num_heads * d), dtype=torch.bfloat16, device=qkv.device)
-    need = _lib.lib().fdattn_append_attention_workspace_bytes(T, batch, num_heads, hkv, d, mb)
+    splits = prefill_auto_splits(prefill_rows, num_heads, max_chunk) if prefill_rows and max_chunk > 0 else 1
+    need = _lib.lib().fdattn_append_attention_workspace_bytes_ex(T, batch, num_heads, hkv, d, mb, splits)
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=qkv.device)
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(d)
-    ep = _epilogue(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, qkv.shape[1], d)
+    ep = _extras(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, qkv.shape[1], d, prefill_rows or 0)
     rc = _lib.lib().fdattn_append_attention_ex(
         p_qkv, p_kc, p_vc, p_ks, p_vs, p_cos, p_sin, p_bt, p_enc, p_dec, p_this, p_cu,
         _chk(out, "out", torch.bfloat16), workspace.data_ptr(), workspace.numel() * workspace.element_size(),

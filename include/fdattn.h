@@ -96,23 +96,30 @@ FDATTN_API int fdattn_write_cache_kv(
     int rope_style, int cache_quant_type, void* stream);
 
 /*
- * The QKV projection's epilogue, fused in front of the cache writer (every member optional;
- * engine-side operators take optional inputs the same way,
- * fastdeploy/runtime/backends/paddle/ops/voxelize_op.cc:194-204 lists inputs and attributes).
+ * Optional extras of a step (every member optional; engine-side operators take optional inputs
+ * the same way, fastdeploy/runtime/backends/paddle/ops/voxelize_op.cc:194-204 lists inputs and
+ * attributes).  The QKV projection's epilogue, fused in front of the cache writer:
  *   qkv_bias        bf16 [(hq + 2*hkv) * head_dim]: x = bf16(x + bias), the result of a bf16 add
  *   q_norm_weight   f32 [head_dim]: every Q head x -> x / sqrt(mean(x^2) + eps) * weight, before
  *   k_norm_weight   f32 [head_dim]  the rotation; the same for every K head (V is not normed)
  * All arithmetic is fp32 with every operation rounded on its own; nothing is rounded to bf16
  * between the norm and the rotation.  The norm needs head_dim = 16 * 2^n.
+ *   prefill_rows    (fdattn_append_attention_ex only) the number of prefill rows of the step, if the
+ *                   host knows it (0 = unknown).  When those rows alone would leave CUs idle - one
+ *                   sequence's chunk of a few hundred tokens among decode rows - every query tile
+ *                   is shared by fdattn_prefill_auto_splits(prefill_rows, hq, max_chunk) workgroups,
+ *                   each walking a part of its keys; the workspace must then come from
+ *                   fdattn_append_attention_workspace_bytes_ex with that number of splits.
  */
-typedef struct fdattn_qkv_epilogue {
+typedef struct fdattn_step_extras {
   const void* qkv_bias;
   const float* q_norm_weight;
   const float* k_norm_weight;
   float rms_norm_eps;
-} fdattn_qkv_epilogue;
+  int prefill_rows;
+} fdattn_step_extras;
 
-/* fdattn_write_cache_kv with the epilogue (host pointer, read during the call; NULL = none). */
+/* fdattn_write_cache_kv with the extras (host pointer, read during the call; NULL = none). */
 FDATTN_API int fdattn_write_cache_kv_ex(
     const void* qkv, void* q_out, void* k_out, void* v_out,
     void* key_cache, void* value_cache,
@@ -122,7 +129,7 @@ FDATTN_API int fdattn_write_cache_kv_ex(
     const int32_t* cu_seqlens_q,
     int num_tokens, int batch, int hq, int hkv, int head_dim, int block_size,
     int max_blocks_per_seq, int num_blocks, int max_pos,
-    int rope_style, int cache_quant_type, const fdattn_qkv_epilogue* epilogue, void* stream);
+    int rope_style, int cache_quant_type, const fdattn_step_extras* extras, void* stream);
 
 /*
  * Bytes of workspace fdattn_decode_attention / fdattn_decode_attention_sparse
@@ -301,6 +308,28 @@ FDATTN_API int fdattn_append_attention_prefill(
     int cache_quant_type, float softmax_scale, void* stream);
 
 /*
+ * fdattn_append_attention_prefill with the keys of every query tile split over num_splits
+ * workgroups (MFMA shapes; elsewhere num_splits is ignored): each walks 1/num_splits of the key
+ * tiles and leaves a partial (o in fp32, exponent reference, weight sum) in workspace, a second
+ * kernel merges them.  For launches whose query tiles alone leave CUs idle - a single sequence's
+ * chunk of a few hundred tokens: fdattn_prefill_auto_splits(rows, hq, max_chunk) says how many
+ * splits fill the GPU (1..8) when `rows` sequences bring at most max_chunk new tokens each.
+ * workspace: fdattn_append_attention_prefill_split_workspace_bytes(num_tokens, hq, num_splits),
+ * no initialisation needed.  Same plug-in position as fdattn_append_attention_prefill.
+ */
+FDATTN_API int fdattn_prefill_auto_splits(int rows, int hq, int max_chunk);
+FDATTN_API size_t fdattn_append_attention_prefill_split_workspace_bytes(int num_tokens, int hq, int num_splits);
+FDATTN_API int fdattn_append_attention_prefill_split(
+    const void* q, const void* k_new, const void* v_new,
+    const void* key_cache, const void* value_cache,
+    const float* cache_k_scale, const float* cache_v_scale,
+    const int32_t* block_tables, const int32_t* seq_lens_decoder,
+    const int32_t* cu_seqlens_q, void* out, void* workspace, size_t workspace_bytes, int num_splits,
+    int num_tokens, int batch, int max_chunk, int hq, int hkv, int head_dim,
+    int block_size, int max_blocks_per_seq, int num_blocks,
+    int cache_quant_type, float softmax_scale, void* stream);
+
+/*
  * The shape-agnostic kernel fdattn_append_attention_prefill falls back to when the
  * MFMA kernel does not cover the shape (it covers head_dim 128, block_size 64),
  * callable directly.  Same arguments and plug-in position.
@@ -321,6 +350,9 @@ FDATTN_API int fdattn_append_attention_prefill_generic(
  */
 FDATTN_API size_t fdattn_append_attention_workspace_bytes(int num_tokens, int batch, int hq, int hkv,
                                                           int head_dim, int max_blocks_per_seq);
+/* The same with room for the partials of prefill_splits key splits (fdattn_step_extras). */
+FDATTN_API size_t fdattn_append_attention_workspace_bytes_ex(int num_tokens, int batch, int hq, int hkv,
+                                                             int head_dim, int max_blocks_per_seq, int prefill_splits);
 
 /*
  * One attention step of a layer over a mixed batch: the whole of what an engine-side
@@ -350,7 +382,7 @@ FDATTN_API int fdattn_append_attention(
     int block_size, int max_blocks_per_seq, int num_blocks, int max_pos,
     int rope_style, int cache_quant_type, float softmax_scale, void* stream);
 
-/* fdattn_append_attention with the QKV projection's epilogue in front of the cache write (NULL = none). */
+/* fdattn_append_attention with the extras of a step (NULL = none). */
 FDATTN_API int fdattn_append_attention_ex(
     const void* qkv, void* key_cache, void* value_cache,
     const float* cache_k_scale, const float* cache_v_scale,
@@ -360,7 +392,7 @@ FDATTN_API int fdattn_append_attention_ex(
     const int32_t* cu_seqlens_q, void* out, void* workspace, size_t workspace_bytes,
     int num_tokens, int batch, int max_chunk, int hq, int hkv, int head_dim,
     int block_size, int max_blocks_per_seq, int num_blocks, int max_pos,
-    int rope_style, int cache_quant_type, float softmax_scale, const fdattn_qkv_epilogue* epilogue, void* stream);
+    int rope_style, int cache_quant_type, float softmax_scale, const fdattn_step_extras* extras, void* stream);
 
 /*
  * Host-side block pool: the producer of block_tables (no counterpart in the reference,

@@ -204,3 +204,29 @@ def test_prefill_config5_shape_sampled_rows(oracle):
     ref = fd.append_attention_prefill(*args, num_heads=32, max_chunk=2048, impl="generic")
     ok, mx, bad = bf16_close(bits(out), bits(ref), 4e-3, 2e-2)
     assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
+
+
+@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+def test_prefill_key_splits(oracle, quant):
+    """Every query tile's keys shared by 2 .. 8 workgroups (partials + merge) against the oracle and against the
+    unsplit kernel: one sequence's chunk on a long prefix (what the split is for), shares that end inside the
+    prefix, start in the chunk or are empty, a ragged batch, and no prefix at all."""
+    from fastdeploy_amd.ops import prefill_auto_splits
+    assert prefill_auto_splits(1, 32, 512) >= 2 and prefill_auto_splits(64, 32, 2048) == 1
+    for prefix, chunks, splits in (([64 * 70 + 17], [300], None), ([64 * 300], [130], 8), ([0, 4500, 64], [129, 5, 256], 4),
+                                   ([0, 0], [40, 200], 3)):
+        c = _prefill_case(len(chunks) * 7 + (splits or 0), prefix, chunks, quant)
+        dev = syn.to_device(c, "cuda")
+        args = (dev["q_new"], dev["k_new"], dev["v_new"], dev["key_cache"], dev["value_cache"], dev["cache_k_scale"],
+                dev["cache_v_scale"], dev["block_tables"], dev["seq_lens_decoder"], dev["cu_seqlens_q"])
+        out = fd.append_attention_prefill(*args, num_heads=32, max_chunk=max(chunks), cache_quant_type=quant, num_splits=splits)
+        one = fd.append_attention_prefill(*args, num_heads=32, max_chunk=max(chunks), cache_quant_type=quant, num_splits=1)
+        torch.cuda.synchronize()
+        want = oracle.append_attention_prefill(bits(c["q_new"]), bits(c["k_new"]), bits(c["v_new"]), np_of(c["key_cache"]),
+                                               np_of(c["value_cache"]), np_of(c["cache_k_scale"]), np_of(c["cache_v_scale"]),
+                                               np_of(c["block_tables"]), np_of(c["seq_lens_decoder"]), np_of(c["cu_seqlens_q"]),
+                                               32, 8, 128, quant)
+        ok, mx, bad = bf16_close(bits(out), want)
+        assert ok, "splits %r: %d out of tolerance, max %.4g" % (splits, bad, mx)
+        ok, mx, bad = bf16_close(bits(one), want)
+        assert ok, "unsplit: %d out of tolerance, max %.4g" % (bad, mx)
