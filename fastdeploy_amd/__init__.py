@@ -12,6 +12,7 @@ from .ops import (  # noqa: F401
     decode_attention_sparse,
     decode_uses_mfma,
     decode_workspace,
+    prefill_auto_splits,
     splitkv_combine,
     sqattn_select,
     write_cache_kv,

@@ -104,6 +104,41 @@ def test_mixed_batch_step_with_projection_epilogue(oracle):
     assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
 
 
+def test_mixed_step_with_key_splits_for_the_prefill_row(oracle):
+    """One prefill row on a long prefix among decode rows, the host saying so (prefill_rows=1): its query tiles'
+    keys are shared by several workgroups; same cache bytes and outputs as the oracle."""
+    enc, dec = [0, 200, 0, 0], [700, 4500, 64, 3000]
+    c = mixed_case(enc, dec, CACHE_INT8, seed=15, max_pos=8192)
+    assert fd.ops.prefill_auto_splits(1, 32, 200) > 1
+    dev = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
+    out = fd.append_attention(dev["qkv"], dev["key_cache"], dev["value_cache"], dev["seq_lens_encoder"],
+                              dev["seq_lens_decoder"], dev["seq_lens_this_time"], dev["block_tables"],
+                              (dev["rope_cos"], dev["rope_sin"]), dev["cache_k_scale"], dev["cache_v_scale"],
+                              num_heads=32, kv_num_heads=8, max_chunk=200, cu_seqlens_q=dev["cu_seqlens_q"], prefill_rows=1)
+    torch.cuda.synchronize()
+    want, kc, vc = oracle_step(oracle, c, CACHE_INT8)
+    assert np.array_equal(np_of(dev["key_cache"]), kc) and np.array_equal(np_of(dev["value_cache"]), vc)
+    ok, mx, bad = bf16_close(bits(out), want)
+    assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
+    # a workspace sized without the splits still works: as many splits as it holds (none)
+    ws = fd.append_attention_workspace(c["T"], 4, 32, 8, 128, dev["block_tables"].shape[1])
+    kc2, vc2 = c["key_cache"].cuda(), c["value_cache"].cuda()
+    import ctypes
+    from fastdeploy_amd import _lib
+    ex = _lib.StepExtras(None, None, None, 0.0, 1)
+    o2 = torch.empty_like(out)
+    rc = _lib.lib().fdattn_append_attention_ex(
+        dev["qkv"].data_ptr(), kc2.data_ptr(), vc2.data_ptr(), dev["cache_k_scale"].data_ptr(), dev["cache_v_scale"].data_ptr(),
+        dev["rope_cos"].data_ptr(), dev["rope_sin"].data_ptr(), dev["block_tables"].data_ptr(), dev["seq_lens_encoder"].data_ptr(),
+        dev["seq_lens_decoder"].data_ptr(), dev["seq_lens_this_time"].data_ptr(), dev["cu_seqlens_q"].data_ptr(), o2.data_ptr(),
+        ws.data_ptr(), ws.numel(), c["T"], 4, 200, 32, 8, 128, 64, dev["block_tables"].shape[1], kc2.shape[0],
+        dev["rope_cos"].shape[0], 1, CACHE_INT8, 1.0 / 128 ** 0.5, ctypes.addressof(ex), torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert rc == 0
+    ok, mx, bad = bf16_close(bits(o2), want)
+    assert ok, "small workspace: %d out of tolerance, max %.4g" % (bad, mx)
+
+
 def test_decode_only_and_prefill_only_steps_through_the_same_entry(oracle):
     for enc, dec, mc in (([0, 0, 0, 0], [5, 64, 1000, 0], 0), ([64, 1, 257, 0], [0, 0, 100, 0], 257)):
         c = mixed_case(enc, dec, CACHE_INT8, seed=9)
