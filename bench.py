@@ -146,6 +146,35 @@ def other_workloads(args):
         ms = time_events(pf, max(args.steps // 10, 5), 3)
         line("configs[4] append attention (2 x 2048 new on 8192 cached)", ms, "mfma", 2 * syn.prefill_flops(8192, 2048),
              2500.0, "TFLOP/s")
+    if args.workload in ("mixed", "all"):
+        # a serving step: 63 decode rows (ctx U[3584,4608]) and one prefill row appending 512 tokens to 8192 cached ones,
+        # in ONE call (cache write, decode rows, prefill row); with and without the host's hint that one row is a prefill row
+        from fastdeploy_amd.rope import rope_table
+        gm = torch.Generator().manual_seed(3)
+        lens = torch.randint(3584, 4609, (63,), generator=gm).tolist() + [8192]
+        c = syn.decode_case(batch=64, ctx=[n + 1 for n in lens[:63]] + [8192 + 512], seed=2, device=dev, direct_bytes=True)
+        enc = torch.tensor([0] * 63 + [512], dtype=torch.int32, device=dev)
+        dec = torch.tensor(lens, dtype=torch.int32, device=dev)
+        this = torch.tensor([1] * 63 + [512], dtype=torch.int32, device=dev)
+        cu = torch.tensor([0] + list(range(1, 64)) + [63 + 512], dtype=torch.int32, device=dev)
+        T = 63 + 512
+        qkv = torch.randn((T, 48 * 128), generator=g, device=dev).to(torch.bfloat16)
+        rot = rope_table(16384, 128, 500000.0, dev)
+        mb = c["block_tables"].shape[1]
+        outm = torch.empty((T, 32 * 128), dtype=torch.bfloat16, device=dev)
+        for rows in (None, 1):
+            splits = fd.prefill_auto_splits(rows, 32, 512) if rows else 1
+            wsm = fd.append_attention_workspace(T, 64, 32, 8, 128, mb, dev, prefill_splits=splits)
+            stepm = lambda: fd.append_attention(qkv, c["key_cache"], c["value_cache"], enc, dec, this, c["block_tables"], rot,
+                                                c["cache_k_scale"], c["cache_v_scale"], num_heads=32, kv_num_heads=8,
+                                                max_chunk=512, cu_seqlens_q=cu, workspace=wsm, out=outm, prefill_rows=rows)
+            ms = time_events(stepm, max(args.steps // 4, 5), 3)
+            kvb = syn.decode_kv_bytes([n + 1 for n in lens[:63]])
+            line("mixed step: 63 decode rows + 1 prefill row (512 new on 8192 cached), one call%s" %
+                 (", prefill_rows hint -> %d key splits" % splits if rows else ""), ms, "hbm", kvb, HBM_PEAK_GBPS, "GB/s",
+                 {"note": "roofline counts the decode rows' K/V bytes only; the prefill row adds %.1f GFLOP" %
+                          (syn.prefill_flops(8192, 512) / 1e9)})
+        del c
     if args.workload in ("kv_wire", "all"):
         # the sequences of configs[1] leave the cache in wire form and enter another one: HBM copies (read + write)
         from fastdeploy_amd import kv_wire
@@ -173,7 +202,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--pools", type=int, default=2, help="distinct cache pools rotated between steps")
-    ap.add_argument("--workload", default="decode", choices=["decode", "write_decode", "sqattn", "prefill", "kv_wire", "all"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "write_decode", "sqattn", "prefill", "mixed", "kv_wire", "all"],
                     help="decode = the headline metric (default); the others print one line per kernel of that row")
     ap.add_argument("--calibrate", action="store_true",
                     help="kept for the profiling command line: the 1 GiB device copy (the yardstick the HBM byte "

@@ -38,7 +38,7 @@ class ForwardMeta:
     max_enc_len_this_time: Optional[int] = None  # host-side bound on seq_lens_encoder (0: no prefill row); found with one sync if None
     cu_seqlens_q: Optional[torch.Tensor] = None  # filled by init_attention_metadata
     num_tokens: int = 0                          # filled by init_attention_metadata
-    prefill_rows: Optional[int] = None           # host-side count of prefill rows (None: unknown, no key splits)
+    prefill_rows: Optional[int] = None           # exact count of rows with seq_lens_encoder > 0, if known (None: unknown)
     prefill_splits: int = 1                      # filled by init_attention_metadata
     extra: dict = field(default_factory=dict)
 

@@ -24,6 +24,7 @@ struct PrefillArgs {
   // key tiles and leaves a partial (unnormalised o in fp32, exponent reference m, weight sum l) for the merge
   int n_splits;
   int tile_tokens;  // queries per workgroup of this launch (128 or 256), for the merge kernel
+  int rows;         // MFMA kernel: sequences the grid covers - the batch, or the number of prefill rows when the host gave it
   float* part_o;   // [n_splits][num_tokens][hq][128]
   float* part_ml;  // [n_splits][num_tokens][hq][2]
 };

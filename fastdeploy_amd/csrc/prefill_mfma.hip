@@ -126,6 +126,27 @@ __device__ __forceinline__ u32 lds_addr(const void* p) {
 
 }  // namespace
 
+// The sequence a grid row stands for.  A grid over the whole batch: the row itself.  A grid over the prefill rows
+// only (the host said how many there are): the r-th sequence with seq_lens_encoder > 0, found by every wavefront
+// with ballots over the batch; -1 if there are fewer.
+__device__ __forceinline__ int sequence_of_row(const PrefillArgs& a, int r) {
+  if (a.rows >= a.batch || !a.seq_lens_encoder) return r;
+  const int lane = threadIdx.x & 63;
+  int seen = 0;
+  for (int base = 0; base < a.batch; base += 64) {
+    const int idx = base + lane;
+    const unsigned long long m = __ballot(idx < a.batch && a.seq_lens_encoder[idx] > 0);
+    const int c = __popcll(m);
+    if (r < seen + c) {
+      unsigned long long mm = m;
+      for (int k = seen; k < r; ++k) mm &= mm - 1;  // drop the set bits before the wanted one
+      return base + __ffsll((long long)mm) - 1;
+    }
+    seen += c;
+  }
+  return -1;
+}
+
 // how many of the launch's max_splits key splits a walk of n_tiles tiles uses
 __device__ __forceinline__ int splits_of(int n_tiles, int max_splits) { return min(max(n_tiles / 32, 1), max_splits); }
 
@@ -142,8 +163,8 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   // head) pair - every workgroup that reads one pair's K and V shares one L2 - and inside an XCD the
   // query tiles come longest first (the causal rows of late tokens walk more keys), so every XCD gets
   // the same mix of long and short workgroups and the short ones fill the end of the launch.
-  const int G = a.hq / a.hkv, pairs = a.batch * a.hkv, units = a.batch * a.hq;
-  int qt, b, qh;
+  const int G = a.hq / a.hkv, pairs = a.rows * a.hkv, units = a.rows * a.hq;
+  int qt, b, qh;  // b: the grid row first, the sequence below
   if ((pairs & 7) == 0) {
     const int ppx = pairs >> 3;  // pairs per XCD
     const int x = blockIdx.x & 7, jx = blockIdx.x >> 3;
@@ -158,6 +179,8 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
     qh = u - b * a.hq;
   }
   const int h = qh / G;
+  b = sequence_of_row(a, b);
+  if (b < 0) return;
   const int tok0 = a.cu_seqlens_q[b], n_b = a.cu_seqlens_q[b + 1] - tok0, p = a.seq_lens_decoder[b];
   const int q0 = qt * BM;
   if (q0 >= n_b) return;
@@ -487,7 +510,8 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
 // Merge of the split partials: one wavefront per new token of a prefill row, looping over the query heads;
 // lane = two channels.  grid (ceil(max_chunk / 4), batch), 256 threads.
 __global__ __launch_bounds__(256) void prefill_merge_kernel(PrefillArgs a) {
-  const int b = blockIdx.y, lane = threadIdx.x & 63;
+  const int b = sequence_of_row(a, blockIdx.y), lane = threadIdx.x & 63;
+  if (b < 0) return;
   if (a.seq_lens_encoder && a.seq_lens_encoder[b] <= 0) return;
   const int tok0 = a.cu_seqlens_q[b], n_b = a.cu_seqlens_q[b + 1] - tok0;
   const int i = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -533,7 +557,7 @@ hipError_t launch_one(const PrefillArgs& a, int max_chunk, hipStream_t s) {
   PrefillArgs args = a;
   args.q_tiles = (max_chunk + BM - 1) / BM;
   args.tile_tokens = BM;
-  const dim3 grid((unsigned)a.batch * a.hq * args.q_tiles, a.n_splits), block(64 * NW);
+  const dim3 grid((unsigned)a.rows * a.hq * args.q_tiles, a.n_splits), block(64 * NW);
   const size_t shm = (size_t)kSlots * BUF_ELEMS * sizeof(uint16_t);  // 151,552 B
   // the dynamic LDS limit is a per-device property of the kernel: raise it once on each device
   static std::atomic<unsigned long long> raised{0};  // bit d: done on device d (one word per instantiation)
@@ -585,15 +609,16 @@ int prefill_mfma_launch(const PrefillArgs& a_in, int max_chunk, int quant, hipSt
   if (n_splits > kMaxSplits) n_splits = kMaxSplits;
   while (n_splits > 1 && (!workspace || workspace_bytes < prefill_split_workspace_bytes(a.num_tokens, a.hq, n_splits))) --n_splits;
   a.n_splits = n_splits < 1 ? 1 : n_splits;
+  a.rows = rows_hint > 0 && rows_hint < a.batch && a.seq_lens_encoder ? rows_hint : a.batch;
   a.part_o = (float*)workspace;
   a.part_ml = a.part_o + (size_t)a.n_splits * a.num_tokens * a.hq * HD;
-  if ((long long)a.batch * a.hq * ((max_chunk + 127) / 128) > 0x7fffffffLL)
+  if ((long long)a_in.batch * a_in.hq * ((max_chunk + 127) / 128) > 0x7fffffffLL)
     return fail(FDATTN_ERR_SHAPE, "fdattn_append_attention_prefill: too many workgroups for one launch");
   // 256-token workgroups share each staged tile among 8 wavefronts (their two groups alternate between the MFMA
   // units and the vector ALU); short chunks keep 128
   // when they would still leave CUs without a workgroup (one fits a CU), 128-token workgroups cover twice as
   // many CUs: 10-14 % faster at e.g. 2 x 512 tokens, although a 4-wavefront workgroup overlaps nothing
-  const bool wide = wide_workgroups(rows_hint > 0 ? rows_hint : a.batch, a.hq, max_chunk, a.n_splits);
+  const bool wide = wide_workgroups(a.rows, a.hq, max_chunk, a.n_splits);
   hipError_t e;
   if (quant == FDATTN_CACHE_INT8)
     e = wide ? launch_one<FDATTN_CACHE_INT8, 8>(a, max_chunk, s) : launch_one<FDATTN_CACHE_INT8, 4>(a, max_chunk, s);
@@ -604,7 +629,7 @@ int prefill_mfma_launch(const PrefillArgs& a_in, int max_chunk, int quant, hipSt
   int rc = check_launch("fdattn_append_attention_prefill (mfma)");
   if (rc || a.n_splits <= 1) return rc;
   a.tile_tokens = wide ? 256 : 128;
-  hipLaunchKernelGGL(prefill_merge_kernel, dim3((max_chunk + 3) / 4, a.batch), dim3(256), 0, s, a);
+  hipLaunchKernelGGL(prefill_merge_kernel, dim3((max_chunk + 3) / 4, a.rows), dim3(256), 0, s, a);
   return check_launch("fdattn_append_attention_prefill (merge)");
 }
 

@@ -375,9 +375,10 @@ def append_attention(qkv, key_cache, value_cache, seq_lens_encoder, seq_lens_dec
     to their cached prefix and causally to their own chunk; slots without a token
     are skipped.  max_chunk bounds the tokens of a prefill row (0: the step has none, decode only).
     qkv_bias / q_norm_weight / k_norm_weight / rms_norm_eps: the projection's epilogue, as in write_cache_kv.
-    prefill_rows: how many rows of the step are prefill rows, if the host knows (None: unknown).  When those rows
-    alone would leave CUs idle, every query tile is shared by prefill_auto_splits(prefill_rows, num_heads,
-    max_chunk) workgroups; a workspace passed in must have been sized with that number of splits.
+    prefill_rows: how many sequences of the step have seq_lens_encoder > 0, if the host knows (None: unknown).  A
+    promise, not a guess - the prefill pass then covers that many prefill rows only (no workgroups for decode rows),
+    and when they alone would leave CUs idle every query tile is shared by prefill_auto_splits(prefill_rows,
+    num_heads, max_chunk) workgroups (as many as a workspace passed in has room for).
     Returns bf16 [num_tokens, num_heads*head_dim]."""
     nb, hkv, bs, d = _cache_dims(key_cache, value_cache)
     if hkv != kv_num_heads:

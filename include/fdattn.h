@@ -104,12 +104,15 @@ FDATTN_API int fdattn_write_cache_kv(
  *   k_norm_weight   f32 [head_dim]  the rotation; the same for every K head (V is not normed)
  * All arithmetic is fp32 with every operation rounded on its own; nothing is rounded to bf16
  * between the norm and the rotation.  The norm needs head_dim = 16 * 2^n.
- *   prefill_rows    (fdattn_append_attention_ex only) the number of prefill rows of the step, if the
- *                   host knows it (0 = unknown).  When those rows alone would leave CUs idle - one
- *                   sequence's chunk of a few hundred tokens among decode rows - every query tile
- *                   is shared by fdattn_prefill_auto_splits(prefill_rows, hq, max_chunk) workgroups,
- *                   each walking a part of its keys; the workspace must then come from
- *                   fdattn_append_attention_workspace_bytes_ex with that number of splits.
+ *   prefill_rows    (fdattn_append_attention_ex only) the number of sequences with
+ *                   seq_lens_encoder > 0 in this step, if the host knows it (0 = unknown: the prefill
+ *                   pass covers the whole batch).  It is a promise, not a guess: the prefill pass
+ *                   then covers the first prefill_rows such sequences only.  With it the pass launches
+ *                   no workgroups for decode rows, and when the prefill rows alone would leave CUs
+ *                   idle - one sequence's chunk of a few hundred tokens among decode rows - every
+ *                   query tile is shared by fdattn_prefill_auto_splits(prefill_rows, hq, max_chunk)
+ *                   workgroups, each walking a part of its keys, if the workspace has room for their
+ *                   partials (fdattn_append_attention_workspace_bytes_ex with that number of splits).
  */
 typedef struct fdattn_step_extras {
   const void* qkv_bias;
