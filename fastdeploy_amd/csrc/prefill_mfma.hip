@@ -56,6 +56,7 @@ constexpr int LDK = 136;  // 16-bit elements per K row in LDS (272 B)
 constexpr int LDV = 160;  // 16-bit elements per V row in LDS (320 B)
 constexpr int K_ELEMS = BN * LDK, BUF_ELEMS = BN * (LDK + LDV);
 constexpr int kSlots = 4;  // K/V tile slots in LDS (three are live at a time; four make the slot of a tile a mask)
+constexpr int kMaxSplits = 8;  // workgroups that may share one query tile's keys
 constexpr float kSumLimit = 1024.0f;  // a query's weight sum over one tile above which its exponent reference is raised
 
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
@@ -507,39 +508,50 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
     }
 }
 
-// Merge of the split partials: one wavefront per new token of a prefill row, looping over the query heads;
-// lane = two channels.  grid (ceil(max_chunk / 4), batch), 256 threads.
+// Merge of the split partials: one wavefront per (new token of a prefill row, query head), lane = two channels.
+// grid (ceil(max_chunk * hq / 4), rows), 256 threads.
 __global__ __launch_bounds__(256) void prefill_merge_kernel(PrefillArgs a) {
   const int b = sequence_of_row(a, blockIdx.y), lane = threadIdx.x & 63;
   if (b < 0) return;
   if (a.seq_lens_encoder && a.seq_lens_encoder[b] <= 0) return;
   const int tok0 = a.cu_seqlens_q[b], n_b = a.cu_seqlens_q[b + 1] - tok0;
-  const int i = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int unit = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int i = unit / a.hq, qh = unit - i * a.hq;
   if (i >= n_b) return;
   // the split count of this token's query tile, as the main kernel worked it out
   const int q0 = i / a.tile_tokens * a.tile_tokens;
   const int n_tiles = (a.seq_lens_decoder[b] + BN - 1) / BN + (min(n_b, q0 + a.tile_tokens) + BN - 1) / BN;
   const int n_splits = splits_of(n_tiles, a.n_splits);
   if (n_splits <= 1) return;  // the row is final already
-  for (int qh = 0; qh < a.hq; ++qh) {
-    const size_t row0 = ((size_t)(tok0 + i)) * a.hq + qh, stride = (size_t)a.num_tokens * a.hq;
-    float M = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) M = fmaxf(M, a.part_ml[(row0 + s * stride) * 2]);
-    float L = 0.f, o0 = 0.f, o1 = 0.f;
-    if (M > -INFINITY) {
-      for (int s = 0; s < n_splits; ++s) {
-        const float ms = a.part_ml[(row0 + s * stride) * 2];
-        if (ms == -INFINITY) continue;
-        const float f = __builtin_amdgcn_exp2f(ms - M);
-        L += a.part_ml[(row0 + s * stride) * 2 + 1] * f;
-        const float2 v = *reinterpret_cast<const float2*>(a.part_o + (row0 + s * stride) * HD + 2 * lane);
-        o0 += v.x * f;
-        o1 += v.y * f;
-      }
+  const size_t row0 = ((size_t)(tok0 + i)) * a.hq + qh, stride = (size_t)a.num_tokens * a.hq;
+  // every partial is requested before any is used: one round trip to memory, not one per split
+  float ms[kMaxSplits], ls[kMaxSplits];
+  float2 v[kMaxSplits];
+#pragma unroll
+  for (int s = 0; s < kMaxSplits; ++s)
+    if (s < n_splits) {
+      ms[s] = a.part_ml[(row0 + s * stride) * 2];
+      ls[s] = a.part_ml[(row0 + s * stride) * 2 + 1];
+      // an empty share (m = -inf) has no o: the load is skipped by the weight 0 below, its address is still valid memory
+      v[s] = *reinterpret_cast<const float2*>(a.part_o + (row0 + s * stride) * HD + 2 * lane);
     }
-    const float inv = L > 0.f ? 1.0f / L : 0.f;
-    *reinterpret_cast<u32*>(a.out + row0 * HD + 2 * lane) = pack_bf16(o0 * inv, o1 * inv);
+  float M = -INFINITY;
+#pragma unroll
+  for (int s = 0; s < kMaxSplits; ++s)
+    if (s < n_splits) M = fmaxf(M, ms[s]);
+  float L = 0.f, o0 = 0.f, o1 = 0.f;
+  if (M > -INFINITY) {
+#pragma unroll
+    for (int s = 0; s < kMaxSplits; ++s)
+      if (s < n_splits && ms[s] > -INFINITY) {
+        const float f = __builtin_amdgcn_exp2f(ms[s] - M);
+        L += ls[s] * f;
+        o0 += v[s].x * f;
+        o1 += v[s].y * f;
+      }
   }
+  const float inv = L > 0.f ? 1.0f / L : 0.f;
+  *reinterpret_cast<u32*>(a.out + row0 * HD + 2 * lane) = pack_bf16(o0 * inv, o1 * inv);
 }
 
 bool prefill_mfma_supported(int hq, int hkv, int d, int bs, int quant) {
@@ -548,8 +560,6 @@ bool prefill_mfma_supported(int hq, int hkv, int d, int bs, int quant) {
 }
 
 namespace {
-
-constexpr int kMaxSplits = 8;
 
 template <int QUANT, int NW>
 hipError_t launch_one(const PrefillArgs& a, int max_chunk, hipStream_t s) {
@@ -629,7 +639,7 @@ int prefill_mfma_launch(const PrefillArgs& a_in, int max_chunk, int quant, hipSt
   int rc = check_launch("fdattn_append_attention_prefill (mfma)");
   if (rc || a.n_splits <= 1) return rc;
   a.tile_tokens = wide ? 256 : 128;
-  hipLaunchKernelGGL(prefill_merge_kernel, dim3((max_chunk + 3) / 4, a.rows), dim3(256), 0, s, a);
+  hipLaunchKernelGGL(prefill_merge_kernel, dim3(((long long)max_chunk * a.hq + 3) / 4, a.rows), dim3(256), 0, s, a);
   return check_launch("fdattn_append_attention_prefill (merge)");
 }
 
