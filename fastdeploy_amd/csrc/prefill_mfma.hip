@@ -149,7 +149,7 @@ __device__ __forceinline__ int sequence_of_row(const PrefillArgs& a, int r) {
 }
 
 // how many of the launch's max_splits key splits a walk of n_tiles tiles uses
-__device__ __forceinline__ int splits_of(int n_tiles, int max_splits) { return min(max(n_tiles / 32, 1), max_splits); }
+__device__ __forceinline__ int splits_of(int n_tiles, int max_splits) { return min(max(n_tiles / 16, 1), max_splits); }
 
 template <int QUANT, int NW>
 __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
@@ -198,7 +198,7 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   const int n_chk = (min(n_b, q0 + BM) + BN - 1) / BN;
   const int n_tiles = n_pre + n_chk;
   // this workgroup's share of the key tiles: [t0, t1).  A share is worth its fixed costs (prologue, partial,
-  // merge) from about 32 tiles on: shorter walks are split less, or not at all - then split 0 walks everything
+  // merge) from about 16 tiles on: shorter walks are split less, or not at all - then split 0 walks everything
   // and writes the final rows itself.
   const int n_splits = splits_of(n_tiles, a.n_splits);
   if ((int)blockIdx.y >= n_splits) return;
