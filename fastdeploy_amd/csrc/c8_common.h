@@ -89,11 +89,29 @@ __device__ __forceinline__ void dma_tile(const uint8_t* gtile_in, u32 lds_addr, 
       : "memory", "scc");
 }
 
+// Direct global->LDS load of 64 consecutive floats (one per lane, lane l lands at byte 4l): the scale row of one
+// (block, head) tile of the formats that keep one scale per stored row.  One load for the vmcnt bookkeeping.
+__device__ __forceinline__ void dma_row64(const float* grow_in, u32 lds_addr, u32 lane_x4) {
+  const unsigned long long gp = (unsigned long long)grow_in;
+  const u32 glo = __builtin_amdgcn_readfirstlane((u32)gp), ghi = __builtin_amdgcn_readfirstlane((u32)(gp >> 32));
+  const float* grow = (const float*)(((unsigned long long)ghi << 32) | glo);
+  u32 saved_m0;
+  asm volatile(
+      "s_mov_b32 %[sv], m0\n\t"
+      "s_mov_b32 m0, %[l]\n\ts_nop 0\n\t"
+      "global_load_lds_dword %[o], %[g]\n\t"
+      "s_mov_b32 m0, %[sv]\n\t"
+      : [sv] "=&s"(saved_m0)
+      : [l] "s"(lds_addr), [g] "s"(grow), [o] "v"(lane_x4)
+      : "memory", "scc");
+}
+
 __device__ __forceinline__ u32 lds_addr_of(const void* p) {
   return (u32)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
 }
 
 __device__ __forceinline__ void wait_vm8() { asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); }
+__device__ __forceinline__ void wait_vm10() { asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); }
 __device__ __forceinline__ void wait_vm0() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ void wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ void wave_sync() {
@@ -119,6 +137,8 @@ struct PairRaw {
   float4 ks[2][4];  // their K scales
 };
 
+// k_scale: the per-channel K scales [hkv, 128], or NULL (all ones: the scales are per stored row and are applied
+// to the scores)
 __device__ __forceinline__ PairRaw load_pair_issue(const uint16_t* q, const float* k_scale, int hkv, int p, int row, int lane) {
   const int h = p % hkv;  // row: the sequence's row of q
   const int m = lane & 15, g = lane >> 4, head = m >> 2;
@@ -131,7 +151,8 @@ __device__ __forceinline__ PairRaw load_pair_issue(const uint16_t* q, const floa
     r.w[s][0] = *reinterpret_cast<const uint4*>(qrow + c0);
     r.w[s][1] = *reinterpret_cast<const uint4*>(qrow + c0 + 8);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) r.ks[s][i] = *reinterpret_cast<const float4*>(ks + c0 + 4 * i);
+    for (int i = 0; i < 4; ++i)
+      r.ks[s][i] = k_scale ? *reinterpret_cast<const float4*>(ks + c0 + 4 * i) : make_float4(1.f, 1.f, 1.f, 1.f);
   }
   return r;
 }

@@ -18,7 +18,7 @@ struct WriterArgs {
   uint16_t* v_out;
   uint8_t* key_cache;
   uint8_t* value_cache;
-  const float* k_scale;
+  const float* k_scale;  // per channel [hkv, d]; DYN: the scale cache [num_blocks, hkv, bs], written here
   const float* v_scale;
   const float* rope_cos;
   const float* rope_sin;
@@ -51,7 +51,8 @@ __device__ __forceinline__ u32 quant1(float x, float s) {
 //   heads [0, hq)            Q   : rotate, round to bf16, store to q_out
 //   heads [hq, hq+hkv)       K   : rotate, (bf16 -> k_out), quantise, store to key_cache
 //   heads [hq+hkv, hq+2hkv)  V   : (copy -> v_out), quantise, store to value_cache
-template <int QUANT>
+// DYN: one scale per stored row, (largest magnitude of the row) / 127 or / 448, stored beside the row.
+template <int QUANT, bool DYN>
 __global__ __launch_bounds__(256) void write_cache_kv_kernel(WriterArgs a) {
   // grid (units of a token / 256, tokens): the token - and with it the sequence, the position and the
   // cache slot - is uniform over the workgroup and is worked out in scalar registers
@@ -224,12 +225,29 @@ __global__ __launch_bounds__(256) void write_cache_kv_kernel(WriterArgs a) {
   if (lb >= a.max_blocks) return;
   const int pb = a.block_tables[(size_t)b * a.max_blocks + lb];
   if (pb < 0 || pb >= a.num_blocks) return;
-  const float* sc = (is_k ? a.k_scale : a.v_scale) + (size_t)h * a.d;
   uint8_t* dst = (is_k ? a.key_cache : a.value_cache) + (((size_t)pb * a.hkv + h) * a.bs + slot) * a.d;
-  float4 s1a = *reinterpret_cast<const float4*>(sc + c1), s1b = *reinterpret_cast<const float4*>(sc + c1 + 4);
-  float4 s2a = *reinterpret_cast<const float4*>(sc + c2), s2b = *reinterpret_cast<const float4*>(sc + c2 + 4);
-  float s1[8] = {s1a.x, s1a.y, s1a.z, s1a.w, s1b.x, s1b.y, s1b.z, s1b.w};
-  float s2[8] = {s2a.x, s2a.y, s2a.z, s2a.w, s2b.x, s2b.y, s2b.z, s2b.w};
+  float s1[8], s2[8];
+  if (DYN) {
+    // the row's largest magnitude: over this thread's 16 channels, then over the d/16 threads of the head
+    // (a butterfly; the host checked that d/16 is a power of two).  fmaxf drops NaNs, as the oracle's does.
+    float m = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) m = fmaxf(m, fmaxf(fabsf(g1[i]), fabsf(g2[i])));
+    for (int o = 1; o < units_per_head; o <<= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    const float sc = m > 0.f ? __fdiv_rn(m, QUANT == FDATTN_CACHE_INT8 ? 127.0f : 448.0f) : 1.0f;
+    if (u == 0)
+      const_cast<float*>(is_k ? a.k_scale : a.v_scale)[((size_t)pb * a.hkv + h) * a.bs + slot] = sc;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s1[i] = s2[i] = sc;
+  } else {
+    const float* sc = (is_k ? a.k_scale : a.v_scale) + (size_t)h * a.d;
+    float4 s1a = *reinterpret_cast<const float4*>(sc + c1), s1b = *reinterpret_cast<const float4*>(sc + c1 + 4);
+    float4 s2a = *reinterpret_cast<const float4*>(sc + c2), s2b = *reinterpret_cast<const float4*>(sc + c2 + 4);
+    const float t1[8] = {s1a.x, s1a.y, s1a.z, s1a.w, s1b.x, s1b.y, s1b.z, s1b.w};
+    const float t2[8] = {s2a.x, s2a.y, s2a.z, s2a.w, s2b.x, s2b.y, s2b.z, s2b.w};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { s1[i] = t1[i]; s2[i] = t2[i]; }
+  }
   u32 q1[2] = {0, 0}, q2[2] = {0, 0};
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
@@ -266,6 +284,12 @@ extern "C" int fdattn_write_cache_kv_ex(
     int cache_quant_type, const fdattn_step_extras* extras, void* stream) {
   const fdattn_step_extras none = {nullptr, nullptr, nullptr, 0.f, 0};
   const fdattn_step_extras& ep = extras ? *extras : none;
+  if (quant_dynamic(cache_quant_type)) {
+    const int u = head_dim / 16;
+    if (head_dim % 16 != 0 || u <= 0 || (u & (u - 1)) != 0 || u > 64)
+      return fail(FDATTN_ERR_SHAPE, "fdattn_write_cache_kv: the dynamic cache formats need head_dim = 16 * a power "
+                  "of two up to 1024, got %d", head_dim);
+  }
   if (ep.q_norm_weight || ep.k_norm_weight) {
     const int u = head_dim / 16;
     if (head_dim % 16 != 0 || u <= 0 || (u & (u - 1)) != 0 || u > 64)
@@ -289,7 +313,7 @@ extern "C" int fdattn_write_cache_kv_ex(
     return fail(FDATTN_ERR_SHAPE, "fdattn_write_cache_kv: max_pos must be positive with a rope table");
   if (rope_style != FDATTN_ROPE_INTERLEAVED && rope_style != FDATTN_ROPE_NEOX)
     return fail(FDATTN_ERR_QUANT, "fdattn_write_cache_kv: unknown rope_style %d", rope_style);
-  if (cache_quant_type != FDATTN_CACHE_INT8 && cache_quant_type != FDATTN_CACHE_FP8_E4M3)
+  if (!quant_known(cache_quant_type))
     return fail(FDATTN_ERR_QUANT, "fdattn_write_cache_kv: unknown cache_quant_type %d", cache_quant_type);
   if (num_tokens == 0) return 0;
   WriterArgs a{(const uint16_t*)qkv, (uint16_t*)q_out, (uint16_t*)k_out, (uint16_t*)v_out,
@@ -304,9 +328,13 @@ extern "C" int fdattn_write_cache_kv_ex(
     a.tok0 = t0;
     const dim3 grid((units + 255) / 256, num_tokens - t0 < 65535 ? num_tokens - t0 : 65535);
     if (cache_quant_type == FDATTN_CACHE_INT8)
-      hipLaunchKernelGGL(write_cache_kv_kernel<FDATTN_CACHE_INT8>, grid, dim3(256), 0, s, a);
+      hipLaunchKernelGGL((write_cache_kv_kernel<FDATTN_CACHE_INT8, false>), grid, dim3(256), 0, s, a);
+    else if (cache_quant_type == FDATTN_CACHE_FP8_E4M3)
+      hipLaunchKernelGGL((write_cache_kv_kernel<FDATTN_CACHE_FP8_E4M3, false>), grid, dim3(256), 0, s, a);
+    else if (cache_quant_type == FDATTN_CACHE_INT8_DYNAMIC)
+      hipLaunchKernelGGL((write_cache_kv_kernel<FDATTN_CACHE_INT8, true>), grid, dim3(256), 0, s, a);
     else
-      hipLaunchKernelGGL(write_cache_kv_kernel<FDATTN_CACHE_FP8_E4M3>, grid, dim3(256), 0, s, a);
+      hipLaunchKernelGGL((write_cache_kv_kernel<FDATTN_CACHE_FP8_E4M3, true>), grid, dim3(256), 0, s, a);
   }
   return check_launch("fdattn_write_cache_kv");
 }

@@ -15,7 +15,7 @@ static int check_decode_args(const char* fn, const void* q, const void* kc, cons
       num_blocks <= 0)
     return fail(FDATTN_ERR_SHAPE, "%s: bad shape batch=%d hq=%d hkv=%d head_dim=%d block_size=%d max_blocks=%d "
                 "num_blocks=%d", fn, batch, hq, hkv, d, bs, max_blocks, num_blocks);
-  if (quant != FDATTN_CACHE_INT8 && quant != FDATTN_CACHE_FP8_E4M3)
+  if (!quant_known(quant))
     return fail(FDATTN_ERR_QUANT, "%s: unknown cache_quant_type %d", fn, quant);
   return 0;
 }

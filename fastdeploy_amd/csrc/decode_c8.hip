@@ -4,10 +4,10 @@
 // Work unit: one (sequence, KV head, cache block) = an 8 KiB K tile + an 8 KiB V tile,
 // each contiguous in HBM.  The block list of every (sequence, KV head) pair is cut into
 // chunks of `chunk` units; one workgroup of 4 wavefronts takes one chunk (grid = chunks
-// per pair x pairs, workgroups past the end of a list do nothing).  Chunks are short
-// (24 units = 384 KiB by default), so the hardware dispatcher balances uneven sequence
-// lengths, and they need no scan to be found: pair and chunk follow from the block index,
-// the physical blocks from one coalesced read of the block table.
+// per pair x pairs, workgroups past the end of a list do nothing).  The chunk length is
+// picked so that the launch fills the GPU's workgroup slots once (c8_pick_chunk): as
+// few, as long workgroups as that allows, up to 128 units each.  Pair and chunk follow
+// from the block index, the physical blocks from one coalesced read of the block table.
 //
 // Inside a workgroup every wavefront is autonomous: it takes units wave, wave+4, ... of
 // the chunk, owns a K slot, a V slot and a P slot in LDS, fills them with direct
@@ -23,6 +23,10 @@
 //     e4m3 residual limbs (16 significant bits).
 // The per-channel K scale is folded into q, the V scale is applied once to the output.
 // V tiles are transposed for free by ds_read_b64_tr_b8.
+// The formats with one scale per stored row (DYN) bring a unit's 64 K scales and 64 V
+// scales into LDS with two more direct loads; the K scale multiplies the token's score,
+// the V scale - relative to the unit's largest - rides on the token's softmax weight
+// before the weight is cut into limbs, and the unit's largest scales its P.V product.
 //
 // At the end the 4 wavefronts merge their (m, l, o) through LDS.  A pair with a single
 // chunk is finished on the spot (bf16 output written); otherwise the workgroup leaves one
@@ -42,7 +46,7 @@ struct C8Args {
   const uint16_t* q;
   const uint8_t* key_cache;
   const uint8_t* value_cache;
-  const float* k_scale;
+  const float* k_scale;  // [hkv, 128] per channel; DYN: [num_blocks, hkv, 64] per stored row
   const float* v_scale;
   const int32_t* block_tables;
   const int32_t* seq_lens_decoder;
@@ -58,6 +62,7 @@ struct C8Args {
   int chunk;            // units per workgroup
   int chunks_per_pair;  // grid.x
   float sm_scale_log2;  // softmax_scale * log2(e)
+  int dyn;              // scales per stored row: the output takes no per-channel V scale
 };
 
 // Length of the pair's block list: every block of the sequence, or the kept ones.
@@ -67,11 +72,12 @@ __device__ __forceinline__ int pair_units(const C8Args& a, int p, int kv_len) {
   return min((max(kv_len, 0) + kBS - 1) / kBS, a.max_blocks);
 }
 
-template <int QUANT, bool SPARSE>
+template <int QUANT, bool SPARSE, bool DYN>
 __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
   __shared__ __attribute__((aligned(16))) uint8_t ldsK[kWaves][kTileB];
   __shared__ __attribute__((aligned(16))) uint8_t ldsV[kWaves][kTileB];
   __shared__ __attribute__((aligned(16))) uint8_t ldsP[kWaves][1024];
+  __shared__ __attribute__((aligned(16))) float ldsS[DYN ? kWaves : 1][2 * kBS];  // DYN: a unit's K scales, V scales
   const int lane = threadIdx.x & 63;
   const int wv = uni(threadIdx.x >> 6);
   const int ticket = blockIdx.x;
@@ -101,7 +107,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
   }
   int row;
   if (!decode_row(a.rows, b, row)) return;
-  const PairRaw raw = load_pair_issue(a.q, a.k_scale, a.hkv, p, row, lane);  // in flight with the table entries
+  const PairRaw raw = load_pair_issue(a.q, DYN ? nullptr : a.k_scale, a.hkv, p, row, lane);  // in flight with the table entries
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
   const int n_p = pair_units<SPARSE>(a, p, kv_len);
   const int cnt = min(a.chunk, n_p - first);  // <= 0: past the end of this pair's list
@@ -142,6 +148,18 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
   const uint8_t* const kbase = a.key_cache + (size_t)h * tile_stride;
   const uint8_t* const vbase = a.value_cache + (size_t)h * tile_stride;
   const size_t blk_stride = (size_t)a.hkv * tile_stride;
+  // DYN: the scale rows of a unit travel with its K tile (the V row too: it is needed before the V tile is)
+  const float* const sbuf = ldsS[DYN ? wv : 0];
+  const u32 saddr = uni((int)lds_addr_of(sbuf));
+  const u32 lane_x4 = (u32)lane * 4u;
+  auto fetch_k = [&](int blk) {
+    dma_tile(kbase + (size_t)blk * blk_stride, kaddr, offK);
+    if (DYN) {
+      const size_t srow = ((size_t)blk * a.hkv + h) * kBS;
+      dma_row64(a.k_scale + srow, saddr, lane_x4);
+      dma_row64(a.v_scale + srow, saddr + 4 * kBS, lane_x4);
+    }
+  };
 
   PairState st;
   st.m = -INFINITY;
@@ -152,7 +170,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
   if (wv < cnt) {  // this wavefront has units wv, wv + 4, ...
     int pb = unit_pb(wv);
     int valid = unit_valid(wv);
-    dma_tile(kbase + (size_t)pb * blk_stride, kaddr, offK);
+    fetch_k(pb);
     dma_tile(vbase + (size_t)pb * blk_stride, vaddr, offV);
     load_pair_finish<QUANT>(raw, a.sm_scale_log2, lane, st);
 
@@ -165,7 +183,14 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
       }
 
       // ---------------- S = Q K^T : rows = head*4 + limb, columns = token slots
-      wait_vm8();  // K(j) landed; V(j) may still be in flight
+      wait_vm8();  // K(j) landed (DYN: and the unit's scale rows); V(j) may still be in flight
+      float kt[4] = {1.f, 1.f, 1.f, 1.f}, vt[4] = {1.f, 1.f, 1.f, 1.f};  // scales of this lane's tokens 4n .. 4n+3
+      if (DYN) {
+        const float4 k4 = *reinterpret_cast<const float4*>(sbuf + 4 * n16);
+        const float4 v4 = *reinterpret_cast<const float4*>(sbuf + kBS + 4 * n16);
+        kt[0] = k4.x; kt[1] = k4.y; kt[2] = k4.z; kt[3] = k4.w;
+        vt[0] = v4.x; vt[1] = v4.y; vt[2] = v4.z; vt[3] = v4.w;
+      }
       v4i S[4];
       v4f Sf[4];
 #pragma unroll
@@ -196,8 +221,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
           Sf[stl] = acc;
         }
       }
-      wait_lgkm0();  // K tile is in registers: its slot may be refilled
-      if (has_next) dma_tile(kbase + (size_t)pbn * blk_stride, kaddr, offK);
+      wait_lgkm0();  // K tile (and the scale rows) are in registers: their slots may be refilled
+      if (has_next) fetch_k(pbn);
 
       // ---------------- online softmax in the S layout: lane = (token slot n, head g)
       float sv[4];
@@ -209,7 +234,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
           s = st.rs * ((float)S[stl].x + 128.0f * (float)S[stl].y + 16384.0f * (float)S[stl].z);
         else
           s = st.rs * ((Sf[stl].x + Sf[stl].y) + (Sf[stl].z + Sf[stl].w));
-        s = (4 * n16 + stl < valid) ? s : -INFINITY;
+        if (DYN) s *= kt[stl];
+        s = (4 * n16 + stl < valid) ? s : -INFINITY;  // (a slot past the end may hold any scale, NaN included)
         sv[stl] = s;
         mb = fmaxf(mb, s);
       }
@@ -221,13 +247,33 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
       st.m = m_new;
       u32 pw[4] = {0, 0, 0, 0};
       float lsum = 0.f;
+      float prs[4];
+#pragma unroll
+      for (int stl = 0; stl < 4; ++stl) prs[stl] = __builtin_amdgcn_exp2f(sv[stl] - m_use);  // in [0, 1]
+      // DYN: what is cut into limbs is weight x V scale of the token, relative to the largest such product of the
+      // unit (so the unit's heaviest contribution always has full precision); that largest product scales the
+      // unit's P.V.  The weight sum takes the plain weights.
+      float vmax = 1.f;
+      if (DYN) {
+        float wm = 0.f;
+#pragma unroll
+        for (int stl = 0; stl < 4; ++stl) {
+          lsum += prs[stl] * (QUANT == FDATTN_CACHE_INT8 ? 268435456.0f : 256.0f);
+          prs[stl] *= (4 * n16 + stl < valid) ? vt[stl] : 0.f;  // (a slot past the end may hold any scale)
+          wm = fmaxf(wm, prs[stl]);
+        }
+        vmax = row_max16(wm);
+        const float inv = vmax > 0.f ? 1.0f / vmax : 0.f;
+#pragma unroll
+        for (int stl = 0; stl < 4; ++stl) prs[stl] *= inv;
+      }
 #pragma unroll
       for (int stl = 0; stl < 4; ++stl) {
-        const float pr = __builtin_amdgcn_exp2f(sv[stl] - m_use);  // in [0, 1]
+        const float pr = prs[stl];
         if (QUANT == FDATTN_CACHE_INT8) {
           u32 x = (u32)__builtin_rintf(pr * 268435456.0f);  // 2^28
           x = min(x, 268435455u);
-          lsum += (float)x;
+          if (!DYN) lsum += (float)x;
           pw[0] |= (x & 127u) << (8 * stl);
           pw[1] |= ((x >> 7) & 127u) << (8 * stl);
           pw[2] |= ((x >> 14) & 127u) << (8 * stl);
@@ -242,7 +288,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
             x -= dv;
             used += dv;
           }
-          lsum += used;
+          if (!DYN) lsum += used;
         }
       }
       st.l = st.l * alpha + lsum;
@@ -252,7 +298,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
       wave_sync();
 
       // ---------------- O += P V : V^T operands come transposed out of LDS
-      if (has_next) wait_vm8(); else wait_vm0();  // V(j) landed; K(j+1) may still be in flight
+      // V(j) landed; K(j+1) (DYN: with its two scale rows) may still be in flight
+      if (!has_next) wait_vm0(); else if (DYN) wait_vm10(); else wait_vm8();
       if (QUANT != FDATTN_CACHE_INT8 && valid < kBS) {
         // e4m3 has NaN codes: a stale byte in a row past the sequence end would poison 0 * NaN
         for (int r = valid + (lane >> 3); r < kBS; r += 8)
@@ -283,7 +330,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
           d = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a1, b1, d, 0, 0, 0);
           ob = (d.x + d.y) + (d.z + d.w);
         }
-        st.o[ct] = st.o[ct] * alpha + ob;
+        st.o[ct] = st.o[ct] * alpha + (DYN ? ob * vmax : ob);
       }
       wait_lgkm0();  // V tile consumed
       if (has_next) dma_tile(vbase + (size_t)pbn * blk_stride, vaddr, offV);
@@ -327,7 +374,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
     if (single) {
       // the only chunk of this pair: finish here
       const float inv = L > 0.f ? 1.0f / L : 0.f;
-      const float r0 = o0 * inv * a.v_scale[h * kD + c2], r1 = o1 * inv * a.v_scale[h * kD + c2 + 1];
+      const float r0 = o0 * inv * (DYN ? 1.f : a.v_scale[h * kD + c2]), r1 = o1 * inv * (DYN ? 1.f : a.v_scale[h * kD + c2 + 1]);
       uint16_t* o = a.out + ((size_t)row * a.hkv * kG + h * kG + head) * kD + c2;
       *reinterpret_cast<u32*>(o) = (u32)f32_to_bf16(r0) | ((u32)f32_to_bf16(r1) << 16);
     } else {
@@ -371,7 +418,7 @@ __global__ __launch_bounds__(256) void decode_c8_combine_kernel(C8Args a) {
     }
   }
   const float inv = L > 0.f ? 1.0f / L : 0.f;
-  const float r0 = o0 * inv * a.v_scale[h * kD + c2], r1 = o1 * inv * a.v_scale[h * kD + c2 + 1];
+  const float r0 = o0 * inv * (a.dyn ? 1.f : a.v_scale[h * kD + c2]), r1 = o1 * inv * (a.dyn ? 1.f : a.v_scale[h * kD + c2 + 1]);
   uint16_t* o = a.out + ((size_t)row * a.hkv * kG + h * kG + head) * kD + c2;
   *reinterpret_cast<u32*>(o) = (u32)f32_to_bf16(r0) | ((u32)f32_to_bf16(r1) << 16);
 }
@@ -414,8 +461,7 @@ size_t c8_workspace_bytes(int batch, int hkv, int max_units) {
 }
 
 bool c8_supported(int hq, int hkv, int d, int bs, int quant) {
-  return d == kD && hq == kG * hkv && bs == kBS &&
-         (quant == FDATTN_CACHE_INT8 || quant == FDATTN_CACHE_FP8_E4M3);
+  return d == kD && hq == kG * hkv && bs == kBS && quant_known(quant);
 }
 
 int decode_c8_launch(const void* q, const void* key_cache, const void* value_cache, const float* k_scale,
@@ -443,15 +489,21 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
   C8Args a{(const uint16_t*)q, (const uint8_t*)key_cache, (const uint8_t*)value_cache, k_scale, v_scale,
            block_tables, seq_lens_decoder, seq_lens_this_time, kept_blocks, kept_counts, max_kept, part_o,
            part_ml, (uint16_t*)out, rows, batch, hkv, max_blocks, num_blocks, chunk, cpp,
-           sm_scale * 1.4426950408889634f};
+           sm_scale * 1.4426950408889634f, quant_dynamic(quant) ? 1 : 0};
   const dim3 grid(cpp * pairs), block(kWaves * 64);
   if (!(stages & 1)) {
   } else if (quant == FDATTN_CACHE_INT8) {
-    if (sparse) hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_INT8, true>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_INT8, false>), grid, block, 0, s, a);
+    if (sparse) hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_INT8, true, false>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_INT8, false, false>), grid, block, 0, s, a);
+  } else if (quant == FDATTN_CACHE_FP8_E4M3) {
+    if (sparse) hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_FP8_E4M3, true, false>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_FP8_E4M3, false, false>), grid, block, 0, s, a);
+  } else if (quant == FDATTN_CACHE_INT8_DYNAMIC) {
+    if (sparse) hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_INT8, true, true>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_INT8, false, true>), grid, block, 0, s, a);
   } else {
-    if (sparse) hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_FP8_E4M3, true>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_FP8_E4M3, false>), grid, block, 0, s, a);
+    if (sparse) hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_FP8_E4M3, true, true>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_FP8_E4M3, false, true>), grid, block, 0, s, a);
   }
   int rc = check_launch("fdattn_decode_attention (mfma)");
   if (rc || !(stages & 2)) return rc;

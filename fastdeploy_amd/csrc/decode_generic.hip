@@ -35,7 +35,8 @@ __device__ __forceinline__ float dq(u32 byte) {
 
 constexpr int kMaxD = 256;
 
-template <int QUANT>
+// DYN: cache scales per stored row ([num_blocks, hkv, bs]) instead of per channel.
+template <int QUANT, bool DYN>
 __global__ __launch_bounds__(64) void decode_generic_kernel(GenericDecodeArgs a) {
   __shared__ float qs[kMaxD];
   __shared__ float pbuf[64];
@@ -48,7 +49,7 @@ __global__ __launch_bounds__(64) void decode_generic_kernel(GenericDecodeArgs a)
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
 
   for (int c = lane; c < d; c += 64)
-    qs[c] = bf16_to_f32(a.q[((size_t)qrow * a.hq + qh) * d + c]) * a.k_scale[h * d + c] * a.sm_scale;
+    qs[c] = bf16_to_f32(a.q[((size_t)qrow * a.hq + qh) * d + c]) * (DYN ? 1.0f : a.k_scale[h * d + c]) * a.sm_scale;
   __syncthreads();
 
   int nblk = (kv_len + bs - 1) / bs;
@@ -72,6 +73,7 @@ __global__ __launch_bounds__(64) void decode_generic_kernel(GenericDecodeArgs a)
     if (pb < 0 || pb >= a.num_blocks) continue;
     const uint8_t* kp = a.key_cache + ((size_t)pb * a.hkv + h) * bs * d;
     const uint8_t* vp = a.value_cache + ((size_t)pb * a.hkv + h) * bs * d;
+    const size_t srow = ((size_t)pb * a.hkv + h) * bs;  // DYN: this tile's rows in the scale caches
     for (int t0 = 0; t0 < bs; t0 += 64) {
       const int t = t0 + lane;
       const bool valid = t < bs && lb * bs + t < kv_len;
@@ -84,6 +86,7 @@ __global__ __launch_bounds__(64) void decode_generic_kernel(GenericDecodeArgs a)
           s += qs[c] * dq<QUANT>(w & 0xff) + qs[c + 1] * dq<QUANT>((w >> 8) & 0xff) +
                qs[c + 2] * dq<QUANT>((w >> 16) & 0xff) + qs[c + 3] * dq<QUANT>(w >> 24);
         }
+        if (DYN) s *= a.k_scale[srow + t];
       }
       const float mb = wave_max(s);
       if (mb == -INFINITY) continue;  // uniform: no valid token in this group
@@ -93,7 +96,7 @@ __global__ __launch_bounds__(64) void decode_generic_kernel(GenericDecodeArgs a)
       l = l * alpha + wave_sum(p);
       m = m_new;
       __syncthreads();
-      pbuf[lane] = p;
+      pbuf[lane] = (DYN && valid) ? p * a.v_scale[srow + t] : p;  // the V row's scale rides on its weight
       __syncthreads();
       const int nt = min(64, bs - t0);
 #pragma unroll
@@ -111,7 +114,7 @@ __global__ __launch_bounds__(64) void decode_generic_kernel(GenericDecodeArgs a)
 #pragma unroll
   for (int i = 0; i < kMaxD / 64; ++i) {
     const int c = lane + 64 * i;
-    if (c < d) a.part_o[slot * d + c] = acc[i] * a.v_scale[h * d + c];
+    if (c < d) a.part_o[slot * d + c] = DYN ? acc[i] : acc[i] * a.v_scale[h * d + c];
   }
   if (lane == 0) {
     a.part_m[slot] = m;
@@ -180,10 +183,15 @@ int decode_generic_launch(const void* q, const void* key_cache, const void* valu
                       k_scale, v_scale, block_tables, seq_lens_decoder, seq_lens_this_time,
                       kept_blocks, kept_counts, max_kept, part_o, part_m, part_l, rmap, batch, hq, hkv,
                       d, bs, max_blocks, num_blocks, nsplit, sm_scale};
+  const dim3 grid(rows, nsplit);
   if (quant == FDATTN_CACHE_INT8)
-    hipLaunchKernelGGL(decode_generic_kernel<FDATTN_CACHE_INT8>, dim3(rows, nsplit), dim3(64), 0, s, a);
+    hipLaunchKernelGGL((decode_generic_kernel<FDATTN_CACHE_INT8, false>), grid, dim3(64), 0, s, a);
+  else if (quant == FDATTN_CACHE_FP8_E4M3)
+    hipLaunchKernelGGL((decode_generic_kernel<FDATTN_CACHE_FP8_E4M3, false>), grid, dim3(64), 0, s, a);
+  else if (quant == FDATTN_CACHE_INT8_DYNAMIC)
+    hipLaunchKernelGGL((decode_generic_kernel<FDATTN_CACHE_INT8, true>), grid, dim3(64), 0, s, a);
   else
-    hipLaunchKernelGGL(decode_generic_kernel<FDATTN_CACHE_FP8_E4M3>, dim3(rows, nsplit), dim3(64), 0, s, a);
+    hipLaunchKernelGGL((decode_generic_kernel<FDATTN_CACHE_FP8_E4M3, true>), grid, dim3(64), 0, s, a);
   int rc = check_launch("fdattn_decode_attention (generic)");
   if (rc) return rc;
   hipLaunchKernelGGL(splitkv_combine_kernel, dim3(rows), dim3(128), 0, s, part_o, part_m, part_l,

@@ -30,6 +30,15 @@ __device__ __forceinline__ bool prefill_row(const RowMap& m, int b) {
   return !m.seq_lens_encoder || m.seq_lens_encoder[b] > 0;
 }
 
+// cache_quant_type -> how the bytes are encoded / whether the scales are per stored row
+__host__ __device__ constexpr int quant_bytes(int q) {
+  return q == FDATTN_CACHE_INT8_DYNAMIC ? FDATTN_CACHE_INT8 : (q == FDATTN_CACHE_FP8_E4M3_DYNAMIC ? FDATTN_CACHE_FP8_E4M3 : q);
+}
+__host__ __device__ constexpr bool quant_dynamic(int q) {
+  return q == FDATTN_CACHE_INT8_DYNAMIC || q == FDATTN_CACHE_FP8_E4M3_DYNAMIC;
+}
+__host__ __device__ constexpr bool quant_known(int q) { return q >= FDATTN_CACHE_INT8 && q <= FDATTN_CACHE_FP8_E4M3_DYNAMIC; }
+
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
 typedef float v4f __attribute__((ext_vector_type(4)));

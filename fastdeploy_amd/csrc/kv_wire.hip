@@ -167,7 +167,7 @@ __global__ __launch_bounds__(256) void kv_wire_kernel(WireArgs a) {
 int check_shape(const char* what, int batch, int max_tokens, int hkv, int d, int bs, int max_blocks, int num_blocks,
                 int quant) {
   if (quant != FDATTN_CACHE_INT8 && quant != FDATTN_CACHE_FP8_E4M3)
-    return fail(FDATTN_ERR_QUANT, "%s: cache_quant_type %d is not a one-byte cache format", what, quant);
+    return fail(FDATTN_ERR_QUANT, "%s: cache_quant_type %d is not a format with per-channel scales", what, quant);
   if (batch < 0 || max_tokens < 0 || hkv <= 0 || d <= 0 || bs <= 0 || max_blocks <= 0 || num_blocks <= 0 || d % 16 != 0 ||
       batch > 65535)
     return fail(FDATTN_ERR_SHAPE, "%s: bad shape batch=%d max_tokens=%d hkv=%d head_dim=%d block_size=%d "

@@ -15,7 +15,8 @@ __device__ __forceinline__ float pdq(u32 byte) {
 // Shape-agnostic kernel: one wavefront per (new token, query head); lanes own keys for
 // q.K and channels for P.V.  Keys [0, p) come from the quantised pages, keys [p, p+ci]
 // from the chunk's bf16 K/V.
-template <int QUANT>
+// DYN: cache scales per stored row ([num_blocks, hkv, bs]) instead of per channel.
+template <int QUANT, bool DYN>
 __global__ __launch_bounds__(64) void prefill_generic_kernel(PrefillArgs a) {
   __shared__ float qf[kPfMaxD];
   __shared__ float pbuf[64];
@@ -47,10 +48,19 @@ __global__ __launch_bounds__(64) void prefill_generic_kernel(PrefillArgs a) {
       if (kk < p) {
         const int pb = table[kk / bs];
         const uint8_t* kr = a.key_cache + (((size_t)pb * a.hkv + h) * bs + kk % bs) * d;
-        for (int c = 0; c < d; c += 4) {
-          const u32 w = *reinterpret_cast<const u32*>(kr + c);
-          s += qf[c] * (pdq<QUANT>(w & 0xff) * ks[c]) + qf[c + 1] * (pdq<QUANT>((w >> 8) & 0xff) * ks[c + 1]) +
-               qf[c + 2] * (pdq<QUANT>((w >> 16) & 0xff) * ks[c + 2]) + qf[c + 3] * (pdq<QUANT>(w >> 24) * ks[c + 3]);
+        if (DYN) {
+          for (int c = 0; c < d; c += 4) {
+            const u32 w = *reinterpret_cast<const u32*>(kr + c);
+            s += qf[c] * pdq<QUANT>(w & 0xff) + qf[c + 1] * pdq<QUANT>((w >> 8) & 0xff) +
+                 qf[c + 2] * pdq<QUANT>((w >> 16) & 0xff) + qf[c + 3] * pdq<QUANT>(w >> 24);
+          }
+          s *= a.k_scale[((size_t)pb * a.hkv + h) * bs + kk % bs];
+        } else {
+          for (int c = 0; c < d; c += 4) {
+            const u32 w = *reinterpret_cast<const u32*>(kr + c);
+            s += qf[c] * (pdq<QUANT>(w & 0xff) * ks[c]) + qf[c + 1] * (pdq<QUANT>((w >> 8) & 0xff) * ks[c + 1]) +
+                 qf[c + 2] * (pdq<QUANT>((w >> 16) & 0xff) * ks[c + 2]) + qf[c + 3] * (pdq<QUANT>(w >> 24) * ks[c + 3]);
+          }
         }
       } else {
         const uint16_t* kr = a.k_new + ((size_t)(a.cu_seqlens_q[b] + kk - p) * a.hkv + h) * d;
@@ -80,7 +90,8 @@ __global__ __launch_bounds__(64) void prefill_generic_kernel(PrefillArgs a) {
           float v;
           if (kk2 < p) {
             const int pb = table[kk2 / bs];
-            v = pdq<QUANT>(a.value_cache[(((size_t)pb * a.hkv + h) * bs + kk2 % bs) * d + c]) * vs[c];
+            v = pdq<QUANT>(a.value_cache[(((size_t)pb * a.hkv + h) * bs + kk2 % bs) * d + c]) *
+                (DYN ? a.v_scale[((size_t)pb * a.hkv + h) * bs + kk2 % bs] : vs[c]);
           } else {
             v = bf16_to_f32(a.v_new[((size_t)(a.cu_seqlens_q[b] + kk2 - p) * a.hkv + h) * d + c]);
           }
@@ -113,7 +124,7 @@ int prefill_launch(const void* q, const void* k_new, const void* v_new, const vo
     return fail(FDATTN_ERR_SHAPE,
                 "fdattn_append_attention_prefill: unsupported shape tokens=%d batch=%d max_chunk=%d hq=%d hkv=%d "
                 "head_dim=%d block_size=%d", num_tokens, batch, max_chunk, hq, hkv, head_dim, block_size);
-  if (cache_quant_type != FDATTN_CACHE_INT8 && cache_quant_type != FDATTN_CACHE_FP8_E4M3)
+  if (!quant_known(cache_quant_type))
     return fail(FDATTN_ERR_QUANT, "fdattn_append_attention_prefill: unknown cache_quant_type %d", cache_quant_type);
   if (num_tokens == 0) return 0;
   PrefillArgs a{(const uint16_t*)q, (const uint16_t*)k_new, (const uint16_t*)v_new, (const uint8_t*)key_cache,
@@ -122,10 +133,15 @@ int prefill_launch(const void* q, const void* k_new, const void* v_new, const vo
                 max_blocks_per_seq, num_blocks, softmax_scale};
   if (!force_generic && prefill_mfma_supported(hq, hkv, head_dim, block_size, cache_quant_type))
     return prefill_mfma_launch(a, max_chunk, cache_quant_type, s, workspace, workspace_bytes, n_splits, rows_hint);
+  const dim3 grid(num_tokens, hq);
   if (cache_quant_type == FDATTN_CACHE_INT8)
-    hipLaunchKernelGGL(prefill_generic_kernel<FDATTN_CACHE_INT8>, dim3(num_tokens, hq), dim3(64), 0, s, a);
+    hipLaunchKernelGGL((prefill_generic_kernel<FDATTN_CACHE_INT8, false>), grid, dim3(64), 0, s, a);
+  else if (cache_quant_type == FDATTN_CACHE_FP8_E4M3)
+    hipLaunchKernelGGL((prefill_generic_kernel<FDATTN_CACHE_FP8_E4M3, false>), grid, dim3(64), 0, s, a);
+  else if (cache_quant_type == FDATTN_CACHE_INT8_DYNAMIC)
+    hipLaunchKernelGGL((prefill_generic_kernel<FDATTN_CACHE_INT8, true>), grid, dim3(64), 0, s, a);
   else
-    hipLaunchKernelGGL(prefill_generic_kernel<FDATTN_CACHE_FP8_E4M3>, dim3(num_tokens, hq), dim3(64), 0, s, a);
+    hipLaunchKernelGGL((prefill_generic_kernel<FDATTN_CACHE_FP8_E4M3, true>), grid, dim3(64), 0, s, a);
   return check_launch("fdattn_append_attention_prefill");
 }
 

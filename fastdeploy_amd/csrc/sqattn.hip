@@ -557,7 +557,8 @@ static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_ca
                 "max_blocks=%d top_k=%d (group <= %d, head_dim <= %d multiple of 4, max_blocks <= 4096)",
                 batch, hq, hkv, head_dim, block_size, max_blocks_per_seq, top_k, kSelMaxG, kSelMaxD);
   if (cache_quant_type != FDATTN_CACHE_INT8 && cache_quant_type != FDATTN_CACHE_FP8_E4M3)
-    return fail(FDATTN_ERR_QUANT, "fdattn_sqattn_select: unknown cache_quant_type %d", cache_quant_type);
+    return fail(FDATTN_ERR_QUANT, "fdattn_sqattn_select: cache_quant_type %d is not a format with per-channel scales",
+                cache_quant_type);
   const size_t need = (size_t)batch * hkv * ((size_t)max_blocks_per_seq * sizeof(double) + sizeof(float));
   if (workspace_bytes < need)
     return fail(FDATTN_ERR_WORKSPACE, "fdattn_sqattn_select: workspace %zu B < required %zu B", workspace_bytes, need);

@@ -20,14 +20,31 @@ from . import _lib
 
 CACHE_INT8 = 1
 CACHE_FP8 = 2
+# the same byte formats with one scale per stored row (token, KV head), computed by the cache writer:
+# the scale tensors are then float32 [num_blocks, kv_num_heads, block_size] and the writer fills them
+CACHE_INT8_DYNAMIC = 3
+CACHE_FP8_DYNAMIC = 4
 _QUANT = {"cache_int8": CACHE_INT8, "int8": CACHE_INT8, CACHE_INT8: CACHE_INT8,
-          "cache_fp8": CACHE_FP8, "fp8": CACHE_FP8, "fp8_e4m3": CACHE_FP8, CACHE_FP8: CACHE_FP8}
+          "cache_fp8": CACHE_FP8, "fp8": CACHE_FP8, "fp8_e4m3": CACHE_FP8, CACHE_FP8: CACHE_FP8,
+          "cache_int8_dynamic": CACHE_INT8_DYNAMIC, CACHE_INT8_DYNAMIC: CACHE_INT8_DYNAMIC,
+          "cache_fp8_dynamic": CACHE_FP8_DYNAMIC, CACHE_FP8_DYNAMIC: CACHE_FP8_DYNAMIC}
+
+
+def is_dynamic(cache_quant_type):
+    """True for the formats that carry one scale per stored row."""
+    return _QUANT.get(cache_quant_type) in (CACHE_INT8_DYNAMIC, CACHE_FP8_DYNAMIC)
+
+
+def byte_format(cache_quant_type):
+    """CACHE_INT8 or CACHE_FP8: how the cache bytes of this format are encoded."""
+    q = _QUANT[cache_quant_type]
+    return {CACHE_INT8_DYNAMIC: CACHE_INT8, CACHE_FP8_DYNAMIC: CACHE_FP8}.get(q, q)
 _ROPE = {"interleaved": 0, 0: 0, False: 0, "neox": 1, 1: 1, True: 1}
 
 
 def _quant(t):
     if t not in _QUANT:
-        raise ValueError("unknown cache_quant_type %r (cache_int8 | cache_fp8)" % (t,))
+        raise ValueError("unknown cache_quant_type %r (cache_int8 | cache_fp8 | cache_int8_dynamic | cache_fp8_dynamic)" % (t,))
     return _QUANT[t]
 
 
@@ -63,10 +80,14 @@ def _cache_dims(key_cache, value_cache):
     return key_cache.shape  # num_blocks, hkv, block_size, head_dim
 
 
-def _scales(cache_k_scale, cache_v_scale, hkv, d):
+def _scales(cache_k_scale, cache_v_scale, hkv, d, quant=CACHE_INT8, nb=0, bs=0):
     pk = _chk(cache_k_scale, "cache_k_scale", torch.float32)
     pv = _chk(cache_v_scale, "cache_v_scale", torch.float32)
-    if cache_k_scale.numel() != hkv * d or cache_v_scale.numel() != hkv * d:
+    if is_dynamic(quant):
+        if cache_k_scale.numel() != nb * hkv * bs or cache_v_scale.numel() != nb * hkv * bs:
+            raise ValueError("the dynamic formats' cache scales must hold num_blocks*kv_num_heads*block_size = %d "
+                             "values" % (nb * hkv * bs))
+    elif cache_k_scale.numel() != hkv * d or cache_v_scale.numel() != hkv * d:
         raise ValueError("cache scales must hold kv_num_heads*head_dim = %d values" % (hkv * d))
     return pk, pv
 
@@ -127,7 +148,7 @@ def write_cache_kv(qkv, key_cache, value_cache, cache_k_scale, cache_v_scale, bl
                          (qkv.shape[1], (num_heads + 2 * hkv) * d))
     p_kc = _chk(key_cache, "key_cache", _CACHE_DT, 4)
     p_vc = _chk(value_cache, "value_cache", _CACHE_DT, 4)
-    p_ks, p_vs = _scales(cache_k_scale, cache_v_scale, hkv, d)
+    p_ks, p_vs = _scales(cache_k_scale, cache_v_scale, hkv, d, cache_quant_type, nb, bs)
     p_bt = _chk(block_tables, "block_tables", torch.int32, 2)
     batch, mb = block_tables.shape
     p_dec = _chk(seq_lens_decoder, "seq_lens_decoder", torch.int32, 1)
@@ -181,7 +202,7 @@ def decode_uses_mfma(num_heads, kv_num_heads, head_dim, block_size, cache_quant_
 
 
 def _decode_common(q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
-                   seq_lens_decoder, seq_lens_this_time, num_heads, out, workspace):
+                   seq_lens_decoder, seq_lens_this_time, num_heads, out, workspace, cache_quant_type):
     nb, hkv, bs, d = _cache_dims(key_cache, value_cache)
     p_q = _chk(q, "q", torch.bfloat16)
     batch, mb = block_tables.shape
@@ -190,7 +211,7 @@ def _decode_common(q, key_cache, value_cache, cache_k_scale, cache_v_scale, bloc
                          (q.numel(), batch * num_heads * d))
     p_kc = _chk(key_cache, "key_cache", _CACHE_DT, 4)
     p_vc = _chk(value_cache, "value_cache", _CACHE_DT, 4)
-    p_ks, p_vs = _scales(cache_k_scale, cache_v_scale, hkv, d)
+    p_ks, p_vs = _scales(cache_k_scale, cache_v_scale, hkv, d, cache_quant_type, nb, bs)
     p_bt = _chk(block_tables, "block_tables", torch.int32, 2)
     p_dec = _chk(seq_lens_decoder, "seq_lens_decoder", torch.int32, 1)
     p_tt = _chk(seq_lens_this_time, "seq_lens_this_time", torch.int32, 1, optional=True)
@@ -215,7 +236,7 @@ def decode_attention(q, key_cache, value_cache, cache_k_scale, cache_v_scale, bl
     impl: "auto" (MFMA kernel when the shape allows) or "generic"."""
     ptrs, out, p_out, p_ws, workspace, dims = _decode_common(
         q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables, seq_lens_decoder,
-        seq_lens_this_time, num_heads, out, workspace)
+        seq_lens_this_time, num_heads, out, workspace, cache_quant_type)
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(dims[3])
     if impl == "generic":
         rc = _lib.lib().fdattn_decode_attention_generic(
@@ -241,7 +262,7 @@ def decode_attention_sparse(q, key_cache, value_cache, cache_k_scale, cache_v_sc
     (ascending logical block indices) / kept_counts int32 [batch, kv_num_heads]."""
     ptrs, out, p_out, p_ws, workspace, dims = _decode_common(
         q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables, seq_lens_decoder,
-        seq_lens_this_time, num_heads, out, workspace)
+        seq_lens_this_time, num_heads, out, workspace, cache_quant_type)
     batch, _, hkv = dims[0], dims[1], dims[2]
     p_kb = _chk(kept_blocks, "kept_blocks", torch.int32, 3)
     p_kn = _chk(kept_counts, "kept_counts", torch.int32, 2)
@@ -319,7 +340,7 @@ def append_attention_prefill(q, k_new, v_new, key_cache, value_cache, cache_k_sc
         raise ValueError("q must be [T, num_heads*head_dim], k_new / v_new [T, kv_num_heads*head_dim]")
     p_kc = _chk(key_cache, "key_cache", _CACHE_DT, 4)
     p_vc = _chk(value_cache, "value_cache", _CACHE_DT, 4)
-    p_ks, p_vs = _scales(cache_k_scale, cache_v_scale, hkv, d)
+    p_ks, p_vs = _scales(cache_k_scale, cache_v_scale, hkv, d, cache_quant_type, nb, bs)
     p_bt = _chk(block_tables, "block_tables", torch.int32, 2)
     batch, mb = block_tables.shape
     p_dec = _chk(seq_lens_decoder, "seq_lens_decoder", torch.int32, 1)
@@ -390,7 +411,7 @@ def append_attention(qkv, key_cache, value_cache, seq_lens_encoder, seq_lens_dec
                          (qkv.shape[1], (num_heads + 2 * hkv) * d))
     p_kc = _chk(key_cache, "key_cache", _CACHE_DT, 4)
     p_vc = _chk(value_cache, "value_cache", _CACHE_DT, 4)
-    p_ks, p_vs = _scales(cache_k_scale, cache_v_scale, hkv, d)
+    p_ks, p_vs = _scales(cache_k_scale, cache_v_scale, hkv, d, cache_quant_type, nb, bs)
     p_bt = _chk(block_tables, "block_tables", torch.int32, 2)
     batch, mb = block_tables.shape
     p_enc = _chk(seq_lens_encoder, "seq_lens_encoder", torch.int32, 1)

@@ -9,7 +9,7 @@ import math
 
 import torch
 
-from .ops import CACHE_FP8, CACHE_INT8
+from .ops import CACHE_FP8, CACHE_INT8, byte_format, is_dynamic
 
 HQ, HKV, D, BS = 32, 8, 128, 64
 
@@ -17,13 +17,13 @@ HQ, HKV, D, BS = 32, 8, 128, 64
 def quantize_ref(x, scale, quant):
     """fp32 x / scale -> cache bytes (uint8 view), the formulas of the cache format."""
     r = x.float() / scale
-    if quant == CACHE_INT8:
+    if byte_format(quant) == CACHE_INT8:
         return torch.clamp(torch.round(r), -127, 127).to(torch.int8).view(torch.uint8)
     return torch.clamp(r, -448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8)
 
 
 def dequantize_ref(c, scale, quant):
-    if quant == CACHE_INT8:
+    if byte_format(quant) == CACHE_INT8:
         return c.view(torch.int8).float() * scale
     return c.view(torch.float8_e4m3fn).float() * scale
 
@@ -57,6 +57,9 @@ def decode_case(batch=4, ctx=1024, pool_blocks=None, quant=CACHE_INT8, seed=0, d
     direct_bytes: draw the cache bytes directly (values do not matter for bandwidth);
     otherwise K, V ~ N(0,1) bf16 quantised with per-channel scales = max-abs/127 (int8)
     or max-abs/448 (fp8).  salient: fraction of (sequence, block) pairs whose K is x4.
+    The dynamic formats get scale caches [pool, hkv, bs]: every stored row's own max-abs/127 (/448)
+    with the rows scaled by 2^U{-3..3} so that the scales differ widely, or (direct_bytes) random ones;
+    the slots of no token hold NaN there, which nothing may read.
     """
     g = _gen(seed, device)
     if isinstance(ctx, tuple):
@@ -69,11 +72,12 @@ def decode_case(batch=4, ctx=1024, pool_blocks=None, quant=CACHE_INT8, seed=0, d
     pool = pool_blocks or (need + extra_blocks)
     bt = make_block_tables(lens, pool, bs, g, device, max_blocks)
     q = torch.randn((batch, hq * d), generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
-    qmax = 127.0 if quant == CACHE_INT8 else 448.0
+    dyn, fmt = is_dynamic(quant), byte_format(quant)
+    qmax = 127.0 if fmt == CACHE_INT8 else 448.0
     kc = torch.zeros((pool, hkv, bs, d), dtype=torch.uint8, device=device)
     vc = torch.zeros((pool, hkv, bs, d), dtype=torch.uint8, device=device)
     if direct_bytes:
-        if quant == CACHE_INT8:
+        if fmt == CACHE_INT8:
             kc = torch.randint(-127, 128, kc.shape, generator=g, device=device, dtype=torch.int8).view(torch.uint8)
             vc = torch.randint(-127, 128, vc.shape, generator=g, device=device, dtype=torch.int8).view(torch.uint8)
         else:  # any finite e4m3 code: magnitude field 0..0x7e, random sign
@@ -84,8 +88,41 @@ def decode_case(batch=4, ctx=1024, pool_blocks=None, quant=CACHE_INT8, seed=0, d
             kc, vc = mk | sk, mv | sv
         ks = (torch.rand((hkv, d), generator=g, device=device) * 0.02 + 0.02) * (127.0 / qmax)
         vs = (torch.rand((hkv, d), generator=g, device=device) * 0.02 + 0.02) * (127.0 / qmax)
-        if quant == CACHE_FP8:
+        if fmt == CACHE_FP8:
             ks, vs = ks * 0.05, vs * 0.05  # e4m3 codes reach 448: keep logits in a sane range
+        if dyn:
+            sc = 127.0 / qmax * (0.05 if fmt == CACHE_FP8 else 1.0)
+            ks = (torch.rand((pool, hkv, bs), generator=g, device=device) * 0.03 + 0.01) * sc
+            vs = (torch.rand((pool, hkv, bs), generator=g, device=device) * 0.03 + 0.01) * sc
+    elif dyn:
+        ks = torch.full((pool, hkv, bs), float("nan"), device=device)
+        vs = torch.full((pool, hkv, bs), float("nan"), device=device)
+        for b, n in enumerate(lens):
+            if n == 0:
+                continue
+            k = torch.randn((n, hkv, d), generator=g, device=device).to(torch.bfloat16).float()
+            v = torch.randn((n, hkv, d), generator=g, device=device).to(torch.bfloat16).float()
+            k = k * torch.exp2(torch.randint(-3, 4, (n, hkv, 1), generator=g, device=device).float())
+            v = v * torch.exp2(torch.randint(-3, 4, (n, hkv, 1), generator=g, device=device).float())
+            if salient > 0:
+                nb = (n + bs - 1) // bs
+                pick = torch.rand((nb,), generator=g, device=device) < salient
+                k = k * (1.0 + 3.0 * pick.repeat_interleave(bs)[:n].float())[:, None, None]
+            sk, sv = k.abs().amax(-1) / qmax, v.abs().amax(-1) / qmax  # [n, hkv]
+            sk, sv = torch.where(sk > 0, sk, torch.ones_like(sk)), torch.where(sv > 0, sv, torch.ones_like(sv))
+            nb = (n + bs - 1) // bs
+            pad = nb * bs - n
+            kq, vq = quantize_ref(k, sk[..., None], quant), quantize_ref(v, sv[..., None], quant)
+            if pad:
+                z = torch.zeros((pad, hkv, d), dtype=torch.uint8, device=device)
+                kq, vq = torch.cat([kq, z]), torch.cat([vq, z])
+                nanpad = torch.full((pad, hkv), float("nan"), device=device)
+                sk, sv = torch.cat([sk, nanpad]), torch.cat([sv, nanpad])
+            idx = bt[b, :nb].long()
+            kc[idx] = kq.view(nb, bs, hkv, d).permute(0, 2, 1, 3)
+            vc[idx] = vq.view(nb, bs, hkv, d).permute(0, 2, 1, 3)
+            ks[idx] = sk.view(nb, bs, hkv).permute(0, 2, 1)
+            vs[idx] = sv.view(nb, bs, hkv).permute(0, 2, 1)
     else:
         ks_acc = torch.zeros((hkv, d), device=device)
         vs_acc = torch.zeros((hkv, d), device=device)
@@ -137,12 +174,16 @@ def write_case(num_seqs=256, max_pos=8192, quant=CACHE_INT8, seed=0, device="cpu
     bt = perm.view(num_seqs, mb).contiguous()
     kc = torch.randint(0, 256, (pool, hkv, bs, d), generator=g, device=device, dtype=torch.uint8)
     vc = torch.randint(0, 256, (pool, hkv, bs, d), generator=g, device=device, dtype=torch.uint8)
-    if quant == CACHE_FP8:  # no NaN codes in the prior contents
+    if byte_format(quant) == CACHE_FP8:  # no NaN codes in the prior contents
         kc = torch.where((kc & 0x7F) == 0x7F, kc & 0xFE, kc)
         vc = torch.where((vc & 0x7F) == 0x7F, vc & 0xFE, vc)
-    qmax = 127.0 if quant == CACHE_INT8 else 448.0
-    ks = (torch.rand((hkv, d), generator=g, device=device) * 2.0 + 3.0) / qmax
-    vs = (torch.rand((hkv, d), generator=g, device=device) * 2.0 + 3.0) / qmax
+    qmax = 127.0 if byte_format(quant) == CACHE_INT8 else 448.0
+    if is_dynamic(quant):  # scale caches with prior contents: the rows already stored
+        ks = (torch.rand((pool, hkv, bs), generator=g, device=device) * 2.0 + 3.0) / qmax
+        vs = (torch.rand((pool, hkv, bs), generator=g, device=device) * 2.0 + 3.0) / qmax
+    else:
+        ks = (torch.rand((hkv, d), generator=g, device=device) * 2.0 + 3.0) / qmax
+        vs = (torch.rand((hkv, d), generator=g, device=device) * 2.0 + 3.0) / qmax
     cos, sin = rope_table(max_pos, d, theta, device)
     this = torch.full((num_seqs,), chunk, dtype=torch.int32, device=device)
     cu = torch.arange(0, T + 1, chunk, dtype=torch.int32, device=device)

@@ -52,6 +52,18 @@ extern "C" {
 /* cache_quant_type */
 #define FDATTN_CACHE_INT8 1     /* q = clamp(rne(x / scale), -127, 127), stored as int8 */
 #define FDATTN_CACHE_FP8_E4M3 2 /* q = e4m3fn(clamp(x / scale, -448, 448)), RNE        */
+/*
+ * The dynamic formats: the same bytes, but one scale per stored row - per (token, KV head) - that the
+ * cache writer derives from the row itself: scale = max_c |x[c]| / 127 (/ 448 for fp8), one IEEE
+ * division, NaNs ignored by the maximum, 1.0 for a row of zeros.  Wherever an entry point takes
+ * cache_k_scale / cache_v_scale, they are then the scale CACHES, f32 [num_blocks, hkv, block_size],
+ * indexed like the rows of key_cache / value_cache; the cache writer (and the one-call step, which
+ * contains it) STORES into them despite the const qualifier, every attention entry point reads them.
+ * K scales are taken after the rotation.  Dequantised value = byte * scale of its row.
+ * Not accepted by the block selector and the wire form, which are defined on per-channel scales.
+ */
+#define FDATTN_CACHE_INT8_DYNAMIC 3
+#define FDATTN_CACHE_FP8_E4M3_DYNAMIC 4
 
 /* rope_style */
 #define FDATTN_ROPE_INTERLEAVED 0 /* pairs (2j, 2j+1)          */

@@ -16,6 +16,13 @@
  *     complex multiplication in fp64), |x - q*s| <= s/2, max-abs -> +-127;
  *     its epilogue (bias, RMS norm of Q and K heads): torch's bf16 add and an
  *     fp64 RMS norm, unit weights -> unit mean square, scale invariance;
+ *     its dynamic formats (one scale per stored row): the stored scale is the
+ *     row's numpy max-abs / 127 (/ 448), the row's largest element maps to
+ *     +-127 (+-448), and the bytes equal those of the static writer run with
+ *     that row's scale in every channel;
+ *   - decode / prefill over the dynamic formats: equal to the same functions
+ *     over a static cache when every row of a head carries the same scale, and
+ *     to fp64 SDPA on the dequantised cache otherwise;
  *   - fdo_decode_attention: torch CPU scaled_dot_product_attention in fp64 on
  *     the dequantised gathered cache, block-table permutation invariance,
  *     kv_len 1 = V row, constant K = mean of V; its softmax against the
@@ -47,6 +54,15 @@
 
 #define FDO_CACHE_INT8 1
 #define FDO_CACHE_FP8 2
+/* the same byte formats with one scale per (token, KV head), computed by the writer from the row it
+ * stores: scale caches fp32 [num_blocks, kv_heads, block_size] in place of the [kv_heads, head_dim] ones */
+#define FDO_CACHE_INT8_DYNAMIC 3
+#define FDO_CACHE_FP8_DYNAMIC 4
+
+static inline int is_dynamic(int cache_type) { return cache_type == FDO_CACHE_INT8_DYNAMIC || cache_type == FDO_CACHE_FP8_DYNAMIC; }
+static inline int byte_format(int cache_type) {
+  return cache_type == FDO_CACHE_INT8_DYNAMIC ? FDO_CACHE_INT8 : (cache_type == FDO_CACHE_FP8_DYNAMIC ? FDO_CACHE_FP8 : cache_type);
+}
 
 /* ---------------------------------------------------------------- scalars */
 
@@ -111,7 +127,18 @@ int8_t fdo_quant_int8(float x, float scale) {
 uint8_t fdo_quant_fp8(float x, float scale) { return fdo_f32_to_e4m3(x / scale); }
 
 static inline float dequant(uint8_t byte, int cache_type) {
-  return cache_type == FDO_CACHE_INT8 ? (float)(int8_t)byte : fdo_e4m3_to_f32(byte);
+  return byte_format(cache_type) == FDO_CACHE_INT8 ? (float)(int8_t)byte : fdo_e4m3_to_f32(byte);
+}
+
+/*
+ * The scale of one stored row of the dynamic formats: (largest magnitude of the row) / 127 for int8,
+ * / 448 for fp8, one IEEE division; a row of zeros gets the scale 1.  NaNs do not take part in the maximum.
+ */
+float fdo_row_scale(const float* x, int d, int cache_type) {
+  float m = 0.f;
+  for (int c = 0; c < d; ++c) m = fmaxf(m, fabsf(x[c]));
+  if (!(m > 0.f)) return 1.0f;
+  return m / (byte_format(cache_type) == FDO_CACHE_INT8 ? 127.0f : 448.0f);
 }
 
 /* ------------------------------------------------------------ cache writer */
@@ -224,13 +251,22 @@ int fdo_write_cache_kv_ex(const uint16_t* qkv, uint16_t* q_out, uint16_t* k_out,
       rope_row(x, y, d, cs, sn, rope_style);
       epilogue_row(vr, qkv_bias ? qkv_bias + (size_t)(hq + hkv + h) * d : NULL, NULL, 0.f, d, rope_style, vx);
       size_t base = (((size_t)pb * hkv + h) * block_size + slot) * d;
+      int dyn = is_dynamic(cache_type);
+      float dk = 1.f, dv = 1.f;
+      if (dyn && pb >= 0) {
+        /* the scale caches are outputs here: the writer stores the scale beside the row */
+        dk = fdo_row_scale(y, d, cache_type);
+        dv = fdo_row_scale(vx, d, cache_type);
+        ((float*)k_scale)[((size_t)pb * hkv + h) * block_size + slot] = dk;
+        ((float*)v_scale)[((size_t)pb * hkv + h) * block_size + slot] = dv;
+      }
       for (int c = 0; c < d; ++c) {
-        float sk = k_scale[h * d + c], sv = v_scale[h * d + c];
+        float sk = dyn ? dk : k_scale[h * d + c], sv = dyn ? dv : v_scale[h * d + c];
         float v = vx[c];
         if (k_out) k_out[((size_t)i * hkv + h) * d + c] = fdo_f32_to_bf16(y[c]);
         if (v_out) v_out[((size_t)i * hkv + h) * d + c] = fdo_f32_to_bf16(v); /* exact: v is a bf16 value */
         if (pb < 0) continue;
-        if (cache_type == FDO_CACHE_INT8) {
+        if (byte_format(cache_type) == FDO_CACHE_INT8) {
           key_cache[base + c] = (uint8_t)fdo_quant_int8(y[c], sk);
           value_cache[base + c] = (uint8_t)fdo_quant_int8(v, sv);
         } else {
@@ -266,9 +302,11 @@ int fdo_write_cache_kv(const uint16_t* qkv, uint16_t* q_out, uint16_t* k_out, ui
  */
 static void attend_row(const float* qs /* q*k_scale, [d] */, const uint8_t* key_cache,
                        const uint8_t* value_cache, const float* v_scale /* [d] */,
-                       const int32_t* table, const int32_t* blk, int nblk, int kv_len, int h,
+                       const float* k_tok /* dynamic formats: [num_blocks,hkv,bs], else NULL */,
+                       const float* v_tok, const int32_t* table, const int32_t* blk, int nblk, int kv_len, int h,
                        int hkv, int d, int bs, int cache_type, float sm_scale, float* logits,
                        float* acc, uint16_t* out) {
+  cache_type = byte_format(cache_type);
   int n = 0;
   float mx = -INFINITY;
   for (int bi = 0; bi < nblk; ++bi) {
@@ -282,6 +320,7 @@ static void attend_row(const float* qs /* q*k_scale, [d] */, const uint8_t* key_
         for (int c = 0; c < d; ++c) s += qs[c] * (float)(int8_t)kr[c];
       else
         for (int c = 0; c < d; ++c) s += qs[c] * fdo_e4m3_to_f32(kr[c]);
+      if (k_tok) s *= k_tok[((size_t)table[lb] * hkv + h) * bs + (t - t0)];
       s *= sm_scale;
       logits[n++] = s;
       if (s > mx) mx = s;
@@ -297,6 +336,7 @@ static void attend_row(const float* qs /* q*k_scale, [d] */, const uint8_t* key_
     for (int t = t0; t < t1; ++t) {
       float p = expf(logits[n++] - mx);
       l += p;
+      if (v_tok) p *= v_tok[((size_t)table[lb] * hkv + h) * bs + (t - t0)];
       const uint8_t* vr = vp + (size_t)(t - t0) * d;
       if (cache_type == FDO_CACHE_INT8)
         for (int c = 0; c < d; ++c) acc[c] += p * (float)(int8_t)vr[c];
@@ -304,7 +344,7 @@ static void attend_row(const float* qs /* q*k_scale, [d] */, const uint8_t* key_
         for (int c = 0; c < d; ++c) acc[c] += p * fdo_e4m3_to_f32(vr[c]);
     }
   }
-  for (int c = 0; c < d; ++c) out[c] = fdo_f32_to_bf16(n ? acc[c] * v_scale[c] / l : 0.f);
+  for (int c = 0; c < d; ++c) out[c] = fdo_f32_to_bf16(n ? acc[c] * (v_tok ? 1.0f : v_scale[c]) / l : 0.f);
 }
 
 /*
@@ -329,15 +369,16 @@ int fdo_decode_attention(const uint16_t* q, const uint8_t* key_cache, const uint
         int h = qh / g;
         int kv_len = kv_lens[b];
         const uint16_t* qr = q + ((size_t)b * hq + qh) * d;
-        for (int c = 0; c < d; ++c) qs[c] = fdo_bf16_to_f32(qr[c]) * k_scale[h * d + c];
+        int dyn = is_dynamic(cache_type);
+        for (int c = 0; c < d; ++c) qs[c] = fdo_bf16_to_f32(qr[c]) * (dyn ? 1.0f : k_scale[h * d + c]);
         const int32_t* blk = NULL;
         int nblk = (kv_len + bs - 1) / bs;
         if (kept_blocks) {
           blk = kept_blocks + ((size_t)b * hkv + h) * max_kept;
           nblk = kept_counts[b * hkv + h];
         }
-        attend_row(qs, key_cache, value_cache, v_scale + h * d,
-                   block_tables + (size_t)b * max_blocks_per_seq, blk, nblk, kv_len, h, hkv, d,
+        attend_row(qs, key_cache, value_cache, dyn ? NULL : v_scale + h * d, dyn ? k_scale : NULL,
+                   dyn ? v_scale : NULL, block_tables + (size_t)b * max_blocks_per_seq, blk, nblk, kv_len, h, hkv, d,
                    bs, cache_type, sm_scale, logits, acc, out + ((size_t)b * hq + qh) * d);
       }
     free(logits);
@@ -498,7 +539,12 @@ int fdo_append_attention_prefill(const uint16_t* q, const uint16_t* k_new, const
           const uint8_t* kr =
               key_cache + (((size_t)table[t / bs] * hkv + h) * bs + t % bs) * d;
           float s = 0.f;
-          for (int c = 0; c < d; ++c) s += qf[c] * (dequant(kr[c], cache_type) * k_scale[h * d + c]);
+          if (is_dynamic(cache_type)) {
+            for (int c = 0; c < d; ++c) s += qf[c] * dequant(kr[c], cache_type);
+            s *= k_scale[((size_t)table[t / bs] * hkv + h) * bs + t % bs];
+          } else {
+            for (int c = 0; c < d; ++c) s += qf[c] * (dequant(kr[c], cache_type) * k_scale[h * d + c]);
+          }
           s *= sm_scale;
           logits[t] = s;
           if (s > mx) mx = s;
@@ -518,7 +564,12 @@ int fdo_append_attention_prefill(const uint16_t* q, const uint16_t* k_new, const
               value_cache + (((size_t)table[t / bs] * hkv + h) * bs + t % bs) * d;
           float pr = expf(logits[t] - mx);
           l += pr;
-          for (int c = 0; c < d; ++c) acc[c] += pr * (dequant(vr[c], cache_type) * v_scale[h * d + c]);
+          if (is_dynamic(cache_type)) {
+            float pv = pr * v_scale[((size_t)table[t / bs] * hkv + h) * bs + t % bs];
+            for (int c = 0; c < d; ++c) acc[c] += pv * dequant(vr[c], cache_type);
+          } else {
+            for (int c = 0; c < d; ++c) acc[c] += pr * (dequant(vr[c], cache_type) * v_scale[h * d + c]);
+          }
         }
         for (int j = 0; j <= ci; ++j) {
           const uint16_t* vr = v_new + ((size_t)(cu_seqlens_q[b] + j) * hkv + h) * d;

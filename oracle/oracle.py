@@ -16,6 +16,9 @@ _SO = os.path.join(_HERE, "libfdattn_oracle.so")
 
 CACHE_INT8 = 1
 CACHE_FP8 = 2
+CACHE_INT8_DYNAMIC = 3   # one scale per stored row: scale caches float32 [num_blocks, hkv, bs]
+CACHE_FP8_DYNAMIC = 4
+DYNAMIC = (CACHE_INT8_DYNAMIC, CACHE_FP8_DYNAMIC)
 
 
 def build(force=False):
@@ -48,6 +51,8 @@ def lib():
         _lib.fdo_quant_int8.argtypes = [ctypes.c_float, ctypes.c_float]
         _lib.fdo_quant_fp8.restype = ctypes.c_uint8
         _lib.fdo_quant_fp8.argtypes = [ctypes.c_float, ctypes.c_float]
+        _lib.fdo_row_scale.restype = ctypes.c_float
+        _lib.fdo_row_scale.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int]
     return _lib
 
 
@@ -94,6 +99,12 @@ def quant_int8(x, scale):
     return f(np.asarray(x, dtype=np.float32), np.asarray(scale, dtype=np.float32))
 
 
+def row_scale(x, cache_type):
+    """The scale the dynamic formats store for the row x (float32 [d])."""
+    x = _c(x, np.float32)
+    return float(lib().fdo_row_scale(_p(x), x.size, cache_type))
+
+
 def softmax_row(x):
     x = _c(x, np.float32)
     y = np.empty_like(x)
@@ -107,7 +118,8 @@ def write_cache_kv(qkv, key_cache, value_cache, k_scale, v_scale, rope_cos, rope
                    block_tables, seq_lens_decoder, cu_seqlens_q, hq, hkv, d, rope_style,
                    cache_type, want_kv_out=True, qkv_bias=None, q_norm_weight=None, k_norm_weight=None,
                    rms_norm_eps=0.0):
-    """Mutates key_cache / value_cache (uint8 [num_blocks,hkv,bs,d]) in place.
+    """Mutates key_cache / value_cache (uint8 [num_blocks,hkv,bs,d]) in place - and, for the dynamic
+    formats, k_scale / v_scale (float32 [num_blocks,hkv,bs]), which receive the stored rows' scales.
 
     qkv_bias: uint16 bf16 patterns [(hq+2hkv)*d]; q_norm_weight / k_norm_weight: float32 [d].
     Returns (q_out, k_out, v_out) as uint16 bf16 patterns.
@@ -117,6 +129,9 @@ def write_cache_kv(qkv, key_cache, value_cache, k_scale, v_scale, rope_cos, rope
     assert key_cache.dtype == np.uint8 and key_cache.flags.c_contiguous
     assert value_cache.dtype == np.uint8 and value_cache.flags.c_contiguous
     num_blocks, _, bs, _ = key_cache.shape
+    if cache_type in DYNAMIC:
+        for sc in (k_scale, v_scale):
+            assert sc.dtype == np.float32 and sc.flags.c_contiguous and sc.shape == (num_blocks, hkv, bs)
     k_scale, v_scale = _c(k_scale, np.float32), _c(v_scale, np.float32)
     rope_cos, rope_sin = _c(rope_cos, np.float32), _c(rope_sin, np.float32)
     bt = _c(block_tables, np.int32)

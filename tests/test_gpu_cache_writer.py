@@ -6,7 +6,9 @@ import torch
 import fastdeploy_amd as fd
 from conftest import bits, np_of
 from fastdeploy_amd import synthetic as syn
-from fastdeploy_amd.ops import CACHE_FP8, CACHE_INT8
+from fastdeploy_amd.ops import CACHE_FP8, CACHE_FP8_DYNAMIC, CACHE_INT8, CACHE_INT8_DYNAMIC, is_dynamic
+
+ALL_FORMATS = [CACHE_INT8, CACHE_FP8, CACHE_INT8_DYNAMIC, CACHE_FP8_DYNAMIC]
 
 pytestmark = pytest.mark.gpu
 
@@ -21,20 +23,24 @@ def _run_both(oracle, case, want_kv=True, rope=True):
         cache_quant_type=case["quant"], want_kv_out=want_kv)
     torch.cuda.synchronize()
     kc, vc = np_of(case["key_cache"]).copy(), np_of(case["value_cache"]).copy()
+    ks, vs = np_of(case["cache_k_scale"]).copy(), np_of(case["cache_v_scale"]).copy()  # the dynamic formats store into them
     oq, ok, ov = oracle.write_cache_kv(
-        bits(case["qkv"]), kc, vc, np_of(case["cache_k_scale"]), np_of(case["cache_v_scale"]),
+        bits(case["qkv"]), kc, vc, ks, vs,
         np_of(case["rope_cos"]) if rope else None, np_of(case["rope_sin"]) if rope else None,
         np_of(case["block_tables"]), np_of(case["seq_lens_decoder"]), np_of(case["cu_seqlens_q"]), case["hq"],
         case["hkv"], case["d"], 1 if case["rope_style"] == "neox" else 0, case["quant"], want_kv)
     assert np.array_equal(np_of(dev["key_cache"]), kc), "key cache bytes differ"
     assert np.array_equal(np_of(dev["value_cache"]), vc), "value cache bytes differ"
+    if is_dynamic(case["quant"]):
+        assert np.array_equal(np_of(dev["cache_k_scale"]).view(np.uint32), ks.view(np.uint32)), "K scale cache differs"
+        assert np.array_equal(np_of(dev["cache_v_scale"]).view(np.uint32), vs.view(np.uint32)), "V scale cache differs"
     assert np.array_equal(bits(q), oq), "rotated Q differs"
     if want_kv:
         assert np.array_equal(bits(k), ok) and np.array_equal(bits(v), ov)
     return dev
 
 
-@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+@pytest.mark.parametrize("quant", ALL_FORMATS)
 @pytest.mark.parametrize("style", ["neox", "interleaved"])
 def test_writer_bit_exact_small(oracle, quant, style):
     for seed in range(3):
@@ -47,7 +53,20 @@ def test_writer_config3_shape_bit_exact(oracle):
         _run_both(oracle, syn.write_case(num_seqs=256, max_pos=8192, seed=seed, blocks_per_seq=128))
 
 
-@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+@pytest.mark.parametrize("quant", [CACHE_INT8_DYNAMIC, CACHE_FP8_DYNAMIC])
+def test_writer_dynamic_formats_other_head_dims_and_odd_rows(oracle, quant):
+    """One scale per stored row for head_dim 128 / 64 / 32 (8, 4, 2 threads share a row), rows of zeros and rows
+    holding a NaN: bytes and scale caches bit for bit as the oracle's."""
+    for d, hq, hkv in ((128, 8, 2), (64, 4, 2), (32, 2, 1)):
+        case = syn.write_case(num_seqs=9, max_pos=400, quant=quant, seed=3 + d, hq=hq, hkv=hkv, d=d, chunk=4)
+        x = case["qkv"].view(36, hq + 2 * hkv, d)
+        x[3, hq] = 0                       # a K row of zeros: scale 1, bytes 0
+        x[5, hq + hkv, 7] = float("nan")   # a NaN does not take part in the row's maximum
+        x[7, hq + hkv + hkv - 1] *= 300.0  # a large row
+        _run_both(oracle, case)
+
+
+@pytest.mark.parametrize("quant", ALL_FORMATS)
 def test_writer_chunks_ragged_and_no_rope(oracle, quant):
     case = syn.write_case(num_seqs=5, max_pos=700, quant=quant, seed=4, chunk=37)
     _run_both(oracle, case)

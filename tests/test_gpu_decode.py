@@ -6,7 +6,9 @@ import torch
 import fastdeploy_amd as fd
 from conftest import bf16_close, bits, np_of
 from fastdeploy_amd import synthetic as syn
-from fastdeploy_amd.ops import CACHE_FP8, CACHE_INT8
+from fastdeploy_amd.ops import CACHE_FP8, CACHE_FP8_DYNAMIC, CACHE_INT8, CACHE_INT8_DYNAMIC
+
+ALL_FORMATS = [CACHE_INT8, CACHE_FP8, CACHE_INT8_DYNAMIC, CACHE_FP8_DYNAMIC]
 
 pytestmark = pytest.mark.gpu
 
@@ -35,7 +37,7 @@ def check(got, want, what=""):
 
 
 @pytest.mark.parametrize("impl", ["generic", "auto"])
-@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+@pytest.mark.parametrize("quant", ALL_FORMATS)
 def test_decode_config1(oracle, impl, quant):
     """batch 4, 32/8 heads, head_dim 128, ctx 1024, 64 physical blocks in a random permutation."""
     for seed in range(3):
@@ -44,7 +46,7 @@ def test_decode_config1(oracle, impl, quant):
 
 
 @pytest.mark.parametrize("impl", ["generic", "auto"])
-@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+@pytest.mark.parametrize("quant", ALL_FORMATS)
 def test_decode_ragged_and_edge_lengths(oracle, impl, quant):
     lens = [1, 2, 63, 64, 65, 127, 128, 129, 700, 0, 1000, 31]
     case = syn.decode_case(batch=len(lens), ctx=lens, quant=quant, seed=5, extra_blocks=7, max_blocks=20)
@@ -76,6 +78,21 @@ def test_decode_this_time_adds_to_kv_len(oracle, impl):
     check(bits(out), oracle_decode(oracle, case), "this_time")
 
 
+@pytest.mark.parametrize("impl", ["generic", "auto"])
+@pytest.mark.parametrize("quant", [CACHE_INT8_DYNAMIC, CACHE_FP8_DYNAMIC])
+def test_decode_dynamic_formats_with_widely_different_row_scales(oracle, impl, quant):
+    """One scale per stored row; the rows of one block differ in scale by up to 2^16 for V and 2^12 for K, and the
+    slots past a sequence's end hold NaN scales.  The dequantised magnitudes stay at the scale the absolute part of
+    the tolerance is meant for (|V| up to about 8)."""
+    case = syn.decode_case(batch=5, ctx=[1, 64, 200, 1000, 2500], quant=quant, seed=12, extra_blocks=3)
+    g = torch.Generator().manual_seed(5)
+    for name, lo, hi in (("cache_k_scale", -6, 0), ("cache_v_scale", -12, -2)):
+        sc = case[name]
+        mult = torch.exp2(torch.randint(lo, hi + 1, sc.shape, generator=g).float())
+        case[name] = torch.where(sc.isnan(), sc, sc * mult)
+    check(gpu_decode(case, impl), oracle_decode(oracle, case), "row scales")
+
+
 def test_decode_generic_other_shapes(oracle):
     """Shapes outside the MFMA kernel: head_dim 64, group 2, block_size 16."""
     case = syn.decode_case(batch=3, ctx=[50, 200, 333], seed=8, hq=8, hkv=4, d=64, bs=16)
@@ -87,7 +104,7 @@ def test_decode_generic_other_shapes(oracle):
 
 
 @pytest.mark.parametrize("impl", ["generic", "auto"])
-@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+@pytest.mark.parametrize("quant", ALL_FORMATS)
 def test_sparse_decode(oracle, impl, quant):
     case = syn.decode_case(batch=3, ctx=[2000, 1500, 64 * 40 + 5], quant=quant, seed=9)
     rng = np.random.default_rng(1)

@@ -6,7 +6,8 @@ import torch
 
 import fastdeploy_amd as fd
 from conftest import bf16_close, bits, np_of
-from fastdeploy_amd.ops import CACHE_FP8, CACHE_INT8, cu_seqlens_of, seq_lens_this_time_of
+from fastdeploy_amd.ops import (CACHE_FP8, CACHE_FP8_DYNAMIC, CACHE_INT8, CACHE_INT8_DYNAMIC, byte_format, cu_seqlens_of,
+                                is_dynamic, seq_lens_this_time_of)
 from fastdeploy_amd.rope import rope_table
 
 pytestmark = pytest.mark.gpu
@@ -24,15 +25,16 @@ def mixed_case(enc, dec, quant, seed, hq=32, hkv=8, d=128, bs=64, max_pos=4096):
     bt = torch.randperm(pool, generator=g).to(torch.int32).view(batch, mb).contiguous()
     kc = torch.randint(0, 256, (pool, hkv, bs, d), generator=g, dtype=torch.uint8)
     vc = torch.randint(0, 256, (pool, hkv, bs, d), generator=g, dtype=torch.uint8)
-    if quant == CACHE_FP8:  # no NaN codes in the prior contents
+    if byte_format(quant) == CACHE_FP8:  # no NaN codes in the prior contents
         kc = torch.where((kc & 0x7F) == 0x7F, kc & 0xFE, kc)
         vc = torch.where((vc & 0x7F) == 0x7F, vc & 0xFE, vc)
     # The prior cache bytes are uniform over all codes - far heavier-tailed than quantised activations - so the
     # scales put the dequantised range at +-(1..1.5): the prefill kernel carries q*k_scale and the softmax weights
     # in fp16, and its error grows with the magnitude of the dequantised cache.
-    qmax = 127.0 if quant == CACHE_INT8 else 448.0
-    ks = ((torch.rand((hkv, d), generator=g) * 0.5 + 1.0) / qmax).contiguous()
-    vs = ((torch.rand((hkv, d), generator=g) * 0.5 + 1.0) / qmax).contiguous()
+    qmax = 127.0 if byte_format(quant) == CACHE_INT8 else 448.0
+    shape = (pool, hkv, bs) if is_dynamic(quant) else (hkv, d)  # one scale per stored row / per channel
+    ks = ((torch.rand(shape, generator=g) * 0.5 + 1.0) / qmax).contiguous()
+    vs = ((torch.rand(shape, generator=g) * 0.5 + 1.0) / qmax).contiguous()
     qkv = torch.randn((T, (hq + 2 * hkv) * d), generator=g).to(torch.bfloat16)
     cos, sin = rope_table(max_pos, d, 500000.0, "cpu")
     return dict(qkv=qkv, key_cache=kc, value_cache=vc, cache_k_scale=ks, cache_v_scale=vs, block_tables=bt,
@@ -42,9 +44,11 @@ def mixed_case(enc, dec, quant, seed, hq=32, hkv=8, d=128, bs=64, max_pos=4096):
 
 def oracle_step(oracle, c, quant, hq=32, hkv=8, d=128, **epilogue):
     """The step composed from the oracle's pieces; returns (out bf16 bits [T, hq*d] with NaN-free rows only where
-    a token exists, key cache, value cache)."""
+    a token exists, key cache, value cache).  For the dynamic formats the scale caches the step leaves behind are
+    put into c["scales_after"]."""
     kc, vc = np_of(c["key_cache"]).copy(), np_of(c["value_cache"]).copy()
-    ks, vs = np_of(c["cache_k_scale"]), np_of(c["cache_v_scale"])
+    ks, vs = np_of(c["cache_k_scale"]).copy(), np_of(c["cache_v_scale"]).copy()
+    c["scales_after"] = (ks, vs)
     bt, dec, cu = np_of(c["block_tables"]), np_of(c["seq_lens_decoder"]), np_of(c["cu_seqlens_q"])
     enc, this = np_of(c["seq_lens_encoder"]), np_of(c["seq_lens_this_time"])
     q, k_new, v_new = oracle.write_cache_kv(bits(c["qkv"]), kc, vc, ks, vs, np_of(c["rope_cos"]), np_of(c["rope_sin"]),
@@ -65,7 +69,7 @@ def oracle_step(oracle, c, quant, hq=32, hkv=8, d=128, **epilogue):
     return out, kc, vc
 
 
-@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8, CACHE_INT8_DYNAMIC, CACHE_FP8_DYNAMIC])
 def test_mixed_batch_step(oracle, quant):
     enc = [0, 150, 0, 0, 70, 0, 1, 300]
     dec = [700, 0, 0, 63, 200, 1, 0, 129]
@@ -79,6 +83,10 @@ def test_mixed_batch_step(oracle, quant):
     torch.cuda.synchronize()
     want, kc, vc = oracle_step(oracle, c, quant)
     assert np.array_equal(np_of(dev["key_cache"]), kc) and np.array_equal(np_of(dev["value_cache"]), vc)
+    if is_dynamic(quant):  # the writer stored the new rows' scales
+        assert np.array_equal(np_of(dev["cache_k_scale"]), c["scales_after"][0])
+        assert np.array_equal(np_of(dev["cache_v_scale"]), c["scales_after"][1])
+        assert not np.array_equal(np_of(c["cache_k_scale"]), c["scales_after"][0])
     ok, mx, bad = bf16_close(bits(out), want)
     assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
 
@@ -137,6 +145,50 @@ def test_mixed_step_with_key_splits_for_the_prefill_row(oracle):
     assert rc == 0
     ok, mx, bad = bf16_close(bits(o2), want)
     assert ok, "small workspace: %d out of tolerance, max %.4g" % (bad, mx)
+
+
+def test_mixed_step_with_key_splits_replays_from_a_hip_graph():
+    """The mixed step with key splits (writer, decode + its merge, prefill shares, prefill merge) captured in a HIP
+    graph: every replay, with eager work and synchronisations in between, equals the eager step on a copy of the
+    state bit for bit (outputs and cache bytes)."""
+    enc, dec = [0, 160, 0, 0, 0], [900, 4200, 63, 2100, 4600]
+    c = mixed_case(enc, dec, CACHE_INT8, seed=21, max_pos=8192)
+    dev = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
+    eag = {k: (v.clone() if isinstance(v, torch.Tensor) else v) for k, v in dev.items()}
+    splits = fd.ops.prefill_auto_splits(1, 32, 160)
+    assert splits > 1
+    mb = dev["block_tables"].shape[1]
+    ws_g = fd.append_attention_workspace(c["T"], 5, 32, 8, 128, mb, prefill_splits=splits)
+    ws_e = fd.append_attention_workspace(c["T"], 5, 32, 8, 128, mb, prefill_splits=splits)
+
+    def step(s, ws):
+        return fd.append_attention(s["qkv"], s["key_cache"], s["value_cache"], s["seq_lens_encoder"],
+                                   s["seq_lens_decoder"], s["seq_lens_this_time"], s["block_tables"],
+                                   (s["rope_cos"], s["rope_sin"]), s["cache_k_scale"], s["cache_v_scale"],
+                                   num_heads=32, kv_num_heads=8, max_chunk=160, cu_seqlens_q=s["cu_seqlens_q"],
+                                   prefill_rows=1, workspace=ws)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up outside the capture, on a throw-away copy
+        tmp = {k: (v.clone() if isinstance(v, torch.Tensor) else v) for k, v in dev.items()}
+        step(tmp, ws_g)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_g = step(dev, ws_g)
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    for r in range(3):
+        new_qkv = torch.randn(dev["qkv"].shape, generator=gen, device="cuda").to(torch.bfloat16)
+        dev["qkv"].copy_(new_qkv)  # eager work between the replays
+        eag["qkv"].copy_(new_qkv)
+        torch.cuda.synchronize()
+        graph.replay()
+        want = step(eag, ws_e)
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, want), "replay %d: outputs differ" % r
+        assert torch.equal(dev["key_cache"], eag["key_cache"]) and torch.equal(dev["value_cache"], eag["value_cache"]), r
 
 
 def test_decode_only_and_prefill_only_steps_through_the_same_entry(oracle):

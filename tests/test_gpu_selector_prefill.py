@@ -6,7 +6,9 @@ import torch
 import fastdeploy_amd as fd
 from conftest import bf16_close, bits, np_of
 from fastdeploy_amd import synthetic as syn
-from fastdeploy_amd.ops import CACHE_FP8, CACHE_INT8
+from fastdeploy_amd.ops import CACHE_FP8, CACHE_FP8_DYNAMIC, CACHE_INT8, CACHE_INT8_DYNAMIC
+
+ALL_FORMATS = [CACHE_INT8, CACHE_FP8, CACHE_INT8_DYNAMIC, CACHE_FP8_DYNAMIC]
 
 pytestmark = pytest.mark.gpu
 
@@ -84,6 +86,14 @@ def test_selector_config4_shape_indices_bit_exact(oracle):
     assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
 
 
+def test_selector_rejects_the_dynamic_formats():
+    """The block scores are defined on per-channel scales: the formats with one scale per stored row are refused."""
+    case = syn.to_device(syn.decode_case(batch=2, ctx=[300, 500], quant=CACHE_FP8_DYNAMIC, seed=1), "cuda")
+    with pytest.raises(ValueError, match="per-channel"):
+        fd.sqattn_select(case["q"], case["key_cache"], case["cache_k_scale"], case["block_tables"],
+                         case["seq_lens_decoder"], num_heads=32, top_k=4, cache_quant_type=CACHE_FP8_DYNAMIC)
+
+
 def _prefill_case(seed, prefix, chunks, quant=CACHE_INT8):
     batch = len(chunks)
     base = syn.decode_case(batch=batch, ctx=prefix, quant=quant, seed=seed, extra_blocks=4)
@@ -97,7 +107,7 @@ def _prefill_case(seed, prefix, chunks, quant=CACHE_INT8):
 
 
 @pytest.mark.parametrize("impl", ["generic", "auto"])
-@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+@pytest.mark.parametrize("quant", ALL_FORMATS)
 def test_prefill_small(oracle, impl, quant):
     c = _prefill_case(1, [200, 64, 0, 333], [70, 128, 5, 1], quant)
     dev = syn.to_device(c, "cuda")
@@ -113,7 +123,7 @@ def test_prefill_small(oracle, impl, quant):
     assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
 
 
-@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+@pytest.mark.parametrize("quant", ALL_FORMATS)
 def test_prefill_ragged_edges(oracle, quant):
     """Prefix lengths around the tile size, chunks around the workgroup size, an empty prefix."""
     c = _prefill_case(2, [0, 63, 64, 65, 1000, 129], [129, 128, 1, 127, 257, 64], quant)

@@ -15,7 +15,7 @@ import torch
 
 from conftest import bf16_close, bits, np_of
 from fastdeploy_amd import synthetic as syn
-from fastdeploy_amd.ops import CACHE_FP8, CACHE_INT8
+from fastdeploy_amd.ops import CACHE_FP8, CACHE_FP8_DYNAMIC, CACHE_INT8, CACHE_INT8_DYNAMIC, is_dynamic
 from fastdeploy_amd.rope import rope_table
 
 def assert_is_bf16_of(got, want, extra=3e-4):
@@ -291,6 +291,60 @@ def test_writer_bytes_match_torch_formulas(oracle, quant):
             assert np.array_equal(vc[blk, :, slot], wv[b, i])
 
 
+@pytest.mark.parametrize("quant", [CACHE_INT8_DYNAMIC, CACHE_FP8_DYNAMIC])
+def test_writer_dynamic_formats_scale_and_bytes(oracle, quant):
+    """One scale per stored row.  Without rotation: scale = numpy's max-abs / 127 (/ 448) of the row and the bytes
+    are torch's x / scale -> round / clamp (-> e4m3 cast); the row's largest element maps to the largest code.
+    With rotation: the bytes are those of the (pinned) per-channel writer run with the row's scale in every channel."""
+    fmt = CACHE_INT8 if quant == CACHE_INT8_DYNAMIC else CACHE_FP8
+    qmax = np.float32(127.0 if fmt == CACHE_INT8 else 448.0)
+    case = syn.write_case(num_seqs=6, max_pos=300, seed=21, quant=quant, chunk=2)
+    hq, hkv, d = case["hq"], case["hkv"], case["d"]
+    args = (np_of(case["block_tables"]), np_of(case["seq_lens_decoder"]), np_of(case["cu_seqlens_q"]), hq, hkv, d, 1)
+    # a row of zeros and a row with a NaN among the inputs
+    qkv = case["qkv"].clone().view(12, hq + 2 * hkv, d)
+    qkv[0, hq + 1] = 0
+    qkv[1, hq + hkv + 2, 5] = float("nan")
+    qkv = qkv.view(12, -1)
+    kc, vc = np_of(case["key_cache"]).copy(), np_of(case["value_cache"]).copy()
+    ks, vs = np_of(case["cache_k_scale"]).copy(), np_of(case["cache_v_scale"]).copy()
+    ks0, vs0 = ks.copy(), vs.copy()
+    oracle.write_cache_kv(bits(qkv), kc, vc, ks, vs, None, None, *args, quant)
+    x = qkv.float().view(6, 2, hq + 2 * hkv, d).numpy()
+    touched = np.zeros(ks.shape, bool)
+    for b in range(6):
+        for i in range(2):
+            p = int(case["seq_lens_decoder"][b]) + i
+            blk, slot = int(case["block_tables"][b, p // 64]), p % 64
+            touched[blk, :, slot] = True
+            for h in range(hkv):
+                for row, cache, sc in ((x[b, i, hq + h], kc, ks), (x[b, i, hq + hkv + h], vc, vs)):
+                    m = np.nanmax(np.abs(row)).astype(np.float32)
+                    want_s = np.float32(m / qmax) if m > 0 else np.float32(1.0)
+                    assert sc[blk, h, slot] == want_s
+                    wb = syn.quantize_ref(torch.from_numpy(row), float(want_s), quant).numpy()
+                    assert np.array_equal(cache[blk, h, slot], wb)
+                    if m > 0:  # the largest element takes the largest code
+                        top = cache[blk, h, slot][np.nanargmax(np.abs(row))]
+                        assert (int(np.int8(top)) in (-127, 127)) if fmt == CACHE_INT8 else (top & 0x7F) == 0x7E
+    assert np.array_equal(ks[~touched], ks0[~touched]) and np.array_equal(vs[~touched], vs0[~touched])
+    assert ks[int(case["block_tables"][0, int(case["seq_lens_decoder"][0]) // 64]), 1, int(case["seq_lens_decoder"][0]) % 64] == 1.0
+    # with rotation: token by token against the per-channel writer carrying that row's scale
+    rope = (np_of(case["rope_cos"]), np_of(case["rope_sin"]))
+    kc, vc = np_of(case["key_cache"]).copy(), np_of(case["value_cache"]).copy()
+    oracle.write_cache_kv(bits(case["qkv"]), kc, vc, ks, vs, *rope, *args, quant)
+    for b in range(6):
+        p = int(case["seq_lens_decoder"][b])
+        blk, slot = int(case["block_tables"][b, p // 64]), p % 64
+        kc2, vc2 = np_of(case["key_cache"]).copy(), np_of(case["value_cache"]).copy()
+        sk = np.repeat(ks[blk, :, slot][:, None], d, 1).astype(np.float32)
+        sv = np.repeat(vs[blk, :, slot][:, None], d, 1).astype(np.float32)
+        oracle.write_cache_kv(bits(case["qkv"]), kc2, vc2, sk, sv, *rope, *args, fmt)
+        assert np.array_equal(kc[blk, :, slot], kc2[blk, :, slot]) and np.array_equal(vc[blk, :, slot], vc2[blk, :, slot])
+        k8 = kc[blk, :, slot].view(np.int8) if fmt == CACHE_INT8 else kc[blk, :, slot] & 0x7F
+        assert (np.abs(k8.astype(np.int32)).max(-1) == (127 if fmt == CACHE_INT8 else 0x7E)).all()
+
+
 # ------------------------------------------------------------ decode attention
 
 def _gather_dense(case, b):
@@ -298,8 +352,12 @@ def _gather_dense(case, b):
     n = int(case["seq_lens_decoder"][b])
     nb = (n + case["bs"] - 1) // case["bs"]
     idx = case["block_tables"][b, :nb].long()
-    k = syn.dequantize_ref(case["key_cache"][idx], case["cache_k_scale"][:, None, :], case["quant"])
-    v = syn.dequantize_ref(case["value_cache"][idx], case["cache_v_scale"][:, None, :], case["quant"])
+    if is_dynamic(case["quant"]):  # one scale per stored row: [pool, hkv, bs]
+        sk, sv = case["cache_k_scale"][idx][..., None], case["cache_v_scale"][idx][..., None]
+    else:
+        sk, sv = case["cache_k_scale"][:, None, :], case["cache_v_scale"][:, None, :]
+    k = syn.dequantize_ref(case["key_cache"][idx], sk, case["quant"])
+    v = syn.dequantize_ref(case["value_cache"][idx], sv, case["quant"])
     k = k.permute(0, 2, 1, 3).reshape(nb * case["bs"], case["hkv"], case["d"])[:n].double()
     v = v.permute(0, 2, 1, 3).reshape(nb * case["bs"], case["hkv"], case["d"])[:n].double()
     return k, v
@@ -330,6 +388,36 @@ def test_decode_matches_torch_sdpa_fp64(oracle, quant):
     got = oracle.bf16_to_f32(_decode(oracle, case)).astype(np.float64)
     want = _sdpa_decode(case).numpy()
     assert_is_bf16_of(got, want)
+
+
+@pytest.mark.parametrize("quant", [CACHE_INT8_DYNAMIC, CACHE_FP8_DYNAMIC])
+def test_decode_dynamic_formats_match_sdpa_and_the_per_channel_path(oracle, quant):
+    """Scales per stored row: fp64 SDPA on the dequantised cache (rows scaled over 2^-3 .. 2^3); and when every row
+    of a head carries one scale, the result of the per-channel path with that scale in every channel."""
+    case = syn.decode_case(batch=3, ctx=[1, 63, 330], quant=quant, seed=1, extra_blocks=5)
+    got = oracle.bf16_to_f32(_decode(oracle, case)).astype(np.float64)
+    assert_is_bf16_of(got, _sdpa_decode(case).numpy())
+    fmt = CACHE_INT8 if quant == CACHE_INT8_DYNAMIC else CACHE_FP8
+    stat = syn.decode_case(batch=2, ctx=[200, 77], quant=fmt, seed=3, extra_blocks=2, direct_bytes=True)
+    dyn = dict(stat)
+    dyn["quant"] = quant
+    pool = stat["key_cache"].shape[0]
+    head_k, head_v = stat["cache_k_scale"][:, 0], stat["cache_v_scale"][:, 0]
+    stat["cache_k_scale"] = head_k[:, None].repeat(1, 128).contiguous()
+    stat["cache_v_scale"] = head_v[:, None].repeat(1, 128).contiguous()
+    dyn["cache_k_scale"] = head_k[None, :, None].repeat(pool, 1, 64).contiguous()
+    dyn["cache_v_scale"] = head_v[None, :, None].repeat(pool, 1, 64).contiguous()
+    a, b = _decode(oracle, stat), _decode(oracle, dyn)
+    ok, mx, bad = bf16_close(b, a, atol=1e-4, rtol=2 ** -7)
+    assert ok, (mx, bad)
+    # sparse lists read the same scale rows
+    kept = np.full((2, 8, 4), -1, np.int32)
+    kept[0, :, :3] = [0, 2, 3]
+    kept[1, :, :2] = [0, 1]
+    cnt = np.array([[3] * 8, [2] * 8], np.int32)
+    a, b = _decode(oracle, stat, kept_blocks=kept, kept_counts=cnt), _decode(oracle, dyn, kept_blocks=kept, kept_counts=cnt)
+    ok, mx, bad = bf16_close(b, a, atol=1e-4, rtol=2 ** -7)
+    assert ok, (mx, bad)
 
 
 def test_decode_config1_shape_and_block_table_permutation_invariance(oracle):
@@ -515,6 +603,22 @@ def test_prefill_matches_dense_causal_sdpa(oracle, quant):
         mask = torch.arange(p + n)[None, :] <= (p + torch.arange(n))[:, None]
         want = torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask).permute(1, 0, 2).reshape(n, -1)
         assert_is_bf16_of(got[cu[b]:cu[b + 1]], want.numpy())
+
+
+@pytest.mark.parametrize("quant", [CACHE_INT8_DYNAMIC, CACHE_FP8_DYNAMIC])
+def test_prefill_dynamic_formats_match_dense_causal_sdpa(oracle, quant):
+    c = _prefill_case(4, 2, [70, 129], [33, 20], quant)
+    got = oracle.bf16_to_f32(_prefill(oracle, c)).astype(np.float64)
+    cu = c["cu_seqlens_q"].tolist()
+    for b in range(2):
+        kp, vp = _gather_dense(c, b)
+        n, p = cu[b + 1] - cu[b], kp.shape[0]
+        k = torch.cat([kp, c["k_new"][cu[b]:cu[b + 1]].double().view(n, 8, 128)]).permute(1, 0, 2).repeat_interleave(4, 0)
+        v = torch.cat([vp, c["v_new"][cu[b]:cu[b + 1]].double().view(n, 8, 128)]).permute(1, 0, 2).repeat_interleave(4, 0)
+        q = c["q_new"][cu[b]:cu[b + 1]].double().view(n, 32, 128).permute(1, 0, 2)
+        mask = torch.arange(p + n)[None, :] <= (p + torch.arange(n))[:, None]
+        want = torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask).permute(1, 0, 2).reshape(n, -1)
+        assert_is_bf16_of(got[cu[b]:cu[b + 1]], want.numpy(), extra=1e-3)
 
 
 def test_prefill_row_subset_and_one_token_chunk_equals_decode(oracle):
