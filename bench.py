@@ -175,6 +175,56 @@ def other_workloads(args):
                  {"note": "roofline counts the decode rows' K/V bytes only; the prefill row adds %.1f GFLOP" %
                           (syn.prefill_flops(8192, 512) / 1e9)})
         del c
+    if args.workload in ("dynamic", "all"):
+        # the formats with one scale per stored row: configs[1]'s decode (two pools rotated, as the headline run) and
+        # the prefill-sized cache write; the scale caches add 2 x 4 B per token and KV head to the bytes moved
+        lens = torch.randint(3584, 4609, (64,), generator=torch.Generator().manual_seed(0)).tolist()
+        for name in ("cache_int8_dynamic", "cache_fp8_dynamic"):
+            cs = [syn.decode_case(batch=64, ctx=lens, pool_blocks=6000, seed=sd, device=dev, direct_bytes=True,
+                                  max_blocks=72, quant=name) for sd in range(2)]
+            ws = fd.decode_workspace(64, 32, 8, 128, 72, dev)
+            out = torch.empty((64, 32 * 128), dtype=torch.bfloat16, device=dev)
+            n = [0]
+
+            def dec_dyn():
+                c = cs[n[0] % 2]
+                n[0] += 1
+                fd.decode_attention(c["q"], c["key_cache"], c["value_cache"], c["cache_k_scale"], c["cache_v_scale"],
+                                    c["block_tables"], c["seq_lens_decoder"], num_heads=32, cache_quant_type=name,
+                                    out=out, workspace=ws)
+            ms = time_events(dec_dyn, args.steps, args.warmup)
+            work = syn.decode_algorithmic_bytes(lens, 64) - 2 * 8 * 128 * 4 + sum(lens) * 8 * 2 * 4
+            line("configs[1] decode over the %s cache (one scale per stored row)" % name, ms, "hbm", work,
+                 HBM_PEAK_GBPS, "GB/s")
+            del cs
+        cw = syn.write_case(num_seqs=2, max_pos=8192 + 2048, seed=1, device=dev, chunk=2048, blocks_per_seq=160,
+                            quant="cache_int8_dynamic")
+        cw["seq_lens_decoder"].fill_(8192)
+        rotw = (cw["rope_cos"], cw["rope_sin"])
+
+        def wr_dyn():
+            return fd.write_cache_kv(cw["qkv"], cw["key_cache"], cw["value_cache"], cw["cache_k_scale"], cw["cache_v_scale"],
+                                     cw["block_tables"], cw["seq_lens_encoder"], cw["seq_lens_decoder"], cw["seq_lens_this_time"],
+                                     cw["cu_seqlens_q"], rotw, num_heads=32, kv_num_heads=8, want_kv_out=True,
+                                     cache_quant_type="cache_int8_dynamic")
+        ms = time_events(wr_dyn, args.steps, args.warmup)
+        line("configs[4] cache write, cache_int8_dynamic (4096 tokens, q/k/v handed on)", ms, "hbm",
+             4096 * (48 * 128 * 2 * 2 + 2 * 8 * 128 + 2 * 64 * 4 + 2 * 8 * 4), HBM_PEAK_GBPS, "GB/s")
+        del cw
+        for name in ("cache_int8_dynamic", "cache_fp8_dynamic"):
+            c = syn.decode_case(batch=2, ctx=8192, seed=0, device=dev, direct_bytes=True, extra_blocks=8, quant=name)
+            q = torch.randn((4096, 4096), generator=g, device=dev).to(torch.bfloat16)
+            k = torch.randn((4096, 1024), generator=g, device=dev).to(torch.bfloat16)
+            v = torch.randn((4096, 1024), generator=g, device=dev).to(torch.bfloat16)
+            cu = torch.tensor([0, 2048, 4096], dtype=torch.int32, device=dev)
+            out = torch.empty_like(q)
+            pf = lambda: fd.append_attention_prefill(q, k, v, c["key_cache"], c["value_cache"], c["cache_k_scale"],
+                                                     c["cache_v_scale"], c["block_tables"], c["seq_lens_decoder"], cu,
+                                                     num_heads=32, max_chunk=2048, out=out, cache_quant_type=name)
+            ms = time_events(pf, max(args.steps // 10, 5), 3)
+            line("configs[4] append attention over the %s cache" % name, ms, "mfma", 2 * syn.prefill_flops(8192, 2048),
+                 2500.0, "TFLOP/s")
+
     if args.workload in ("kv_wire", "all"):
         # the sequences of configs[1] leave the cache in wire form and enter another one: HBM copies (read + write)
         from fastdeploy_amd import kv_wire
@@ -202,7 +252,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--pools", type=int, default=2, help="distinct cache pools rotated between steps")
-    ap.add_argument("--workload", default="decode", choices=["decode", "write_decode", "sqattn", "prefill", "mixed", "kv_wire", "all"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "write_decode", "sqattn", "prefill", "mixed", "dynamic", "kv_wire", "all"],
                     help="decode = the headline metric (default); the others print one line per kernel of that row")
     ap.add_argument("--calibrate", action="store_true",
                     help="kept for the profiling command line: the 1 GiB device copy (the yardstick the HBM byte "

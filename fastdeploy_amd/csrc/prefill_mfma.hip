@@ -67,11 +67,12 @@ typedef short v8s __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v2f __attribute__((ext_vector_type(2)));
 
-// how a cache byte sits in fp16: value = kMul^-1 (byte value + kOff)
-template <int QUANT>
+// how a cache byte sits in fp16: value = kMul^-1 (byte value + kOff).  DYN (one scale per stored row): the staged
+// fp16 number is the dequantised value itself, byte x scale of its row.
+template <int QUANT, bool DYN>
 struct ByteFmt {
-  static constexpr float kMul = QUANT == FDATTN_CACHE_INT8 ? 16777216.0f : 1.0f;
-  static constexpr float kOff = QUANT == FDATTN_CACHE_INT8 ? 128.0f : 0.0f;
+  static constexpr float kMul = (QUANT == FDATTN_CACHE_INT8 && !DYN) ? 16777216.0f : 1.0f;
+  static constexpr float kOff = (QUANT == FDATTN_CACHE_INT8 && !DYN) ? 128.0f : 0.0f;
 };
 
 __device__ __forceinline__ u32 pack_bf16(float lo, float hi) {
@@ -100,6 +101,30 @@ __device__ __forceinline__ uint4 cvt8(u32 w0, u32 w1) {
   const v2f c = __builtin_amdgcn_cvt_pk_f32_fp8((int)w1, false), d = __builtin_amdgcn_cvt_pk_f32_fp8((int)w1, true);
   return make_uint4(pack_f16_fast(a[0], a[1]), pack_f16_fast(b[0], b[1]), pack_f16_fast(c[0], c[1]),
                     pack_f16_fast(d[0], d[1]));
+}
+
+// 8 cache bytes of one stored row -> 8 fp16 dequantised values, byte x s, each rounded to nearest once
+template <int QUANT>
+__device__ __forceinline__ uint4 cvt8_scaled(u32 w0, u32 w1, float s) {
+  float f[8];
+  if (QUANT == FDATTN_CACHE_INT8) {
+    // (b + 128) as an unsigned byte -> float, then (b + 128) s - 128 s in one fused step: b s rounded once
+    const u32 x[2] = {w0 ^ 0x80808080u, w1 ^ 0x80808080u};
+    const float c = -128.0f * s;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      f[4 * i + 0] = __builtin_fmaf((float)(x[i] & 0xffu), s, c);
+      f[4 * i + 1] = __builtin_fmaf((float)((x[i] >> 8) & 0xffu), s, c);
+      f[4 * i + 2] = __builtin_fmaf((float)((x[i] >> 16) & 0xffu), s, c);
+      f[4 * i + 3] = __builtin_fmaf((float)(x[i] >> 24), s, c);
+    }
+  } else {
+    const v2f a = __builtin_amdgcn_cvt_pk_f32_fp8((int)w0, false), b = __builtin_amdgcn_cvt_pk_f32_fp8((int)w0, true);
+    const v2f c = __builtin_amdgcn_cvt_pk_f32_fp8((int)w1, false), d = __builtin_amdgcn_cvt_pk_f32_fp8((int)w1, true);
+    f[0] = a[0] * s; f[1] = a[1] * s; f[2] = b[0] * s; f[3] = b[1] * s;
+    f[4] = c[0] * s; f[5] = c[1] * s; f[6] = d[0] * s; f[7] = d[1] * s;
+  }
+  return make_uint4(pack_f16(f[0], f[1]), pack_f16(f[2], f[3]), pack_f16(f[4], f[5]), pack_f16(f[6], f[7]));
 }
 
 // ---- the matrix phase, hand-scheduled (generated by gen_prefill_sched.py).  Operands stream
@@ -151,7 +176,7 @@ __device__ __forceinline__ int sequence_of_row(const PrefillArgs& a, int r) {
 // how many of the launch's max_splits key splits a walk of n_tiles tiles uses
 __device__ __forceinline__ int splits_of(int n_tiles, int max_splits) { return min(max(n_tiles / 16, 1), max_splits); }
 
-template <int QUANT, int NW>
+template <int QUANT, int NW, bool DYN>
 __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   constexpr int BM = 32 * NW;       // queries per workgroup
   constexpr int PASSES = 16 / NW;   // 16-byte LDS chunks a thread stages per tile and tensor
@@ -226,8 +251,10 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
       const int c0 = 16 * s + 8 * hf;
       uint4 w = *reinterpret_cast<const uint4*>(qrow + c0);
       if (scaled) {
-        const float4 s0 = *reinterpret_cast<const float4*>(a.k_scale + h * HD + c0);
-        const float4 s1 = *reinterpret_cast<const float4*>(a.k_scale + h * HD + c0 + 4);
+        // DYN: the K scales sit in the staged tile, q goes to fp16 as it is
+        const float4 one = make_float4(1.f, 1.f, 1.f, 1.f);
+        const float4 s0 = DYN ? one : *reinterpret_cast<const float4*>(a.k_scale + h * HD + c0);
+        const float4 s1 = DYN ? one : *reinterpret_cast<const float4*>(a.k_scale + h * HD + c0 + 4);
         const v2h h0 = {(_Float16)(bf16lo_to_f32(w.x) * s0.x), (_Float16)(bf16hi_to_f32(w.x) * s0.y)};
         const v2h h1 = {(_Float16)(bf16lo_to_f32(w.y) * s0.z), (_Float16)(bf16hi_to_f32(w.y) * s0.w)};
         const v2h h2 = {(_Float16)(bf16lo_to_f32(w.z) * s1.x), (_Float16)(bf16hi_to_f32(w.z) * s1.y)};
@@ -259,6 +286,7 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   // LDS byte addresses of its K and V chunk of pass 0 in slot 0
   const u32 kw0 = lds_addr(lds + srow * LDK + scc), vw0 = lds_addr(lds + K_ELEMS + srow * LDV + scc);
   uint4 stg_k[PASSES], stg_v[PASSES];
+  float stg_ks[DYN ? PASSES : 1], stg_vs[DYN ? PASSES : 1];  // DYN: the scales of the fetched rows
   // The physical block of the next prefix tile to fetch is requested one fetch ahead and kept
   // in a vector register until it is needed (vzero hides from the compiler that the index is
   // uniform: it would otherwise move the value to a scalar register - and wait for the load -
@@ -283,6 +311,14 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
         const uint2 vv = *reinterpret_cast<const uint2*>(vb + (goff + (u32)(i * ROWS * HD)));
         stg_k[i].x = kk.x, stg_k[i].y = kk.y, stg_v[i].x = vv.x, stg_v[i].y = vv.y;
       }
+      if (DYN) {
+        const size_t srow0 = ((size_t)pb * a.hkv + h) * BN + srow;
+#pragma unroll
+        for (int i = 0; i < PASSES; ++i) {
+          stg_ks[i] = a.k_scale[srow0 + i * ROWS];
+          stg_vs[i] = a.v_scale[srow0 + i * ROWS];
+        }
+      }
     } else {
 #pragma unroll
       for (int i = 0; i < PASSES; ++i) {
@@ -305,12 +341,20 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
       if ((t + 1) * BN > p) {
 #pragma unroll
         for (int i = 0; i < PASSES; ++i)
-          if (t * BN + srow + i * ROWS >= p) stg_k[i].x = stg_k[i].y = stg_v[i].x = stg_v[i].y = 0u;
+          if (t * BN + srow + i * ROWS >= p) {
+            stg_k[i].x = stg_k[i].y = stg_v[i].x = stg_v[i].y = 0u;
+            if (DYN) stg_ks[i] = stg_vs[i] = 0.f;  // their scale slots may hold anything
+          }
       }
 #pragma unroll
       for (int i = 0; i < PASSES; ++i) {
-        lds_store16(kd + i * ROWS * LDK * 2, cvt8<QUANT>(stg_k[i].x, stg_k[i].y));
-        lds_store16(vd + i * ROWS * LDV * 2, cvt8<QUANT>(stg_v[i].x, stg_v[i].y));
+        if (DYN) {
+          lds_store16(kd + i * ROWS * LDK * 2, cvt8_scaled<QUANT>(stg_k[i].x, stg_k[i].y, stg_ks[i]));
+          lds_store16(vd + i * ROWS * LDV * 2, cvt8_scaled<QUANT>(stg_v[i].x, stg_v[i].y, stg_vs[i]));
+        } else {
+          lds_store16(kd + i * ROWS * LDK * 2, cvt8<QUANT>(stg_k[i].x, stg_k[i].y));
+          lds_store16(vd + i * ROWS * LDV * 2, cvt8<QUANT>(stg_v[i].x, stg_v[i].y));
+        }
       }
     } else {
 #pragma unroll
@@ -340,7 +384,7 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
 
   load_q(t0 < n_pre);
   // log2-domain constant that removes the byte offset from the prefix scores
-  const float qbias = -ByteFmt<QUANT>::kOff * sc * (qsum + __shfl_xor(qsum, 32, 64));
+  const float qbias = -ByteFmt<QUANT, DYN>::kOff * sc * (qsum + __shfl_xor(qsum, 32, 64));
 
   // prologue: the first tile (and group 1's rows of the second) into LDS
   fetch(t0);
@@ -355,16 +399,17 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   // leaving the quantised prefix: o holds sums over offset bytes; remove the offset and give the channels
   // their scale
   auto leave_prefix = [&]() {
-    const float l_off = -ByteFmt<QUANT>::kOff * (l_run + __shfl_xor(l_run, 32, 64));
+    if (DYN) return;  // the staged values were the dequantised ones: nothing to remove, nothing to scale
+    const float l_off = -ByteFmt<QUANT, DYN>::kOff * (l_run + __shfl_xor(l_run, 32, 64));
 #pragma unroll
     for (int ct = 0; ct < 4; ++ct)
 #pragma unroll
       for (int rb = 0; rb < 4; ++rb) {
         const float4 vs = *reinterpret_cast<const float4*>(a.v_scale + h * HD + 32 * ct + 8 * rb + 4 * hf);
-        o[ct][4 * rb + 0] = (o[ct][4 * rb + 0] * ByteFmt<QUANT>::kMul + l_off) * vs.x;
-        o[ct][4 * rb + 1] = (o[ct][4 * rb + 1] * ByteFmt<QUANT>::kMul + l_off) * vs.y;
-        o[ct][4 * rb + 2] = (o[ct][4 * rb + 2] * ByteFmt<QUANT>::kMul + l_off) * vs.z;
-        o[ct][4 * rb + 3] = (o[ct][4 * rb + 3] * ByteFmt<QUANT>::kMul + l_off) * vs.w;
+        o[ct][4 * rb + 0] = (o[ct][4 * rb + 0] * ByteFmt<QUANT, DYN>::kMul + l_off) * vs.x;
+        o[ct][4 * rb + 1] = (o[ct][4 * rb + 1] * ByteFmt<QUANT, DYN>::kMul + l_off) * vs.y;
+        o[ct][4 * rb + 2] = (o[ct][4 * rb + 2] * ByteFmt<QUANT, DYN>::kMul + l_off) * vs.z;
+        o[ct][4 * rb + 3] = (o[ct][4 * rb + 3] * ByteFmt<QUANT, DYN>::kMul + l_off) * vs.w;
       }
   };
 
@@ -409,7 +454,7 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
           }
       }
       // logit (log2 domain) = accumulator * scl + add
-      const float scl = pre ? sc * ByteFmt<QUANT>::kMul : sc;
+      const float scl = pre ? sc * ByteFmt<QUANT, DYN>::kMul : sc;
       const float add = pre ? qbias : 0.f;
       // fp16 P^T operands and this lane's weight sum for the exponent reference m_ref
       float tsum;
@@ -555,13 +600,12 @@ __global__ __launch_bounds__(256) void prefill_merge_kernel(PrefillArgs a) {
 }
 
 bool prefill_mfma_supported(int hq, int hkv, int d, int bs, int quant) {
-  return d == HD && bs == BN && hq % hkv == 0 &&
-         (quant == FDATTN_CACHE_INT8 || quant == FDATTN_CACHE_FP8_E4M3);
+  return d == HD && bs == BN && hq % hkv == 0 && quant_known(quant);
 }
 
 namespace {
 
-template <int QUANT, int NW>
+template <int QUANT, int NW, bool DYN>
 hipError_t launch_one(const PrefillArgs& a, int max_chunk, hipStream_t s) {
   constexpr int BM = 32 * NW;
   PrefillArgs args = a;
@@ -575,12 +619,12 @@ hipError_t launch_one(const PrefillArgs& a, int max_chunk, hipStream_t s) {
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
   if (dev >= 64 || !(raised.load(std::memory_order_relaxed) >> dev & 1ull)) {
-    e = hipFuncSetAttribute((const void*)prefill_mfma_kernel<QUANT, NW>, hipFuncAttributeMaxDynamicSharedMemorySize,
+    e = hipFuncSetAttribute((const void*)prefill_mfma_kernel<QUANT, NW, DYN>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)shm);
     if (e != hipSuccess) return e;
     if (dev < 64) raised.fetch_or(1ull << dev, std::memory_order_relaxed);
   }
-  hipLaunchKernelGGL((prefill_mfma_kernel<QUANT, NW>), grid, block, shm, s, args);
+  hipLaunchKernelGGL((prefill_mfma_kernel<QUANT, NW, DYN>), grid, block, shm, s, args);
   return hipSuccess;
 }
 
@@ -631,10 +675,15 @@ int prefill_mfma_launch(const PrefillArgs& a_in, int max_chunk, int quant, hipSt
   const bool wide = wide_workgroups(a.rows, a.hq, max_chunk, a.n_splits);
   hipError_t e;
   if (quant == FDATTN_CACHE_INT8)
-    e = wide ? launch_one<FDATTN_CACHE_INT8, 8>(a, max_chunk, s) : launch_one<FDATTN_CACHE_INT8, 4>(a, max_chunk, s);
+    e = wide ? launch_one<FDATTN_CACHE_INT8, 8, false>(a, max_chunk, s) : launch_one<FDATTN_CACHE_INT8, 4, false>(a, max_chunk, s);
+  else if (quant == FDATTN_CACHE_FP8_E4M3)
+    e = wide ? launch_one<FDATTN_CACHE_FP8_E4M3, 8, false>(a, max_chunk, s)
+             : launch_one<FDATTN_CACHE_FP8_E4M3, 4, false>(a, max_chunk, s);
+  else if (quant == FDATTN_CACHE_INT8_DYNAMIC)
+    e = wide ? launch_one<FDATTN_CACHE_INT8, 8, true>(a, max_chunk, s) : launch_one<FDATTN_CACHE_INT8, 4, true>(a, max_chunk, s);
   else
-    e = wide ? launch_one<FDATTN_CACHE_FP8_E4M3, 8>(a, max_chunk, s)
-             : launch_one<FDATTN_CACHE_FP8_E4M3, 4>(a, max_chunk, s);
+    e = wide ? launch_one<FDATTN_CACHE_FP8_E4M3, 8, true>(a, max_chunk, s)
+             : launch_one<FDATTN_CACHE_FP8_E4M3, 4, true>(a, max_chunk, s);
   if (e != hipSuccess) return fail((int)e, "fdattn_append_attention_prefill: %s", hipGetErrorString(e));
   int rc = check_launch("fdattn_append_attention_prefill (mfma)");
   if (rc || a.n_splits <= 1) return rc;

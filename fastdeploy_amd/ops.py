@@ -39,6 +39,8 @@ def byte_format(cache_quant_type):
     """CACHE_INT8 or CACHE_FP8: how the cache bytes of this format are encoded."""
     q = _QUANT[cache_quant_type]
     return {CACHE_INT8_DYNAMIC: CACHE_INT8, CACHE_FP8_DYNAMIC: CACHE_FP8}.get(q, q)
+
+
 _ROPE = {"interleaved": 0, 0: 0, False: 0, "neox": 1, 1: 1, True: 1}
 
 

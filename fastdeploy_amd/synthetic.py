@@ -50,7 +50,7 @@ def make_block_tables(ctx_lens, pool_blocks, bs, gen, device, max_blocks=None):
 
 def decode_case(batch=4, ctx=1024, pool_blocks=None, quant=CACHE_INT8, seed=0, device="cpu",
                 hq=HQ, hkv=HKV, d=D, bs=BS, direct_bytes=False, extra_blocks=0, salient=0.0,
-                max_blocks=None):
+                max_blocks=None, row_log2=(-3, 3)):
     """A decode-attention case with a pre-filled cache.
 
     ctx: an int (every sequence), a (lo, hi) tuple (uniform, inclusive) or a list.
@@ -58,7 +58,7 @@ def decode_case(batch=4, ctx=1024, pool_blocks=None, quant=CACHE_INT8, seed=0, d
     otherwise K, V ~ N(0,1) bf16 quantised with per-channel scales = max-abs/127 (int8)
     or max-abs/448 (fp8).  salient: fraction of (sequence, block) pairs whose K is x4.
     The dynamic formats get scale caches [pool, hkv, bs]: every stored row's own max-abs/127 (/448)
-    with the rows scaled by 2^U{-3..3} so that the scales differ widely, or (direct_bytes) random ones;
+    with the rows scaled by 2^U{row_log2} so that the scales differ widely, or (direct_bytes) random ones;
     the slots of no token hold NaN there, which nothing may read.
     """
     g = _gen(seed, device)
@@ -102,8 +102,8 @@ def decode_case(batch=4, ctx=1024, pool_blocks=None, quant=CACHE_INT8, seed=0, d
                 continue
             k = torch.randn((n, hkv, d), generator=g, device=device).to(torch.bfloat16).float()
             v = torch.randn((n, hkv, d), generator=g, device=device).to(torch.bfloat16).float()
-            k = k * torch.exp2(torch.randint(-3, 4, (n, hkv, 1), generator=g, device=device).float())
-            v = v * torch.exp2(torch.randint(-3, 4, (n, hkv, 1), generator=g, device=device).float())
+            k = k * torch.exp2(torch.randint(row_log2[0], row_log2[1] + 1, (n, hkv, 1), generator=g, device=device).float())
+            v = v * torch.exp2(torch.randint(row_log2[0], row_log2[1] + 1, (n, hkv, 1), generator=g, device=device).float())
             if salient > 0:
                 nb = (n + bs - 1) // bs
                 pick = torch.rand((nb,), generator=g, device=device) < salient

@@ -96,7 +96,10 @@ def test_selector_rejects_the_dynamic_formats():
 
 def _prefill_case(seed, prefix, chunks, quant=CACHE_INT8):
     batch = len(chunks)
-    base = syn.decode_case(batch=batch, ctx=prefix, quant=quant, seed=seed, extra_blocks=4)
+    # the dynamic formats: the stored rows differ in scale by up to 2^6, the largest staying at unit scale - the
+    # MFMA kernel carries the softmax weights in fp16, so its absolute error grows with the largest dequantised V
+    # it mixes, and the 2e-3 part of the tolerance is meant for unit-scale activations
+    base = syn.decode_case(batch=batch, ctx=prefix, quant=quant, seed=seed, extra_blocks=4, row_log2=(-6, 0))
     g = torch.Generator().manual_seed(seed + 100)
     T = sum(chunks)
     base["q_new"] = torch.randn((T, 32 * 128), generator=g).to(torch.bfloat16)
