@@ -44,6 +44,7 @@ SIGNATURES = {
     "fdattn_pool_refcount": (_i, [_vp, _i]),
     "fdattn_pool_block_tables": (ctypes.POINTER(ctypes.c_int32), [_vp]),
     "fdattn_kv_wire_bytes": (_sz, [_i] * 4),
+    "fdattn_kv_wire_bytes_for": (_sz, [_i] * 5),
     "fdattn_kv_export": (_i, [_vp] * 8 + [_i] * 8 + [_vp]),
     "fdattn_kv_import": (_i, [_vp] * 9 + [_i] * 8 + [_vp]),
 }

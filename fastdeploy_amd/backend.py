@@ -20,8 +20,8 @@ class AttentionLayer:
     """Per-layer constants: the layer's caches, their scales and the optional projection epilogue."""
     key_cache: torch.Tensor                      # uint8 / int8 / fp8 [num_blocks, kv_num_heads, block_size, head_dim]
     value_cache: torch.Tensor
-    cache_k_scale: torch.Tensor                  # float32 [kv_num_heads, head_dim]
-    cache_v_scale: torch.Tensor
+    cache_k_scale: torch.Tensor                  # float32 [kv_num_heads, head_dim]; the dynamic formats: the scale
+    cache_v_scale: torch.Tensor                  # caches [num_blocks, kv_num_heads, block_size] the cache writer fills
     qkv_bias: Optional[torch.Tensor] = None
     q_norm_weight: Optional[torch.Tensor] = None
     k_norm_weight: Optional[torch.Tensor] = None
@@ -58,17 +58,28 @@ class AppendAttentionBackend:
         self._out = None
 
     # ---- cache allocation -------------------------------------------------------------------------------
-    def allocate_layer(self, num_blocks, cache_k_scale, cache_v_scale, **epilogue):
-        """Zeroed caches of one layer ([num_blocks, kv_num_heads, block_size, head_dim] bytes each)."""
+    def allocate_layer(self, num_blocks, cache_k_scale=None, cache_v_scale=None, **epilogue):
+        """Zeroed caches of one layer ([num_blocks, kv_num_heads, block_size, head_dim] bytes each).  The per-channel
+        formats need their scales (float32 [kv_num_heads, head_dim]); the dynamic formats get scale caches
+        ([num_blocks, kv_num_heads, block_size], ones) that the cache writer fills row by row."""
+        from .ops import is_dynamic
         shape = (num_blocks, self.kv_num_heads, self.block_size, self.head_dim)
         kc = torch.zeros(shape, dtype=torch.uint8, device=self.device)
         vc = torch.zeros(shape, dtype=torch.uint8, device=self.device)
+        if is_dynamic(self.cache_quant_type):
+            if cache_k_scale is not None or cache_v_scale is not None:
+                raise ValueError("the dynamic cache formats take no scales: the cache writer computes them")
+            cache_k_scale = torch.ones(shape[:3], dtype=torch.float32, device=self.device)
+            cache_v_scale = torch.ones(shape[:3], dtype=torch.float32, device=self.device)
+        elif cache_k_scale is None or cache_v_scale is None:
+            raise ValueError("cache_k_scale and cache_v_scale are required for %r" % (self.cache_quant_type,))
         return AttentionLayer(kc, vc, cache_k_scale.to(self.device).contiguous(),
                               cache_v_scale.to(self.device).contiguous(), **epilogue)
 
     @staticmethod
     def blocks_for_memory(num_bytes, num_layers, kv_num_heads, head_dim, block_size=64):
-        """How many blocks per layer fit into num_bytes of cache memory (K and V, one byte per value)."""
+        """How many blocks per layer fit into num_bytes of cache memory (K and V, one byte per value; the dynamic
+        formats' scale caches add 4 bytes per stored row, 1/32 more at head_dim 128)."""
         per_block = 2 * kv_num_heads * block_size * head_dim * num_layers
         return int(num_bytes // per_block)
 

@@ -6,8 +6,9 @@
 // Wire layout of one sequence (little-endian, every section 256-byte aligned):
 //   header   256 B   u32 magic 'FDKV', version, cache_quant_type, hkv, head_dim, block_size,
 //                    num_tokens, num_pages; u64 scales_off, sums_off, pages_off, total_bytes
-//   scales           f32 K [hkv, head_dim], f32 V [hkv, head_dim]
-//   sums             u64 [num_pages][2][hkv]: sum of the unit's 32-bit words
+//   scales           f32 K [hkv, head_dim], f32 V [hkv, head_dim];
+//                    dynamic formats: f32 [num_pages][2][hkv][block_size], the stored rows' scales (0 past num_tokens)
+//   sums             u64 [num_pages][2][hkv]: sum of the unit's 32-bit words (dynamic: its scale row included)
 //   pages            [num_pages][2][hkv][block_size][head_dim] bytes; rows past num_tokens are zero
 #include "fdattn_common.h"
 
@@ -24,11 +25,14 @@ struct WireLayout {
   size_t scales_off, sums_off, pages_off, total;
   int pages;
 };
-__host__ __device__ inline WireLayout wire_layout(int num_tokens, int hkv, int d, int bs) {
+__host__ __device__ inline size_t scale_bytes(int pages, int hkv, int d, int bs, bool dyn) {
+  return (dyn ? (size_t)pages * 2 * hkv * bs : (size_t)2 * hkv * d) * sizeof(float);
+}
+__host__ __device__ inline WireLayout wire_layout(int num_tokens, int hkv, int d, int bs, bool dyn) {
   WireLayout w;
   w.pages = (num_tokens + bs - 1) / bs;
   w.scales_off = kHeaderBytes;
-  w.sums_off = align256(w.scales_off + (size_t)2 * hkv * d * sizeof(float));
+  w.sums_off = align256(w.scales_off + scale_bytes(w.pages, hkv, d, bs, dyn));
   w.pages_off = align256(w.sums_off + (size_t)w.pages * 2 * hkv * sizeof(unsigned long long));
   w.total = align256(w.pages_off + (size_t)w.pages * 2 * hkv * bs * d);
   return w;
@@ -37,7 +41,7 @@ __host__ __device__ inline WireLayout wire_layout(int num_tokens, int hkv, int d
 struct WireArgs {
   uint8_t* key_cache;
   uint8_t* value_cache;
-  const float* k_scale;
+  const float* k_scale;  // dynamic formats: the scale caches [num_blocks, hkv, bs], written by the import
   const float* v_scale;
   const int32_t* block_tables;  // [batch, max_blocks]
   const int32_t* num_tokens;    // [batch]
@@ -84,7 +88,8 @@ __global__ __launch_bounds__(256) void kv_wire_kernel(WireArgs a) {
   __shared__ unsigned long long sh[4];
   const int b = blockIdx.y;
   const int tokens = min(max(a.num_tokens[b], 0), a.max_tokens);
-  const WireLayout w = wire_layout(tokens, a.hkv, a.d, a.bs);
+  const bool dyn = quant_dynamic(a.quant);
+  const WireLayout w = wire_layout(tokens, a.hkv, a.d, a.bs, dyn);
   const int unit = blockIdx.x;
   uint8_t* wire = a.wire + a.wire_offsets[b];
   u32* hdr = reinterpret_cast<u32*>(wire);
@@ -107,16 +112,17 @@ __global__ __launch_bounds__(256) void kv_wire_kernel(WireArgs a) {
     if (!IMPORT) {
       if (threadIdx.x < 64) hdr[threadIdx.x] = header_word(threadIdx.x, a, tokens, w);
       float* sc = reinterpret_cast<float*>(wire + w.scales_off);
-      for (int i = threadIdx.x; i < ns; i += 256) sc[i] = a.k_scale[i], sc[ns + i] = a.v_scale[i];
+      if (!dyn)  // (the dynamic formats' scale rows travel with their units)
+        for (int i = threadIdx.x; i < ns; i += 256) sc[i] = a.k_scale[i], sc[ns + i] = a.v_scale[i];
       // the alignment gaps behind the three sections (each under 256 bytes) are zero: the buffer's
       // bytes are a function of the sequence alone
-      const size_t gap[3][2] = {{w.scales_off + (size_t)2 * ns * sizeof(float), w.sums_off},
+      const size_t gap[3][2] = {{w.scales_off + scale_bytes(w.pages, a.hkv, a.d, a.bs, dyn), w.sums_off},
                                 {w.sums_off + (size_t)w.pages * 2 * a.hkv * sizeof(unsigned long long), w.pages_off},
                                 {w.pages_off + (size_t)w.pages * 2 * a.hkv * a.bs * a.d, w.total}};
 #pragma unroll
       for (int g = 0; g < 3; ++g)
         if (gap[g][0] + threadIdx.x < gap[g][1]) wire[gap[g][0] + threadIdx.x] = 0;
-    } else if (a.k_scale && hdr_ok) {
+    } else if (a.k_scale && hdr_ok && !dyn) {
       const float* sc = reinterpret_cast<const float*>(wire + w.scales_off);
       bool bad = false;
       for (int i = threadIdx.x; i < ns; i += 256)
@@ -150,6 +156,21 @@ __global__ __launch_bounds__(256) void kv_wire_kernel(WireArgs a) {
       if (pb_ok) *reinterpret_cast<uint4*>(cache + off) = v;
     }
   }
+  if (dyn && (int)threadIdx.x < a.bs) {
+    // the unit's scale row: bs floats beside the tile, zero for the rows past the sequence's end
+    float* crow = const_cast<float*>(kv ? a.v_scale : a.k_scale) + ((size_t)pb * a.hkv + h) * a.bs;
+    u32* wrow = reinterpret_cast<u32*>(wire + w.scales_off) + (size_t)unit * a.bs;
+    const int t = threadIdx.x;
+    if (!IMPORT) {
+      const u32 v = (t < valid && pb_ok) ? __float_as_uint(crow[t]) : 0u;
+      wrow[t] = v;
+      s += v;
+    } else {
+      const u32 v = wrow[t];
+      s += v;
+      if (pb_ok) crow[t] = __uint_as_float(v);
+    }
+  }
   s = block_sum(s, sh);
   if (threadIdx.x == 0) {
     if (!IMPORT) {
@@ -166,8 +187,9 @@ __global__ __launch_bounds__(256) void kv_wire_kernel(WireArgs a) {
 
 int check_shape(const char* what, int batch, int max_tokens, int hkv, int d, int bs, int max_blocks, int num_blocks,
                 int quant) {
-  if (quant != FDATTN_CACHE_INT8 && quant != FDATTN_CACHE_FP8_E4M3)
-    return fail(FDATTN_ERR_QUANT, "%s: cache_quant_type %d is not a format with per-channel scales", what, quant);
+  if (!quant_known(quant)) return fail(FDATTN_ERR_QUANT, "%s: unknown cache_quant_type %d", what, quant);
+  if (quant_dynamic(quant) && bs > 256)
+    return fail(FDATTN_ERR_SHAPE, "%s: the dynamic formats' scale rows need block_size <= 256, got %d", what, bs);
   if (batch < 0 || max_tokens < 0 || hkv <= 0 || d <= 0 || bs <= 0 || max_blocks <= 0 || num_blocks <= 0 || d % 16 != 0 ||
       batch > 65535)
     return fail(FDATTN_ERR_SHAPE, "%s: bad shape batch=%d max_tokens=%d hkv=%d head_dim=%d block_size=%d "
@@ -184,9 +206,13 @@ int check_shape(const char* what, int batch, int max_tokens, int hkv, int d, int
 
 using namespace fdattn;
 
+extern "C" size_t fdattn_kv_wire_bytes_for(int num_tokens, int hkv, int head_dim, int block_size, int cache_quant_type) {
+  if (num_tokens < 0 || hkv <= 0 || head_dim <= 0 || block_size <= 0 || !quant_known(cache_quant_type)) return 0;
+  return wire_layout(num_tokens, hkv, head_dim, block_size, quant_dynamic(cache_quant_type)).total;
+}
+
 extern "C" size_t fdattn_kv_wire_bytes(int num_tokens, int hkv, int head_dim, int block_size) {
-  if (num_tokens < 0 || hkv <= 0 || head_dim <= 0 || block_size <= 0) return 0;
-  return wire_layout(num_tokens, hkv, head_dim, block_size).total;
+  return fdattn_kv_wire_bytes_for(num_tokens, hkv, head_dim, block_size, FDATTN_CACHE_INT8);
 }
 
 extern "C" int fdattn_kv_export(const void* key_cache, const void* value_cache, const float* k_scale,
@@ -217,6 +243,8 @@ extern "C" int fdattn_kv_import(const void* wire, const int64_t* wire_offsets, v
     return fail(FDATTN_ERR_NULL, "fdattn_kv_import: NULL pointer argument");
   if ((k_scale == nullptr) != (v_scale == nullptr))
     return fail(FDATTN_ERR_NULL, "fdattn_kv_import: pass both scale tables or neither");
+  if (quant_dynamic(cache_quant_type) && !k_scale)
+    return fail(FDATTN_ERR_NULL, "fdattn_kv_import: the dynamic formats need the scale caches to import into");
   if (int rc = check_shape("fdattn_kv_import", batch, max_tokens, hkv, head_dim, block_size, max_blocks_per_seq,
                            num_blocks, cache_quant_type))
     return rc;

@@ -60,7 +60,7 @@ extern "C" {
  * indexed like the rows of key_cache / value_cache; the cache writer (and the one-call step, which
  * contains it) STORES into them despite the const qualifier, every attention entry point reads them.
  * K scales are taken after the rotation.  Dequantised value = byte * scale of its row.
- * Not accepted by the block selector and the wire form, which are defined on per-channel scales.
+ * Not accepted by the block selector, which is defined on per-channel scales.
  */
 #define FDATTN_CACHE_INT8_DYNAMIC 3
 #define FDATTN_CACHE_FP8_E4M3_DYNAMIC 4
@@ -456,6 +456,11 @@ FDATTN_API const int32_t* fdattn_pool_block_tables(const fdattn_block_pool* pool
  * <= max_tokens.  One launch per call, nothing synchronises.
  */
 FDATTN_API size_t fdattn_kv_wire_bytes(int num_tokens, int hkv, int head_dim, int block_size);
+/* The same for any cache format.  The dynamic formats carry their scales page by page: the scales section is
+ * f32 [num_pages][2][hkv][block_size] (zero for rows past num_tokens), every tile's sum includes its scale row,
+ * the import stores the rows into k_scale / v_scale (the scale caches, required then) and status bit 4 is
+ * not used. */
+FDATTN_API size_t fdattn_kv_wire_bytes_for(int num_tokens, int hkv, int head_dim, int block_size, int cache_quant_type);
 /* cache -> wire.  A table entry outside [0, num_blocks) exports as a page of zeros. */
 FDATTN_API int fdattn_kv_export(const void* key_cache, const void* value_cache, const float* k_scale,
                                 const float* v_scale, const int32_t* block_tables, const int32_t* num_tokens,

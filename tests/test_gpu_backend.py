@@ -7,16 +7,18 @@ import torch
 
 import fastdeploy_amd as fd
 from conftest import bf16_close, bits, np_of
-from fastdeploy_amd.ops import CACHE_INT8
+from fastdeploy_amd.ops import CACHE_INT8, CACHE_INT8_DYNAMIC, is_dynamic
 from test_gpu_mixed_step import oracle_step
 
 pytestmark = pytest.mark.gpu
 
 
-def test_generation_over_steps_and_layers(oracle):
+@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_INT8_DYNAMIC])
+def test_generation_over_steps_and_layers(oracle, quant):
     hq, hkv, d, bs, layers = 32, 8, 128, 64, 2
     g = torch.Generator().manual_seed(31)
-    be = fd.AppendAttentionBackend(hq, hkv, d, block_size=bs, max_position=1024, rope_theta=500000.0)
+    be = fd.AppendAttentionBackend(hq, hkv, d, block_size=bs, max_position=1024, rope_theta=500000.0,
+                                   cache_quant_type=quant)
     pool = fd.BlockPool(num_blocks=40, block_size=bs, max_seqs=5, max_blocks_per_seq=8)
     book = fd.SequenceBook(pool)
     lay = []
@@ -28,7 +30,7 @@ def test_generation_over_steps_and_layers(oracle):
             extra = dict(qkv_bias=(torch.randn((48 * d,), generator=g) * 0.25).to(torch.bfloat16).cuda(),
                          q_norm_weight=(torch.rand((d,), generator=g) + 0.5).cuda(),
                          k_norm_weight=(torch.rand((d,), generator=g) + 0.5).cuda(), rms_norm_eps=1e-6)
-        lay.append(be.allocate_layer(40, ks, vs, **extra))
+        lay.append(be.allocate_layer(40, **extra) if is_dynamic(quant) else be.allocate_layer(40, ks, vs, **extra))
     cos, sin = (t.cpu() for t in be.rotary_embs)
 
     def run_step(new_tokens):
@@ -46,8 +48,11 @@ def test_generation_over_steps_and_layers(oracle):
             if layer.qkv_bias is not None:
                 ep = dict(qkv_bias=bits(layer.qkv_bias), q_norm_weight=np_of(layer.q_norm_weight),
                           k_norm_weight=np_of(layer.k_norm_weight), rms_norm_eps=layer.rms_norm_eps)
-            want, kc, vc = oracle_step(oracle, before, CACHE_INT8, **ep)
+            want, kc, vc = oracle_step(oracle, before, quant, **ep)
             assert np.array_equal(np_of(layer.key_cache), kc) and np.array_equal(np_of(layer.value_cache), vc)
+            if is_dynamic(quant):  # the scale caches follow the stored rows
+                assert np.array_equal(np_of(layer.cache_k_scale), before["scales_after"][0])
+                assert np.array_equal(np_of(layer.cache_v_scale), before["scales_after"][1])
             ok, mx, bad = bf16_close(bits(out), want)
             assert ok, "layer %d, step %r: %d out of tolerance, max %.4g" % (l, new_tokens, bad, mx)
         book.commit()

@@ -8,7 +8,7 @@ import torch
 import fastdeploy_amd as fd
 from conftest import np_of
 from fastdeploy_amd import kv_wire
-from fastdeploy_amd.ops import CACHE_FP8, CACHE_INT8
+from fastdeploy_amd.ops import CACHE_FP8, CACHE_FP8_DYNAMIC, CACHE_INT8, CACHE_INT8_DYNAMIC
 from oracle import kv_wire as ow
 
 pytestmark = pytest.mark.gpu
@@ -50,6 +50,46 @@ def test_export_import_match_the_numpy_restatement(shape):
         bits |= r[0]
     assert bits == 16 and st.tolist() == [16, 0]
     assert np.array_equal(np_of(kc2), kc_w) and np.array_equal(np_of(vc2), vc_w)
+
+
+@pytest.mark.parametrize("shape", [(8, 64, 128), (2, 16, 32)])
+def test_dynamic_formats_export_import_match_the_numpy_restatement(shape):
+    """The formats with one scale per stored row: wire bytes (scale rows, sums over tile + row) and the imported
+    caches and scale caches bit for bit as the restatement's; a flipped scale bit fails its tile's sum."""
+    hkv, bs, d = shape
+    tokens = [0, 1, bs, bs + 1, 3 * bs - 1, 4 * bs]
+    kc, vc, _, _, bt = make(5, 40, hkv, bs, d, len(tokens), 5)
+    g = torch.Generator().manual_seed(6)
+    ks, vs = torch.rand((40, hkv, bs), generator=g) + 0.5, torch.rand((40, hkv, bs), generator=g) + 0.5
+    bt[2, 0] = -1
+    wire, offs = kv_wire.kv_export(kc.cuda(), vc.cuda(), ks.cuda(), vs.cuda(), bt.cuda(), tokens,
+                                   cache_quant_type=CACHE_FP8_DYNAMIC)
+    torch.cuda.synchronize()
+    want = ow.export_batch(np_of(kc), np_of(vc), np_of(ks), np_of(vs), np_of(bt), tokens, CACHE_FP8_DYNAMIC)
+    assert np.array_equal(np_of(wire), want)
+    bt2 = (torch.randperm(40, generator=g)[:bt.numel()].to(torch.int32).view_as(bt)).contiguous()
+    kc2, vc2 = torch.zeros_like(kc).cuda(), torch.zeros_like(vc).cuda()
+    ks2, vs2 = torch.full_like(ks, 7.0).cuda(), torch.full_like(vs, 7.0).cuda()
+    st = kv_wire.kv_import(wire, kc2, vc2, bt2.cuda(), tokens, cache_k_scale=ks2, cache_v_scale=vs2,
+                           cache_quant_type=CACHE_FP8_DYNAMIC)
+    torch.cuda.synchronize()
+    kc_w, vc_w = np.zeros_like(np_of(kc)), np.zeros_like(np_of(vc))
+    ks_w, vs_w = np.full_like(np_of(ks), 7.0), np.full_like(np_of(vs), 7.0)
+    for b, n in enumerate(tokens):
+        assert ow.import_seq(want[offs[b]:], kc_w, vc_w, np_of(bt2)[b], n, CACHE_FP8_DYNAMIC, ks_w, vs_w) == (0, 0)
+    assert st.tolist() == [0, 0]
+    assert np.array_equal(np_of(kc2), kc_w) and np.array_equal(np_of(vc2), vc_w)
+    assert np.array_equal(np_of(ks2), ks_w) and np.array_equal(np_of(vs2), vs_w)
+    bad = wire.clone()
+    bad[offs[3] + 256 + 1] ^= 0x04                            # inside the first scale row of sequence 3
+    st = kv_wire.kv_import(bad, kc2, vc2, bt2.cuda(), tokens, cache_k_scale=ks2, cache_v_scale=vs2,
+                           cache_quant_type=CACHE_FP8_DYNAMIC)
+    assert st.tolist() == [8, 1]
+    with pytest.raises(ValueError):                           # the dynamic formats need somewhere to put the scales
+        kv_wire.kv_import(wire, kc2, vc2, bt2.cuda(), tokens, cache_quant_type=CACHE_FP8_DYNAMIC)
+    with pytest.raises(ValueError):                           # a plan sized for the per-channel formats
+        kv_wire.kv_export(kc.cuda(), vc.cuda(), ks.cuda(), vs.cuda(), bt.cuda(),
+                          kv_wire.WirePlan(tokens, hkv, d, bs), cache_quant_type=CACHE_FP8_DYNAMIC)
 
 
 def test_import_reports_bad_buffers_and_leaves_the_cache_alone():

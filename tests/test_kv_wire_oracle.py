@@ -82,6 +82,50 @@ def test_round_trip_into_other_blocks_and_error_bits():
     assert ow.import_seq(buf, k3, v3, np.array([1, 99, 4, 0, 0, 0], np.int32), tokens, 2)[0] == 16
 
 
+@pytest.mark.parametrize("tokens", [0, 1, 16, 41])
+def test_dynamic_formats_carry_their_scale_rows(tokens):
+    """One scale per stored row: the scales section holds [pages][2][hkv][bs] floats (zero past the end), every
+    tile's sum covers its scale row, and the import stores the rows into the scale caches of the new blocks."""
+    rng, kc, vc, _, _ = case(40 + tokens)
+    nb, hkv, bs, d = kc.shape
+    ks = rng.random((nb, hkv, bs), dtype=np.float32) + 0.5
+    vs = rng.random((nb, hkv, bs), dtype=np.float32) + 0.5
+    src = rng.permutation(nb)[:6].astype(np.int32)
+    buf = ow.export_seq(kc, vc, ks, vs, src, tokens, 3)
+    h = parse_header(buf.tobytes())
+    pages = (tokens + bs - 1) // bs
+    assert h["cache_quant_type"] == 3 and h["num_pages"] == pages and h["total_bytes"] == len(buf)
+    assert len(buf) == wire_bytes(tokens, hkv, d, bs, 3)
+    assert h["sums_off"] >= 256 + pages * 2 * hkv * bs * 4 and h["sums_off"] % 256 == 0
+    raw = buf.tobytes()
+    for p in range(pages):
+        valid = min(bs, tokens - p * bs)
+        for kv, (cache, sc) in enumerate(((kc, ks), (vc, vs))):
+            for hh in range(hkv):
+                unit = (p * 2 + kv) * hkv + hh
+                srow = raw[256 + unit * bs * 4: 256 + (unit + 1) * bs * 4]
+                want = sc[src[p], hh].copy()
+                want[valid:] = 0
+                assert srow == want.tobytes()
+                tile = raw[h["pages_off"] + unit * bs * d: h["pages_off"] + (unit + 1) * bs * d]
+                s = sum(int.from_bytes(x[i:i + 4], "little") for x in (tile, srow) for i in range(0, len(x), 4))
+                assert struct.unpack_from("<Q", raw, h["sums_off"] + 8 * unit)[0] == s
+    # round trip into other blocks
+    dst = np.array([b for b in range(nb) if b not in src[:pages]][:6], np.int32)
+    kc2, vc2, ks2, vs2 = np.zeros_like(kc), np.zeros_like(vc), np.zeros_like(ks), np.zeros_like(vs)
+    assert ow.import_seq(buf, kc2, vc2, dst, tokens, 3, ks2, vs2) == (0, 0)
+    for p in range(pages):
+        valid = min(bs, tokens - p * bs)
+        assert np.array_equal(kc2[dst[p], :, :valid], kc[src[p], :, :valid])
+        assert np.array_equal(ks2[dst[p], :, :valid], ks[src[p], :, :valid]) and not ks2[dst[p], :, valid:].any()
+        assert np.array_equal(vs2[dst[p], :, :valid], vs[src[p], :, :valid])
+    assert np.array_equal(ow.export_seq(kc2, vc2, ks2, vs2, dst, tokens, 3), buf)
+    if pages:  # a flipped bit in a scale row fails that tile's sum
+        bad = buf.copy(); bad[256 + 2] ^= 0x10
+        assert ow.import_seq(bad, kc2, vc2, dst, tokens, 3, ks2, vs2) == (8, 1)
+    assert ow.import_seq(buf, kc2, vc2, dst, tokens, 1, ks2, vs2)[0] == 2      # read as a per-channel format
+
+
 def test_offsets_of_a_packed_batch():
     offs, total = wire_offsets([0, 5, 130], 8, 128, 64)
     sizes = [wire_bytes(n, 8, 128, 64) for n in (0, 5, 130)]
