@@ -108,16 +108,22 @@ template <int QUANT>
 __device__ __forceinline__ uint4 cvt8_scaled(u32 w0, u32 w1, float s) {
   float f[8];
   if (QUANT == FDATTN_CACHE_INT8) {
-    // (b + 128) as an unsigned byte -> float, then (b + 128) s - 128 s in one fused step: b s rounded once
+    // byte b -> the fp16 number 1024 + (b + 128) (exponent byte 0x64 in front of the offset byte: one permute per two
+    // bytes), then (1024 + b + 128) s - 1152 s = b s as one fused multiply-add in fp32, rounded to fp16 once
+    // (the mixed-precision fma takes the fp16 operand and writes the fp16 result directly)
     const u32 x[2] = {w0 ^ 0x80808080u, w1 ^ 0x80808080u};
-    const float c = -128.0f * s;
+    const float c = -1152.0f * s;
+    u32 out[4];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      f[4 * i + 0] = __builtin_fmaf((float)(x[i] & 0xffu), s, c);
-      f[4 * i + 1] = __builtin_fmaf((float)((x[i] >> 8) & 0xffu), s, c);
-      f[4 * i + 2] = __builtin_fmaf((float)((x[i] >> 16) & 0xffu), s, c);
-      f[4 * i + 3] = __builtin_fmaf((float)(x[i] >> 24), s, c);
+      const v2h lo = __builtin_bit_cast(v2h, __builtin_amdgcn_perm(0x64646464u, x[i], 0x04010400u));
+      const v2h hi = __builtin_bit_cast(v2h, __builtin_amdgcn_perm(0x64646464u, x[i], 0x04030402u));
+      const v2h rl = {(_Float16)__builtin_fmaf((float)lo[0], s, c), (_Float16)__builtin_fmaf((float)lo[1], s, c)};
+      const v2h rh = {(_Float16)__builtin_fmaf((float)hi[0], s, c), (_Float16)__builtin_fmaf((float)hi[1], s, c)};
+      out[2 * i] = __builtin_bit_cast(u32, rl);
+      out[2 * i + 1] = __builtin_bit_cast(u32, rh);
     }
+    return make_uint4(out[0], out[1], out[2], out[3]);
   } else {
     const v2f a = __builtin_amdgcn_cvt_pk_f32_fp8((int)w0, false), b = __builtin_amdgcn_cvt_pk_f32_fp8((int)w0, true);
     const v2f c = __builtin_amdgcn_cvt_pk_f32_fp8((int)w1, false), d = __builtin_amdgcn_cvt_pk_f32_fp8((int)w1, true);
