@@ -164,16 +164,18 @@ def test_workspace_is_reusable_across_calls_and_shapes(oracle):
             check(got, oracle_decode(oracle, case), "reuse rep %d" % rep)
 
 
-def test_decode_config2_full_size(oracle):
-    """batch 64, ctx U[3584, 4608], int8 KV, block tables a random permutation over a 6000-block pool:
+@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_INT8_DYNAMIC])
+def test_decode_config2_full_size(oracle, quant):
+    """batch 64, ctx U[3584, 4608], int8 KV (per-channel scales, and one scale per stored row), block tables a random permutation over a 6000-block pool:
     the full-size launch against the oracle, plus two size-independent properties: the result does not
     depend on where the blocks sit in the pool, and it is the same whatever the split-KV chunking is
     (dense call == sparse call that keeps every block)."""
     g = torch.Generator().manual_seed(0)
     lens = torch.randint(3584, 4609, (64,), generator=g).tolist()
-    case = syn.decode_case(batch=64, ctx=lens, pool_blocks=6000, seed=1, device="cuda", max_blocks=72)
+    case = syn.decode_case(batch=64, ctx=lens, pool_blocks=6000, seed=1, device="cuda", max_blocks=72, quant=quant)
     out = fd.decode_attention(case["q"], case["key_cache"], case["value_cache"], case["cache_k_scale"],
-                              case["cache_v_scale"], case["block_tables"], case["seq_lens_decoder"], num_heads=32)
+                              case["cache_v_scale"], case["block_tables"], case["seq_lens_decoder"], num_heads=32,
+                              cache_quant_type=quant)
     torch.cuda.synchronize()
     cpu = syn.to_device(case, "cpu")
     check(bits(out), oracle_decode(oracle, cpu), "cfg2")
@@ -182,8 +184,11 @@ def test_decode_config2_full_size(oracle):
     inv = torch.empty_like(perm)
     inv[perm] = torch.arange(6000, device="cuda")
     bt2 = torch.where(case["block_tables"] >= 0, inv[case["block_tables"].clamp(min=0).long()].to(torch.int32), -1)
-    out2 = fd.decode_attention(case["q"], case["key_cache"][perm], case["value_cache"][perm], case["cache_k_scale"],
-                               case["cache_v_scale"], bt2.contiguous(), case["seq_lens_decoder"], num_heads=32)
+    dyn = quant == CACHE_INT8_DYNAMIC   # the scale caches move with their blocks
+    ks2 = case["cache_k_scale"][perm].contiguous() if dyn else case["cache_k_scale"]
+    vs2 = case["cache_v_scale"][perm].contiguous() if dyn else case["cache_v_scale"]
+    out2 = fd.decode_attention(case["q"], case["key_cache"][perm], case["value_cache"][perm], ks2, vs2,
+                               bt2.contiguous(), case["seq_lens_decoder"], num_heads=32, cache_quant_type=quant)
     assert torch.equal(out, out2)
     # keep-everything sparse call: same blocks, different chunk geometry -> same within a bf16 ulp of rounding noise
     nb = torch.tensor([(n + 63) // 64 for n in lens], dtype=torch.int32, device="cuda")
@@ -192,11 +197,11 @@ def test_decode_config2_full_size(oracle):
     cnt = nb[:, None].repeat(1, 8).contiguous()
     out3 = fd.decode_attention_sparse(case["q"], case["key_cache"], case["value_cache"], case["cache_k_scale"],
                                       case["cache_v_scale"], case["block_tables"], case["seq_lens_decoder"],
-                                      kept_blocks=kept, kept_counts=cnt, num_heads=32)
+                                      kept_blocks=kept, kept_counts=cnt, num_heads=32, cache_quant_type=quant)
     check(bits(out3), bits(out), "dense vs keep-all sparse")
 
 
-@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+@pytest.mark.parametrize("quant", ALL_FORMATS)
 def test_decode_launch_shapes(oracle, quant):
     """The chunking follows the launch size (as few chunks per block list as fill the GPU's workgroup slots):
     long lists in a small batch are cut into several chunks of more than 64 units (second unit-table entry
