@@ -388,37 +388,74 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
   }
 }
 
-// One workgroup per (sequence, KV head) whose list spans several chunks: merges their
-// partials, applies the V scale and writes bf16.  Single-chunk pairs were finished by the
-// main kernel.
+// One workgroup per (sequence, KV head, query head) whose list spans several chunks: merges their partials,
+// applies the V scale and writes bf16.  Single-chunk pairs were finished by the main kernel.  The four
+// wavefronts take the chunks in turn (wavefront w: chunks w, w + 4, ...), four chunks' loads in flight at a
+// time - a list of 64 chunks costs 4 round trips to memory, not 64 - and meet in LDS.  Lane = two channels.
 template <bool SPARSE>
 __global__ __launch_bounds__(256) void decode_c8_combine_kernel(C8Args a) {
-  const int p = blockIdx.x, tid = threadIdx.x;
+  __shared__ float red[kWaves][2 + 2 * 64];  // per wavefront: m, l, o[64][2]
+  const int p = blockIdx.x >> 2, head = blockIdx.x & 3, tid = threadIdx.x;
   const int b = p / a.hkv, h = p - b * a.hkv;
   int row;
   if (!decode_row(a.rows, b, row)) return;
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
   const int n_p = pair_units<SPARSE>(a, p, kv_len);
   if (n_p <= a.chunk) return;
-  const int head = tid >> 6, c2 = (tid & 63) * 2;
+  const int wv = tid >> 6, lane = tid & 63, c2 = lane * 2;
   const int nch = (n_p + a.chunk - 1) / a.chunk;
   const size_t s0 = (size_t)p * a.chunks_per_pair;
-  float M = -INFINITY;
-  for (int c = 0; c < nch; ++c) M = fmaxf(M, a.part_ml[(s0 + c) * 8 + head]);
-  float L = 0.f, o0 = 0.f, o1 = 0.f;
-  if (M > -INFINITY) {
-    for (int c = 0; c < nch; ++c) {
-      const float ms = a.part_ml[(s0 + c) * 8 + head];
-      if (ms == -INFINITY) continue;
-      const float f = __builtin_amdgcn_exp2f(ms - M);
-      L += a.part_ml[(s0 + c) * 8 + 4 + head] * f;
-      const float2 v = *reinterpret_cast<const float2*>(a.part_o + (s0 + c) * kSlotFloats + head * kD + c2);
-      o0 += v.x * f;
-      o1 += v.y * f;
+  // this wavefront's chunks against its own running reference
+  float M = -INFINITY, L = 0.f, o0 = 0.f, o1 = 0.f;
+  for (int c0 = wv; c0 < nch; c0 += 4 * kWaves) {
+    float ms[4], ls[4];
+    float2 v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int c = c0 + k * kWaves;
+      ms[k] = -INFINITY, ls[k] = 0.f, v[k] = make_float2(0.f, 0.f);
+      if (c < nch) {
+        ms[k] = a.part_ml[(s0 + c) * 8 + head];
+        ls[k] = a.part_ml[(s0 + c) * 8 + 4 + head];
+        v[k] = *reinterpret_cast<const float2*>(a.part_o + (s0 + c) * kSlotFloats + head * kD + c2);
+      }
+    }
+    float m_new = M;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) m_new = fmaxf(m_new, ms[k]);
+    if (m_new == -INFINITY) continue;
+    const float alpha = __builtin_amdgcn_exp2f(M - m_new);  // M = -inf: 0
+    L *= alpha, o0 *= alpha, o1 *= alpha;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float f = __builtin_amdgcn_exp2f(ms[k] - m_new);  // an empty chunk (m = -inf) weighs 0, its l and o are 0
+      L += ls[k] * f;
+      o0 += v[k].x * f;
+      o1 += v[k].y * f;
+    }
+    M = m_new;
+  }
+  if (lane == 0) red[wv][0] = M, red[wv][1] = L;
+  red[wv][2 + c2] = o0;
+  red[wv][3 + c2] = o1;
+  __syncthreads();
+  if (wv != 0) return;
+  float Mt = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) Mt = fmaxf(Mt, red[w][0]);
+  float Lt = 0.f, r0 = 0.f, r1 = 0.f;
+  if (Mt > -INFINITY) {
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const float f = __builtin_amdgcn_exp2f(red[w][0] - Mt);
+      Lt += red[w][1] * f;
+      r0 += red[w][2 + c2] * f;
+      r1 += red[w][3 + c2] * f;
     }
   }
-  const float inv = L > 0.f ? 1.0f / L : 0.f;
-  const float r0 = o0 * inv * (a.dyn ? 1.f : a.v_scale[h * kD + c2]), r1 = o1 * inv * (a.dyn ? 1.f : a.v_scale[h * kD + c2 + 1]);
+  const float inv = Lt > 0.f ? 1.0f / Lt : 0.f;
+  r0 *= inv * (a.dyn ? 1.f : a.v_scale[h * kD + c2]);
+  r1 *= inv * (a.dyn ? 1.f : a.v_scale[h * kD + c2 + 1]);
   uint16_t* o = a.out + ((size_t)row * a.hkv * kG + h * kG + head) * kD + c2;
   *reinterpret_cast<u32*>(o) = (u32)f32_to_bf16(r0) | ((u32)f32_to_bf16(r1) << 16);
 }
@@ -478,7 +515,7 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
   const int cpp = ((max_units + chunk - 1) / chunk);
   if (pairs > kMaxPairs)
     return fail(FDATTN_ERR_SHAPE, "fdattn_decode_attention: batch*kv_heads = %d exceeds %d", pairs, kMaxPairs);
-  if ((long long)pairs * cpp > 0x7fffffffLL)
+  if ((long long)pairs * (cpp > kG ? cpp : kG) > 0x7fffffffLL)
     return fail(FDATTN_ERR_SHAPE, "fdattn_decode_attention: %d pairs x %d chunks exceed the grid limit", pairs, cpp);
   const size_t slots = (size_t)pairs * cpp;
   const size_t need = slots * (kSlotFloats + 8) * sizeof(float);
@@ -508,8 +545,8 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
   int rc = check_launch("fdattn_decode_attention (mfma)");
   if (rc || !(stages & 2)) return rc;
   if (cpp == 1) return 0;  // every pair was one chunk and has been finished by the main kernel
-  if (sparse) hipLaunchKernelGGL(decode_c8_combine_kernel<true>, dim3(pairs), dim3(256), 0, s, a);
-  else hipLaunchKernelGGL(decode_c8_combine_kernel<false>, dim3(pairs), dim3(256), 0, s, a);
+  if (sparse) hipLaunchKernelGGL(decode_c8_combine_kernel<true>, dim3(pairs * kG), dim3(256), 0, s, a);
+  else hipLaunchKernelGGL(decode_c8_combine_kernel<false>, dim3(pairs * kG), dim3(256), 0, s, a);
   return check_launch("fdattn_decode_attention (merge)");
 }
 
