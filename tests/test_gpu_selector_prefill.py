@@ -192,11 +192,12 @@ def test_prefill_constant_value_bytes(oracle, fill):
     _run_prefill_vs_oracle(oracle, c, CACHE_INT8, 300)
 
 
-def test_prefill_config5_shape_sampled_rows(oracle):
+@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_INT8_DYNAMIC])
+def test_prefill_config5_shape_sampled_rows(oracle, quant):
     """batch 2, 2048 new tokens on 8192 cached (int8 paged), causal: the full-size launch, checked on a
     sample of rows against the oracle and, on the GPU, against the shape-agnostic kernel on every row."""
     g = torch.Generator(device="cuda").manual_seed(0)
-    c = syn.decode_case(batch=2, ctx=8192, seed=0, device="cuda", direct_bytes=True, extra_blocks=8)
+    c = syn.decode_case(batch=2, ctx=8192, seed=0, device="cuda", direct_bytes=True, extra_blocks=8, quant=quant)
     T = 2 * 2048
     c["q_new"] = torch.randn((T, 32 * 128), generator=g, device="cuda").to(torch.bfloat16)
     c["k_new"] = torch.randn((T, 8 * 128), generator=g, device="cuda").to(torch.bfloat16)
@@ -204,22 +205,22 @@ def test_prefill_config5_shape_sampled_rows(oracle):
     cu = torch.tensor([0, 2048, 4096], dtype=torch.int32, device="cuda")
     args = (c["q_new"], c["k_new"], c["v_new"], c["key_cache"], c["value_cache"], c["cache_k_scale"],
             c["cache_v_scale"], c["block_tables"], c["seq_lens_decoder"], cu)
-    out = fd.append_attention_prefill(*args, num_heads=32, max_chunk=2048)
+    out = fd.append_attention_prefill(*args, num_heads=32, max_chunk=2048, cache_quant_type=quant)
     torch.cuda.synchronize()
     ids = np.array([0, 1, 63, 64, 127, 128, 1000, 2047, 2048, 2049, 3000, 4095], np.int32)
     want = oracle.append_attention_prefill(bits(c["q_new"]), bits(c["k_new"]), bits(c["v_new"]), np_of(c["key_cache"]),
                                            np_of(c["value_cache"]), np_of(c["cache_k_scale"]), np_of(c["cache_v_scale"]),
                                            np_of(c["block_tables"]), np_of(c["seq_lens_decoder"]), np_of(cu),
-                                           32, 8, 128, CACHE_INT8, token_ids=ids)
+                                           32, 8, 128, quant, token_ids=ids)
     ok, mx, bad = bf16_close(bits(out)[ids], want[ids])
     assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
     # every row: the two GPU kernels agree within twice the tolerance (each is within it of the truth)
-    ref = fd.append_attention_prefill(*args, num_heads=32, max_chunk=2048, impl="generic")
+    ref = fd.append_attention_prefill(*args, num_heads=32, max_chunk=2048, impl="generic", cache_quant_type=quant)
     ok, mx, bad = bf16_close(bits(out), bits(ref), 4e-3, 2e-2)
     assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
 
 
-@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+@pytest.mark.parametrize("quant", ALL_FORMATS)
 def test_prefill_key_splits(oracle, quant):
     """Every query tile's keys shared by 2 .. 8 workgroups (partials + merge) against the oracle and against the
     unsplit kernel: one sequence's chunk on a long prefix (what the split is for), shares that end inside the
