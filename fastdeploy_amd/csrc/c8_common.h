@@ -111,6 +111,7 @@ __device__ __forceinline__ u32 lds_addr_of(const void* p) {
 }
 
 __device__ __forceinline__ void wait_vm8() { asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); }
+__device__ __forceinline__ void wait_vm9() { asm volatile("s_waitcnt vmcnt(9)" ::: "memory"); }
 __device__ __forceinline__ void wait_vm10() { asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); }
 __device__ __forceinline__ void wait_vm0() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ void wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }

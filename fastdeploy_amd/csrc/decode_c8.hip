@@ -263,6 +263,9 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
           wm = fmaxf(wm, prs[stl]);
         }
         vmax = row_max16(wm);
+        // a unit whose heaviest product has all but vanished (its reciprocal would overflow, and 0 x inf is a
+        // NaN) contributes nothing
+        vmax = vmax > 7.9e-31f ? vmax : 0.f;  // 2^-100
         const float inv = vmax > 0.f ? 1.0f / vmax : 0.f;
 #pragma unroll
         for (int stl = 0; stl < 4; ++stl) prs[stl] *= inv;

@@ -5,6 +5,8 @@
 // ascending order.  Every product (fp32 q*scale times an int8 / e4m3 value) is exact in
 // fp64, so only the order of the additions matters for the bits of a score, and that
 // order is fixed: the kept indices are reproducible bit for bit on a CPU.
+// The formats with one scale per stored row (DYN) take q unscaled and multiply a token's
+// sum by its row's scale at the end (one more fp64 rounding).
 //
 // Two implementations give the same indices:
 //  * exact: every block scored in fp64, one token per lane (any shape; fp64-VALU bound);
@@ -42,7 +44,7 @@ __device__ __forceinline__ double dq64(u32 byte) {
 }
 
 // grid (max_blocks, hkv, batch), one wavefront: lane = token of the block
-template <int QUANT>
+template <int QUANT, bool DYN>
 __global__ __launch_bounds__(64) void sqattn_block_scores_kernel(ScoreArgs a) {
   __shared__ float qs[kSelMaxG][kSelMaxD];
   const int j = blockIdx.x, h = blockIdx.y, b = blockIdx.z, lane = threadIdx.x;
@@ -62,7 +64,8 @@ __global__ __launch_bounds__(64) void sqattn_block_scores_kernel(ScoreArgs a) {
   for (int i = lane; i < g * d; i += 64) {
     const int gi = i / d, c = i % d;
     // one fp32 rounding, as the definition of the score says
-    qs[gi][c] = __fmul_rn(bf16_to_f32(a.q[((size_t)b * a.hq + h * g + gi) * d + c]), a.k_scale[h * d + c]);
+    const float qv = bf16_to_f32(a.q[((size_t)b * a.hq + h * g + gi) * d + c]);
+    qs[gi][c] = DYN ? qv : __fmul_rn(qv, a.k_scale[h * d + c]);
   }
   __syncthreads();
   double best = -INFINITY;
@@ -83,9 +86,10 @@ __global__ __launch_bounds__(64) void sqattn_block_scores_kernel(ScoreArgs a) {
           if (gi < g) s[gi] = __dadd_rn(s[gi], __dmul_rn((double)qs[gi][c + e], kv));
       }
     }
+    const double kt = DYN ? (double)a.k_scale[((size_t)pb * a.hkv + h) * bs + t] : 1.0;
 #pragma unroll
     for (int gi = 0; gi < kSelMaxG; ++gi)
-      if (gi < g) best = fmax(best, s[gi]);
+      if (gi < g) best = fmax(best, DYN ? __dmul_rn(s[gi], kt) : s[gi]);
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) best = fmax(best, __shfl_xor(best, off, 64));
@@ -158,7 +162,7 @@ struct SelArgs {
   const int32_t* seq_lens_this_time;
   float* approx;  // [pairs][max_blocks]
   float* eps;     // [pairs]: bound that holds for every block of the pair
-  float* ebound;  // [pairs][max_blocks]: per-block bound (fp8 only, else NULL)
+  float* ebound;  // [pairs][max_blocks]: per-block bound (fp8 and the dynamic formats, else NULL)
   float* scores_out;  // optional copy of approx
   int32_t* kept_blocks;
   int32_t* kept_counts;
@@ -168,9 +172,10 @@ struct SelArgs {
 // One workgroup = `chunk` consecutive blocks of one (sequence, KV head); each wavefront
 // streams blocks wave, wave+4, ... through two LDS slots (one tile computing, one or two
 // in flight) and leaves one fp32 score per block.
-template <int QUANT>
+template <int QUANT, bool DYN>
 __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelArgs a) {
   __shared__ __attribute__((aligned(16))) uint8_t ldsK[kWaves][2][kTileB];  // two K slots per wavefront
+  __shared__ __attribute__((aligned(16))) float ldsS[DYN ? kWaves : 1][2][kBS];  // DYN: the slots' scale rows
   const int lane = threadIdx.x & 63;
   const int wv = uni(threadIdx.x >> 6);
   // chunk-major: every XCD (workgroups are dealt to them in turn) sees every chunk position
@@ -187,7 +192,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
     const int u = lane + 64 * e;
     if (u < a.chunk && first + u < a.max_blocks) pb_raw[e] = a.block_tables[(size_t)b * a.max_blocks + first + u];
   }
-  const PairRaw raw = load_pair_issue(a.q, a.k_scale, a.hkv, p, b, lane);
+  const PairRaw raw = load_pair_issue(a.q, DYN ? nullptr : a.k_scale, a.hkv, p, b, lane);
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
   const int n_p = min((max(kv_len, 0) + kBS - 1) / kBS, a.max_blocks);
   const int cnt = min(a.chunk, n_p - first);
@@ -219,9 +224,15 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
   const uint8_t* const kbase = a.key_cache + (size_t)h * tile_stride;
   const size_t blk_stride = (size_t)a.hkv * tile_stride;
 
-  if (wv < cnt) dma_tile(kbase + (size_t)unit_pb(wv) * blk_stride, saddr0, offK);
-  if (wv + kWaves < cnt)
-    dma_tile(kbase + (size_t)unit_pb(wv + kWaves) * blk_stride, saddr0 + kTileB, offK);
+  // DYN: a tile's 64 row scales follow it into LDS (one more direct load, counted by the waits below)
+  const u32 ssaddr0 = (u32)uni((int)lds_addr_of(ldsS[DYN ? wv : 0][0]));
+  const u32 lane_x4 = (u32)lane * 4u;
+  auto fetch = [&](int blk, int slot) {
+    dma_tile(kbase + (size_t)blk * blk_stride, saddr0 + (u32)slot * kTileB, offK);
+    if (DYN) dma_row64(a.k_scale + ((size_t)blk * a.hkv + h) * kBS, ssaddr0 + (u32)slot * (kBS * 4), lane_x4);
+  };
+  if (wv < cnt) fetch(unit_pb(wv), 0);
+  if (wv + kWaves < cnt) fetch(unit_pb(wv + kWaves), 1);
 
   if (ck == 0 && wv == 0) {
     // error bound of the MFMA scores of this pair (see the top of the file): q*scale is cut to
@@ -230,7 +241,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
     for (int g = 0; g < kG; ++g) {
       float sa = 0.f, am = 0.f;
       for (int c = lane; c < kD; c += 64) {
-        const float qs = fabsf(bf16_to_f32(a.q[((size_t)b * a.hkv * kG + h * kG + g) * kD + c]) * a.k_scale[h * kD + c]);
+        const float qs = fabsf(bf16_to_f32(a.q[((size_t)b * a.hkv * kG + h * kG + g) * kD + c]) * (DYN ? 1.0f : a.k_scale[h * kD + c]));
         sa += qs;
         am = fmaxf(am, qs);
       }
@@ -246,6 +257,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
     float e;
     if (QUANT == FDATTN_CACHE_INT8) e = amax * ((128.0f * 127.0f * 0.5f + 2048.0f) / 1048575.0f);
     else e = sabs * 448.0f * 3.0517578125e-5f + amax * (128.0f * 448.0f * 3.814697265625e-6f);
+    // DYN: this is the bound before the row scale; every block multiplies it by its largest scale (below)
     if (lane == 0) a.eps[p] = e * 1.0001f;
   }
 
@@ -280,8 +292,19 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
   for (int j = wv; j < cnt; j += kWaves, ++it) {
     const int valid = unit_valid(j);
     const uint8_t* kbuf = ldsK[wv][it & 1];  // indexed, not picked from a pointer array: stays an LDS address
-    if (j + kWaves < cnt) wait_vm8(); else wait_vm0();
+    if (j + kWaves >= cnt) wait_vm0(); else if (DYN) wait_vm9(); else wait_vm8();
     float sv = -INFINITY, bv = 0.f;
+    float kt[4] = {1.f, 1.f, 1.f, 1.f}, ktmax = 0.f;  // DYN: scales of this lane's tokens; the block's largest
+    if (DYN) {
+      const float4 k4 = *reinterpret_cast<const float4*>(&ldsS[wv][it & 1][4 * n16]);
+      kt[0] = k4.x; kt[1] = k4.y; kt[2] = k4.z; kt[3] = k4.w;
+#pragma unroll
+      for (int stl = 0; stl < 4; ++stl) {
+        kt[stl] = (4 * n16 + stl < valid) ? kt[stl] : 0.f;  // (a slot past the end may hold anything)
+        ktmax = fmaxf(ktmax, fabsf(kt[stl]));
+      }
+      ktmax = row_max16(ktmax);
+    }
 #pragma unroll
     for (int stl = 0; stl < 4; ++stl) {
       const int tok = 4 * n16 + stl;
@@ -295,6 +318,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
           acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(st.aq[k2], kb, acc, 0, 0, 0);
         }
         s = st.rs * ((float)acc.x + 128.0f * (float)acc.y + 16384.0f * (float)acc.z);
+        if (DYN) s *= kt[stl];
       } else {
         v4f acc = {0.f, 0.f, 0.f, 0.f}, ab = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -313,13 +337,13 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
           ab = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(m1, b1 & 0x7f7f7f7f7f7f7f7fL, ab, 0, 0, 0);
         }
         s = st.rs * ((acc.x + acc.y) + (acc.z + acc.w));
-        bv = fmaxf(bv, tok < valid ? st.rs * ab.x : 0.f);
+        if (DYN) s *= kt[stl];
+        bv = fmaxf(bv, tok < valid ? st.rs * ab.x * (DYN ? fabsf(kt[stl]) : 1.0f) : 0.f);
       }
       sv = fmaxf(sv, tok < valid ? s : -INFINITY);
     }
     wait_lgkm0();  // tile consumed: refill its slot with the block two steps ahead
-    if (j + 2 * kWaves < cnt)
-      dma_tile(kbase + (size_t)unit_pb(j + 2 * kWaves) * blk_stride, saddr0 + (u32)(it & 1) * kTileB, offK);
+    if (j + 2 * kWaves < cnt) fetch(unit_pb(j + 2 * kWaves), it & 1);
     sv = row_max16(sv);                          // over the tokens of this head
     sv = fmaxf(sv, __shfl_xor(sv, 16, 64));      // over the 4 heads of the group
     sv = fmaxf(sv, __shfl_xor(sv, 32, 64));
@@ -330,11 +354,19 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
       // residual of the four limbs <= 2^-16 |q*scale| per channel (or the e4m3 subnormal floor, 2^-10 in units
       // of amax/256); fp32 accumulation <= 2^-17 of sum |q*scale||k|; the one-limb |q*scale| is itself up to
       // 2^-4 low: (2^-16 + 2^-17) * (1 + 2^-4) < 2^-15.3 -> 2.5e-5
-      bv = bv * 2.5e-5f + amax_pair * (128.0f * 448.0f * 3.814697265625e-6f) * 1.0001f;
+      // DYN: the product with the row scale is one more fp32 rounding, at most 2^-24 of |score| <= the token's
+      // sum |q||k| x scale, which bv holds (up to 2^-4 low): + 1.3e-7
+      bv = bv * (DYN ? 2.513e-5f : 2.5e-5f) + amax_pair * (128.0f * 448.0f * 3.814697265625e-6f) * 1.0001f * (DYN ? ktmax : 1.0f);
+    }
+    if (DYN && QUANT == FDATTN_CACHE_INT8) {
+      // the per-channel format's bound for this pair (from q alone) times the block's largest row scale, plus
+      // the rounding of the product with the row scale: 2^-24 of |score| <= 128 * 127 * amax * scale
+      const float amax_q = fmaxf(fmaxf(__shfl(st.rs, 0, 64), __shfl(st.rs, 16, 64)), fmaxf(__shfl(st.rs, 32, 64), __shfl(st.rs, 48, 64))) * 1048575.0f;
+      bv = amax_q * ktmax * (((128.0f * 127.0f * 0.5f + 2048.0f) / 1048575.0f) * 1.0001f + 128.0f * 127.0f * 1.2e-7f);
     }
     if (lane == 0) {
       srow[first + j] = sv;
-      if (QUANT != FDATTN_CACHE_INT8) a.ebound[(size_t)p * a.max_blocks + first + j] = bv;
+      if (QUANT != FDATTN_CACHE_INT8 || DYN) a.ebound[(size_t)p * a.max_blocks + first + j] = bv;
       if (a.scores_out) a.scores_out[(size_t)p * a.max_blocks + first + j] = sv;
     }
   }
@@ -403,7 +435,7 @@ __device__ void radix_select2_desc(const float* v, const float* e, int n, int r0
 }
 
 // One workgroup per (sequence, KV head): classify, re-score the undecided blocks in fp64, emit.
-template <int QUANT>
+template <int QUANT, bool DYN>
 __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs a) {
   extern __shared__ double smd[];                  // exact scores of undecided blocks [max_blocks]
   float* sf = reinterpret_cast<float*>(smd + a.max_blocks);      // approx scores [max_blocks]
@@ -430,7 +462,8 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
   }
   for (int i = tid; i < kG * kD; i += kResolveThreads) {
     const int g = i / kD, c = i % kD;
-    qs[g][c] = __fmul_rn(bf16_to_f32(a.q[((size_t)b * a.hkv * kG + h * kG + g) * kD + c]), a.k_scale[h * kD + c]);
+    const float qv = bf16_to_f32(a.q[((size_t)b * a.hkv * kG + h * kG + g) * kD + c]);
+    qs[g][c] = DYN ? qv : __fmul_rn(qv, a.k_scale[h * kD + c]);
   }
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
   const int nblk = min((max(kv_len, 0) + kBS - 1) / kBS, a.max_blocks);
@@ -478,6 +511,11 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
 #pragma unroll
               for (int g = 0; g < kG; ++g) acc[g] = __fma_rn((double)qs[g][c + e], kv, acc[g]);
             }
+          }
+          if (DYN) {
+            const double kt = (double)a.k_scale[((size_t)pb * a.hkv + h) * kBS + lane];
+#pragma unroll
+            for (int g = 0; g < kG; ++g) acc[g] = __dmul_rn(acc[g], kt);
           }
           best = fmax(fmax(acc[0], acc[1]), fmax(acc[2], acc[3]));
         }
@@ -556,9 +594,8 @@ static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_ca
                 "fdattn_sqattn_select: unsupported shape batch=%d hq=%d hkv=%d head_dim=%d block_size=%d "
                 "max_blocks=%d top_k=%d (group <= %d, head_dim <= %d multiple of 4, max_blocks <= 4096)",
                 batch, hq, hkv, head_dim, block_size, max_blocks_per_seq, top_k, kSelMaxG, kSelMaxD);
-  if (cache_quant_type != FDATTN_CACHE_INT8 && cache_quant_type != FDATTN_CACHE_FP8_E4M3)
-    return fail(FDATTN_ERR_QUANT, "fdattn_sqattn_select: cache_quant_type %d is not a format with per-channel scales",
-                cache_quant_type);
+  if (!quant_known(cache_quant_type))
+    return fail(FDATTN_ERR_QUANT, "fdattn_sqattn_select: unknown cache_quant_type %d", cache_quant_type);
   const size_t need = (size_t)batch * hkv * ((size_t)max_blocks_per_seq * sizeof(double) + sizeof(float));
   if (workspace_bytes < need)
     return fail(FDATTN_ERR_WORKSPACE, "fdattn_sqattn_select: workspace %zu B < required %zu B", workspace_bytes, need);
@@ -571,15 +608,23 @@ static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_ca
     float* ebound = approx + (size_t)pairs * max_blocks_per_seq;
     float* eps = ebound + (size_t)pairs * max_blocks_per_seq;
     SelArgs sa{(const uint16_t*)q, (const uint8_t*)key_cache, cache_k_scale, block_tables, seq_lens_decoder,
-               seq_lens_this_time, approx, eps, cache_quant_type == FDATTN_CACHE_INT8 ? nullptr : ebound, scores, kept_blocks, kept_counts, batch, hkv,
+               seq_lens_this_time, approx, eps, cache_quant_type == FDATTN_CACHE_INT8 ? nullptr : ebound, scores,
+               kept_blocks, kept_counts, batch, hkv,
                max_blocks_per_seq, num_blocks, chunk, cpp, top_k};
     const size_t shm2 = (size_t)max_blocks_per_seq * (sizeof(double) + 2 * sizeof(float) + 3 * sizeof(int));
+    const dim3 g1(pairs * cpp), g2(pairs), b1(256), b2(kResolveThreads);
     if (cache_quant_type == FDATTN_CACHE_INT8) {
-      hipLaunchKernelGGL(sqattn_scores_mfma_kernel<FDATTN_CACHE_INT8>, dim3(pairs * cpp), dim3(256), 0, s, sa);
-      hipLaunchKernelGGL(sqattn_resolve_kernel<FDATTN_CACHE_INT8>, dim3(pairs), dim3(kResolveThreads), shm2, s, sa);
+      hipLaunchKernelGGL((sqattn_scores_mfma_kernel<FDATTN_CACHE_INT8, false>), g1, b1, 0, s, sa);
+      hipLaunchKernelGGL((sqattn_resolve_kernel<FDATTN_CACHE_INT8, false>), g2, b2, shm2, s, sa);
+    } else if (cache_quant_type == FDATTN_CACHE_FP8_E4M3) {
+      hipLaunchKernelGGL((sqattn_scores_mfma_kernel<FDATTN_CACHE_FP8_E4M3, false>), g1, b1, 0, s, sa);
+      hipLaunchKernelGGL((sqattn_resolve_kernel<FDATTN_CACHE_FP8_E4M3, false>), g2, b2, shm2, s, sa);
+    } else if (cache_quant_type == FDATTN_CACHE_INT8_DYNAMIC) {
+      hipLaunchKernelGGL((sqattn_scores_mfma_kernel<FDATTN_CACHE_INT8, true>), g1, b1, 0, s, sa);
+      hipLaunchKernelGGL((sqattn_resolve_kernel<FDATTN_CACHE_INT8, true>), g2, b2, shm2, s, sa);
     } else {
-      hipLaunchKernelGGL(sqattn_scores_mfma_kernel<FDATTN_CACHE_FP8_E4M3>, dim3(pairs * cpp), dim3(256), 0, s, sa);
-      hipLaunchKernelGGL(sqattn_resolve_kernel<FDATTN_CACHE_FP8_E4M3>, dim3(pairs), dim3(kResolveThreads), shm2, s, sa);
+      hipLaunchKernelGGL((sqattn_scores_mfma_kernel<FDATTN_CACHE_FP8_E4M3, true>), g1, b1, 0, s, sa);
+      hipLaunchKernelGGL((sqattn_resolve_kernel<FDATTN_CACHE_FP8_E4M3, true>), g2, b2, shm2, s, sa);
     }
     return check_launch("fdattn_sqattn_select (mfma)");
   }
@@ -588,9 +633,13 @@ static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_ca
               max_blocks_per_seq, num_blocks};
   dim3 grid(max_blocks_per_seq, hkv, batch);
   if (cache_quant_type == FDATTN_CACHE_INT8)
-    hipLaunchKernelGGL(sqattn_block_scores_kernel<FDATTN_CACHE_INT8>, grid, dim3(64), 0, s, a);
+    hipLaunchKernelGGL((sqattn_block_scores_kernel<FDATTN_CACHE_INT8, false>), grid, dim3(64), 0, s, a);
+  else if (cache_quant_type == FDATTN_CACHE_FP8_E4M3)
+    hipLaunchKernelGGL((sqattn_block_scores_kernel<FDATTN_CACHE_FP8_E4M3, false>), grid, dim3(64), 0, s, a);
+  else if (cache_quant_type == FDATTN_CACHE_INT8_DYNAMIC)
+    hipLaunchKernelGGL((sqattn_block_scores_kernel<FDATTN_CACHE_INT8, true>), grid, dim3(64), 0, s, a);
   else
-    hipLaunchKernelGGL(sqattn_block_scores_kernel<FDATTN_CACHE_FP8_E4M3>, grid, dim3(64), 0, s, a);
+    hipLaunchKernelGGL((sqattn_block_scores_kernel<FDATTN_CACHE_FP8_E4M3, true>), grid, dim3(64), 0, s, a);
   int rc = check_launch("fdattn_sqattn_select (scores)");
   if (rc) return rc;
   const size_t shm = (size_t)max_blocks_per_seq * (sizeof(double) + sizeof(int));

@@ -28,7 +28,8 @@
  *     kv_len 1 = V row, constant K = mean of V; its softmax against the
  *     known-answer vectors of tests/function/test_softmax.cc:28-33;
  *   - fdo_splitkv_combine: split-count invariance against the unsplit result;
- *   - fdo_sqattn_block_scores: brute force in numpy fp64;
+ *   - fdo_sqattn_block_scores: brute force in numpy fp64 (per-channel and
+ *     dynamic formats);
  *   - fdo_topk_select: torch.topk / stable argsort, the tie rule of
  *     fastdeploy/vision/utils/utils.h:41-60 and the sort vectors of
  *     tests/function/test_sort.cc:26-106;
@@ -423,7 +424,9 @@ int fdo_splitkv_combine(const float* part_o, const float* part_m, const float* p
  * summed over c = 0..d-1 in that order in fp64.  The fp32 product q*scale is a
  * single rounding; K8 (an int8 integer or an e4m3 value) is exact in fp64, and
  * so is every product (24 + 8 significant bits).  Blocks past the sequence get
- * -inf.
+ * -inf.  Dynamic formats (k_scale = the scale cache [num_blocks, hkv, bs]): q enters
+ * unscaled and the token's sum is multiplied by its row's scale at the end, one more
+ * fp64 rounding:  (double)k_scale[row of t] * sum_c (double)q[b,g,c] * (double)K8[t,c].
  */
 int fdo_sqattn_block_scores(const uint16_t* q, const uint8_t* key_cache, const float* k_scale,
                             const int32_t* block_tables, const int32_t* kv_lens, double* scores,
@@ -436,7 +439,8 @@ int fdo_sqattn_block_scores(const uint16_t* q, const uint8_t* key_cache, const f
       double* qs = (double*)malloc(sizeof(double) * g * d);
       for (int gi = 0; gi < g; ++gi)
         for (int c = 0; c < d; ++c) {
-          float f = fdo_bf16_to_f32(q[((size_t)b * hq + h * g + gi) * d + c]) * k_scale[h * d + c];
+          float f = fdo_bf16_to_f32(q[((size_t)b * hq + h * g + gi) * d + c]);
+          if (!is_dynamic(cache_type)) f = f * k_scale[h * d + c];
           qs[gi * d + c] = (double)f;
         }
       int kv_len = kv_lens[b];
@@ -444,13 +448,14 @@ int fdo_sqattn_block_scores(const uint16_t* q, const uint8_t* key_cache, const f
         double best = -INFINITY;
         int t0 = j * bs, t1 = t0 + bs < kv_len ? t0 + bs : kv_len;
         if (t0 < kv_len) {
-          const uint8_t* kp =
-              key_cache + ((size_t)block_tables[(size_t)b * max_blocks_per_seq + j] * hkv + h) * bs * d;
+          size_t tile = (size_t)block_tables[(size_t)b * max_blocks_per_seq + j] * hkv + h;
+          const uint8_t* kp = key_cache + tile * bs * d;
           for (int t = t0; t < t1; ++t)
             for (int gi = 0; gi < g; ++gi) {
               double s = 0.0;
               for (int c = 0; c < d; ++c)
                 s += qs[gi * d + c] * (double)dequant(kp[(size_t)(t - t0) * d + c], cache_type);
+              if (is_dynamic(cache_type)) s = s * (double)k_scale[tile * bs + (t - t0)];
               if (s > best) best = s;
             }
         }

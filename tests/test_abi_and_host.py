@@ -76,8 +76,8 @@ def test_version_and_argument_errors_need_no_gpu():
 
 
 def test_dynamic_formats_in_the_argument_checks_and_the_host_helpers():
-    """The formats with one scale per stored row: names, what the selector and odd head sizes answer (before any
-    device call), the decode kernel choice and the size of their wire form."""
+    """The formats with one scale per stored row: names, what odd head sizes and unknown format numbers answer
+    (before any device call), the decode kernel choice and the size of their wire form."""
     lib = _lib.lib()
     one = ctypes.c_void_p(16)
     assert ops._quant("cache_int8_dynamic") == 3 and ops._quant("cache_fp8_dynamic") == 4
@@ -86,8 +86,8 @@ def test_dynamic_formats_in_the_argument_checks_and_the_host_helpers():
     assert lib.fdattn_decode_uses_mfma(32, 8, 128, 64, 3) == 1 and lib.fdattn_decode_uses_mfma(32, 8, 128, 64, 4) == 1
     rc = lib.fdattn_write_cache_kv(*([one] * 13), 1, 1, 4, 2, 96, 64, 1, 1, 8, 1, 3, None)    # 96 / 16 = 6 threads a row
     assert rc == -2 and b"dynamic" in lib.fdattn_last_error()
-    rc = lib.fdattn_sqattn_select(*([one] * 10), 1 << 30, 2, 32, 8, 128, 64, 8, 8, 4, 4, None)
-    assert rc == -3 and b"per-channel" in lib.fdattn_last_error()
+    rc = lib.fdattn_sqattn_select(*([one] * 10), 1 << 30, 2, 32, 8, 128, 64, 8, 8, 4, 7, None)
+    assert rc == -3 and b"unknown" in lib.fdattn_last_error()
     # wire form: the scales section grows with the pages instead of holding 2 x hkv x head_dim floats
     stat, dyn = lib.fdattn_kv_wire_bytes_for(130, 8, 128, 64, 1), lib.fdattn_kv_wire_bytes_for(130, 8, 128, 64, 3)
     assert stat == lib.fdattn_kv_wire_bytes(130, 8, 128, 64)

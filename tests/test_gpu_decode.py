@@ -93,6 +93,27 @@ def test_decode_dynamic_formats_with_widely_different_row_scales(oracle, impl, q
     check(gpu_decode(case, impl), oracle_decode(oracle, case), "row scales")
 
 
+@pytest.mark.parametrize("quant", [CACHE_INT8_DYNAMIC, CACHE_FP8_DYNAMIC])
+def test_decode_dynamic_formats_with_vanishing_units(oracle, quant):
+    """A query aligned with one key so strongly that the weights of whole blocks fall to the bottom of the fp32
+    range (where the reciprocal of a block's heaviest weight x scale product overflows): those blocks must drop
+    out, not poison the row."""
+    # logit gaps from ~30 to ~500 (and 4 x to 16 x smaller for the heads whose key row has a smaller scale): for
+    # some of them the heaviest weight of a block lands in the band just above the smallest fp32 numbers
+    gains = [3.0, 5.0, 7.0, 8.5, 10.0, 12.0, 16.0, 24.0, 34.0, 48.0]
+    case = syn.decode_case(batch=len(gains), ctx=64 * 12 + 5, quant=quant, seed=21, row_log2=(-2, 0))
+    q = case["q"].view(len(gains), 32, 128)
+    for b, gain in enumerate(gains):
+        blk = int(case["block_tables"][b, 3 + b % 5])
+        k8 = case["key_cache"][blk, :, 7 + b, :]
+        kf = (k8.view(torch.int8) if quant == CACHE_INT8_DYNAMIC else k8.view(torch.float8_e4m3fn)).float()
+        krow = kf * case["cache_k_scale"][blk, :, 7 + b][:, None]
+        q[b] = (krow * gain).repeat_interleave(4, 0).to(torch.bfloat16)
+    got, want = gpu_decode(case, "auto"), oracle_decode(oracle, case)
+    assert np.isfinite(oracle.bf16_to_f32(got)).all()
+    check(got, want, "vanishing units")
+
+
 def test_decode_generic_other_shapes(oracle):
     """Shapes outside the MFMA kernel: head_dim 64, group 2, block_size 16."""
     case = syn.decode_case(batch=3, ctx=[50, 200, 333], seed=8, hq=8, hkv=4, d=64, bs=16)

@@ -22,7 +22,7 @@ def oracle_select(oracle, case, top_k):
 
 
 @pytest.mark.parametrize("impl", ["auto", "exact"])
-@pytest.mark.parametrize("quant", [CACHE_FP8, CACHE_INT8])
+@pytest.mark.parametrize("quant", ALL_FORMATS)
 def test_selector_indices_bit_exact(oracle, quant, impl):
     for seed in range(2):
         case = syn.decode_case(batch=3, ctx=[4096, 3000, 64 * 20 + 1], quant=quant, seed=seed, salient=0.05)
@@ -44,18 +44,23 @@ def test_selector_indices_bit_exact(oracle, quant, impl):
 
 
 @pytest.mark.parametrize("impl", ["auto", "exact"])
-@pytest.mark.parametrize("quant", [CACHE_FP8, CACHE_INT8])
+@pytest.mark.parametrize("quant", ALL_FORMATS)
 def test_selector_ties_near_ties_and_short_sequences(oracle, quant, impl):
     case = syn.decode_case(batch=2, ctx=[64 * 12, 100], quant=quant, seed=3)
     bt = case["block_tables"]
-    # identical K pages -> identical scores -> the lower block index must win
+    dyn = quant in (CACHE_INT8_DYNAMIC, CACHE_FP8_DYNAMIC)
+    # identical K pages (and, for the dynamic formats, scale rows) -> identical scores -> the lower block index must win
     for j in (5, 7, 9):
         case["key_cache"][int(bt[0, j])] = case["key_cache"][int(bt[0, 2])]
+        if dyn:
+            case["cache_k_scale"][int(bt[0, j])] = case["cache_k_scale"][int(bt[0, 2])]
     # near ties: copies that differ by one code step in one channel of every token
     for j, ch in ((3, 0), (10, 77)):
         page = case["key_cache"][int(bt[0, 2])].clone()
         page[:, :, ch] = torch.where((page[:, :, ch] & 0x7F) < 0x70, page[:, :, ch] + 1, page[:, :, ch])
         case["key_cache"][int(bt[0, j])] = page
+        if dyn:
+            case["cache_k_scale"][int(bt[0, j])] = case["cache_k_scale"][int(bt[0, 2])]
     dev = syn.to_device(case, "cuda")
     for k in (1, 2, 3, 4, 5, 6, 7, 11, 12, 64):
         kept, cnt = fd.sqattn_select(dev["q"], dev["key_cache"], dev["cache_k_scale"], dev["block_tables"],
@@ -64,12 +69,15 @@ def test_selector_ties_near_ties_and_short_sequences(oracle, quant, impl):
         assert np.array_equal(np_of(kept), okept) and np.array_equal(np_of(cnt), ocnt), k
 
 
-def test_selector_config4_shape_indices_bit_exact(oracle):
+@pytest.mark.parametrize("quant", [CACHE_FP8, CACHE_FP8_DYNAMIC])
+def test_selector_config4_shape_indices_bit_exact(oracle, quant):
     """batch 16, ctx 32768, fp8 KV, top-64 of 512 blocks per KV head, 5 % salient blocks (scaled x4):
-    the full-size launch against the oracle."""
-    case = syn.decode_case(batch=16, ctx=32768, quant=CACHE_FP8, seed=0, device="cuda", salient=0.05)
+    the full-size launch against the oracle (per-channel scales, and one scale per stored row)."""
+    # (dynamic format: row scales up to 2^6 apart with the largest rows at unit scale, where the absolute part of
+    # the output tolerance applies; the fp8 weights of the decode kernel carry 16 significant bits)
+    case = syn.decode_case(batch=16, ctx=32768, quant=quant, seed=0, device="cuda", salient=0.05, row_log2=(-6, 0))
     kept, cnt = fd.sqattn_select(case["q"], case["key_cache"], case["cache_k_scale"], case["block_tables"],
-                                 case["seq_lens_decoder"], num_heads=32, top_k=64)
+                                 case["seq_lens_decoder"], num_heads=32, top_k=64, cache_quant_type=quant)
     torch.cuda.synchronize()
     cpu = syn.to_device(case, "cpu")
     _, okept, ocnt = oracle_select(oracle, cpu, 64)
@@ -78,20 +86,12 @@ def test_selector_config4_shape_indices_bit_exact(oracle):
     # and the sparse decode over the kept blocks equals the oracle's
     out = fd.decode_attention_sparse(case["q"], case["key_cache"], case["value_cache"], case["cache_k_scale"],
                                      case["cache_v_scale"], case["block_tables"], case["seq_lens_decoder"],
-                                     kept_blocks=kept, kept_counts=cnt, num_heads=32, cache_quant_type=CACHE_FP8)
+                                     kept_blocks=kept, kept_counts=cnt, num_heads=32, cache_quant_type=quant)
     want = oracle.decode_attention(bits(cpu["q"]), np_of(cpu["key_cache"]), np_of(cpu["value_cache"]),
                                    np_of(cpu["cache_k_scale"]), np_of(cpu["cache_v_scale"]), np_of(cpu["block_tables"]),
-                                   np_of(cpu["seq_lens_decoder"]), 32, 8, 128, CACHE_FP8, kept_blocks=okept, kept_counts=ocnt)
+                                   np_of(cpu["seq_lens_decoder"]), 32, 8, 128, quant, kept_blocks=okept, kept_counts=ocnt)
     ok, mx, bad = bf16_close(bits(out), want)
     assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
-
-
-def test_selector_rejects_the_dynamic_formats():
-    """The block scores are defined on per-channel scales: the formats with one scale per stored row are refused."""
-    case = syn.to_device(syn.decode_case(batch=2, ctx=[300, 500], quant=CACHE_FP8_DYNAMIC, seed=1), "cuda")
-    with pytest.raises(ValueError, match="per-channel"):
-        fd.sqattn_select(case["q"], case["key_cache"], case["cache_k_scale"], case["block_tables"],
-                         case["seq_lens_decoder"], num_heads=32, top_k=4, cache_quant_type=CACHE_FP8_DYNAMIC)
 
 
 def _prefill_case(seed, prefix, chunks, quant=CACHE_INT8):

@@ -537,6 +537,28 @@ def test_block_scores_brute_force_fp64(oracle, quant):
             assert np.allclose(s[b, :, j], want, rtol=1e-12, atol=1e-12)
 
 
+@pytest.mark.parametrize("quant", [CACHE_INT8_DYNAMIC, CACHE_FP8_DYNAMIC])
+def test_block_scores_dynamic_formats_brute_force_fp64(oracle, quant):
+    """One scale per stored row: the block score is the largest, over the block's tokens and the group's heads, of
+    (row scale) x (q . K8) - here by einsum in fp64 over rows whose scales differ by up to 2^6."""
+    case = syn.decode_case(batch=2, ctx=[200, 130], quant=quant, seed=8, salient=0.3)
+    s = oracle.sqattn_block_scores(bits(case["q"]), np_of(case["key_cache"]), np_of(case["cache_k_scale"]),
+                                   np_of(case["block_tables"]), np_of(case["seq_lens_decoder"]), 32, 8, 128, quant)
+    q = case["q"].double().view(2, 8, 4, 128)
+    for b in range(2):
+        n = int(case["seq_lens_decoder"][b])
+        for j in range(case["block_tables"].shape[1]):
+            if j * 64 >= n:
+                assert np.all(s[b, :, j] == -np.inf)
+                continue
+            blk = int(case["block_tables"][b, j])
+            k8 = case["key_cache"][blk]
+            kv = (k8.view(torch.int8) if quant == CACHE_INT8_DYNAMIC else k8.view(torch.float8_e4m3fn)).double()
+            nt = min(64, n - j * 64)
+            dots = torch.einsum("hgc,htc->hgt", q[b], kv[:, :nt]) * case["cache_k_scale"][blk, :, None, :nt].double()
+            assert np.allclose(s[b, :, j], dots.amax((1, 2)).numpy(), rtol=1e-12, atol=1e-12)
+
+
 def test_topk_tie_rule_sort_vectors_and_torch(oracle):
     # ties resolve to the lowest index (fastdeploy/vision/utils/utils.h:41-60)
     sc = np.array([[[1.0, 5.0, 5.0, 2.0, 5.0, 0.0, 2.0, -1.0]]])
