@@ -199,6 +199,14 @@ def other_workloads(args):
             line("configs[1] decode over the %s cache (one scale per stored row)" % name, ms, "hbm", work,
                  HBM_PEAK_GBPS, "GB/s")
             del cs
+        # configs[3]'s selector over the fp8 dynamic format
+        cs = syn.decode_case(batch=16, ctx=32768, quant="cache_fp8_dynamic", seed=0, device=dev, direct_bytes=True)
+        sel = lambda: fd.sqattn_select(cs["q"], cs["key_cache"], cs["cache_k_scale"], cs["block_tables"],
+                                       cs["seq_lens_decoder"], num_heads=32, top_k=64, cache_quant_type="cache_fp8_dynamic")
+        ms = time_events(sel, max(args.steps // 4, 5), 3)
+        line("configs[3] SQAttn selector over the cache_fp8_dynamic cache", ms, "hbm",
+             16 * 32768 * 8 * (128 + 4) + 16 * 4096 * 2, HBM_PEAK_GBPS, "GB/s")
+        del cs
         cw = syn.write_case(num_seqs=2, max_pos=8192 + 2048, seed=1, device=dev, chunk=2048, blocks_per_seq=160,
                             quant="cache_int8_dynamic")
         cw["seq_lens_decoder"].fill_(8192)

@@ -60,7 +60,8 @@ extern "C" {
  * indexed like the rows of key_cache / value_cache; the cache writer (and the one-call step, which
  * contains it) STORES into them despite the const qualifier, every attention entry point reads them.
  * K scales are taken after the rotation.  Dequantised value = byte * scale of its row.
- * Not accepted by the block selector, which is defined on per-channel scales.
+ * The block selector scores a token as (row scale) x sum_c q[c] * K8[t,c] for these formats: q unscaled, the
+ * sum in fp64 in ascending channel order, one more fp64 rounding for the product with the scale.
  */
 #define FDATTN_CACHE_INT8_DYNAMIC 3
 #define FDATTN_CACHE_FP8_E4M3_DYNAMIC 4
