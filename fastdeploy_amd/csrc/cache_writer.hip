@@ -1,7 +1,8 @@
 // Cache writer: rotary embedding on Q/K + int8 / fp8-e4m3 quantisation of K/V into
 // block-tabled pages; optionally the QKV projection's epilogue in front of it (bias, per-head
 // RMS norm of Q and K).  Memory-bound and tiny (launch-bound at decode sizes): one
-// thread per 16 channels, 16-byte loads of qkv, 8/16-byte stores into the page.
+// thread per 16 channels, 16-byte loads of qkv, 8/16-byte stores into the page.  The
+// dynamic formats derive one scale per stored row from the row itself and store it beside it.
 //
 // Bit-exactness contract (shared with the CPU oracle): every fp32 product, sum and
 // the one division are rounded on their own - this file is compiled with

@@ -2,7 +2,8 @@
 // combine.  One wavefront per (sequence, query head, KV split): lanes own tokens for
 // q.K and channels for P.V.  This is the fall-back for shapes the MFMA kernel in
 // decode_c8.hip does not cover (any head_dim <= 256, any group size, any block size);
-// it makes no attempt to reach the HBM roofline.
+// it makes no attempt to reach the HBM roofline.  The formats with one scale per stored
+// row (DYN) multiply a token's score by its K scale and its weight by its V scale.
 #include "launch.h"
 
 namespace fdattn {

@@ -28,9 +28,11 @@
 // O^T = V^T P^T - no trip through LDS.  V^T operands come transposed out of LDS by
 // ds_read_b64_tr_b16.  The exponent reference of a query is raised only when its weight sum
 // over a tile exceeds 1024 (every weight then stays far inside fp16): the tile's maximum is
-// not even computed on the other tiles, and the accumulator is rescaled on a handful of them.  The per-channel K scale is folded into Q for the
-// prefix tiles; the V scale is applied to the accumulator once, when the walk passes from
-// the prefix to the chunk.
+// not even computed on the other tiles, and the accumulator is rescaled on a handful of them.
+// The per-channel K scale is folded into Q for the prefix tiles; the V scale is applied to the
+// accumulator once, when the walk passes from the prefix to the chunk.  The formats with one
+// scale per stored row (DYN) are dequantised while they are staged instead: the staged fp16
+// number is byte x row scale, Q stays unscaled and nothing is left to apply at the end.
 //
 // Schedule.  The wavefronts form two groups that alternate between a matrix phase (the two
 // MFMA streams of a tile, hand-scheduled: LDS operand reads six deep in flight, exact

@@ -33,6 +33,7 @@
  *   value_cache   u8    same
  *   cache_k_scale f32   [hkv, head_dim]  dequantisation multiplier (max-abs/127 or max-abs/448)
  *   cache_v_scale f32   [hkv, head_dim]
+ *                       dynamic formats: [num_blocks, hkv, block_size], one scale per stored row (see below)
  *   block_tables  i32   [batch, max_blocks_per_seq]  physical block per logical block, -1 = none
  *   seq_lens_*    i32   [batch]
  *   rope_cos/sin  f32   [max_pos, head_dim/2]  host-built table shared with the CPU oracle
