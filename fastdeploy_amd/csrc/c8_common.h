@@ -8,8 +8,9 @@ namespace fdattn {
 
 constexpr int kWaves = 4;      // wavefronts per workgroup
 constexpr int kTileB = 8192;   // bytes of one K or V tile (64 tokens x 128 channels)
-constexpr int kD = 128, kG = 4, kBS = 64;
-constexpr int kSlotFloats = kG * kD;  // partial o per slot
+constexpr int kD = 128, kG = 4, kBS = 64;  // kG: query heads per MFMA row set (16 rows = 4 heads x 4 limbs)
+constexpr int kSlotFloats = kG * kD;       // partial o of one row set
+constexpr int kMaxSets = 2;                // row sets a decode wavefront carries: up to 8 query heads per KV head
 constexpr int kMaxChunk = 128;        // units per chunk: two unit-table entries per lane
 
 __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
@@ -139,18 +140,21 @@ struct PairRaw {
 };
 
 // k_scale: the per-channel K scales [hkv, 128], or NULL (all ones: the scales are per stored row and are applied
-// to the scores)
-__device__ __forceinline__ PairRaw load_pair_issue(const uint16_t* q, const float* k_scale, int hkv, int p, int row, int lane) {
+// to the scores).  group: query heads per KV head; set: which four of them (heads 4 set .. 4 set + 3; heads
+// past the group read as zeros).
+__device__ __forceinline__ PairRaw load_pair_issue(const uint16_t* q, const float* k_scale, int hkv, int p, int row, int lane,
+                                                   int group = kG, int set = 0) {
   const int h = p % hkv;  // row: the sequence's row of q
-  const int m = lane & 15, g = lane >> 4, head = m >> 2;
-  const uint16_t* qrow = q + ((size_t)row * hkv * kG + h * kG + head) * kD;
+  const int m = lane & 15, g = lane >> 4, head = 4 * set + (m >> 2);
+  const bool live = head < group;
+  const uint16_t* qrow = q + ((size_t)row * hkv * group + h * group + (live ? head : 0)) * kD;
   const float* ks = k_scale + (size_t)h * kD;
   PairRaw r;
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
     const int c0 = 16 * (g + 4 * s);
-    r.w[s][0] = *reinterpret_cast<const uint4*>(qrow + c0);
-    r.w[s][1] = *reinterpret_cast<const uint4*>(qrow + c0 + 8);
+    r.w[s][0] = live ? *reinterpret_cast<const uint4*>(qrow + c0) : make_uint4(0u, 0u, 0u, 0u);
+    r.w[s][1] = live ? *reinterpret_cast<const uint4*>(qrow + c0 + 8) : make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       r.ks[s][i] = k_scale ? *reinterpret_cast<const float4*>(ks + c0 + 4 * i) : make_float4(1.f, 1.f, 1.f, 1.f);

@@ -27,7 +27,7 @@ using namespace fdattn;
 extern "C" size_t fdattn_decode_workspace_bytes(int batch, int hq, int hkv, int head_dim, int max_blocks_per_seq) {
   if (batch <= 0 || hq <= 0 || hkv <= 0 || head_dim <= 0 || max_blocks_per_seq <= 0) return 256;
   size_t a = generic_workspace_bytes(batch, hq, head_dim);
-  size_t b = c8_workspace_bytes(batch, hkv, max_blocks_per_seq);
+  size_t b = hq % hkv == 0 ? c8_workspace_bytes(batch, hkv, max_blocks_per_seq, hq / hkv) : 0;
   size_t n = a > b ? a : b;
   return (n + 255) & ~(size_t)255;
 }

@@ -1,5 +1,5 @@
-// Decode attention over the int8 / fp8-e4m3 paged cache for head_dim 128, 4 query heads
-// per KV head, block_size 64 - the HBM-bound kernel of the path.
+// Decode attention over the int8 / fp8-e4m3 paged cache for head_dim 128, 1 .. 8 query
+// heads per KV head, block_size 64 - the HBM-bound kernel of the path.
 //
 // Work unit: one (sequence, KV head, cache block) = an 8 KiB K tile + an 8 KiB V tile,
 // each contiguous in HBM.  The block list of every (sequence, KV head) pair is cut into
@@ -21,6 +21,8 @@
 //     products are exact; the limbs are recombined in fp32.
 //   fp8 cache: v_mfma_f32_16x16x32_fp8_fp8 with q*k_scale and the weights split into 4
 //     e4m3 residual limbs (16 significant bits).
+//   Groups of up to 4 query heads use one such set of 16 rows (rows of absent heads are
+//   zero); 5 .. 8 heads use two sets, and every K and V operand read from LDS feeds both.
 // The per-channel K scale is folded into q, the V scale is applied once to the output.
 // V tiles are transposed for free by ds_read_b64_tr_b8.
 // The formats with one scale per stored row (DYN) bring a unit's 64 K scales and 64 V
@@ -54,8 +56,8 @@ struct C8Args {
   const int32_t* kept_blocks;
   const int32_t* kept_counts;
   int max_kept;
-  float* part_o;   // [pairs * chunks_per_pair][4][128]
-  float* part_ml;  // [pairs * chunks_per_pair][8]: m[4] (log2 domain), l[4]
+  float* part_o;   // [pairs * chunks_per_pair][sets * 4][128], sets = ceil(group / 4)
+  float* part_ml;  // [pairs * chunks_per_pair][sets][8]: m[4] (log2 domain), l[4]
   uint16_t* out;
   RowMap rows;  // which sequences are decode rows and where their q / out rows are
   int batch, hkv, max_blocks, num_blocks;
@@ -63,6 +65,7 @@ struct C8Args {
   int chunks_per_pair;  // grid.x
   float sm_scale_log2;  // softmax_scale * log2(e)
   int dyn;              // scales per stored row: the output takes no per-channel V scale
+  int group;            // query heads per KV head, 1 .. 8
 };
 
 // Length of the pair's block list: every block of the sequence, or the kept ones.
@@ -72,11 +75,13 @@ __device__ __forceinline__ int pair_units(const C8Args& a, int p, int kv_len) {
   return min((max(kv_len, 0) + kBS - 1) / kBS, a.max_blocks);
 }
 
-template <int QUANT, bool SPARSE, bool DYN>
+// NSET: row sets of 4 query heads a wavefront carries (1: up to 4 query heads per KV head, 2: up to 8); every K
+// and V operand read from LDS feeds the MFMAs of all sets.
+template <int QUANT, bool SPARSE, bool DYN, int NSET>
 __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
   __shared__ __attribute__((aligned(16))) uint8_t ldsK[kWaves][kTileB];
   __shared__ __attribute__((aligned(16))) uint8_t ldsV[kWaves][kTileB];
-  __shared__ __attribute__((aligned(16))) uint8_t ldsP[kWaves][1024];
+  __shared__ __attribute__((aligned(16))) uint8_t ldsP[kWaves][NSET][1024];
   __shared__ __attribute__((aligned(16))) float ldsS[DYN ? kWaves : 1][2 * kBS];  // DYN: a unit's K scales, V scales
   const int lane = threadIdx.x & 63;
   const int wv = uni(threadIdx.x >> 6);
@@ -107,22 +112,25 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
   }
   int row;
   if (!decode_row(a.rows, b, row)) return;
-  const PairRaw raw = load_pair_issue(a.q, DYN ? nullptr : a.k_scale, a.hkv, p, row, lane);  // in flight with the table entries
+  PairRaw raw[NSET];  // in flight with the table entries
+#pragma unroll
+  for (int t = 0; t < NSET; ++t) raw[t] = load_pair_issue(a.q, DYN ? nullptr : a.k_scale, a.hkv, p, row, lane, a.group, t);
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
   const int n_p = pair_units<SPARSE>(a, p, kv_len);
   const int cnt = min(a.chunk, n_p - first);  // <= 0: past the end of this pair's list
   const bool single = n_p <= a.chunk;
+  // q / out row of query head `head` of this pair
+  auto out_row = [&](int head) { return a.out + ((size_t)row * a.hkv * a.group + h * a.group + head) * kD; };
   if (cnt <= 0) {
     if (n_p == 0 && ck == 0) {  // empty sequence: its output rows are zeros
-      uint16_t* o = a.out + ((size_t)row * a.hkv * kG + h * kG + (threadIdx.x >> 6)) * kD + (threadIdx.x & 63) * 2;
-      *reinterpret_cast<u32*>(o) = 0u;
+      for (int head = threadIdx.x >> 6; head < a.group; head += kWaves)
+        *reinterpret_cast<u32*>(out_row(head) + (threadIdx.x & 63) * 2) = 0u;
     }
     return;
   }
 
   uint8_t* const kbuf = ldsK[wv];
   uint8_t* const vbuf = ldsV[wv];
-  uint8_t* const pbuf = ldsP[wv];
   const u32 kaddr = uni((int)lds_addr_of(kbuf)), vaddr = uni((int)lds_addr_of(vbuf));
   const DmaOffsets offK = dma_offsets<kShiftK>(lane), offV = dma_offsets<kShiftV>(lane);
   const int n16 = lane & 15, g4 = lane >> 4;
@@ -161,18 +169,22 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
     }
   };
 
-  PairState st;
-  st.m = -INFINITY;
-  st.l = 0.f;
+  PairState st[NSET];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) st.o[i] = 0.f;
+  for (int t = 0; t < NSET; ++t) {
+    st[t].m = -INFINITY;
+    st[t].l = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) st[t].o[i] = 0.f;
+  }
 
   if (wv < cnt) {  // this wavefront has units wv, wv + 4, ...
     int pb = unit_pb(wv);
     int valid = unit_valid(wv);
     fetch_k(pb);
     dma_tile(vbase + (size_t)pb * blk_stride, vaddr, offV);
-    load_pair_finish<QUANT>(raw, a.sm_scale_log2, lane, st);
+#pragma unroll
+    for (int t = 0; t < NSET; ++t) load_pair_finish<QUANT>(raw[t], a.sm_scale_log2, lane, st[t]);
 
     for (int j = wv; j < cnt; j += kWaves) {
       const bool has_next = j + kWaves < cnt;
@@ -191,113 +203,122 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
         kt[0] = k4.x; kt[1] = k4.y; kt[2] = k4.z; kt[3] = k4.w;
         vt[0] = v4.x; vt[1] = v4.y; vt[2] = v4.z; vt[3] = v4.w;
       }
-      v4i S[4];
-      v4f Sf[4];
+      v4i S[NSET][4];
+      v4f Sf[NSET][4];
 #pragma unroll
       for (int stl = 0; stl < 4; ++stl) {
         const int tok = 4 * n16 + stl;  // this lane's column of tile stl is token 4n + stl
-        if (QUANT == FDATTN_CACHE_INT8) {
-          v4i acc = {0, 0, 0, 0};
+        v4i kb[2];
 #pragma unroll
-          for (int s = 0; s < 2; ++s) {
-            const int c = g4 + 4 * s;
-            const v4i kb = *reinterpret_cast<const v4i*>(kbuf + tok * 128 + ((c ^ ((tok >> kShiftK) & 7)) * 16));
-            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(st.aq[s], kb, acc, 0, 0, 0);
-          }
-          S[stl] = acc;
-        } else {
-          v4f acc = {0.f, 0.f, 0.f, 0.f};
+        for (int s = 0; s < 2; ++s) {
+          const int c = g4 + 4 * s;
+          kb[s] = *reinterpret_cast<const v4i*>(kbuf + tok * 128 + ((c ^ ((tok >> kShiftK) & 7)) * 16));
+        }
 #pragma unroll
-          for (int s = 0; s < 2; ++s) {
-            const int c = g4 + 4 * s;
-            const v4i kb = *reinterpret_cast<const v4i*>(kbuf + tok * 128 + ((c ^ ((tok >> kShiftK) & 7)) * 16));
-            const long a0 = ((long)(u32)st.aq[s].y << 32) | (u32)st.aq[s].x;
-            const long a1 = ((long)(u32)st.aq[s].w << 32) | (u32)st.aq[s].z;
-            const long b0 = ((long)(u32)kb.y << 32) | (u32)kb.x;
-            const long b1 = ((long)(u32)kb.w << 32) | (u32)kb.z;
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a0, b0, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a1, b1, acc, 0, 0, 0);
+        for (int t = 0; t < NSET; ++t) {
+          if (QUANT == FDATTN_CACHE_INT8) {
+            v4i acc = {0, 0, 0, 0};
+#pragma unroll
+            for (int s = 0; s < 2; ++s) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(st[t].aq[s], kb[s], acc, 0, 0, 0);
+            S[t][stl] = acc;
+          } else {
+            v4f acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+              const long a0 = ((long)(u32)st[t].aq[s].y << 32) | (u32)st[t].aq[s].x;
+              const long a1 = ((long)(u32)st[t].aq[s].w << 32) | (u32)st[t].aq[s].z;
+              const long b0 = ((long)(u32)kb[s].y << 32) | (u32)kb[s].x;
+              const long b1 = ((long)(u32)kb[s].w << 32) | (u32)kb[s].z;
+              acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a0, b0, acc, 0, 0, 0);
+              acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a1, b1, acc, 0, 0, 0);
+            }
+            Sf[t][stl] = acc;
           }
-          Sf[stl] = acc;
         }
       }
       wait_lgkm0();  // K tile (and the scale rows) are in registers: their slots may be refilled
       if (has_next) fetch_k(pbn);
 
-      // ---------------- online softmax in the S layout: lane = (token slot n, head g)
-      float sv[4];
-      float mb = -INFINITY;
+      // ---------------- online softmax in the S layout: lane = (token slot n, head g), one row set at a time
+      float alpha[NSET], vmax[NSET];
 #pragma unroll
-      for (int stl = 0; stl < 4; ++stl) {
-        float s;
-        if (QUANT == FDATTN_CACHE_INT8)
-          s = st.rs * ((float)S[stl].x + 128.0f * (float)S[stl].y + 16384.0f * (float)S[stl].z);
-        else
-          s = st.rs * ((Sf[stl].x + Sf[stl].y) + (Sf[stl].z + Sf[stl].w));
-        if (DYN) s *= kt[stl];
-        s = (4 * n16 + stl < valid) ? s : -INFINITY;  // (a slot past the end may hold any scale, NaN included)
-        sv[stl] = s;
-        mb = fmaxf(mb, s);
-      }
-      mb = row_max16(mb);
-      const float m_new = fmaxf(st.m, mb);
-      // void unit (no valid token) and nothing seen yet: keep everything at zero
-      const float m_use = m_new == -INFINITY ? 0.f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f(st.m - m_use);
-      st.m = m_new;
-      u32 pw[4] = {0, 0, 0, 0};
-      float lsum = 0.f;
-      float prs[4];
-#pragma unroll
-      for (int stl = 0; stl < 4; ++stl) prs[stl] = __builtin_amdgcn_exp2f(sv[stl] - m_use);  // in [0, 1]
-      // DYN: what is cut into limbs is weight x V scale of the token, relative to the largest such product of the
-      // unit (so the unit's heaviest contribution always has full precision); that largest product scales the
-      // unit's P.V.  The weight sum takes the plain weights.
-      float vmax = 1.f;
-      if (DYN) {
-        float wm = 0.f;
+      for (int t = 0; t < NSET; ++t) {
+        float sv[4];
+        float mb = -INFINITY;
 #pragma unroll
         for (int stl = 0; stl < 4; ++stl) {
-          lsum += prs[stl] * (QUANT == FDATTN_CACHE_INT8 ? 268435456.0f : 256.0f);
-          prs[stl] *= (4 * n16 + stl < valid) ? vt[stl] : 0.f;  // (a slot past the end may hold any scale)
-          wm = fmaxf(wm, prs[stl]);
+          float s;
+          if (QUANT == FDATTN_CACHE_INT8)
+            s = st[t].rs * ((float)S[t][stl].x + 128.0f * (float)S[t][stl].y + 16384.0f * (float)S[t][stl].z);
+          else
+            s = st[t].rs * ((Sf[t][stl].x + Sf[t][stl].y) + (Sf[t][stl].z + Sf[t][stl].w));
+          if (DYN) s *= kt[stl];
+          s = (4 * n16 + stl < valid) ? s : -INFINITY;  // (a slot past the end may hold any scale, NaN included)
+          sv[stl] = s;
+          mb = fmaxf(mb, s);
         }
-        vmax = row_max16(wm);
-        // a unit whose heaviest product has all but vanished (its reciprocal would overflow, and 0 x inf is a
-        // NaN) contributes nothing
-        vmax = vmax > 7.9e-31f ? vmax : 0.f;  // 2^-100
-        const float inv = vmax > 0.f ? 1.0f / vmax : 0.f;
+        mb = row_max16(mb);
+        const float m_new = fmaxf(st[t].m, mb);
+        // void unit (no valid token) and nothing seen yet: keep everything at zero
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        alpha[t] = __builtin_amdgcn_exp2f(st[t].m - m_use);
+        st[t].m = m_new;
+        u32 pw[4] = {0, 0, 0, 0};
+        float lsum = 0.f;
+        float prs[4];
 #pragma unroll
-        for (int stl = 0; stl < 4; ++stl) prs[stl] *= inv;
-      }
+        for (int stl = 0; stl < 4; ++stl) prs[stl] = __builtin_amdgcn_exp2f(sv[stl] - m_use);  // in [0, 1]
+        // DYN: what is cut into limbs is weight x V scale of the token, relative to the largest such product of the
+        // unit (so the unit's heaviest contribution always has full precision); that largest product scales the
+        // unit's P.V.  The weight sum takes the plain weights.
+        vmax[t] = 1.f;
+        if (DYN) {
+          float wm = 0.f;
 #pragma unroll
-      for (int stl = 0; stl < 4; ++stl) {
-        const float pr = prs[stl];
-        if (QUANT == FDATTN_CACHE_INT8) {
-          u32 x = (u32)__builtin_rintf(pr * 268435456.0f);  // 2^28
-          x = min(x, 268435455u);
-          if (!DYN) lsum += (float)x;
-          pw[0] |= (x & 127u) << (8 * stl);
-          pw[1] |= ((x >> 7) & 127u) << (8 * stl);
-          pw[2] |= ((x >> 14) & 127u) << (8 * stl);
-          pw[3] |= (x >> 21) << (8 * stl);
-        } else {
-          float x = pr * 256.0f, used = 0.f;
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const u32 c = (u32)__builtin_amdgcn_cvt_pk_fp8_f32(x, x, 0, false) & 0xffu;
-            const float dv = __builtin_amdgcn_cvt_f32_fp8((int)c, 0);
-            pw[t] |= c << (8 * stl);
-            x -= dv;
-            used += dv;
+          for (int stl = 0; stl < 4; ++stl) {
+            lsum += prs[stl] * (QUANT == FDATTN_CACHE_INT8 ? 268435456.0f : 256.0f);
+            prs[stl] *= (4 * n16 + stl < valid) ? vt[stl] : 0.f;  // (a slot past the end may hold any scale)
+            wm = fmaxf(wm, prs[stl]);
           }
-          if (!DYN) lsum += used;
-        }
-      }
-      st.l = st.l * alpha + lsum;
-      // P rows = head*4 + limb, 64 token bytes per row; this lane owns tokens 4n..4n+3
+          float vm = row_max16(wm);
+          // a unit whose heaviest product has all but vanished (its reciprocal would overflow, and 0 x inf is a
+          // NaN) contributes nothing
+          vm = vm > 7.9e-31f ? vm : 0.f;  // 2^-100
+          const float inv = vm > 0.f ? 1.0f / vm : 0.f;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) *reinterpret_cast<u32*>(pbuf + (4 * g4 + r) * 64 + 4 * n16) = pw[r];
+          for (int stl = 0; stl < 4; ++stl) prs[stl] *= inv;
+          vmax[t] = vm;
+        }
+#pragma unroll
+        for (int stl = 0; stl < 4; ++stl) {
+          const float pr = prs[stl];
+          if (QUANT == FDATTN_CACHE_INT8) {
+            u32 x = (u32)__builtin_rintf(pr * 268435456.0f);  // 2^28
+            x = min(x, 268435455u);
+            if (!DYN) lsum += (float)x;
+            pw[0] |= (x & 127u) << (8 * stl);
+            pw[1] |= ((x >> 7) & 127u) << (8 * stl);
+            pw[2] |= ((x >> 14) & 127u) << (8 * stl);
+            pw[3] |= (x >> 21) << (8 * stl);
+          } else {
+            float x = pr * 256.0f, used = 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const u32 c = (u32)__builtin_amdgcn_cvt_pk_fp8_f32(x, x, 0, false) & 0xffu;
+              const float dv = __builtin_amdgcn_cvt_f32_fp8((int)c, 0);
+              pw[e] |= c << (8 * stl);
+              x -= dv;
+              used += dv;
+            }
+            if (!DYN) lsum += used;
+          }
+        }
+        st[t].l = st[t].l * alpha[t] + lsum;
+        // P rows = head*4 + limb, 64 token bytes per row; this lane owns tokens 4n..4n+3
+        uint8_t* const pbuf = ldsP[wv][t];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) *reinterpret_cast<u32*>(pbuf + (4 * g4 + r) * 64 + 4 * n16) = pw[r];
+      }
       wave_sync();
 
       // ---------------- O += P V : V^T operands come transposed out of LDS
@@ -309,7 +330,9 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
           *reinterpret_cast<uint4*>(vbuf + r * 128 + (lane & 7) * 16) = make_uint4(0, 0, 0, 0);
         wave_sync();
       }
-      const v4i pa = *reinterpret_cast<const v4i*>(pbuf + n16 * 64 + 16 * g4);
+      v4i pa[NSET];
+#pragma unroll
+      for (int t = 0; t < NSET; ++t) pa[t] = *reinterpret_cast<const v4i*>(ldsP[wv][t] + n16 * 64 + 16 * g4);
 #pragma unroll
       for (int ct = 0; ct < 8; ++ct) {
         v2i vr[2];
@@ -319,21 +342,24 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
           const uint8_t* src = vbuf + tok * 128 + ((ct ^ ((tok >> kShiftV) & 7)) * 16) + 8 * (n16 & 1);
           vr[r] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i*)src);
         }
-        float ob;
-        if (QUANT == FDATTN_CACHE_INT8) {
-          const v4i vb = {vr[0].x, vr[0].y, vr[1].x, vr[1].y};
-          const v4i z = {0, 0, 0, 0};
-          const v4i d = __builtin_amdgcn_mfma_i32_16x16x64_i8(pa, vb, z, 0, 0, 0);
-          ob = (float)d.x + 128.0f * (float)d.y + 16384.0f * (float)d.z + 2097152.0f * (float)d.w;
-        } else {
-          v4f d = {0.f, 0.f, 0.f, 0.f};
-          const long a0 = ((long)(u32)pa.y << 32) | (u32)pa.x, a1 = ((long)(u32)pa.w << 32) | (u32)pa.z;
-          const long b0 = ((long)(u32)vr[0].y << 32) | (u32)vr[0].x, b1 = ((long)(u32)vr[1].y << 32) | (u32)vr[1].x;
-          d = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a0, b0, d, 0, 0, 0);
-          d = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a1, b1, d, 0, 0, 0);
-          ob = (d.x + d.y) + (d.z + d.w);
+#pragma unroll
+        for (int t = 0; t < NSET; ++t) {
+          float ob;
+          if (QUANT == FDATTN_CACHE_INT8) {
+            const v4i vb = {vr[0].x, vr[0].y, vr[1].x, vr[1].y};
+            const v4i z = {0, 0, 0, 0};
+            const v4i d = __builtin_amdgcn_mfma_i32_16x16x64_i8(pa[t], vb, z, 0, 0, 0);
+            ob = (float)d.x + 128.0f * (float)d.y + 16384.0f * (float)d.z + 2097152.0f * (float)d.w;
+          } else {
+            v4f d = {0.f, 0.f, 0.f, 0.f};
+            const long a0 = ((long)(u32)pa[t].y << 32) | (u32)pa[t].x, a1 = ((long)(u32)pa[t].w << 32) | (u32)pa[t].z;
+            const long b0 = ((long)(u32)vr[0].y << 32) | (u32)vr[0].x, b1 = ((long)(u32)vr[1].y << 32) | (u32)vr[1].x;
+            d = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a0, b0, d, 0, 0, 0);
+            d = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a1, b1, d, 0, 0, 0);
+            ob = (d.x + d.y) + (d.z + d.w);
+          }
+          st[t].o[ct] = st[t].o[ct] * alpha[t] + (DYN ? ob * vmax[t] : ob);
         }
-        st.o[ct] = st.o[ct] * alpha + (DYN ? ob * vmax : ob);
       }
       wait_lgkm0();  // V tile consumed
       if (has_next) dma_tile(vbase + (size_t)pbn * blk_stride, vaddr, offV);
@@ -343,33 +369,39 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
     }
   }
 
-  // ---- merge the 4 wavefronts through LDS (their K slots are free now)
+  // ---- merge the 4 wavefronts through LDS (their K slots are free now): [set][4 heads][128] floats of this
+  // wavefront in its K slot, m[4], l[4] per set in its P slots
   {
-    float* const mo = reinterpret_cast<float*>(kbuf);  // [4 heads][128] of this wavefront
-    float* const mml = reinterpret_cast<float*>(pbuf);  // m[4], l[4]
-    const float l = row_sum16(st.l);
+    float* const mo = reinterpret_cast<float*>(kbuf);
 #pragma unroll
-    for (int ct = 0; ct < 8; ++ct) mo[g4 * kD + 16 * ct + n16] = st.o[ct];
-    if (n16 == 0) {
-      mml[g4] = st.m;
-      mml[4 + g4] = l;
+    for (int t = 0; t < NSET; ++t) {
+      float* const mml = reinterpret_cast<float*>(ldsP[wv][t]);
+      const float l = row_sum16(st[t].l);
+#pragma unroll
+      for (int ct = 0; ct < 8; ++ct) mo[t * kSlotFloats + g4 * kD + 16 * ct + n16] = st[t].o[ct];
+      if (n16 == 0) {
+        mml[g4] = st[t].m;
+        mml[4 + g4] = l;
+      }
     }
   }
   __syncthreads();
-  {
-    const int tid = threadIdx.x, head = tid >> 6, c2 = (tid & 63) * 2;
+#pragma unroll
+  for (int t = 0; t < NSET; ++t) {
+    const int tid = threadIdx.x, hs = tid >> 6, head = 4 * t + hs, c2 = (tid & 63) * 2;
+    if (head >= a.group) continue;
     float M = -INFINITY;
 #pragma unroll
-    for (int w2 = 0; w2 < kWaves; ++w2) M = fmaxf(M, reinterpret_cast<const float*>(ldsP[w2])[head]);
+    for (int w2 = 0; w2 < kWaves; ++w2) M = fmaxf(M, reinterpret_cast<const float*>(ldsP[w2][t])[hs]);
     float L = 0.f, o0 = 0.f, o1 = 0.f;
     if (M > -INFINITY) {
 #pragma unroll
       for (int w2 = 0; w2 < kWaves; ++w2) {
-        const float* ml = reinterpret_cast<const float*>(ldsP[w2]);
-        const float ms = ml[head];
+        const float* ml = reinterpret_cast<const float*>(ldsP[w2][t]);
+        const float ms = ml[hs];
         const float f = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - M);
-        L += ml[4 + head] * f;
-        const float2 v = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(ldsK[w2]) + head * kD + c2);
+        L += ml[4 + hs] * f;
+        const float2 v = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(ldsK[w2]) + t * kSlotFloats + hs * kD + c2);
         o0 += v.x * f;
         o1 += v.y * f;
       }
@@ -378,14 +410,14 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
       // the only chunk of this pair: finish here
       const float inv = L > 0.f ? 1.0f / L : 0.f;
       const float r0 = o0 * inv * (DYN ? 1.f : a.v_scale[h * kD + c2]), r1 = o1 * inv * (DYN ? 1.f : a.v_scale[h * kD + c2 + 1]);
-      uint16_t* o = a.out + ((size_t)row * a.hkv * kG + h * kG + head) * kD + c2;
-      *reinterpret_cast<u32*>(o) = (u32)f32_to_bf16(r0) | ((u32)f32_to_bf16(r1) << 16);
+      *reinterpret_cast<u32*>(out_row(head) + c2) = (u32)f32_to_bf16(r0) | ((u32)f32_to_bf16(r1) << 16);
     } else {
+      // partial of (pair, chunk): o [sets * 4 heads][128], then m[4], l[4] per set
       const size_t slot = (size_t)p * a.chunks_per_pair + ck;
-      *reinterpret_cast<float2*>(a.part_o + slot * kSlotFloats + head * kD + c2) = make_float2(o0, o1);
+      *reinterpret_cast<float2*>(a.part_o + slot * (NSET * kSlotFloats) + head * kD + c2) = make_float2(o0, o1);
       if ((tid & 63) == 0) {
-        a.part_ml[slot * 8 + head] = M;
-        a.part_ml[slot * 8 + 4 + head] = L;
+        a.part_ml[slot * (NSET * 8) + t * 8 + hs] = M;
+        a.part_ml[slot * (NSET * 8) + t * 8 + 4 + hs] = L;
       }
     }
   }
@@ -398,8 +430,9 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
 template <bool SPARSE>
 __global__ __launch_bounds__(256) void decode_c8_combine_kernel(C8Args a) {
   __shared__ float red[kWaves][2 + 2 * 64];  // per wavefront: m, l, o[64][2]
-  const int p = blockIdx.x >> 2, head = blockIdx.x & 3, tid = threadIdx.x;
+  const int p = blockIdx.x / a.group, head = blockIdx.x - p * a.group, tid = threadIdx.x;
   const int b = p / a.hkv, h = p - b * a.hkv;
+  const int sets = (a.group + kG - 1) / kG, set = head >> 2, hs = head & 3;  // the partial's layout: see the main kernel
   int row;
   if (!decode_row(a.rows, b, row)) return;
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
@@ -418,9 +451,9 @@ __global__ __launch_bounds__(256) void decode_c8_combine_kernel(C8Args a) {
       const int c = c0 + k * kWaves;
       ms[k] = -INFINITY, ls[k] = 0.f, v[k] = make_float2(0.f, 0.f);
       if (c < nch) {
-        ms[k] = a.part_ml[(s0 + c) * 8 + head];
-        ls[k] = a.part_ml[(s0 + c) * 8 + 4 + head];
-        v[k] = *reinterpret_cast<const float2*>(a.part_o + (s0 + c) * kSlotFloats + head * kD + c2);
+        ms[k] = a.part_ml[(s0 + c) * (sets * 8) + set * 8 + hs];
+        ls[k] = a.part_ml[(s0 + c) * (sets * 8) + set * 8 + 4 + hs];
+        v[k] = *reinterpret_cast<const float2*>(a.part_o + (s0 + c) * (sets * kSlotFloats) + head * kD + c2);
       }
     }
     float m_new = M;
@@ -459,7 +492,7 @@ __global__ __launch_bounds__(256) void decode_c8_combine_kernel(C8Args a) {
   const float inv = Lt > 0.f ? 1.0f / Lt : 0.f;
   r0 *= inv * (a.dyn ? 1.f : a.v_scale[h * kD + c2]);
   r1 *= inv * (a.dyn ? 1.f : a.v_scale[h * kD + c2 + 1]);
-  uint16_t* o = a.out + ((size_t)row * a.hkv * kG + h * kG + head) * kD + c2;
+  uint16_t* o = a.out + ((size_t)row * a.hkv * a.group + h * a.group + head) * kD + c2;
   *reinterpret_cast<u32*>(o) = (u32)f32_to_bf16(r0) | ((u32)f32_to_bf16(r1) << 16);
 }
 
@@ -493,16 +526,35 @@ int c8_pick_chunk(int pairs, int max_units) {
 
 constexpr int kMaxPairs = 1 << 20;
 
-size_t c8_workspace_bytes(int batch, int hkv, int max_units) {
+size_t c8_workspace_bytes(int batch, int hkv, int max_units, int group) {
   const int pairs = batch * hkv;
   const int chunk = c8_pick_chunk(pairs, max_units);
   const size_t slots = (size_t)pairs * ((max_units + chunk - 1) / chunk);
-  return slots * (kSlotFloats + 8) * sizeof(float);
+  const int sets = (group + kG - 1) / kG;
+  return slots * sets * (kSlotFloats + 8) * sizeof(float);
 }
 
 bool c8_supported(int hq, int hkv, int d, int bs, int quant) {
-  return d == kD && hq == kG * hkv && bs == kBS && quant_known(quant);
+  return d == kD && hkv > 0 && hq % hkv == 0 && hq / hkv >= 1 && hq / hkv <= kG * kMaxSets && bs == kBS && quant_known(quant);
 }
+
+namespace {
+
+template <int QUANT, bool DYN, int NSET>
+void launch_main(bool sparse, dim3 grid, dim3 block, hipStream_t s, const C8Args& a) {
+  if (sparse) hipLaunchKernelGGL((decode_c8_kernel<QUANT, true, DYN, NSET>), grid, block, 0, s, a);
+  else hipLaunchKernelGGL((decode_c8_kernel<QUANT, false, DYN, NSET>), grid, block, 0, s, a);
+}
+
+template <int NSET>
+void launch_main_sets(int quant, bool sparse, dim3 grid, dim3 block, hipStream_t s, const C8Args& a) {
+  if (quant == FDATTN_CACHE_INT8) launch_main<FDATTN_CACHE_INT8, false, NSET>(sparse, grid, block, s, a);
+  else if (quant == FDATTN_CACHE_FP8_E4M3) launch_main<FDATTN_CACHE_FP8_E4M3, false, NSET>(sparse, grid, block, s, a);
+  else if (quant == FDATTN_CACHE_INT8_DYNAMIC) launch_main<FDATTN_CACHE_INT8, true, NSET>(sparse, grid, block, s, a);
+  else launch_main<FDATTN_CACHE_FP8_E4M3, true, NSET>(sparse, grid, block, s, a);
+}
+
+}  // namespace
 
 int decode_c8_launch(const void* q, const void* key_cache, const void* value_cache, const float* k_scale,
                      const float* v_scale, const int32_t* block_tables, const int32_t* seq_lens_decoder,
@@ -510,46 +562,36 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
                      int max_kept, void* out, void* workspace, size_t workspace_bytes, int batch, int hq,
                      int hkv, int d, int bs, int max_blocks, int num_blocks, int quant, float sm_scale,
                      hipStream_t s, int stages, RowMap rows) {
-  (void)hq; (void)d; (void)bs;
+  (void)d; (void)bs;
   const bool sparse = kept_blocks != nullptr;
-  const int pairs = batch * hkv;
+  const int pairs = batch * hkv, group = hq / hkv, sets = (group + kG - 1) / kG;
   const int max_units = sparse ? (max_kept < max_blocks ? max_kept : max_blocks) : max_blocks;
   const int chunk = c8_pick_chunk(pairs, max_units);
   const int cpp = ((max_units + chunk - 1) / chunk);
   if (pairs > kMaxPairs)
     return fail(FDATTN_ERR_SHAPE, "fdattn_decode_attention: batch*kv_heads = %d exceeds %d", pairs, kMaxPairs);
-  if ((long long)pairs * (cpp > kG ? cpp : kG) > 0x7fffffffLL)
+  if ((long long)pairs * (cpp > group ? cpp : group) > 0x7fffffffLL)
     return fail(FDATTN_ERR_SHAPE, "fdattn_decode_attention: %d pairs x %d chunks exceed the grid limit", pairs, cpp);
   const size_t slots = (size_t)pairs * cpp;
-  const size_t need = slots * (kSlotFloats + 8) * sizeof(float);
+  const size_t need = slots * sets * (kSlotFloats + 8) * sizeof(float);
   if (workspace_bytes < need)
     return fail(FDATTN_ERR_WORKSPACE, "fdattn_decode_attention: workspace %zu B < required %zu B", workspace_bytes, need);
   float* part_o = (float*)workspace;
-  float* part_ml = part_o + slots * kSlotFloats;
+  float* part_ml = part_o + slots * sets * kSlotFloats;
   C8Args a{(const uint16_t*)q, (const uint8_t*)key_cache, (const uint8_t*)value_cache, k_scale, v_scale,
            block_tables, seq_lens_decoder, seq_lens_this_time, kept_blocks, kept_counts, max_kept, part_o,
            part_ml, (uint16_t*)out, rows, batch, hkv, max_blocks, num_blocks, chunk, cpp,
-           sm_scale * 1.4426950408889634f, quant_dynamic(quant) ? 1 : 0};
+           sm_scale * 1.4426950408889634f, quant_dynamic(quant) ? 1 : 0, group};
   const dim3 grid(cpp * pairs), block(kWaves * 64);
-  if (!(stages & 1)) {
-  } else if (quant == FDATTN_CACHE_INT8) {
-    if (sparse) hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_INT8, true, false>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_INT8, false, false>), grid, block, 0, s, a);
-  } else if (quant == FDATTN_CACHE_FP8_E4M3) {
-    if (sparse) hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_FP8_E4M3, true, false>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_FP8_E4M3, false, false>), grid, block, 0, s, a);
-  } else if (quant == FDATTN_CACHE_INT8_DYNAMIC) {
-    if (sparse) hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_INT8, true, true>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_INT8, false, true>), grid, block, 0, s, a);
-  } else {
-    if (sparse) hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_FP8_E4M3, true, true>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((decode_c8_kernel<FDATTN_CACHE_FP8_E4M3, false, true>), grid, block, 0, s, a);
+  if (stages & 1) {
+    if (sets == 1) launch_main_sets<1>(quant, sparse, grid, block, s, a);
+    else launch_main_sets<2>(quant, sparse, grid, block, s, a);
   }
   int rc = check_launch("fdattn_decode_attention (mfma)");
   if (rc || !(stages & 2)) return rc;
   if (cpp == 1) return 0;  // every pair was one chunk and has been finished by the main kernel
-  if (sparse) hipLaunchKernelGGL(decode_c8_combine_kernel<true>, dim3(pairs * kG), dim3(256), 0, s, a);
-  else hipLaunchKernelGGL(decode_c8_combine_kernel<false>, dim3(pairs * kG), dim3(256), 0, s, a);
+  if (sparse) hipLaunchKernelGGL(decode_c8_combine_kernel<true>, dim3(pairs * group), dim3(256), 0, s, a);
+  else hipLaunchKernelGGL(decode_c8_combine_kernel<false>, dim3(pairs * group), dim3(256), 0, s, a);
   return check_launch("fdattn_decode_attention (merge)");
 }
 

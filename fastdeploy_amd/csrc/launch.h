@@ -18,7 +18,7 @@ int gpu_cu_count();
 // units (cache blocks) per workgroup for `pairs` block lists of at most max_units blocks: as few chunks per
 // list as fill the GPU's workgroup slots once, at most kMaxChunk units each
 int c8_pick_chunk(int pairs, int max_units);
-size_t c8_workspace_bytes(int batch, int hkv, int max_units);
+size_t c8_workspace_bytes(int batch, int hkv, int max_units, int group = 4);
 bool c8_supported(int hq, int hkv, int d, int bs, int quant);
 // stages: 1 = the split-KV kernel, 2 = the merge of its partials, 3 = both
 int decode_c8_launch(const void* q, const void* key_cache, const void* value_cache,

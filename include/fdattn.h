@@ -179,7 +179,7 @@ FDATTN_API int fdattn_decode_attention(
 
 /*
  * 1 if fdattn_decode_attention(_sparse) runs these shapes on the MFMA kernel (head_dim
- * 128, hq/hkv 4, block_size 64, either cache type), 0 if on the shape-agnostic one.
+ * 128, hq/hkv from 1 to 8, block_size 64, any cache format), 0 if on the shape-agnostic one.
  */
 FDATTN_API int fdattn_decode_uses_mfma(int hq, int hkv, int head_dim, int block_size, int cache_quant_type);
 

@@ -114,6 +114,43 @@ def test_decode_dynamic_formats_with_vanishing_units(oracle, quant):
     check(got, want, "vanishing units")
 
 
+@pytest.mark.parametrize("quant", ALL_FORMATS)
+@pytest.mark.parametrize("group", [1, 2, 3, 5, 7, 8])
+def test_decode_other_group_sizes_on_the_mfma_kernel(oracle, group, quant):
+    """1 .. 8 query heads per KV head (head_dim 128, block 64) run on the MFMA kernel: groups up to 4 in one set of
+    MFMA rows with the unused head rows zero, 5 .. 8 in two sets sharing every K / V operand.  Ragged lengths, a
+    multi-chunk launch (partials + merge kernel) and a sparse call, each against the oracle."""
+    hkv = 4
+    hq = group * hkv
+    assert fd.decode_uses_mfma(hq, hkv, 128, 64, quant)
+    lens = [1, 63, 64, 65, 700, 0, 1500, 31]
+    case = syn.decode_case(batch=len(lens), ctx=lens, quant=quant, seed=30 + group, extra_blocks=3, hq=hq, hkv=hkv)
+    got, want = gpu_decode(case), oracle_decode(oracle, case)
+    check(got, want, "group %d ragged" % group)
+    assert not got.reshape(len(lens), -1)[5].any()
+    # few long sequences: several chunks per list
+    case = syn.decode_case(batch=2, ctx=[64 * 150 - 3, 64 * 90], quant=quant, seed=40 + group, hq=hq, hkv=hkv,
+                           direct_bytes=True)
+    from fastdeploy_amd import _lib
+    assert _lib.lib().fdattn_decode_chunks_per_sequence(2, hkv, 150) > 1
+    check(gpu_decode(case), oracle_decode(oracle, case), "group %d chunks" % group)
+    # sparse
+    rng = np.random.default_rng(group)
+    kept = np.full((2, hkv, 9), -1, np.int32)
+    cnt = np.zeros((2, hkv), np.int32)
+    for b, nb in enumerate((150, 90)):
+        for h in range(hkv):
+            k = int(rng.integers(1, 10))
+            kept[b, h, :k] = np.sort(rng.choice(nb, k, replace=False))
+            cnt[b, h] = k
+    dev = syn.to_device(case, "cuda")
+    out = fd.decode_attention_sparse(dev["q"], dev["key_cache"], dev["value_cache"], dev["cache_k_scale"],
+                                     dev["cache_v_scale"], dev["block_tables"], dev["seq_lens_decoder"],
+                                     kept_blocks=torch.from_numpy(kept).cuda(), kept_counts=torch.from_numpy(cnt).cuda(),
+                                     num_heads=hq, cache_quant_type=quant)
+    check(bits(out), oracle_decode(oracle, case, kept_blocks=kept, kept_counts=cnt), "group %d sparse" % group)
+
+
 def test_decode_generic_other_shapes(oracle):
     """Shapes outside the MFMA kernel: head_dim 64, group 2, block_size 16."""
     case = syn.decode_case(batch=3, ctx=[50, 200, 333], seed=8, hq=8, hkv=4, d=64, bs=16)
