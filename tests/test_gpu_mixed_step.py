@@ -223,6 +223,26 @@ def test_mixed_step_other_shape_runs_on_the_generic_kernels(oracle):
     assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
 
 
+@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8_DYNAMIC])
+@pytest.mark.parametrize("group", [2, 8])
+def test_mixed_step_other_group_sizes(oracle, group, quant):
+    """2 and 8 query heads per KV head (head_dim 128, block 64): the whole step stays on the MFMA kernels."""
+    hkv = 4
+    hq = group * hkv
+    c = mixed_case([0, 150, 0, 0, 70, 1], [700, 0, 63, 200, 129, 0], quant, seed=40 + group, hq=hq, hkv=hkv)
+    dev = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
+    out = fd.append_attention(dev["qkv"], dev["key_cache"], dev["value_cache"], dev["seq_lens_encoder"],
+                              dev["seq_lens_decoder"], dev["seq_lens_this_time"], dev["block_tables"],
+                              (dev["rope_cos"], dev["rope_sin"]), dev["cache_k_scale"], dev["cache_v_scale"],
+                              num_heads=hq, kv_num_heads=hkv, max_chunk=150, cache_quant_type=quant,
+                              cu_seqlens_q=dev["cu_seqlens_q"])
+    torch.cuda.synchronize()
+    want, kc, vc = oracle_step(oracle, c, quant, hq, hkv, 128)
+    assert np.array_equal(np_of(dev["key_cache"]), kc) and np.array_equal(np_of(dev["value_cache"]), vc)
+    ok, mx, bad = bf16_close(bits(out), want)
+    assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
+
+
 def test_steps_over_block_pool_tables_with_a_shared_prefix(oracle):
     """Two steps driven by the block pool's tables: a prompt is prefilled, a second sequence forks its
     whole blocks and prefills only its own tail while the first decodes and a third arrives.  Every step is
