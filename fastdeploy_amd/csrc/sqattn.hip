@@ -10,7 +10,7 @@
 //
 // Two implementations give the same indices:
 //  * exact: every block scored in fp64, one token per lane (any shape; fp64-VALU bound);
-//  * fast (head_dim 128, 4 query heads per KV head, block_size 64): every block scored on
+//  * fast (head_dim 128, up to 8 query heads per KV head, block_size 64): every block scored on
 //    the MFMA units straight from the cache bytes (the streaming machinery of the decode
 //    kernel, K tiles only - HBM bound), together with a bound eps on the error of those
 //    scores.  The top-k kernel then classifies each block as surely kept (fewer than k
@@ -167,12 +167,14 @@ struct SelArgs {
   int32_t* kept_blocks;
   int32_t* kept_counts;
   int batch, hkv, max_blocks, num_blocks, chunk, chunks_per_pair, top_k;
+  int group;  // query heads per KV head, 1 .. 8
 };
 
 // One workgroup = `chunk` consecutive blocks of one (sequence, KV head); each wavefront
 // streams blocks wave, wave+4, ... through two LDS slots (one tile computing, one or two
 // in flight) and leaves one fp32 score per block.
-template <int QUANT, bool DYN>
+// NSET: sets of 4 query heads (MFMA rows), as in the decode kernel: 1 for groups up to 4, 2 for 5 .. 8.
+template <int QUANT, bool DYN, int NSET>
 __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelArgs a) {
   __shared__ __attribute__((aligned(16))) uint8_t ldsK[kWaves][2][kTileB];  // two K slots per wavefront
   __shared__ __attribute__((aligned(16))) float ldsS[DYN ? kWaves : 1][2][kBS];  // DYN: the slots' scale rows
@@ -192,7 +194,9 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
     const int u = lane + 64 * e;
     if (u < a.chunk && first + u < a.max_blocks) pb_raw[e] = a.block_tables[(size_t)b * a.max_blocks + first + u];
   }
-  const PairRaw raw = load_pair_issue(a.q, DYN ? nullptr : a.k_scale, a.hkv, p, b, lane);
+  PairRaw raw[NSET];
+#pragma unroll
+  for (int t = 0; t < NSET; ++t) raw[t] = load_pair_issue(a.q, DYN ? nullptr : a.k_scale, a.hkv, p, b, lane, a.group, t);
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
   const int n_p = min((max(kv_len, 0) + kBS - 1) / kBS, a.max_blocks);
   const int cnt = min(a.chunk, n_p - first);
@@ -238,10 +242,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
     // error bound of the MFMA scores of this pair (see the top of the file): q*scale is cut to
     // 21 bits (int8) or 16 significant bits in e4m3 limbs (fp8), and sums are kept in fp32
     float amax = 0.f, sabs = 0.f;
-    for (int g = 0; g < kG; ++g) {
+    for (int g = 0; g < a.group; ++g) {
       float sa = 0.f, am = 0.f;
       for (int c = lane; c < kD; c += 64) {
-        const float qs = fabsf(bf16_to_f32(a.q[((size_t)b * a.hkv * kG + h * kG + g) * kD + c]) * (DYN ? 1.0f : a.k_scale[h * kD + c]));
+        const float qs = fabsf(bf16_to_f32(a.q[((size_t)b * a.hkv * a.group + h * a.group + g) * kD + c]) * (DYN ? 1.0f : a.k_scale[h * kD + c]));
         sa += qs;
         am = fmaxf(am, qs);
       }
@@ -262,30 +266,35 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
   }
 
   if (wv >= cnt) return;
-  PairState st;
-  float qs[2][16];
-  load_pair_finish<QUANT>(raw, 1.0f, lane, st, qs);  // scores in natural units
+  PairState st[NSET];
   // fp8: a second operand, |q*scale| in one e4m3 limb, gives sum_c |q*scale||k| per token next to the score;
   // the error of a block's score is a small multiple of that sum (see the bound below)
-  v4i aabs[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
-  float amax_pair = 0.f;
-  if (QUANT != FDATTN_CACHE_INT8) {
-    const int m = lane & 15, head = m >> 2, limb = m & 3;
-    // st.rs = amax / 256 of this lane's S-layout head; the A layout wants the head of row m
-    const float rs_row = __shfl(st.rs, 16 * head, 64);
-    const float inv = rs_row > 0.f ? 1.0f / rs_row : 0.f;
+  v4i aabs[NSET][2];
+  float amax_pair = 0.f;  // largest |q*scale| over the channels of the pair's heads
 #pragma unroll
-    for (int k2 = 0; k2 < 2; ++k2) {
-      u32 pk[4] = {0, 0, 0, 0};
+  for (int t = 0; t < NSET; ++t) {
+    float qs[2][16];
+    load_pair_finish<QUANT>(raw[t], 1.0f, lane, st[t], qs);  // scores in natural units
+    aabs[t][0] = aabs[t][1] = (v4i){0, 0, 0, 0};
+    if (QUANT != FDATTN_CACHE_INT8) {
+      const int m = lane & 15, head = m >> 2, limb = m & 3;
+      // st.rs = amax / 256 of this lane's S-layout head; the A layout wants the head of row m
+      const float rs_row = __shfl(st[t].rs, 16 * head, 64);
+      const float inv = rs_row > 0.f ? 1.0f / rs_row : 0.f;
 #pragma unroll
-      for (int jj = 0; jj < 16; ++jj) {
-        const float x = fabsf(qs[k2][jj]) * inv;
-        const u32 code = limb == 0 ? ((u32)__builtin_amdgcn_cvt_pk_fp8_f32(x, x, 0, false) & 0xffu) : 0u;
-        pk[jj >> 2] |= code << (8 * (jj & 3));
+      for (int k2 = 0; k2 < 2; ++k2) {
+        u32 pk[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int jj = 0; jj < 16; ++jj) {
+          const float x = fabsf(qs[k2][jj]) * inv;
+          const u32 code = limb == 0 ? ((u32)__builtin_amdgcn_cvt_pk_fp8_f32(x, x, 0, false) & 0xffu) : 0u;
+          pk[jj >> 2] |= code << (8 * (jj & 3));
+        }
+        aabs[t][k2] = (v4i){(int)pk[0], (int)pk[1], (int)pk[2], (int)pk[3]};
       }
-      aabs[k2] = (v4i){(int)pk[0], (int)pk[1], (int)pk[2], (int)pk[3]};
     }
-    amax_pair = fmaxf(fmaxf(__shfl(st.rs, 0, 64), __shfl(st.rs, 16, 64)), fmaxf(__shfl(st.rs, 32, 64), __shfl(st.rs, 48, 64))) * 256.0f;
+    const float rs_max = fmaxf(fmaxf(__shfl(st[t].rs, 0, 64), __shfl(st[t].rs, 16, 64)), fmaxf(__shfl(st[t].rs, 32, 64), __shfl(st[t].rs, 48, 64)));
+    amax_pair = fmaxf(amax_pair, rs_max * (QUANT == FDATTN_CACHE_INT8 ? 1048575.0f : 256.0f));
   }
 
   int it = 0;
@@ -308,39 +317,43 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
 #pragma unroll
     for (int stl = 0; stl < 4; ++stl) {
       const int tok = 4 * n16 + stl;
-      float s;
-      if (QUANT == FDATTN_CACHE_INT8) {
-        v4i acc = {0, 0, 0, 0};
+      v4i kb[2];
 #pragma unroll
-        for (int k2 = 0; k2 < 2; ++k2) {
-          const int c = g4 + 4 * k2;
-          const v4i kb = *reinterpret_cast<const v4i*>(kbuf + tok * 128 + ((c ^ ((tok >> kShiftK) & 7)) * 16));
-          acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(st.aq[k2], kb, acc, 0, 0, 0);
-        }
-        s = st.rs * ((float)acc.x + 128.0f * (float)acc.y + 16384.0f * (float)acc.z);
-        if (DYN) s *= kt[stl];
-      } else {
-        v4f acc = {0.f, 0.f, 0.f, 0.f}, ab = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int k2 = 0; k2 < 2; ++k2) {
-          const int c = g4 + 4 * k2;
-          const v4i kb = *reinterpret_cast<const v4i*>(kbuf + tok * 128 + ((c ^ ((tok >> kShiftK) & 7)) * 16));
-          const long a0 = ((long)(u32)st.aq[k2].y << 32) | (u32)st.aq[k2].x;
-          const long a1 = ((long)(u32)st.aq[k2].w << 32) | (u32)st.aq[k2].z;
-          const long b0 = ((long)(u32)kb.y << 32) | (u32)kb.x;
-          const long b1 = ((long)(u32)kb.w << 32) | (u32)kb.z;
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a0, b0, acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a1, b1, acc, 0, 0, 0);
-          const long m0 = ((long)(u32)aabs[k2].y << 32) | (u32)aabs[k2].x;
-          const long m1 = ((long)(u32)aabs[k2].w << 32) | (u32)aabs[k2].z;
-          ab = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(m0, b0 & 0x7f7f7f7f7f7f7f7fL, ab, 0, 0, 0);
-          ab = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(m1, b1 & 0x7f7f7f7f7f7f7f7fL, ab, 0, 0, 0);
-        }
-        s = st.rs * ((acc.x + acc.y) + (acc.z + acc.w));
-        if (DYN) s *= kt[stl];
-        bv = fmaxf(bv, tok < valid ? st.rs * ab.x * (DYN ? fabsf(kt[stl]) : 1.0f) : 0.f);
+      for (int k2 = 0; k2 < 2; ++k2) {
+        const int c = g4 + 4 * k2;
+        kb[k2] = *reinterpret_cast<const v4i*>(kbuf + tok * 128 + ((c ^ ((tok >> kShiftK) & 7)) * 16));
       }
-      sv = fmaxf(sv, tok < valid ? s : -INFINITY);
+#pragma unroll
+      for (int t = 0; t < NSET; ++t) {
+        const bool live = tok < valid && 4 * t + g4 < a.group;  // (rows of heads past the group are zero, not scores)
+        float s;
+        if (QUANT == FDATTN_CACHE_INT8) {
+          v4i acc = {0, 0, 0, 0};
+#pragma unroll
+          for (int k2 = 0; k2 < 2; ++k2) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(st[t].aq[k2], kb[k2], acc, 0, 0, 0);
+          s = st[t].rs * ((float)acc.x + 128.0f * (float)acc.y + 16384.0f * (float)acc.z);
+          if (DYN) s *= kt[stl];
+        } else {
+          v4f acc = {0.f, 0.f, 0.f, 0.f}, ab = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int k2 = 0; k2 < 2; ++k2) {
+            const long a0 = ((long)(u32)st[t].aq[k2].y << 32) | (u32)st[t].aq[k2].x;
+            const long a1 = ((long)(u32)st[t].aq[k2].w << 32) | (u32)st[t].aq[k2].z;
+            const long b0 = ((long)(u32)kb[k2].y << 32) | (u32)kb[k2].x;
+            const long b1 = ((long)(u32)kb[k2].w << 32) | (u32)kb[k2].z;
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a0, b0, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a1, b1, acc, 0, 0, 0);
+            const long m0 = ((long)(u32)aabs[t][k2].y << 32) | (u32)aabs[t][k2].x;
+            const long m1 = ((long)(u32)aabs[t][k2].w << 32) | (u32)aabs[t][k2].z;
+            ab = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(m0, b0 & 0x7f7f7f7f7f7f7f7fL, ab, 0, 0, 0);
+            ab = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(m1, b1 & 0x7f7f7f7f7f7f7f7fL, ab, 0, 0, 0);
+          }
+          s = st[t].rs * ((acc.x + acc.y) + (acc.z + acc.w));
+          if (DYN) s *= kt[stl];
+          bv = fmaxf(bv, live ? st[t].rs * ab.x * (DYN ? fabsf(kt[stl]) : 1.0f) : 0.f);
+        }
+        sv = fmaxf(sv, live ? s : -INFINITY);
+      }
     }
     wait_lgkm0();  // tile consumed: refill its slot with the block two steps ahead
     if (j + 2 * kWaves < cnt) fetch(unit_pb(j + 2 * kWaves), it & 1);
@@ -361,8 +374,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
     if (DYN && QUANT == FDATTN_CACHE_INT8) {
       // the per-channel format's bound for this pair (from q alone) times the block's largest row scale, plus
       // the rounding of the product with the row scale: 2^-24 of |score| <= 128 * 127 * amax * scale
-      const float amax_q = fmaxf(fmaxf(__shfl(st.rs, 0, 64), __shfl(st.rs, 16, 64)), fmaxf(__shfl(st.rs, 32, 64), __shfl(st.rs, 48, 64))) * 1048575.0f;
-      bv = amax_q * ktmax * (((128.0f * 127.0f * 0.5f + 2048.0f) / 1048575.0f) * 1.0001f + 128.0f * 127.0f * 1.2e-7f);
+      bv = amax_pair * ktmax * (((128.0f * 127.0f * 0.5f + 2048.0f) / 1048575.0f) * 1.0001f + 128.0f * 127.0f * 1.2e-7f);
     }
     if (lane == 0) {
       srow[first + j] = sv;
@@ -435,15 +447,16 @@ __device__ void radix_select2_desc(const float* v, const float* e, int n, int r0
 }
 
 // One workgroup per (sequence, KV head): classify, re-score the undecided blocks in fp64, emit.
-template <int QUANT, bool DYN>
+template <int QUANT, bool DYN, int NSET>
 __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs a) {
+  constexpr int GH = kG * NSET;  // query heads the re-scoring loop is unrolled for (those past the group are skipped)
   extern __shared__ double smd[];                  // exact scores of undecided blocks [max_blocks]
   float* sf = reinterpret_cast<float*>(smd + a.max_blocks);      // approx scores [max_blocks]
   float* se = sf + a.max_blocks;                                  // error bounds [max_blocks]
   int* state = reinterpret_cast<int*>(se + a.max_blocks);         // 0 dropped, 1 kept, 2 undecided
   int* ulist = state + a.max_blocks;                              // undecided block ids
   int* tbl = ulist + a.max_blocks;                                // this sequence's block table row
-  __shared__ float qs[kG][kD];
+  __shared__ float qs[GH][kD];
   __shared__ int n_in, n_unc, wave_tot[kResolveThreads / 64], running;
   __shared__ __attribute__((aligned(16))) int hist[4 * 512];
   __shared__ unsigned sel[16];
@@ -460,9 +473,10 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
     se[j] = eb ? eb[j] : eps;
     tbl[j] = a.block_tables[(size_t)b * a.max_blocks + j];
   }
-  for (int i = tid; i < kG * kD; i += kResolveThreads) {
+  for (int i = tid; i < GH * kD; i += kResolveThreads) {
     const int g = i / kD, c = i % kD;
-    const float qv = bf16_to_f32(a.q[((size_t)b * a.hkv * kG + h * kG + g) * kD + c]);
+    // rows past the group are zero: the re-scoring loop runs over all GH rows without a test, the maximum skips them
+    const float qv = g < a.group ? bf16_to_f32(a.q[((size_t)b * a.hkv * a.group + h * a.group + g) * kD + c]) : 0.f;
     qs[g][c] = DYN ? qv : __fmul_rn(qv, a.k_scale[h * kD + c]);
   }
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
@@ -500,7 +514,9 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
         double best = -INFINITY;
         if (pb >= 0 && pb < a.num_blocks && j * kBS + lane < kv_len) {
           const uint8_t* kr = a.key_cache + (((size_t)pb * a.hkv + h) * kBS + lane) * kD;
-          double acc[kG] = {0.0, 0.0, 0.0, 0.0};
+          double acc[GH];
+#pragma unroll
+          for (int g = 0; g < GH; ++g) acc[g] = 0.0;
           // the products are exact in fp64, so fma(q, k, acc) rounds exactly like add(acc, mul(q, k))
           for (int c = 0; c < kD; c += 16) {
             const uint4 w4 = *reinterpret_cast<const uint4*>(kr + c);
@@ -509,15 +525,17 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
             for (int e = 0; e < 16; ++e) {
               const double kv = dq64<QUANT>((ws[e >> 2] >> (8 * (e & 3))) & 0xff);
 #pragma unroll
-              for (int g = 0; g < kG; ++g) acc[g] = __fma_rn((double)qs[g][c + e], kv, acc[g]);
+              for (int g = 0; g < GH; ++g) acc[g] = __fma_rn((double)qs[g][c + e], kv, acc[g]);
             }
           }
           if (DYN) {
             const double kt = (double)a.k_scale[((size_t)pb * a.hkv + h) * kBS + lane];
 #pragma unroll
-            for (int g = 0; g < kG; ++g) acc[g] = __dmul_rn(acc[g], kt);
+            for (int g = 0; g < GH; ++g) acc[g] = __dmul_rn(acc[g], kt);
           }
-          best = fmax(fmax(acc[0], acc[1]), fmax(acc[2], acc[3]));
+#pragma unroll
+          for (int g = 0; g < GH; ++g)
+            if (g < a.group) best = fmax(best, acc[g]);
         }
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) best = fmax(best, __shfl_xor(best, off, 64));
@@ -565,7 +583,8 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
 }
 
 static bool sel_fast_supported(int hq, int hkv, int d, int bs, int max_blocks) {
-  return d == kD && hq == kG * hkv && bs == kBS && max_blocks <= 2048;  // 28 B of LDS per block in the resolve kernel
+  return d == kD && hkv > 0 && hq % hkv == 0 && hq / hkv <= kG * kMaxSets && bs == kBS &&
+         max_blocks <= 2048;  // 28 B of LDS per block in the resolve kernel
 }
 
 }  // namespace fdattn
@@ -610,22 +629,25 @@ static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_ca
     SelArgs sa{(const uint16_t*)q, (const uint8_t*)key_cache, cache_k_scale, block_tables, seq_lens_decoder,
                seq_lens_this_time, approx, eps, cache_quant_type == FDATTN_CACHE_INT8 ? nullptr : ebound, scores,
                kept_blocks, kept_counts, batch, hkv,
-               max_blocks_per_seq, num_blocks, chunk, cpp, top_k};
+               max_blocks_per_seq, num_blocks, chunk, cpp, top_k, hq / hkv};
     const size_t shm2 = (size_t)max_blocks_per_seq * (sizeof(double) + 2 * sizeof(float) + 3 * sizeof(int));
     const dim3 g1(pairs * cpp), g2(pairs), b1(256), b2(kResolveThreads);
-    if (cache_quant_type == FDATTN_CACHE_INT8) {
-      hipLaunchKernelGGL((sqattn_scores_mfma_kernel<FDATTN_CACHE_INT8, false>), g1, b1, 0, s, sa);
-      hipLaunchKernelGGL((sqattn_resolve_kernel<FDATTN_CACHE_INT8, false>), g2, b2, shm2, s, sa);
-    } else if (cache_quant_type == FDATTN_CACHE_FP8_E4M3) {
-      hipLaunchKernelGGL((sqattn_scores_mfma_kernel<FDATTN_CACHE_FP8_E4M3, false>), g1, b1, 0, s, sa);
-      hipLaunchKernelGGL((sqattn_resolve_kernel<FDATTN_CACHE_FP8_E4M3, false>), g2, b2, shm2, s, sa);
-    } else if (cache_quant_type == FDATTN_CACHE_INT8_DYNAMIC) {
-      hipLaunchKernelGGL((sqattn_scores_mfma_kernel<FDATTN_CACHE_INT8, true>), g1, b1, 0, s, sa);
-      hipLaunchKernelGGL((sqattn_resolve_kernel<FDATTN_CACHE_INT8, true>), g2, b2, shm2, s, sa);
-    } else {
-      hipLaunchKernelGGL((sqattn_scores_mfma_kernel<FDATTN_CACHE_FP8_E4M3, true>), g1, b1, 0, s, sa);
-      hipLaunchKernelGGL((sqattn_resolve_kernel<FDATTN_CACHE_FP8_E4M3, true>), g2, b2, shm2, s, sa);
-    }
+    const bool two = hq / hkv > kG;
+#define FDATTN_SEL_LAUNCH(Q, D)                                                                                     \
+  do {                                                                                                              \
+    if (two) {                                                                                                      \
+      hipLaunchKernelGGL((sqattn_scores_mfma_kernel<Q, D, 2>), g1, b1, 0, s, sa);                                   \
+      hipLaunchKernelGGL((sqattn_resolve_kernel<Q, D, 2>), g2, b2, shm2, s, sa);                                    \
+    } else {                                                                                                        \
+      hipLaunchKernelGGL((sqattn_scores_mfma_kernel<Q, D, 1>), g1, b1, 0, s, sa);                                   \
+      hipLaunchKernelGGL((sqattn_resolve_kernel<Q, D, 1>), g2, b2, shm2, s, sa);                                    \
+    }                                                                                                               \
+  } while (0)
+    if (cache_quant_type == FDATTN_CACHE_INT8) FDATTN_SEL_LAUNCH(FDATTN_CACHE_INT8, false);
+    else if (cache_quant_type == FDATTN_CACHE_FP8_E4M3) FDATTN_SEL_LAUNCH(FDATTN_CACHE_FP8_E4M3, false);
+    else if (cache_quant_type == FDATTN_CACHE_INT8_DYNAMIC) FDATTN_SEL_LAUNCH(FDATTN_CACHE_INT8, true);
+    else FDATTN_SEL_LAUNCH(FDATTN_CACHE_FP8_E4M3, true);
+#undef FDATTN_SEL_LAUNCH
     return check_launch("fdattn_sqattn_select (mfma)");
   }
   ScoreArgs a{(const uint16_t*)q, (const uint8_t*)key_cache, cache_k_scale, block_tables, seq_lens_decoder,

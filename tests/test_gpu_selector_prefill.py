@@ -69,6 +69,29 @@ def test_selector_ties_near_ties_and_short_sequences(oracle, quant, impl):
         assert np.array_equal(np_of(kept), okept) and np.array_equal(np_of(cnt), ocnt), k
 
 
+@pytest.mark.parametrize("quant", ALL_FORMATS)
+@pytest.mark.parametrize("group", [1, 3, 5, 8])
+def test_selector_other_group_sizes(oracle, group, quant):
+    """1 .. 8 query heads per KV head on the fast path (MFMA scores + exact resolution): indices bit for bit as the
+    oracle's and as the all-fp64 path's, including planted ties."""
+    hkv = 2
+    hq = group * hkv
+    case = syn.decode_case(batch=3, ctx=[64 * 40, 64 * 17 + 9, 100], quant=quant, seed=50 + group, salient=0.1,
+                           hq=hq, hkv=hkv)
+    bt = case["block_tables"]
+    for j in (6, 11):   # identical pages -> identical scores -> the lower index wins
+        case["key_cache"][int(bt[0, j])] = case["key_cache"][int(bt[0, 2])]
+        if quant in (CACHE_INT8_DYNAMIC, CACHE_FP8_DYNAMIC):
+            case["cache_k_scale"][int(bt[0, j])] = case["cache_k_scale"][int(bt[0, 2])]
+    dev = syn.to_device(case, "cuda")
+    for k in (1, 5, 16):
+        _, okept, ocnt = oracle_select(oracle, case, k)
+        for impl in ("auto", "exact"):
+            kept, cnt = fd.sqattn_select(dev["q"], dev["key_cache"], dev["cache_k_scale"], dev["block_tables"],
+                                         dev["seq_lens_decoder"], num_heads=hq, top_k=k, cache_quant_type=quant, impl=impl)
+            assert np.array_equal(np_of(kept), okept) and np.array_equal(np_of(cnt), ocnt), (k, impl)
+
+
 @pytest.mark.parametrize("quant", [CACHE_FP8, CACHE_FP8_DYNAMIC])
 def test_selector_config4_shape_indices_bit_exact(oracle, quant):
     """batch 16, ctx 32768, fp8 KV, top-64 of 512 blocks per KV head, 5 % salient blocks (scaled x4):
