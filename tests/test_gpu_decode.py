@@ -151,6 +151,46 @@ def test_decode_other_group_sizes_on_the_mfma_kernel(oracle, group, quant):
     check(bits(out), oracle_decode(oracle, case, kept_blocks=kept, kept_counts=cnt), "group %d sparse" % group)
 
 
+def test_decode_random_shapes_against_the_oracle(oracle):
+    """40 seeded random cases: batch 1 .. 9, 1 .. 8 query heads per KV head, 1 .. 4 KV heads, any of the four cache
+    formats, lengths that favour block boundaries and zero, dense or sparse lists - the MFMA kernel against the oracle."""
+    rng = np.random.default_rng(2024)
+    for it in range(40):
+        group, hkv = int(rng.integers(1, 9)), int(rng.integers(1, 5))
+        hq, quant = group * hkv, ALL_FORMATS[int(rng.integers(0, 4))]
+        batch = int(rng.integers(1, 10))
+        lens = []
+        for _ in range(batch):
+            kind = int(rng.integers(0, 5))
+            base = int(rng.integers(0, 40)) * 64
+            lens.append([0, base, base + 1, base + 63, int(rng.integers(1, 2600))][kind])
+        if not any(lens):
+            lens[0] = 65
+        mb = max(max(lens) // 64 + 1, 1) + int(rng.integers(0, 3))
+        case = syn.decode_case(batch=batch, ctx=lens, quant=quant, seed=1000 + it, extra_blocks=2, hq=hq, hkv=hkv,
+                               max_blocks=mb, row_log2=(-4, 0))
+        assert fd.decode_uses_mfma(hq, hkv, 128, 64, quant)
+        what = "case %d: group %d hkv %d quant %d lens %r" % (it, group, hkv, quant, lens)
+        if it % 3 == 2:   # sparse: random ascending subsets, some empty
+            mk = int(rng.integers(1, 8))
+            kept = np.full((batch, hkv, mk), -1, np.int32)
+            cnt = np.zeros((batch, hkv), np.int32)
+            for b in range(batch):
+                nb = (lens[b] + 63) // 64
+                for h in range(hkv):
+                    k = int(rng.integers(0, min(mk, nb) + 1))
+                    kept[b, h, :k] = np.sort(rng.choice(nb, k, replace=False)) if k else []
+                    cnt[b, h] = k
+            dev = syn.to_device(case, "cuda")
+            out = fd.decode_attention_sparse(dev["q"], dev["key_cache"], dev["value_cache"], dev["cache_k_scale"],
+                                             dev["cache_v_scale"], dev["block_tables"], dev["seq_lens_decoder"],
+                                             kept_blocks=torch.from_numpy(kept).cuda(), kept_counts=torch.from_numpy(cnt).cuda(),
+                                             num_heads=hq, cache_quant_type=quant)
+            check(bits(out), oracle_decode(oracle, case, kept_blocks=kept, kept_counts=cnt), what + " sparse")
+        else:
+            check(gpu_decode(case), oracle_decode(oracle, case), what)
+
+
 def test_decode_generic_other_shapes(oracle):
     """Shapes outside the MFMA kernel: head_dim 64, group 2, block_size 16."""
     case = syn.decode_case(batch=3, ctx=[50, 200, 333], seed=8, hq=8, hkv=4, d=64, bs=16)

@@ -243,6 +243,42 @@ def test_mixed_step_other_group_sizes(oracle, group, quant):
     assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
 
 
+def test_mixed_step_random_batches_against_the_oracle(oracle):
+    """20 seeded random steps: 1 .. 8 slots that are prefill rows (1 .. 140 new tokens, with or without cached
+    tokens), decode rows or idle; 1 .. 8 query heads per KV head; any cache format; with and without the
+    prefill-row count.  Cache bytes (and scale caches) exact, outputs within tolerance."""
+    rng = np.random.default_rng(7)
+    formats = [CACHE_INT8, CACHE_FP8, CACHE_INT8_DYNAMIC, CACHE_FP8_DYNAMIC]
+    for it in range(20):
+        slots, group, hkv = int(rng.integers(1, 9)), int(rng.integers(1, 9)), int(rng.integers(1, 4))
+        quant = formats[int(rng.integers(0, 4))]
+        enc, dec = [], []
+        for _ in range(slots):
+            kind = int(rng.integers(0, 4))   # prefill on nothing, prefill on a prefix, decode, idle
+            enc.append(int(rng.integers(1, 141)) if kind < 2 else 0)
+            dec.append(0 if kind in (0, 3) else int(rng.integers(1, 600)))
+        if not any(enc) and not any(dec):
+            dec[0] = 77
+        hq = group * hkv
+        c = mixed_case(enc, dec, quant, seed=500 + it, hq=hq, hkv=hkv, max_pos=1024)
+        dev = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
+        rows = sum(1 for e in enc if e > 0)
+        out = fd.append_attention(dev["qkv"], dev["key_cache"], dev["value_cache"], dev["seq_lens_encoder"],
+                                  dev["seq_lens_decoder"], dev["seq_lens_this_time"], dev["block_tables"],
+                                  (dev["rope_cos"], dev["rope_sin"]), dev["cache_k_scale"], dev["cache_v_scale"],
+                                  num_heads=hq, kv_num_heads=hkv, max_chunk=max(enc), cache_quant_type=quant,
+                                  cu_seqlens_q=dev["cu_seqlens_q"], prefill_rows=rows if it % 2 else None)
+        torch.cuda.synchronize()
+        what = "step %d: enc %r dec %r group %d hkv %d quant %d" % (it, enc, dec, group, hkv, quant)
+        want, kc, vc = oracle_step(oracle, c, quant, hq, hkv, 128)
+        assert np.array_equal(np_of(dev["key_cache"]), kc) and np.array_equal(np_of(dev["value_cache"]), vc), what
+        if is_dynamic(quant):
+            assert np.array_equal(np_of(dev["cache_k_scale"]), c["scales_after"][0]), what
+            assert np.array_equal(np_of(dev["cache_v_scale"]), c["scales_after"][1]), what
+        ok, mx, bad = bf16_close(bits(out), want)
+        assert ok, "%s: %d out of tolerance, max %.4g" % (what, bad, mx)
+
+
 def test_steps_over_block_pool_tables_with_a_shared_prefix(oracle):
     """Two steps driven by the block pool's tables: a prompt is prefilled, a second sequence forks its
     whole blocks and prefills only its own tail while the first decodes and a third arrives.  Every step is
