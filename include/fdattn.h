@@ -383,6 +383,10 @@ FDATTN_API size_t fdattn_append_attention_workspace_bytes_ex(int num_tokens, int
  *                  to the cache and attends to seq_lens_decoder[b] + 1 cached tokens
  *                  (fdattn_decode_attention),
  *   idle           otherwise (no token: nothing is read or written for it).
+ * A row that brings several tokens with causal attention among them - a prompt chunk, or the
+ * draft tokens of a speculative step - is a prefill row: give it seq_lens_encoder[b] = its
+ * number of tokens (a row with several tokens and seq_lens_encoder[b] == 0 gets its tokens
+ * written to the cache but no attention output).
  * Every new token is first rotated and written to the cache (fdattn_write_cache_kv).
  * max_chunk bounds the tokens of a prefill row in this step; 0 says that the step has no
  * prefill row (the prefill pass is then not launched at all).
