@@ -69,7 +69,7 @@ extern "C" int fdattn_append_attention_ex(
   if (num_tokens == 0) return 0;
   // key splits for the prefill rows: only when the host says how few they are
   const int prefill_rows = extras && extras->prefill_rows > 0 ? extras->prefill_rows : 0;
-  int splits = prefill_rows > 0 && max_chunk > 0 ? prefill_auto_splits(prefill_rows, hq, max_chunk) : 1;
+  int splits = prefill_rows > 0 && max_chunk > 0 ? prefill_auto_splits(prefill_rows, hq, max_chunk, hkv) : 1;
   StepWorkspace w = step_workspace(num_tokens, batch, hq, hkv, head_dim, max_blocks_per_seq, splits);
   while (splits > 1 && workspace_bytes < w.total)  // a workspace sized for fewer splits: use as many as it holds
     w = step_workspace(num_tokens, batch, hq, hkv, head_dim, max_blocks_per_seq, --splits);

@@ -25,6 +25,10 @@ struct PrefillArgs {
   int n_splits;
   int tile_tokens;  // queries per workgroup of this launch (128 or 256), for the merge kernel
   int rows;         // MFMA kernel: sequences the grid covers - the batch, or the number of prefill rows when the host gave it
+  // MFMA kernel, short chunks: > 0 packs ALL query heads of a KV head into one workgroup - query column x of the
+  // workgroup is head x / pack_slot of the group, token x % pack_slot - so that the staged K / V tiles serve the
+  // whole group (the grid then runs over KV heads, not query heads); 0: one query head per workgroup
+  int pack_slot;
   float* part_o;   // [n_splits][num_tokens][hq][128]
   float* part_ml;  // [n_splits][num_tokens][hq][2]
 };
@@ -34,7 +38,8 @@ bool prefill_mfma_supported(int hq, int hkv, int d, int bs, int quant);
 int prefill_mfma_launch(const PrefillArgs& a, int max_chunk, int quant, hipStream_t s, void* workspace = nullptr,
                         size_t workspace_bytes = 0, int n_splits = 1, int rows_hint = 0);
 size_t prefill_split_workspace_bytes(int num_tokens, int hq, int n_splits);
-// splits that fill the GPU when `rows` sequences bring at most max_chunk new tokens each (1 = none needed)
-int prefill_auto_splits(int rows, int hq, int max_chunk);
+// splits that fill the GPU when `rows` sequences bring at most max_chunk new tokens each (1 = none needed);
+// hkv (optional): with it the count allows for short chunks running one workgroup per KV head
+int prefill_auto_splits(int rows, int hq, int max_chunk, int hkv = 0);
 
 }  // namespace fdattn

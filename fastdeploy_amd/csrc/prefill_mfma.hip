@@ -198,8 +198,13 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   // query tiles come longest first (the causal rows of late tokens walk more keys), so every XCD gets
   // the same mix of long and short workgroups and the short ones fill the end of the launch.
   const int G = a.hq / a.hkv, pairs = a.rows * a.hkv, units = a.rows * a.hq;
-  int qt, b, qh;  // b: the grid row first, the sequence below
-  if ((pairs & 7) == 0) {
+  const bool pack = a.pack_slot > 0;  // short chunks: the workgroup holds every query head of its KV head
+  int qt, b, qh;  // b: the grid row first, the sequence below; qh: the (first) query head
+  if (pack) {
+    qt = 0;
+    b = blockIdx.x / a.hkv;
+    qh = (blockIdx.x - b * a.hkv) * G;
+  } else if ((pairs & 7) == 0) {
     const int ppx = pairs >> 3;  // pairs per XCD
     const int x = blockIdx.x & 7, jx = blockIdx.x >> 3;
     const int r = jx % (ppx * G), pk = (r / G) * 8 + x;
@@ -222,13 +227,19 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
 
   const int j32 = lane & 31, hf = lane >> 5;
   // this lane's query; rows past the chunk behave like its last row and are not stored
-  const int ci_raw = q0 + 32 * wv + j32;
+  int ci_raw = q0 + 32 * wv + j32;
+  int qh_lane = qh;  // packed: query column x = 32 wv + j32 is head x / slot of the group, token x % slot
+  if (pack) {
+    const int x = 32 * wv + j32, hg = x / a.pack_slot;
+    ci_raw = hg < G ? x - hg * a.pack_slot : n_b;
+    qh_lane = qh + min(hg, G - 1);
+  }
   const int ci = min(ci_raw, n_b - 1);
-  const bool wave_active = q0 + 32 * wv < n_b;
-  const int ci_wave_max = min(q0 + 32 * wv + 31, n_b - 1);
+  const bool wave_active = pack ? __ballot(ci_raw < n_b) != 0ull : q0 + 32 * wv < n_b;
+  const int ci_wave_max = pack ? n_b - 1 : min(q0 + 32 * wv + 31, n_b - 1);
 
   const int n_pre = (p + BN - 1) / BN;
-  const int n_chk = (min(n_b, q0 + BM) + BN - 1) / BN;
+  const int n_chk = (min(n_b, pack ? a.pack_slot : q0 + BM) + BN - 1) / BN;
   const int n_tiles = n_pre + n_chk;
   // this workgroup's share of the key tiles: [t0, t1).  A share is worth its fixed costs (prologue, partial,
   // merge) from about 16 tiles on: shorter walks are split less, or not at all - then split 0 walks everything
@@ -238,19 +249,21 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   const int per = (n_tiles + n_splits - 1) / n_splits;
   const int t0 = (int)blockIdx.y * per, t1 = min(t0 + per, n_tiles);
   if (t0 >= t1) {  // nothing to walk (only with splits): an empty partial for each of the tile's queries
-    for (int i = tid; i < BM; i += 64 * NW)
-      if (q0 + i < n_b) {
-        float* ml = a.part_ml + (((size_t)blockIdx.y * a.num_tokens + tok0 + q0 + i) * a.hq + qh) * 2;
+    for (int i = tid; i < BM; i += 64 * NW) {
+      const int hg = pack ? i / a.pack_slot : 0, tk = pack ? i - hg * a.pack_slot : q0 + i;
+      if (hg < G && tk < n_b) {
+        float* ml = a.part_ml + (((size_t)blockIdx.y * a.num_tokens + tok0 + tk) * a.hq + qh + hg) * 2;
         ml[0] = -INFINITY;
         ml[1] = 0.f;
       }
+    }
     return;
   }
   const int32_t* table = a.block_tables + (size_t)b * a.max_blocks;
   const float sc = a.sm_scale * 1.4426950408889634f;  // logits go to the log2 domain
 
   // ---- Q as the B operand: lane = query, 8 channels per k-step
-  const uint16_t* qrow = a.q + ((size_t)(tok0 + ci) * a.hq + qh) * HD;
+  const uint16_t* qrow = a.q + ((size_t)(tok0 + ci) * a.hq + qh_lane) * HD;
   uint4 qf[8];       // fp16 (q * k_scale) while the prefix is walked, bf16 q for the chunk
   float qsum = 0.f;  // sum over this lane's 64 channels of the rounded q * k_scale
   auto load_q = [&](bool scaled) {
@@ -451,7 +464,7 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
       const bool pre = t < n_pre;
       const int key0 = pre ? t * BN : (t - n_pre) * BN;  // index of the tile's first key in its segment
       const int limit = pre ? p - key0 : ci - key0 + 1;  // keys [0, limit) of the tile are visible
-      const bool need_mask = pre ? (key0 + BN > p) : (key0 + BN > q0 + 32 * wv + 1);
+      const bool need_mask = pre ? (key0 + BN > p) : (pack || key0 + BN > q0 + 32 * wv + 1);
       if (need_mask) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
@@ -533,7 +546,7 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
   if (n_splits > 1) {
     // ---- a partial for the merge: o unnormalised in fp32, the exponent reference and the weight sum
-    const size_t row = ((size_t)blockIdx.y * a.num_tokens + tok0 + ci) * a.hq + qh;
+    const size_t row = ((size_t)blockIdx.y * a.num_tokens + tok0 + ci) * a.hq + qh_lane;
     float* po = a.part_o + row * HD;
 #pragma unroll
     for (int ct = 0; ct < 4; ++ct)
@@ -549,7 +562,7 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   }
   // ---- epilogue: normalise and store bf16 (every query saw at least its own chunk tile)
   const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-  uint16_t* orow = a.out + ((size_t)(tok0 + ci) * a.hq + qh) * HD;
+  uint16_t* orow = a.out + ((size_t)(tok0 + ci) * a.hq + qh_lane) * HD;
 #pragma unroll
   for (int ct = 0; ct < 4; ++ct)
 #pragma unroll
@@ -617,9 +630,8 @@ template <int QUANT, int NW, bool DYN>
 hipError_t launch_one(const PrefillArgs& a, int max_chunk, hipStream_t s) {
   constexpr int BM = 32 * NW;
   PrefillArgs args = a;
-  args.q_tiles = (max_chunk + BM - 1) / BM;
-  args.tile_tokens = BM;
-  const dim3 grid((unsigned)a.rows * a.hq * args.q_tiles, a.n_splits), block(64 * NW);
+  args.q_tiles = a.pack_slot > 0 ? 1 : (max_chunk + BM - 1) / BM;
+  const dim3 grid((unsigned)a.rows * (a.pack_slot > 0 ? a.hkv : a.hq) * args.q_tiles, a.n_splits), block(64 * NW);
   const size_t shm = (size_t)kSlots * BUF_ELEMS * sizeof(uint16_t);  // 151,552 B
   // the dynamic LDS limit is a per-device property of the kernel: raise it once on each device
   static std::atomic<unsigned long long> raised{0};  // bit d: done on device d (one word per instantiation)
@@ -650,9 +662,26 @@ static bool wide_workgroups(int rows, int hq, int max_chunk, int n_splits) {
   return max_chunk > 128 && (long long)rows * hq * ((max_chunk + 255) / 256) * n_splits >= gpu_cu_count();
 }
 
-int prefill_auto_splits(int rows, int hq, int max_chunk) {
+// Short chunks: when all query heads of a KV head, times the chunk's tokens, fit the query columns of one
+// workgroup (128 or 256), the workgroup takes the whole group and its staged K / V tiles serve every head.
+// Returns the tokens per head slot (0: not packed) and the workgroup's wavefront count.
+static int pack_slot_for(int hq, int hkv, int max_chunk, int* nw) {
+  const int g = hkv > 0 ? hq / hkv : 0;
+  if (g < 2 || max_chunk <= 0 || (long long)g * max_chunk > 256) return 0;
+  // always the 8-wavefront workgroup: its two wavefront groups overlap MFMA and vector work, and wavefronts whose
+  // columns hold no token (slots are 256 / g tokens wide) only help with the staging
+  *nw = 8;
+  return 32 * *nw / g;
+}
+
+int prefill_auto_splits(int rows, int hq, int max_chunk, int hkv) {
   if (rows <= 0 || hq <= 0 || max_chunk <= 0) return 1;
   const int cus = gpu_cu_count();
+  int nw = 0;
+  if (pack_slot_for(hq, hkv, max_chunk, &nw) > 0) {  // one workgroup per (row, KV head)
+    const long long wgs = (long long)rows * hkv, sp = (cus + wgs - 1) / wgs;
+    return (int)(sp < 1 ? 1 : (sp > kMaxSplits ? kMaxSplits : sp));
+  }
   auto splits_for = [&](int bm) {
     const long long wgs = (long long)rows * hq * ((max_chunk + bm - 1) / bm);
     const long long s = (cus + wgs - 1) / wgs;  // enough to give every CU a workgroup
@@ -680,7 +709,9 @@ int prefill_mfma_launch(const PrefillArgs& a_in, int max_chunk, int quant, hipSt
   // units and the vector ALU); short chunks keep 128
   // when they would still leave CUs without a workgroup (one fits a CU), 128-token workgroups cover twice as
   // many CUs: 10-14 % faster at e.g. 2 x 512 tokens, although a 4-wavefront workgroup overlaps nothing
-  const bool wide = wide_workgroups(a.rows, a.hq, max_chunk, a.n_splits);
+  int pack_nw = 0;
+  a.pack_slot = pack_slot_for(a.hq, a.hkv, max_chunk, &pack_nw);
+  const bool wide = a.pack_slot > 0 ? pack_nw == 8 : wide_workgroups(a.rows, a.hq, max_chunk, a.n_splits);
   hipError_t e;
   if (quant == FDATTN_CACHE_INT8)
     e = wide ? launch_one<FDATTN_CACHE_INT8, 8, false>(a, max_chunk, s) : launch_one<FDATTN_CACHE_INT8, 4, false>(a, max_chunk, s);
@@ -695,7 +726,7 @@ int prefill_mfma_launch(const PrefillArgs& a_in, int max_chunk, int quant, hipSt
   if (e != hipSuccess) return fail((int)e, "fdattn_append_attention_prefill: %s", hipGetErrorString(e));
   int rc = check_launch("fdattn_append_attention_prefill (mfma)");
   if (rc || a.n_splits <= 1) return rc;
-  a.tile_tokens = wide ? 256 : 128;
+  a.tile_tokens = a.pack_slot > 0 ? a.pack_slot : (wide ? 256 : 128);
   hipLaunchKernelGGL(prefill_merge_kernel, dim3(((long long)max_chunk * a.hq + 3) / 4, a.rows), dim3(256), 0, s, a);
   return check_launch("fdattn_append_attention_prefill (merge)");
 }

@@ -166,6 +166,29 @@ def test_prefill_ragged_edges(oracle, quant):
     assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
 
 
+@pytest.mark.parametrize("quant", ALL_FORMATS)
+def test_prefill_short_chunks_share_a_workgroup_per_kv_head(oracle, quant):
+    """Chunks short enough that all query heads of a KV head fit one workgroup's query columns (speculative
+    steps, tails of prompts): 1 .. 32 tokens with 4 heads per KV head, up to 64 with the 8-wavefront workgroup,
+    ragged rows, an empty prefix, and key splits on a long prefix - against the oracle."""
+    for prefix, chunks, mc, splits in (([200, 64, 0, 333, 1000], [4, 32, 5, 1, 17], 32, None),
+                                       ([64 * 9 + 3, 0, 129], [64, 33, 2], 64, None),
+                                       ([64 * 200 + 7], [8], 8, 8), ([64 * 70, 5], [3, 2], 3, 4)):
+        c = _prefill_case(sum(chunks) + len(prefix), prefix, chunks, quant)
+        dev = syn.to_device(c, "cuda")
+        out = fd.append_attention_prefill(dev["q_new"], dev["k_new"], dev["v_new"], dev["key_cache"], dev["value_cache"],
+                                          dev["cache_k_scale"], dev["cache_v_scale"], dev["block_tables"],
+                                          dev["seq_lens_decoder"], dev["cu_seqlens_q"], num_heads=32, max_chunk=mc,
+                                          cache_quant_type=quant, num_splits=splits)
+        torch.cuda.synchronize()
+        want = oracle.append_attention_prefill(bits(c["q_new"]), bits(c["k_new"]), bits(c["v_new"]), np_of(c["key_cache"]),
+                                               np_of(c["value_cache"]), np_of(c["cache_k_scale"]), np_of(c["cache_v_scale"]),
+                                               np_of(c["block_tables"]), np_of(c["seq_lens_decoder"]), np_of(c["cu_seqlens_q"]),
+                                               32, 8, 128, quant)
+        ok, mx, bad = bf16_close(bits(out), want)
+        assert ok, "prefix %r chunks %r splits %r: %d out of tolerance, max %.4g" % (prefix, chunks, splits, bad, mx)
+
+
 def _run_prefill_vs_oracle(oracle, c, quant, max_chunk):
     dev = syn.to_device(c, "cuda")
     out = fd.append_attention_prefill(dev["q_new"], dev["k_new"], dev["v_new"], dev["key_cache"], dev["value_cache"],
