@@ -84,6 +84,11 @@ def test_dynamic_formats_in_the_argument_checks_and_the_host_helpers():
     assert ops.is_dynamic("cache_fp8_dynamic") and not ops.is_dynamic("cache_fp8")
     assert ops.byte_format("cache_int8_dynamic") == ops.CACHE_INT8 and ops.byte_format(4) == ops.CACHE_FP8
     assert lib.fdattn_decode_uses_mfma(32, 8, 128, 64, 3) == 1 and lib.fdattn_decode_uses_mfma(32, 8, 128, 64, 4) == 1
+    # 1 .. 8 query heads per KV head run on the MFMA decode kernel; more, or a ragged ratio, do not
+    assert [lib.fdattn_decode_uses_mfma(g * 8, 8, 128, 64, 1) for g in (1, 2, 5, 8, 9)] == [1, 1, 1, 1, 0]
+    assert lib.fdattn_decode_uses_mfma(36, 8, 128, 64, 1) == 0
+    # the workspace of two row sets (5 .. 8 heads) is twice that of one
+    assert lib.fdattn_decode_workspace_bytes(1, 64, 8, 128, 2048) > lib.fdattn_decode_workspace_bytes(1, 32, 8, 128, 2048)
     rc = lib.fdattn_write_cache_kv(*([one] * 13), 1, 1, 4, 2, 96, 64, 1, 1, 8, 1, 3, None)    # 96 / 16 = 6 threads a row
     assert rc == -2 and b"dynamic" in lib.fdattn_last_error()
     rc = lib.fdattn_sqattn_select(*([one] * 10), 1 << 30, 2, 32, 8, 128, 64, 8, 8, 4, 7, None)
