@@ -82,6 +82,15 @@ def test_writer_chunks_ragged_and_no_rope(oracle, quant):
     _run_both(oracle, case)
 
 
+@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8_DYNAMIC])
+def test_writer_more_tokens_than_one_grid_dimension_holds(oracle, quant):
+    """66,000 new tokens in one call (a grid dimension holds 65,535 workgroups: the launch goes in slices): every
+    byte, scale and rotated row as the oracle's."""
+    case = syn.write_case(num_seqs=3, max_pos=22050, quant=quant, seed=17, hq=2, hkv=1, d=32, chunk=22000)
+    assert case["qkv"].shape[0] == 66000
+    _run_both(oracle, case)
+
+
 @pytest.mark.parametrize("style", ["neox", "interleaved"])
 @pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
 def test_writer_epilogue_bit_exact(oracle, quant, style):
