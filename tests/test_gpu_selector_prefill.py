@@ -92,6 +92,18 @@ def test_selector_other_group_sizes(oracle, group, quant):
             assert np.array_equal(np_of(kept), okept) and np.array_equal(np_of(cnt), ocnt), (k, impl)
 
 
+def test_selector_longest_sequences_of_the_fast_path_and_beyond(oracle):
+    """2048 blocks per sequence (131,072 tokens) is the most the fast path's resolve kernel holds in LDS; one block
+    more goes to the all-fp64 path.  Both against the oracle."""
+    for ctx in (64 * 2048, 64 * 2049 + 5):
+        case = syn.decode_case(batch=1, ctx=ctx, quant=CACHE_INT8, seed=4, device="cuda", direct_bytes=True)
+        kept, cnt = fd.sqattn_select(case["q"], case["key_cache"], case["cache_k_scale"], case["block_tables"],
+                                     case["seq_lens_decoder"], num_heads=32, top_k=100, cache_quant_type=CACHE_INT8)
+        torch.cuda.synchronize()
+        _, okept, ocnt = oracle_select(oracle, syn.to_device(case, "cpu"), 100)
+        assert np.array_equal(np_of(cnt), ocnt) and np.array_equal(np_of(kept), okept), ctx
+
+
 @pytest.mark.parametrize("quant", [CACHE_FP8, CACHE_FP8_DYNAMIC])
 def test_selector_config4_shape_indices_bit_exact(oracle, quant):
     """batch 16, ctx 32768, fp8 KV, top-64 of 512 blocks per KV head, 5 % salient blocks (scaled x4):
