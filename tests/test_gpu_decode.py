@@ -317,6 +317,19 @@ def test_decode_launch_shapes(oracle, quant):
         check(bits(out), oracle_decode(oracle, syn.to_device(case, "cpu")), "batch %d" % batch)
 
 
+def test_decode_one_very_long_sequence(oracle):
+    """One sequence of 524,288 tokens (8,192 blocks, 1 GiB of K and V): 64 chunks of 128 units per KV head and the
+    merge kernel over all of them."""
+    from fastdeploy_amd import _lib
+    ctx = 64 * 8192 - 9
+    assert _lib.lib().fdattn_decode_chunks_per_sequence(1, 8, 8192) == 64
+    case = syn.decode_case(batch=1, ctx=ctx, seed=3, device="cuda", direct_bytes=True)
+    out = fd.decode_attention(case["q"], case["key_cache"], case["value_cache"], case["cache_k_scale"],
+                              case["cache_v_scale"], case["block_tables"], case["seq_lens_decoder"], num_heads=32)
+    torch.cuda.synchronize()
+    check(bits(out), oracle_decode(oracle, syn.to_device(case, "cpu")), "524k tokens")
+
+
 def test_write_then_decode_config3_full_size(oracle):
     """256 new tokens (bf16 qkv ~ N(0,1)), RoPE theta 500000 at positions U{0..8191}, int8 write into the
     block-tabled slots, then decode over ctx = pos + 1: cache bytes bit-exact, outputs within tolerance."""
