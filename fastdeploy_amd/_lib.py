@@ -29,6 +29,7 @@ SIGNATURES = {
     "fdattn_append_attention_workspace_bytes": (_sz, [_i] * 6),
     "fdattn_append_attention": (_i, [_vp] * 14 + [_sz] + [_i] * 12 + [_f, _vp]),
     "fdattn_prefill_auto_splits": (_i, [_i] * 3),
+    "fdattn_prefill_auto_splits_for": (_i, [_i] * 4),
     "fdattn_append_attention_prefill_split_workspace_bytes": (_sz, [_i] * 3),
     "fdattn_append_attention_prefill_split": (_i, [_vp] * 12 + [_sz] + [_i] * 11 + [_f, _vp]),
     "fdattn_append_attention_workspace_bytes_ex": (_sz, [_i] * 7),
@@ -54,7 +55,7 @@ SIGNATURES = {
 class StepExtras(ctypes.Structure):
     """fdattn_step_extras of include/fdattn.h"""
     _fields_ = [("qkv_bias", _vp), ("q_norm_weight", _vp), ("k_norm_weight", _vp), ("rms_norm_eps", _f),
-                ("prefill_rows", _i)]
+                ("prefill_rows", _i), ("sqattn_top_k", _i)]
 
 
 _lib = None

@@ -45,13 +45,15 @@ class ForwardMeta:
 
 class AppendAttentionBackend:
     def __init__(self, num_heads, kv_num_heads, head_dim, *, block_size=64, max_position=8192, rope_theta=10000.0,
-                 rope_style="neox", cache_quant_type="cache_int8", softmax_scale=None, device="cuda"):
+                 rope_style="neox", cache_quant_type="cache_int8", softmax_scale=None, device="cuda",
+                 sqattn_top_k=None):
         from .rope import rope_table
         if num_heads % kv_num_heads:
             raise ValueError("num_heads %d is not a multiple of kv_num_heads %d" % (num_heads, kv_num_heads))
         self.num_heads, self.kv_num_heads, self.head_dim = num_heads, kv_num_heads, head_dim
         self.block_size, self.rope_style, self.cache_quant_type = block_size, rope_style, cache_quant_type
         self.softmax_scale = softmax_scale
+        self.sqattn_top_k = sqattn_top_k   # > 0: decode rows attend to their top-k blocks only (block-sparse)
         self.device = device
         self.rotary_embs = rope_table(max_position, head_dim, rope_theta, device)
         self._workspace = None
@@ -102,7 +104,8 @@ class AppendAttentionBackend:
         # a step whose few prefill rows would leave CUs idle shares every query tile's keys among several workgroups
         meta.prefill_splits = 1
         if meta.prefill_rows and meta.max_enc_len_this_time > 0:
-            meta.prefill_splits = ops.prefill_auto_splits(meta.prefill_rows, self.num_heads, meta.max_enc_len_this_time)
+            meta.prefill_splits = ops.prefill_auto_splits(meta.prefill_rows, self.num_heads, meta.max_enc_len_this_time,
+                                                           self.kv_num_heads)
         need = ops.append_attention_workspace_bytes(meta.num_tokens, slots, self.num_heads, self.kv_num_heads,
                                                     self.head_dim, meta.block_tables.shape[1], meta.prefill_splits)
         if self._workspace is None or self._workspace.numel() < need:
@@ -123,7 +126,7 @@ class AppendAttentionBackend:
             rope_style=self.rope_style, cache_quant_type=self.cache_quant_type, softmax_scale=self.softmax_scale,
             cu_seqlens_q=meta.cu_seqlens_q, workspace=self._workspace, out=out, qkv_bias=layer.qkv_bias,
             q_norm_weight=layer.q_norm_weight, k_norm_weight=layer.k_norm_weight, rms_norm_eps=layer.rms_norm_eps,
-            prefill_rows=meta.prefill_rows)
+            prefill_rows=meta.prefill_rows, sqattn_top_k=self.sqattn_top_k)
 
 
 class SequenceBook:

@@ -9,7 +9,7 @@ namespace fdattn {
 static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 
 struct StepWorkspace {
-  size_t q_rot, k_new, v_new, decode, split, total;  // byte offsets of the parts, and the sum
+  size_t q_rot, k_new, v_new, decode, select, kept, split, total;  // byte offsets of the parts, and the sum
 };
 
 static StepWorkspace step_workspace(int num_tokens, int batch, int hq, int hkv, int d, int max_blocks, int prefill_splits) {
@@ -18,7 +18,10 @@ static StepWorkspace step_workspace(int num_tokens, int batch, int hq, int hkv, 
   w.k_new = w.q_rot + align256((size_t)num_tokens * hq * d * 2);
   w.v_new = w.k_new + align256((size_t)num_tokens * hkv * d * 2);
   w.decode = w.v_new + align256((size_t)num_tokens * hkv * d * 2);
-  w.split = w.decode + align256(fdattn_decode_workspace_bytes(batch, hq, hkv, d, max_blocks));
+  // the block selector's scores and bounds, then its result (kept blocks - at most every block - and counts)
+  w.select = w.decode + align256(fdattn_decode_workspace_bytes(batch, hq, hkv, d, max_blocks));
+  w.kept = w.select + align256(fdattn_sqattn_workspace_bytes(batch, hkv, max_blocks));
+  w.split = w.kept + align256((size_t)batch * hkv * ((size_t)max_blocks + 1) * sizeof(int32_t));
   w.total = w.split + align256(prefill_split_workspace_bytes(num_tokens, hq, prefill_splits));
   return w;
 }
@@ -89,9 +92,26 @@ extern "C" int fdattn_append_attention_ex(
   if (rc) return rc;
   // 2. decode rows: one token, seq_lens_encoder == 0; they read their own token back from the cache
   const RowMap rows{cu_seqlens_q, seq_lens_encoder};
-  const size_t dws = w.split - w.decode;
+  const size_t dws = w.select - w.decode;
   hipStream_t s = (hipStream_t)stream;
-  if (c8_supported(hq, hkv, head_dim, block_size, cache_quant_type))
+  const int top_k = extras && extras->sqattn_top_k > 0 ? (extras->sqattn_top_k < max_blocks_per_seq ? extras->sqattn_top_k : max_blocks_per_seq) : 0;
+  if (top_k > 0) {
+    // block-sparse decode rows: select with the new query over the cache as the writer left it, then attend to
+    // the kept blocks only
+    if (!c8_supported(hq, hkv, head_dim, block_size, cache_quant_type) ||
+        !sqattn_fast_supported(hq, hkv, head_dim, block_size, max_blocks_per_seq))
+      return fail(FDATTN_ERR_SHAPE, "fdattn_append_attention: sqattn_top_k needs head_dim 128, block_size 64, at most 8 "
+                  "query heads per KV head and at most 2048 blocks per sequence");
+    int32_t* kept = (int32_t*)(ws + w.kept);
+    int32_t* counts = kept + (size_t)batch * hkv * top_k;
+    rc = sqattn_select_launch(q_rot, key_cache, cache_k_scale, block_tables, seq_lens_decoder, seq_lens_this_time, kept,
+                              counts, ws + w.select, w.kept - w.select, batch, hq, hkv, head_dim, block_size,
+                              max_blocks_per_seq, num_blocks, top_k, cache_quant_type, s, rows);
+    if (rc) return rc;
+    rc = decode_c8_launch(q_rot, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables, seq_lens_decoder,
+                          seq_lens_this_time, kept, counts, top_k, out, ws + w.decode, dws, batch, hq, hkv, head_dim,
+                          block_size, max_blocks_per_seq, num_blocks, cache_quant_type, softmax_scale, s, 3, rows);
+  } else if (c8_supported(hq, hkv, head_dim, block_size, cache_quant_type))
     rc = decode_c8_launch(q_rot, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
                           seq_lens_decoder, seq_lens_this_time, nullptr, nullptr, 0, out, ws + w.decode, dws, batch,
                           hq, hkv, head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type,

@@ -28,6 +28,13 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
                      void* out, void* workspace, size_t workspace_bytes, int batch, int hq,
                      int hkv, int d, int bs, int max_blocks, int num_blocks, int quant,
                      float sm_scale, hipStream_t s, int stages, RowMap rows = RowMap{nullptr, nullptr});
+// the block selector on the decode rows of a mixed step (rows), MFMA shapes only
+bool sqattn_fast_supported(int hq, int hkv, int d, int bs, int max_blocks);
+int sqattn_select_launch(const void* q, const void* key_cache, const float* cache_k_scale, const int32_t* block_tables,
+                         const int32_t* seq_lens_decoder, const int32_t* seq_lens_this_time, int32_t* kept_blocks,
+                         int32_t* kept_counts, void* workspace, size_t workspace_bytes, int batch, int hq, int hkv,
+                         int head_dim, int block_size, int max_blocks_per_seq, int num_blocks, int top_k,
+                         int cache_quant_type, hipStream_t s, RowMap rows);
 // append (prefill) attention; seq_lens_encoder may be NULL (every sequence is a prefill row)
 // workspace / n_splits: the MFMA kernel may split every query tile's keys over n_splits workgroups (partials in
 // workspace); rows_hint: how many of the batch's rows are prefill rows, if known (0: all of them)

@@ -162,6 +162,9 @@ extern "C" int fdattn_append_attention_prefill(
 }
 
 extern "C" int fdattn_prefill_auto_splits(int rows, int hq, int max_chunk) { return prefill_auto_splits(rows, hq, max_chunk); }
+extern "C" int fdattn_prefill_auto_splits_for(int rows, int hq, int hkv, int max_chunk) {
+  return prefill_auto_splits(rows, hq, max_chunk, hkv);
+}
 
 extern "C" size_t fdattn_append_attention_prefill_split_workspace_bytes(int num_tokens, int hq, int num_splits) {
   return prefill_split_workspace_bytes(num_tokens, hq, num_splits);

@@ -168,6 +168,7 @@ struct SelArgs {
   int32_t* kept_counts;
   int batch, hkv, max_blocks, num_blocks, chunk, chunks_per_pair, top_k;
   int group;  // query heads per KV head, 1 .. 8
+  RowMap rows;  // inside a mixed step: which sequences are decode rows (the others keep no block) and their q rows
 };
 
 // One workgroup = `chunk` consecutive blocks of one (sequence, KV head); each wavefront
@@ -194,9 +195,11 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
     const int u = lane + 64 * e;
     if (u < a.chunk && first + u < a.max_blocks) pb_raw[e] = a.block_tables[(size_t)b * a.max_blocks + first + u];
   }
+  int qrow;
+  if (!decode_row(a.rows, b, qrow)) return;  // not a decode row of this step: nothing to score
   PairRaw raw[NSET];
 #pragma unroll
-  for (int t = 0; t < NSET; ++t) raw[t] = load_pair_issue(a.q, DYN ? nullptr : a.k_scale, a.hkv, p, b, lane, a.group, t);
+  for (int t = 0; t < NSET; ++t) raw[t] = load_pair_issue(a.q, DYN ? nullptr : a.k_scale, a.hkv, p, qrow, lane, a.group, t);
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
   const int n_p = min((max(kv_len, 0) + kBS - 1) / kBS, a.max_blocks);
   const int cnt = min(a.chunk, n_p - first);
@@ -245,7 +248,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void sqattn_scores_mfma_kernel(SelA
     for (int g = 0; g < a.group; ++g) {
       float sa = 0.f, am = 0.f;
       for (int c = lane; c < kD; c += 64) {
-        const float qs = fabsf(bf16_to_f32(a.q[((size_t)b * a.hkv * a.group + h * a.group + g) * kD + c]) * (DYN ? 1.0f : a.k_scale[h * kD + c]));
+        const float qs = fabsf(bf16_to_f32(a.q[((size_t)qrow * a.hkv * a.group + h * a.group + g) * kD + c]) * (DYN ? 1.0f : a.k_scale[h * kD + c]));
         sa += qs;
         am = fmaxf(am, qs);
       }
@@ -462,6 +465,11 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
   __shared__ unsigned sel[16];
   const int p = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int b = p / a.hkv, h = p - b * a.hkv;
+  int qrow;
+  if (!decode_row(a.rows, b, qrow)) {  // not a decode row of this step: it keeps no block
+    if (tid == 0) a.kept_counts[p] = 0;
+    return;
+  }
   // Everything the kernel will need from memory is requested here, in one round trip: the scores and
   // their bounds, the table row and q * k_scale of the re-scoring step (needed only if a block stays
   // undecided, but a second and third trip would cost more than these few KB).
@@ -476,7 +484,7 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
   for (int i = tid; i < GH * kD; i += kResolveThreads) {
     const int g = i / kD, c = i % kD;
     // rows past the group are zero: the re-scoring loop runs over all GH rows without a test, the maximum skips them
-    const float qv = g < a.group ? bf16_to_f32(a.q[((size_t)b * a.hkv * a.group + h * a.group + g) * kD + c]) : 0.f;
+    const float qv = g < a.group ? bf16_to_f32(a.q[((size_t)qrow * a.hkv * a.group + h * a.group + g) * kD + c]) : 0.f;
     qs[g][c] = DYN ? qv : __fmul_rn(qv, a.k_scale[h * kD + c]);
   }
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
@@ -597,12 +605,17 @@ extern "C" size_t fdattn_sqattn_workspace_bytes(int batch, int hkv, int max_bloc
   return (n + 255) & ~(size_t)255;
 }
 
+namespace fdattn {
+bool sqattn_fast_supported(int hq, int hkv, int d, int bs, int max_blocks) { return sel_fast_supported(hq, hkv, d, bs, max_blocks); }
+}
+
 static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_cache, const float* cache_k_scale,
                                     const int32_t* block_tables, const int32_t* seq_lens_decoder,
                                     const int32_t* seq_lens_this_time, float* scores, int32_t* kept_blocks,
                                     int32_t* kept_counts, void* workspace, size_t workspace_bytes, int batch,
                                     int hq, int hkv, int head_dim, int block_size, int max_blocks_per_seq,
-                                    int num_blocks, int top_k, int cache_quant_type, void* stream) {
+                                    int num_blocks, int top_k, int cache_quant_type, void* stream,
+                                    RowMap rows = RowMap{nullptr, nullptr}) {
   if (!q || !key_cache || !cache_k_scale || !block_tables || !seq_lens_decoder || !kept_blocks ||
       !kept_counts || !workspace)
     return fail(FDATTN_ERR_NULL, "fdattn_sqattn_select: a required pointer is NULL");
@@ -629,7 +642,7 @@ static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_ca
     SelArgs sa{(const uint16_t*)q, (const uint8_t*)key_cache, cache_k_scale, block_tables, seq_lens_decoder,
                seq_lens_this_time, approx, eps, cache_quant_type == FDATTN_CACHE_INT8 ? nullptr : ebound, scores,
                kept_blocks, kept_counts, batch, hkv,
-               max_blocks_per_seq, num_blocks, chunk, cpp, top_k, hq / hkv};
+               max_blocks_per_seq, num_blocks, chunk, cpp, top_k, hq / hkv, rows};
     const size_t shm2 = (size_t)max_blocks_per_seq * (sizeof(double) + 2 * sizeof(float) + 3 * sizeof(int));
     const dim3 g1(pairs * cpp), g2(pairs), b1(256), b2(kResolveThreads);
     const bool two = hq / hkv > kG;
@@ -650,6 +663,8 @@ static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_ca
 #undef FDATTN_SEL_LAUNCH
     return check_launch("fdattn_sqattn_select (mfma)");
   }
+  if (rows.cu_seqlens_q)
+    return fail(FDATTN_ERR_SHAPE, "fdattn_sqattn_select: inside a mixed step only the MFMA selector's shapes are covered");
   ScoreArgs a{(const uint16_t*)q, (const uint8_t*)key_cache, cache_k_scale, block_tables, seq_lens_decoder,
               seq_lens_this_time, (double*)workspace, scores, batch, hq, hkv, head_dim, block_size,
               max_blocks_per_seq, num_blocks};
@@ -692,3 +707,15 @@ extern "C" int fdattn_sqattn_select_exact(const void* q, const void* key_cache, 
                             scores, kept_blocks, kept_counts, workspace, workspace_bytes, batch, hq, hkv, head_dim,
                             block_size, max_blocks_per_seq, num_blocks, top_k, cache_quant_type, stream);
 }
+
+namespace fdattn {
+int sqattn_select_launch(const void* q, const void* key_cache, const float* cache_k_scale, const int32_t* block_tables,
+                         const int32_t* seq_lens_decoder, const int32_t* seq_lens_this_time, int32_t* kept_blocks,
+                         int32_t* kept_counts, void* workspace, size_t workspace_bytes, int batch, int hq, int hkv,
+                         int head_dim, int block_size, int max_blocks_per_seq, int num_blocks, int top_k,
+                         int cache_quant_type, hipStream_t s, RowMap rows) {
+  return sqattn_select_impl(true, q, key_cache, cache_k_scale, block_tables, seq_lens_decoder, seq_lens_this_time,
+                            nullptr, kept_blocks, kept_counts, workspace, workspace_bytes, batch, hq, hkv, head_dim,
+                            block_size, max_blocks_per_seq, num_blocks, top_k, cache_quant_type, (void*)s, rows);
+}
+}  // namespace fdattn

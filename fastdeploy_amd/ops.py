@@ -94,9 +94,9 @@ def _scales(cache_k_scale, cache_v_scale, hkv, d, quant=CACHE_INT8, nb=0, bs=0):
     return pk, pv
 
 
-def _extras(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, width, d, prefill_rows=0):
-    """fdattn_step_extras for the optional projection epilogue / prefill splits, or None"""
-    if qkv_bias is None and q_norm_weight is None and k_norm_weight is None and prefill_rows <= 0:
+def _extras(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, width, d, prefill_rows=0, sqattn_top_k=0):
+    """fdattn_step_extras for the optional projection epilogue / prefill splits / block-sparse decode rows, or None"""
+    if qkv_bias is None and q_norm_weight is None and k_norm_weight is None and prefill_rows <= 0 and sqattn_top_k <= 0:
         return None
     pb = _chk(qkv_bias, "qkv_bias", torch.bfloat16, 1, optional=True)
     if qkv_bias is not None and qkv_bias.numel() != width:
@@ -106,11 +106,13 @@ def _extras(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, width, d, pref
     for name, t in (("q_norm_weight", q_norm_weight), ("k_norm_weight", k_norm_weight)):
         if t is not None and t.numel() != d:
             raise ValueError("%s has %d entries, head_dim is %d" % (name, t.numel(), d))
-    return _lib.StepExtras(pb or None, pq or None, pk or None, float(rms_norm_eps), int(prefill_rows))
+    return _lib.StepExtras(pb or None, pq or None, pk or None, float(rms_norm_eps), int(prefill_rows), int(sqattn_top_k))
 
 
-def prefill_auto_splits(rows, num_heads, max_chunk):
+def prefill_auto_splits(rows, num_heads, max_chunk, kv_num_heads=None):
     """How many key splits fill the GPU when `rows` sequences bring at most max_chunk new tokens each (1..8)."""
+    if kv_num_heads:
+        return _lib.lib().fdattn_prefill_auto_splits_for(int(rows), int(num_heads), int(kv_num_heads), int(max_chunk))
     return _lib.lib().fdattn_prefill_auto_splits(int(rows), int(num_heads), int(max_chunk))
 
 
@@ -391,7 +393,7 @@ def append_attention(qkv, key_cache, value_cache, seq_lens_encoder, seq_lens_dec
                      block_tables, rotary_embs, cache_k_scale, cache_v_scale, *, num_heads, kv_num_heads,
                      max_chunk, rope_style="neox", cache_quant_type="cache_int8", softmax_scale=None,
                      cu_seqlens_q=None, workspace=None, out=None, qkv_bias=None, q_norm_weight=None,
-                     k_norm_weight=None, rms_norm_eps=1e-6, prefill_rows=None):
+                     k_norm_weight=None, rms_norm_eps=1e-6, prefill_rows=None, sqattn_top_k=None):
     """One attention step of a layer over a mixed batch (one call into the library):
     every new token is rotated and written to the cache, decode rows (one token,
     seq_lens_encoder == 0) attend to the cache, prefill rows (seq_lens_encoder > 0)
@@ -401,7 +403,9 @@ def append_attention(qkv, key_cache, value_cache, seq_lens_encoder, seq_lens_dec
     prefill_rows: how many sequences of the step have seq_lens_encoder > 0, if the host knows (None: unknown).  A
     promise, not a guess - the prefill pass then covers that many prefill rows only (no workgroups for decode rows),
     and when they alone would leave CUs idle every query tile is shared by prefill_auto_splits(prefill_rows,
-    num_heads, max_chunk) workgroups (as many as a workspace passed in has room for).
+    num_heads, max_chunk, kv_num_heads) workgroups (as many as a workspace passed in has room for).
+    sqattn_top_k: > 0 makes the decode rows block-sparse - the selector keeps that many blocks per (row, KV head),
+    scored with the row's new query, and the decode attention reads only those (MFMA selector shapes only).
     Returns bf16 [num_tokens, num_heads*head_dim]."""
     nb, hkv, bs, d = _cache_dims(key_cache, value_cache)
     if hkv != kv_num_heads:
@@ -443,12 +447,13 @@ def append_attention(qkv, key_cache, value_cache, seq_lens_encoder, seq_lens_dec
         raise ValueError("max_chunk must be >= 0")
     if out is None:
         out = torch.empty((T, num_heads * d), dtype=torch.bfloat16, device=qkv.device)
-    splits = prefill_auto_splits(prefill_rows, num_heads, max_chunk) if prefill_rows and max_chunk > 0 else 1
+    splits = prefill_auto_splits(prefill_rows, num_heads, max_chunk, hkv) if prefill_rows and max_chunk > 0 else 1
     need = _lib.lib().fdattn_append_attention_workspace_bytes_ex(T, batch, num_heads, hkv, d, mb, splits)
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=qkv.device)
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(d)
-    ep = _extras(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, qkv.shape[1], d, prefill_rows or 0)
+    ep = _extras(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, qkv.shape[1], d, prefill_rows or 0,
+                 sqattn_top_k or 0)
     rc = _lib.lib().fdattn_append_attention_ex(
         p_qkv, p_kc, p_vc, p_ks, p_vs, p_cos, p_sin, p_bt, p_enc, p_dec, p_this, p_cu,
         _chk(out, "out", torch.bfloat16), workspace.data_ptr(), workspace.numel() * workspace.element_size(),

@@ -127,6 +127,12 @@ FDATTN_API int fdattn_write_cache_kv(
  *                   query tile is shared by fdattn_prefill_auto_splits(prefill_rows, hq, max_chunk)
  *                   workgroups, each walking a part of its keys, if the workspace has room for their
  *                   partials (fdattn_append_attention_workspace_bytes_ex with that number of splits).
+ *   sqattn_top_k    (fdattn_append_attention_ex only) > 0: the decode rows of the step run block-sparse - the
+ *                   selector (fdattn_sqattn_select) keeps this many blocks per (row, KV head), scored with the
+ *                   row's new query against the cache that already holds its new token, and the decode
+ *                   attention reads only those (fdattn_decode_attention_sparse); rows with no more blocks
+ *                   than that keep all.  Shapes of the MFMA selector only.  The step's workspace always has
+ *                   room for it.  0: dense.
  */
 typedef struct fdattn_step_extras {
   const void* qkv_bias;
@@ -134,6 +140,7 @@ typedef struct fdattn_step_extras {
   const float* k_norm_weight;
   float rms_norm_eps;
   int prefill_rows;
+  int sqattn_top_k;
 } fdattn_step_extras;
 
 /* fdattn_write_cache_kv with the extras (host pointer, read during the call; NULL = none). */
@@ -335,6 +342,10 @@ FDATTN_API int fdattn_append_attention_prefill(
  * no initialisation needed.  Same plug-in position as fdattn_append_attention_prefill.
  */
 FDATTN_API int fdattn_prefill_auto_splits(int rows, int hq, int max_chunk);
+/* The same when the number of KV heads is known: chunks short enough for one workgroup to hold every query
+ * head of a KV head (hq / hkv x max_chunk <= 256) launch one workgroup per (row, KV head), and need more splits
+ * to fill the GPU.  This is the count fdattn_append_attention_ex uses. */
+FDATTN_API int fdattn_prefill_auto_splits_for(int rows, int hq, int hkv, int max_chunk);
 FDATTN_API size_t fdattn_append_attention_prefill_split_workspace_bytes(int num_tokens, int hq, int num_splits);
 FDATTN_API int fdattn_append_attention_prefill_split(
     const void* q, const void* k_new, const void* v_new,

@@ -243,6 +243,54 @@ def test_mixed_step_other_group_sizes(oracle, group, quant):
     assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
 
 
+@pytest.mark.parametrize("quant", [CACHE_FP8, CACHE_INT8_DYNAMIC])
+def test_mixed_step_with_block_sparse_decode_rows(oracle, quant):
+    """sqattn_top_k in the one-call step: every decode row selects its top-k blocks with its new query over the
+    cache that already holds its new token, and attends to those only; prefill rows are untouched by it.  Against the
+    oracle's pieces: writer, block scores + top-k, sparse decode, prefill."""
+    enc, dec = [0, 90, 0, 0, 0], [64 * 30 + 5, 700, 63, 64 * 11, 64 * 3]
+    top_k = 6
+    c = mixed_case(enc, dec, quant, seed=33, max_pos=4096)
+    dev = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
+    out = fd.append_attention(dev["qkv"], dev["key_cache"], dev["value_cache"], dev["seq_lens_encoder"],
+                              dev["seq_lens_decoder"], dev["seq_lens_this_time"], dev["block_tables"],
+                              (dev["rope_cos"], dev["rope_sin"]), dev["cache_k_scale"], dev["cache_v_scale"],
+                              num_heads=32, kv_num_heads=8, max_chunk=90, cache_quant_type=quant,
+                              cu_seqlens_q=dev["cu_seqlens_q"], prefill_rows=1, sqattn_top_k=top_k)
+    torch.cuda.synchronize()
+    # the oracle's step, with the decode rows done sparsely
+    kc, vc = np_of(c["key_cache"]).copy(), np_of(c["value_cache"]).copy()
+    ks, vs = np_of(c["cache_k_scale"]).copy(), np_of(c["cache_v_scale"]).copy()
+    bt, cu = np_of(c["block_tables"]), np_of(c["cu_seqlens_q"])
+    decs, this = np_of(c["seq_lens_decoder"]), np_of(c["seq_lens_this_time"])
+    q, k_new, v_new = oracle.write_cache_kv(bits(c["qkv"]), kc, vc, ks, vs, np_of(c["rope_cos"]), np_of(c["rope_sin"]),
+                                            bt, decs, cu, 32, 8, 128, 1, quant, want_kv_out=True)
+    assert np.array_equal(np_of(dev["key_cache"]), kc) and np.array_equal(np_of(dev["value_cache"]), vc)
+    want = np.zeros((c["T"], 32 * 128), np.uint16)
+    drows = [b for b in range(len(enc)) if enc[b] == 0 and this[b] == 1]
+    qd = np.ascontiguousarray(q[[cu[b] for b in drows]])
+    btd, kvl = np.ascontiguousarray(bt[drows]), np.ascontiguousarray(decs[drows] + 1)
+    sc = oracle.sqattn_block_scores(qd, kc, ks, btd, kvl, 32, 8, 128, quant)
+    kept, cnt = oracle.topk_select(sc, kvl, 64, top_k)
+    od = oracle.decode_attention(qd, kc, vc, ks, vs, btd, kvl, 32, 8, 128, quant, kept_blocks=kept, kept_counts=cnt)
+    for i, b in enumerate(drows):
+        want[cu[b]] = od[i]
+    ptoks = np.arange(cu[1], cu[2], dtype=np.int32)
+    op = oracle.append_attention_prefill(q, k_new, v_new, kc, vc, ks, vs, bt, decs, cu, 32, 8, 128, quant, token_ids=ptoks)
+    want[ptoks] = op[ptoks]
+    ok, mx, bad = bf16_close(bits(out), want)
+    assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
+    # and it differs from the dense step where a row has more blocks than it keeps
+    dense = fd.append_attention(dev["qkv"], dev["key_cache"], dev["value_cache"], dev["seq_lens_encoder"],
+                                dev["seq_lens_decoder"], dev["seq_lens_this_time"], dev["block_tables"],
+                                (dev["rope_cos"], dev["rope_sin"]), dev["cache_k_scale"], dev["cache_v_scale"],
+                                num_heads=32, kv_num_heads=8, max_chunk=90, cache_quant_type=quant,
+                                cu_seqlens_q=dev["cu_seqlens_q"], prefill_rows=1)
+    assert not torch.equal(dense[0], out[0]) and torch.equal(dense[cu[1]:cu[2]], out[cu[1]:cu[2]])
+    ok, mx, bad = bf16_close(bits(out[int(cu[4])]), bits(dense[int(cu[4])]))   # 4 blocks <= top_k: the row keeps them all
+    assert ok
+
+
 def test_mixed_step_random_batches_against_the_oracle(oracle):
     """20 seeded random steps: 1 .. 8 slots that are prefill rows (1 .. 140 new tokens, with or without cached
     tokens), decode rows or idle; 1 .. 8 query heads per KV head; any cache format; with and without the
