@@ -131,6 +131,24 @@ def other_workloads(args):
                                          c["block_tables"], c["seq_lens_decoder"], num_heads=32, cache_quant_type="cache_fp8", workspace=ws)
         ms = time_events(de, max(args.steps // 4, 5), 3)
         line("configs[3] dense fp8 decode, for comparison", ms, "hbm", 16 * 32768 * 8 * 128 * 2, HBM_PEAK_GBPS, "GB/s")
+        # the same as ONE library call per step: write the 16 new tokens (the last of each 32768), select, sparse decode
+        from fastdeploy_amd.rope import rope_table
+        g = torch.Generator(device=dev).manual_seed(5)
+        qkv = torch.randn((16, 48 * 128), generator=g, device=dev).to(torch.bfloat16)
+        zeros, ones = torch.zeros(16, dtype=torch.int32, device=dev), torch.ones(16, dtype=torch.int32, device=dev)
+        cu = torch.arange(17, dtype=torch.int32, device=dev)
+        cached = c["seq_lens_decoder"] - 1
+        rot = rope_table(32768, 128, 500000.0, dev)
+        sws = fd.append_attention_workspace(16, 16, 32, 8, 128, 512, dev)
+        sout = torch.empty((16, 32 * 128), dtype=torch.bfloat16, device=dev)
+
+        def sparse_step():
+            fd.append_attention(qkv, c["key_cache"], c["value_cache"], zeros, cached, ones, c["block_tables"], rot,
+                                c["cache_k_scale"], c["cache_v_scale"], num_heads=32, kv_num_heads=8, max_chunk=0,
+                                cache_quant_type="cache_fp8", cu_seqlens_q=cu, workspace=sws, out=sout, sqattn_top_k=64)
+        ms = time_events(sparse_step, max(args.steps // 4, 5), 3)
+        line("configs[3] as one call per step: cache write + selector + sparse decode", ms, "hbm",
+             16 * 32768 * 8 * 128 + 16 * 8 * 64 * 64 * 128 * 2, HBM_PEAK_GBPS, "GB/s")
 
     if args.workload in ("prefill", "all"):
         # configs[4]: batch 2, 2048 new tokens on 8192 cached (int8 paged), causal

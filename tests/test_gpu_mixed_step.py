@@ -147,9 +147,10 @@ def test_mixed_step_with_key_splits_for_the_prefill_row(oracle):
     assert ok, "small workspace: %d out of tolerance, max %.4g" % (bad, mx)
 
 
-def test_mixed_step_with_key_splits_replays_from_a_hip_graph():
-    """The mixed step with key splits (writer, decode + its merge, prefill shares, prefill merge) captured in a HIP
-    graph: every replay, with eager work and synchronisations in between, equals the eager step on a copy of the
+@pytest.mark.parametrize("top_k", [None, 8])
+def test_mixed_step_with_key_splits_replays_from_a_hip_graph(top_k):
+    """The mixed step with key splits (writer, decode + its merge - with top_k the block selector and the sparse
+    decode instead -, prefill shares, prefill merge) captured in a HIP graph: every replay, with eager work and synchronisations in between, equals the eager step on a copy of the
     state bit for bit (outputs and cache bytes)."""
     enc, dec = [0, 160, 0, 0, 0], [900, 4200, 63, 2100, 4600]
     c = mixed_case(enc, dec, CACHE_INT8, seed=21, max_pos=8192)
@@ -166,7 +167,7 @@ def test_mixed_step_with_key_splits_replays_from_a_hip_graph():
                                    s["seq_lens_decoder"], s["seq_lens_this_time"], s["block_tables"],
                                    (s["rope_cos"], s["rope_sin"]), s["cache_k_scale"], s["cache_v_scale"],
                                    num_heads=32, kv_num_heads=8, max_chunk=160, cu_seqlens_q=s["cu_seqlens_q"],
-                                   prefill_rows=1, workspace=ws)
+                                   prefill_rows=1, workspace=ws, sqattn_top_k=top_k)
 
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
