@@ -195,6 +195,34 @@ def other_workloads(args):
                  {"note": "roofline counts the decode rows' K/V bytes only; the prefill row adds %.1f GFLOP" %
                           (syn.prefill_flops(8192, 512) / 1e9)})
         del c
+    if args.workload in ("speculative", "all"):
+        # a speculative step: the 64 sequences of configs[1] bring 2 tokens each (the last two of their ctx), one call;
+        # as decode rows of two tokens (one pass of the decode kernel) and as prefill rows of two tokens
+        from fastdeploy_amd.rope import rope_table
+        lens = torch.randint(3584, 4609, (64,), generator=torch.Generator().manual_seed(0)).tolist()
+        c = syn.decode_case(batch=64, ctx=lens, pool_blocks=6000, seed=0, device=dev, direct_bytes=True, max_blocks=72)
+        g = torch.Generator(device=dev).manual_seed(5)
+        qkv = torch.randn((128, 48 * 128), generator=g, device=dev).to(torch.bfloat16)
+        zeros = torch.zeros(64, dtype=torch.int32, device=dev)
+        twos = torch.full((64,), 2, dtype=torch.int32, device=dev)
+        cu = torch.arange(0, 129, 2, dtype=torch.int32, device=dev)
+        cached = c["seq_lens_decoder"] - 2
+        rot = rope_table(8192, 128, 500000.0, dev)
+        sws = fd.append_attention_workspace(128, 64, 32, 8, 128, 72, dev)
+        sout = torch.empty((128, 32 * 128), dtype=torch.bfloat16, device=dev)
+
+        def spec(enc, **kw):
+            fd.append_attention(qkv, c["key_cache"], c["value_cache"], enc, cached, twos, c["block_tables"], rot,
+                                c["cache_k_scale"], c["cache_v_scale"], num_heads=32, kv_num_heads=8,
+                                cu_seqlens_q=cu, workspace=sws, out=sout, **kw)
+        nbytes = syn.decode_algorithmic_bytes(lens, 64) + 128 * (48 * 128 * 2 + 2 * 8 * 128) + 64 * 32 * 128 * 2 * 2
+        ms = time_events(lambda: spec(zeros, max_chunk=0, decode_tokens=2), args.steps, args.warmup)
+        line("speculative step, 64 x 2 tokens on ctx ~4k as decode rows of two tokens (write + one decode pass)", ms,
+             "hbm", nbytes, HBM_PEAK_GBPS, "GB/s")
+        ms = time_events(lambda: spec(twos, max_chunk=2), args.steps, 30)
+        line("the same step as prefill rows of two tokens (write + packed append attention)", ms, "hbm", nbytes,
+             HBM_PEAK_GBPS, "GB/s")
+        del c
     if args.workload in ("dynamic", "all"):
         # the formats with one scale per stored row: configs[1]'s decode (two pools rotated, as the headline run) and
         # the prefill-sized cache write; the scale caches add 2 x 4 B per token and KV head to the bytes moved
@@ -280,7 +308,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--pools", type=int, default=2, help="distinct cache pools rotated between steps")
-    ap.add_argument("--workload", default="decode", choices=["decode", "write_decode", "sqattn", "prefill", "mixed", "dynamic", "kv_wire", "all"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "write_decode", "sqattn", "prefill", "mixed", "speculative", "dynamic", "kv_wire", "all"],
                     help="decode = the headline metric (default); the others print one line per kernel of that row")
     ap.add_argument("--calibrate", action="store_true",
                     help="kept for the profiling command line: the 1 GiB device copy (the yardstick the HBM byte "

@@ -19,7 +19,13 @@ static StepWorkspace step_workspace(int num_tokens, int batch, int hq, int hkv, 
   w.v_new = w.k_new + align256((size_t)num_tokens * hkv * d * 2);
   w.decode = w.v_new + align256((size_t)num_tokens * hkv * d * 2);
   // the block selector's scores and bounds, then its result (kept blocks - at most every block - and counts)
-  w.select = w.decode + align256(fdattn_decode_workspace_bytes(batch, hq, hkv, d, max_blocks));
+  // (decode partials: room for 8 rows per KV head, which decode rows of several tokens may use)
+  size_t dec = fdattn_decode_workspace_bytes(batch, hq, hkv, d, max_blocks);
+  if (hq % hkv == 0 && hq / hkv <= 8) {
+    const size_t spec = c8_workspace_bytes(batch, hkv, max_blocks, 8);
+    if (spec > dec) dec = spec;
+  }
+  w.select = w.decode + align256(dec);
   w.kept = w.select + align256(fdattn_sqattn_workspace_bytes(batch, hkv, max_blocks));
   w.split = w.kept + align256((size_t)batch * hkv * ((size_t)max_blocks + 1) * sizeof(int32_t));
   w.total = w.split + align256(prefill_split_workspace_bytes(num_tokens, hq, prefill_splits));
@@ -79,6 +85,17 @@ extern "C" int fdattn_append_attention_ex(
   if (workspace_bytes < w.total)
     return fail(FDATTN_ERR_WORKSPACE, "fdattn_append_attention: workspace %zu B < required %zu B", workspace_bytes,
                 w.total);
+  // what the decode rows ask for, checked before anything is written
+  const int top_k = extras && extras->sqattn_top_k > 0 ? (extras->sqattn_top_k < max_blocks_per_seq ? extras->sqattn_top_k : max_blocks_per_seq) : 0;
+  const int decode_tokens = extras && extras->decode_tokens > 1 ? extras->decode_tokens : 1;
+  if (decode_tokens > 1 && (top_k > 0 || !c8_supported(hq, hkv, head_dim, block_size, cache_quant_type) ||
+                            decode_tokens * (hq / hkv) > 8))
+    return fail(FDATTN_ERR_SHAPE, "fdattn_append_attention: decode_tokens %d needs head_dim 128, block_size 64, "
+                "decode_tokens x query heads per KV head <= 8, and no sqattn_top_k", decode_tokens);
+  if (top_k > 0 && (!c8_supported(hq, hkv, head_dim, block_size, cache_quant_type) ||
+                    !sqattn_fast_supported(hq, hkv, head_dim, block_size, max_blocks_per_seq)))
+    return fail(FDATTN_ERR_SHAPE, "fdattn_append_attention: sqattn_top_k needs head_dim 128, block_size 64, at most 8 "
+                "query heads per KV head and at most 2048 blocks per sequence");
   char* ws = (char*)workspace;
   void* q_rot = ws + w.q_rot;
   const bool any_prefill = max_chunk > 0;  // the caller's word: 0 = no sequence has seq_lens_encoder > 0
@@ -94,14 +111,9 @@ extern "C" int fdattn_append_attention_ex(
   const RowMap rows{cu_seqlens_q, seq_lens_encoder};
   const size_t dws = w.select - w.decode;
   hipStream_t s = (hipStream_t)stream;
-  const int top_k = extras && extras->sqattn_top_k > 0 ? (extras->sqattn_top_k < max_blocks_per_seq ? extras->sqattn_top_k : max_blocks_per_seq) : 0;
   if (top_k > 0) {
     // block-sparse decode rows: select with the new query over the cache as the writer left it, then attend to
     // the kept blocks only
-    if (!c8_supported(hq, hkv, head_dim, block_size, cache_quant_type) ||
-        !sqattn_fast_supported(hq, hkv, head_dim, block_size, max_blocks_per_seq))
-      return fail(FDATTN_ERR_SHAPE, "fdattn_append_attention: sqattn_top_k needs head_dim 128, block_size 64, at most 8 "
-                  "query heads per KV head and at most 2048 blocks per sequence");
     int32_t* kept = (int32_t*)(ws + w.kept);
     int32_t* counts = kept + (size_t)batch * hkv * top_k;
     rc = sqattn_select_launch(q_rot, key_cache, cache_k_scale, block_tables, seq_lens_decoder, seq_lens_this_time, kept,
@@ -115,7 +127,7 @@ extern "C" int fdattn_append_attention_ex(
     rc = decode_c8_launch(q_rot, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
                           seq_lens_decoder, seq_lens_this_time, nullptr, nullptr, 0, out, ws + w.decode, dws, batch,
                           hq, hkv, head_dim, block_size, max_blocks_per_seq, num_blocks, cache_quant_type,
-                          softmax_scale, s, 3, rows);
+                          softmax_scale, s, 3, rows, decode_tokens);
   else
     rc = decode_generic_launch(q_rot, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
                                seq_lens_decoder, seq_lens_this_time, nullptr, nullptr, 0, out, ws + w.decode, dws,

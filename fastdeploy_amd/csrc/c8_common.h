@@ -141,13 +141,20 @@ struct PairRaw {
 
 // k_scale: the per-channel K scales [hkv, 128], or NULL (all ones: the scales are per stored row and are applied
 // to the scores).  group: query heads per KV head; set: which four of them (heads 4 set .. 4 set + 3; heads
-// past the group read as zeros).
+// past the group read as zeros).  toks > 0: the sequence owns q rows row .. row + toks - 1 and the MFMA rows are
+// (token, head) in that order - row 4 set + i is token (4 set + i) / group, head (4 set + i) % group; rows of
+// tokens past toks read as zeros.
 __device__ __forceinline__ PairRaw load_pair_issue(const uint16_t* q, const float* k_scale, int hkv, int p, int row, int lane,
-                                                   int group = kG, int set = 0) {
-  const int h = p % hkv;  // row: the sequence's row of q
-  const int m = lane & 15, g = lane >> 4, head = 4 * set + (m >> 2);
-  const bool live = head < group;
-  const uint16_t* qrow = q + ((size_t)row * hkv * group + h * group + (live ? head : 0)) * kD;
+                                                   int group = kG, int set = 0, int toks = 0) {
+  const int h = p % hkv;  // row: the sequence's (first) row of q
+  const int m = lane & 15, g = lane >> 4;
+  int head = 4 * set + (m >> 2), tok = 0;
+  if (toks > 0) {
+    tok = head / group;
+    head -= tok * group;
+  }
+  const bool live = toks > 0 ? tok < toks : head < group;
+  const uint16_t* qrow = q + ((size_t)(row + (live ? tok : 0)) * hkv * group + h * group + (live ? head : 0)) * kD;
   const float* ks = k_scale + (size_t)h * kD;
   PairRaw r;
 #pragma unroll

@@ -66,6 +66,7 @@ struct C8Args {
   float sm_scale_log2;  // softmax_scale * log2(e)
   int dyn;              // scales per stored row: the output takes no per-channel V scale
   int group;            // query heads per KV head, 1 .. 8
+  int max_tokens;       // tokens a decode row may bring (1; speculative steps: up to 8 / group)
 };
 
 // Length of the pair's block list: every block of the sequence, or the kept ones.
@@ -77,7 +78,10 @@ __device__ __forceinline__ int pair_units(const C8Args& a, int p, int kv_len) {
 
 // NSET: row sets of 4 query heads a wavefront carries (1: up to 4 query heads per KV head, 2: up to 8); every K
 // and V operand read from LDS feeds the MFMAs of all sets.
-template <int QUANT, bool SPARSE, bool DYN, int NSET>
+// SPEC: a decode row may bring several tokens (a speculative step's drafts, all in the cache already): the MFMA
+// rows are then (token, head) pairs - row v is token v / group, head v % group - and token t of T attends to the
+// sequence's cached tokens and the new ones up to itself, i.e. to T - 1 - t fewer than the last one.
+template <int QUANT, bool SPARSE, bool DYN, int NSET, bool SPEC = false>
 __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
   __shared__ __attribute__((aligned(16))) uint8_t ldsK[kWaves][kTileB];
   __shared__ __attribute__((aligned(16))) uint8_t ldsV[kWaves][kTileB];
@@ -110,20 +114,25 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
       lb[e] = l;
     }
   }
-  int row;
-  if (!decode_row(a.rows, b, row)) return;
+  int row, toks = 1;
+  if (SPEC ? !decode_rows(a.rows, b, a.max_tokens, row, toks) : !decode_row(a.rows, b, row)) return;
   PairRaw raw[NSET];  // in flight with the table entries
 #pragma unroll
-  for (int t = 0; t < NSET; ++t) raw[t] = load_pair_issue(a.q, DYN ? nullptr : a.k_scale, a.hkv, p, row, lane, a.group, t);
+  for (int t = 0; t < NSET; ++t)
+    raw[t] = load_pair_issue(a.q, DYN ? nullptr : a.k_scale, a.hkv, p, row, lane, a.group, t, SPEC ? toks : 0);
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
   const int n_p = pair_units<SPARSE>(a, p, kv_len);
   const int cnt = min(a.chunk, n_p - first);  // <= 0: past the end of this pair's list
   const bool single = n_p <= a.chunk;
-  // q / out row of query head `head` of this pair
-  auto out_row = [&](int head) { return a.out + ((size_t)row * a.hkv * a.group + h * a.group + head) * kD; };
+  const int vg = a.group * toks;  // MFMA rows in use: (token, head) pairs
+  // q / out row of MFMA row `head` of this pair (SPEC: token head / group, head head % group)
+  auto out_row = [&](int head) {
+    const int tok = SPEC ? head / a.group : 0;
+    return a.out + ((size_t)(row + tok) * a.hkv * a.group + h * a.group + (head - tok * a.group)) * kD;
+  };
   if (cnt <= 0) {
     if (n_p == 0 && ck == 0) {  // empty sequence: its output rows are zeros
-      for (int head = threadIdx.x >> 6; head < a.group; head += kWaves)
+      for (int head = threadIdx.x >> 6; head < vg; head += kWaves)
         *reinterpret_cast<u32*>(out_row(head) + (threadIdx.x & 63) * 2) = 0u;
     }
     return;
@@ -145,7 +154,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
     for (int e = 0; e < 2; ++e)
       if (lane + 64 * e < cnt && pb_raw[e] >= 0 && pb_raw[e] < a.num_blocks) {
         my_pb[e] = pb_raw[e];
-        my_valid[e] = min(max(kv_len - lb[e] * kBS, 0), kBS);
+        // SPEC: not cut at the block's size, so that an earlier token's smaller count can be taken from it
+        my_valid[e] = min(max(kv_len - lb[e] * kBS, 0), SPEC ? kBS + 8 : kBS);
       }
   }
   // entry of unit j (uniform)
@@ -168,6 +178,12 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
       dma_row64(a.v_scale + srow, saddr + 4 * kBS, lane_x4);
     }
   };
+
+  // SPEC: this lane's score row of set t is MFMA row 4 t + g4 = token (4 t + g4) / group, which sees
+  // toks - 1 - token fewer keys than the sequence's last token (rows of absent tokens: as the last one)
+  int fewer[NSET];
+#pragma unroll
+  for (int t = 0; t < NSET; ++t) fewer[t] = SPEC ? max(toks - 1 - (4 * t + g4) / a.group, 0) : 0;
 
   PairState st[NSET];
 #pragma unroll
@@ -253,7 +269,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
           else
             s = st[t].rs * ((Sf[t][stl].x + Sf[t][stl].y) + (Sf[t][stl].z + Sf[t][stl].w));
           if (DYN) s *= kt[stl];
-          s = (4 * n16 + stl < valid) ? s : -INFINITY;  // (a slot past the end may hold any scale, NaN included)
+          s = (4 * n16 + stl < valid - fewer[t]) ? s : -INFINITY;  // (a slot past the end may hold any scale, NaN included)
           sv[stl] = s;
           mb = fmaxf(mb, s);
         }
@@ -389,7 +405,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
 #pragma unroll
   for (int t = 0; t < NSET; ++t) {
     const int tid = threadIdx.x, hs = tid >> 6, head = 4 * t + hs, c2 = (tid & 63) * 2;
-    if (head >= a.group) continue;
+    if (head >= vg) continue;
     float M = -INFINITY;
 #pragma unroll
     for (int w2 = 0; w2 < kWaves; ++w2) M = fmaxf(M, reinterpret_cast<const float*>(ldsP[w2][t])[hs]);
@@ -430,11 +446,14 @@ __global__ __launch_bounds__(kWaves * 64, 2) void decode_c8_kernel(C8Args a) {
 template <bool SPARSE>
 __global__ __launch_bounds__(256) void decode_c8_combine_kernel(C8Args a) {
   __shared__ float red[kWaves][2 + 2 * 64];  // per wavefront: m, l, o[64][2]
-  const int p = blockIdx.x / a.group, head = blockIdx.x - p * a.group, tid = threadIdx.x;
+  const int vgmax = a.group * a.max_tokens;  // MFMA rows of a pair: (token, head), token-major
+  const int p = blockIdx.x / vgmax, head = blockIdx.x - p * vgmax, tid = threadIdx.x;
   const int b = p / a.hkv, h = p - b * a.hkv;
-  const int sets = (a.group + kG - 1) / kG, set = head >> 2, hs = head & 3;  // the partial's layout: see the main kernel
-  int row;
-  if (!decode_row(a.rows, b, row)) return;
+  const int sets = (vgmax + kG - 1) / kG, set = head >> 2, hs = head & 3;  // the partial's layout: see the main kernel
+  int row, toks;
+  if (!decode_rows(a.rows, b, a.max_tokens, row, toks)) return;
+  const int tok = head / a.group;
+  if (tok >= toks) return;
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
   const int n_p = pair_units<SPARSE>(a, p, kv_len);
   if (n_p <= a.chunk) return;
@@ -492,7 +511,7 @@ __global__ __launch_bounds__(256) void decode_c8_combine_kernel(C8Args a) {
   const float inv = Lt > 0.f ? 1.0f / Lt : 0.f;
   r0 *= inv * (a.dyn ? 1.f : a.v_scale[h * kD + c2]);
   r1 *= inv * (a.dyn ? 1.f : a.v_scale[h * kD + c2 + 1]);
-  uint16_t* o = a.out + ((size_t)row * a.hkv * a.group + h * a.group + head) * kD + c2;
+  uint16_t* o = a.out + ((size_t)(row + tok) * a.hkv * a.group + h * a.group + (head - tok * a.group)) * kD + c2;
   *reinterpret_cast<u32*>(o) = (u32)f32_to_bf16(r0) | ((u32)f32_to_bf16(r1) << 16);
 }
 
@@ -542,7 +561,8 @@ namespace {
 
 template <int QUANT, bool DYN, int NSET>
 void launch_main(bool sparse, dim3 grid, dim3 block, hipStream_t s, const C8Args& a) {
-  if (sparse) hipLaunchKernelGGL((decode_c8_kernel<QUANT, true, DYN, NSET>), grid, block, 0, s, a);
+  if (a.max_tokens > 1) hipLaunchKernelGGL((decode_c8_kernel<QUANT, false, DYN, NSET, true>), grid, block, 0, s, a);
+  else if (sparse) hipLaunchKernelGGL((decode_c8_kernel<QUANT, true, DYN, NSET>), grid, block, 0, s, a);
   else hipLaunchKernelGGL((decode_c8_kernel<QUANT, false, DYN, NSET>), grid, block, 0, s, a);
 }
 
@@ -561,16 +581,20 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
                      const int32_t* seq_lens_this_time, const int32_t* kept_blocks, const int32_t* kept_counts,
                      int max_kept, void* out, void* workspace, size_t workspace_bytes, int batch, int hq,
                      int hkv, int d, int bs, int max_blocks, int num_blocks, int quant, float sm_scale,
-                     hipStream_t s, int stages, RowMap rows) {
+                     hipStream_t s, int stages, RowMap rows, int max_tokens) {
   (void)d; (void)bs;
   const bool sparse = kept_blocks != nullptr;
-  const int pairs = batch * hkv, group = hq / hkv, sets = (group + kG - 1) / kG;
+  if (max_tokens < 1) max_tokens = 1;
+  const int pairs = batch * hkv, group = hq / hkv, vgmax = group * max_tokens, sets = (vgmax + kG - 1) / kG;
+  if (max_tokens > 1 && (sparse || !rows.cu_seqlens_q || vgmax > kG * kMaxSets))
+    return fail(FDATTN_ERR_SHAPE, "fdattn_decode_attention: decode rows of up to %d tokens need a dense step with "
+                "tokens x query heads per KV head <= %d (here %d)", max_tokens, kG * kMaxSets, vgmax);
   const int max_units = sparse ? (max_kept < max_blocks ? max_kept : max_blocks) : max_blocks;
   const int chunk = c8_pick_chunk(pairs, max_units);
   const int cpp = ((max_units + chunk - 1) / chunk);
   if (pairs > kMaxPairs)
     return fail(FDATTN_ERR_SHAPE, "fdattn_decode_attention: batch*kv_heads = %d exceeds %d", pairs, kMaxPairs);
-  if ((long long)pairs * (cpp > group ? cpp : group) > 0x7fffffffLL)
+  if ((long long)pairs * (cpp > vgmax ? cpp : vgmax) > 0x7fffffffLL)
     return fail(FDATTN_ERR_SHAPE, "fdattn_decode_attention: %d pairs x %d chunks exceed the grid limit", pairs, cpp);
   const size_t slots = (size_t)pairs * cpp;
   const size_t need = slots * sets * (kSlotFloats + 8) * sizeof(float);
@@ -581,7 +605,7 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
   C8Args a{(const uint16_t*)q, (const uint8_t*)key_cache, (const uint8_t*)value_cache, k_scale, v_scale,
            block_tables, seq_lens_decoder, seq_lens_this_time, kept_blocks, kept_counts, max_kept, part_o,
            part_ml, (uint16_t*)out, rows, batch, hkv, max_blocks, num_blocks, chunk, cpp,
-           sm_scale * 1.4426950408889634f, quant_dynamic(quant) ? 1 : 0, group};
+           sm_scale * 1.4426950408889634f, quant_dynamic(quant) ? 1 : 0, group, max_tokens};
   const dim3 grid(cpp * pairs), block(kWaves * 64);
   if (stages & 1) {
     if (sets == 1) launch_main_sets<1>(quant, sparse, grid, block, s, a);
@@ -590,8 +614,8 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
   int rc = check_launch("fdattn_decode_attention (mfma)");
   if (rc || !(stages & 2)) return rc;
   if (cpp == 1) return 0;  // every pair was one chunk and has been finished by the main kernel
-  if (sparse) hipLaunchKernelGGL(decode_c8_combine_kernel<true>, dim3(pairs * group), dim3(256), 0, s, a);
-  else hipLaunchKernelGGL(decode_c8_combine_kernel<false>, dim3(pairs * group), dim3(256), 0, s, a);
+  if (sparse) hipLaunchKernelGGL(decode_c8_combine_kernel<true>, dim3(pairs * vgmax), dim3(256), 0, s, a);
+  else hipLaunchKernelGGL(decode_c8_combine_kernel<false>, dim3(pairs * vgmax), dim3(256), 0, s, a);
   return check_launch("fdattn_decode_attention (merge)");
 }
 

@@ -26,6 +26,16 @@ __device__ __forceinline__ bool decode_row(const RowMap& m, int b, int& row) {
   row = m.cu_seqlens_q[b];
   return m.cu_seqlens_q[b + 1] - row == 1 && (!m.seq_lens_encoder || m.seq_lens_encoder[b] == 0);
 }
+// The same for steps whose decode rows may bring up to max_tokens tokens (the draft tokens of a speculative step):
+// toks = the sequence's tokens; row = the first of its q / out rows.
+__device__ __forceinline__ bool decode_rows(const RowMap& m, int b, int max_tokens, int& row, int& toks) {
+  row = b;
+  toks = 1;
+  if (!m.cu_seqlens_q) return true;
+  row = m.cu_seqlens_q[b];
+  toks = m.cu_seqlens_q[b + 1] - row;
+  return toks >= 1 && toks <= max_tokens && (!m.seq_lens_encoder || m.seq_lens_encoder[b] == 0);
+}
 __device__ __forceinline__ bool prefill_row(const RowMap& m, int b) {
   return !m.seq_lens_encoder || m.seq_lens_encoder[b] > 0;
 }

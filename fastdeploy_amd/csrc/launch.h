@@ -27,7 +27,8 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
                      const int32_t* kept_blocks, const int32_t* kept_counts, int max_kept,
                      void* out, void* workspace, size_t workspace_bytes, int batch, int hq,
                      int hkv, int d, int bs, int max_blocks, int num_blocks, int quant,
-                     float sm_scale, hipStream_t s, int stages, RowMap rows = RowMap{nullptr, nullptr});
+                     float sm_scale, hipStream_t s, int stages, RowMap rows = RowMap{nullptr, nullptr},
+                     int max_tokens = 1);
 // the block selector on the decode rows of a mixed step (rows), MFMA shapes only
 bool sqattn_fast_supported(int hq, int hkv, int d, int bs, int max_blocks);
 int sqattn_select_launch(const void* q, const void* key_cache, const float* cache_k_scale, const int32_t* block_tables,

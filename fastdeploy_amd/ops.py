@@ -94,9 +94,12 @@ def _scales(cache_k_scale, cache_v_scale, hkv, d, quant=CACHE_INT8, nb=0, bs=0):
     return pk, pv
 
 
-def _extras(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, width, d, prefill_rows=0, sqattn_top_k=0):
-    """fdattn_step_extras for the optional projection epilogue / prefill splits / block-sparse decode rows, or None"""
-    if qkv_bias is None and q_norm_weight is None and k_norm_weight is None and prefill_rows <= 0 and sqattn_top_k <= 0:
+def _extras(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, width, d, prefill_rows=0, sqattn_top_k=0,
+            decode_tokens=0):
+    """fdattn_step_extras for the optional projection epilogue / prefill splits / block-sparse decode rows / decode
+    rows of several tokens, or None"""
+    if (qkv_bias is None and q_norm_weight is None and k_norm_weight is None and prefill_rows <= 0
+            and sqattn_top_k <= 0 and decode_tokens <= 1):
         return None
     pb = _chk(qkv_bias, "qkv_bias", torch.bfloat16, 1, optional=True)
     if qkv_bias is not None and qkv_bias.numel() != width:
@@ -106,7 +109,8 @@ def _extras(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, width, d, pref
     for name, t in (("q_norm_weight", q_norm_weight), ("k_norm_weight", k_norm_weight)):
         if t is not None and t.numel() != d:
             raise ValueError("%s has %d entries, head_dim is %d" % (name, t.numel(), d))
-    return _lib.StepExtras(pb or None, pq or None, pk or None, float(rms_norm_eps), int(prefill_rows), int(sqattn_top_k))
+    return _lib.StepExtras(pb or None, pq or None, pk or None, float(rms_norm_eps), int(prefill_rows), int(sqattn_top_k),
+                           int(decode_tokens))
 
 
 def prefill_auto_splits(rows, num_heads, max_chunk, kv_num_heads=None):
@@ -393,7 +397,8 @@ def append_attention(qkv, key_cache, value_cache, seq_lens_encoder, seq_lens_dec
                      block_tables, rotary_embs, cache_k_scale, cache_v_scale, *, num_heads, kv_num_heads,
                      max_chunk, rope_style="neox", cache_quant_type="cache_int8", softmax_scale=None,
                      cu_seqlens_q=None, workspace=None, out=None, qkv_bias=None, q_norm_weight=None,
-                     k_norm_weight=None, rms_norm_eps=1e-6, prefill_rows=None, sqattn_top_k=None):
+                     k_norm_weight=None, rms_norm_eps=1e-6, prefill_rows=None, sqattn_top_k=None,
+                     decode_tokens=None):
     """One attention step of a layer over a mixed batch (one call into the library):
     every new token is rotated and written to the cache, decode rows (one token,
     seq_lens_encoder == 0) attend to the cache, prefill rows (seq_lens_encoder > 0)
@@ -406,6 +411,9 @@ def append_attention(qkv, key_cache, value_cache, seq_lens_encoder, seq_lens_dec
     num_heads, max_chunk, kv_num_heads) workgroups (as many as a workspace passed in has room for).
     sqattn_top_k: > 0 makes the decode rows block-sparse - the selector keeps that many blocks per (row, KV head),
     scored with the row's new query, and the decode attention reads only those (MFMA selector shapes only).
+    decode_tokens: > 1 makes rows with seq_lens_encoder 0 and up to that many tokens (speculative drafts) decode rows:
+    token t attends to the cached tokens and the new ones up to itself, all read from the cache, in one decode pass
+    (head_dim 128, block_size 64, decode_tokens x heads per KV head <= 8).
     Returns bf16 [num_tokens, num_heads*head_dim]."""
     nb, hkv, bs, d = _cache_dims(key_cache, value_cache)
     if hkv != kv_num_heads:
@@ -453,7 +461,7 @@ def append_attention(qkv, key_cache, value_cache, seq_lens_encoder, seq_lens_dec
         workspace = torch.empty(need, dtype=torch.uint8, device=qkv.device)
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(d)
     ep = _extras(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, qkv.shape[1], d, prefill_rows or 0,
-                 sqattn_top_k or 0)
+                 sqattn_top_k or 0, decode_tokens or 0)
     rc = _lib.lib().fdattn_append_attention_ex(
         p_qkv, p_kc, p_vc, p_ks, p_vs, p_cos, p_sin, p_bt, p_enc, p_dec, p_this, p_cu,
         _chk(out, "out", torch.bfloat16), workspace.data_ptr(), workspace.numel() * workspace.element_size(),

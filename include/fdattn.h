@@ -133,6 +133,14 @@ FDATTN_API int fdattn_write_cache_kv(
  *                   attention reads only those (fdattn_decode_attention_sparse); rows with no more blocks
  *                   than that keep all.  Shapes of the MFMA selector only.  The step's workspace always has
  *                   room for it.  0: dense.
+ *   decode_tokens   (fdattn_append_attention_ex only) > 1: a row with seq_lens_encoder[b] == 0 and 2 ..
+ *                   decode_tokens tokens - the draft tokens of a speculative step - is a decode row too: all
+ *                   its tokens are written to the cache first, then token t (0-based) attends to the
+ *                   seq_lens_decoder[b] + t + 1 first tokens of the sequence, read from the cache (so, unlike a
+ *                   prefill row's, its own keys and values are the quantised ones).  One pass of the decode
+ *                   kernel serves all the tokens of a row.  Needs head_dim 128, block_size 64 and
+ *                   decode_tokens x (query heads per KV head) <= 8; not together with sqattn_top_k.  0 / 1: such
+ *                   rows get no attention output (they are prefill rows if seq_lens_encoder says so).
  */
 typedef struct fdattn_step_extras {
   const void* qkv_bias;
@@ -141,6 +149,7 @@ typedef struct fdattn_step_extras {
   float rms_norm_eps;
   int prefill_rows;
   int sqattn_top_k;
+  int decode_tokens;
 } fdattn_step_extras;
 
 /* fdattn_write_cache_kv with the extras (host pointer, read during the call; NULL = none). */
@@ -397,7 +406,8 @@ FDATTN_API size_t fdattn_append_attention_workspace_bytes_ex(int num_tokens, int
  * A row that brings several tokens with causal attention among them - a prompt chunk, or the
  * draft tokens of a speculative step - is a prefill row: give it seq_lens_encoder[b] = its
  * number of tokens (a row with several tokens and seq_lens_encoder[b] == 0 gets its tokens
- * written to the cache but no attention output).
+ * written to the cache but no attention output, unless fdattn_step_extras.decode_tokens makes
+ * it a decode row of several tokens).
  * Every new token is first rotated and written to the cache (fdattn_write_cache_kv).
  * max_chunk bounds the tokens of a prefill row in this step; 0 says that the step has no
  * prefill row (the prefill pass is then not launched at all).

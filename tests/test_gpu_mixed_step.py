@@ -13,11 +13,11 @@ from fastdeploy_amd.rope import rope_table
 pytestmark = pytest.mark.gpu
 
 
-def mixed_case(enc, dec, quant, seed, hq=32, hkv=8, d=128, bs=64, max_pos=4096):
+def mixed_case(enc, dec, quant, seed, hq=32, hkv=8, d=128, bs=64, max_pos=4096, this=None):
     g = torch.Generator().manual_seed(seed)
     batch = len(enc)
     enc_t, dec_t = torch.tensor(enc, dtype=torch.int32), torch.tensor(dec, dtype=torch.int32)
-    this = seq_lens_this_time_of(enc_t, dec_t)
+    this = seq_lens_this_time_of(enc_t, dec_t) if this is None else torch.tensor(this, dtype=torch.int32)
     cu = cu_seqlens_of(this)
     T = int(cu[-1])
     mb = max((int(dec[b]) + int(this[b]) + bs - 1) // bs for b in range(batch)) + 1
@@ -290,6 +290,64 @@ def test_mixed_step_with_block_sparse_decode_rows(oracle, quant):
     assert not torch.equal(dense[0], out[0]) and torch.equal(dense[cu[1]:cu[2]], out[cu[1]:cu[2]])
     ok, mx, bad = bf16_close(bits(out[int(cu[4])]), bits(dense[int(cu[4])]))   # 4 blocks <= top_k: the row keeps them all
     assert ok
+
+
+@pytest.mark.parametrize("quant,hq,hkv,tokens", [(CACHE_INT8, 32, 8, 2), (CACHE_FP8, 32, 8, 2), (CACHE_INT8_DYNAMIC, 32, 8, 2),
+                                                 (CACHE_FP8_DYNAMIC, 16, 8, 4), (CACHE_INT8, 8, 8, 8),
+                                                 (CACHE_INT8, 24, 8, 2)])
+def test_mixed_step_with_decode_rows_of_several_tokens(oracle, quant, hq, hkv, tokens):
+    """decode_tokens in the one-call step: a row with seq_lens_encoder 0 and 2 .. decode_tokens tokens (speculative
+    drafts) is served by the decode kernel in one pass - token t attends to cached + t + 1 tokens, all read back from
+    the quantised cache.  Against the oracle: its writer, then one decode per token with that token's length (block
+    boundaries inside the new tokens, a first step on an empty cache, rows of fewer tokens, a long row in several
+    chunks); the prefill row and the one-token rows as ever; rows with more tokens than decode_tokens get none."""
+    T = tokens
+    enc = [0, 40, 0, 0, 0, 0, 0, 0]
+    dec = [63, 100, 0, 64 * 3 - 1, 500, 64 * 70 + 3, 64 * 2 - T + 1, 77]
+    this = [T, 40, T, T, 1, T, T - 1 if T > 2 else 1, T + 1]
+    c = mixed_case(enc, dec, quant, seed=50 + T, hq=hq, hkv=hkv, max_pos=8192, this=this)
+    dev = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
+    out = torch.full((c["T"], hq * 128), float("nan"), dtype=torch.bfloat16, device="cuda")
+    fd.append_attention(dev["qkv"], dev["key_cache"], dev["value_cache"], dev["seq_lens_encoder"],
+                        dev["seq_lens_decoder"], dev["seq_lens_this_time"], dev["block_tables"],
+                        (dev["rope_cos"], dev["rope_sin"]), dev["cache_k_scale"], dev["cache_v_scale"],
+                        num_heads=hq, kv_num_heads=hkv, max_chunk=40, cache_quant_type=quant,
+                        cu_seqlens_q=dev["cu_seqlens_q"], prefill_rows=1, decode_tokens=T, out=out)
+    torch.cuda.synchronize()
+    kc, vc = np_of(c["key_cache"]).copy(), np_of(c["value_cache"]).copy()
+    ks, vs = np_of(c["cache_k_scale"]).copy(), np_of(c["cache_v_scale"]).copy()
+    bt, cu, decs = np_of(c["block_tables"]), np_of(c["cu_seqlens_q"]), np_of(c["seq_lens_decoder"])
+    q, k_new, v_new = oracle.write_cache_kv(bits(c["qkv"]), kc, vc, ks, vs, np_of(c["rope_cos"]), np_of(c["rope_sin"]),
+                                            bt, decs, cu, hq, hkv, 128, 1, quant, want_kv_out=True)
+    assert np.array_equal(np_of(dev["key_cache"]), kc) and np.array_equal(np_of(dev["value_cache"]), vc)
+    got = bits(out)
+    for b in range(len(enc)):
+        rows = list(range(cu[b], cu[b + 1]))
+        if enc[b] > 0:
+            want = oracle.append_attention_prefill(q, k_new, v_new, kc, vc, ks, vs, bt, decs, cu, hq, hkv, 128, quant,
+                                                   token_ids=np.array(rows, np.int32))[rows]
+        elif this[b] <= T:   # every token of the row: one decode over its own length
+            want = oracle.decode_attention(np.ascontiguousarray(q[rows]), kc, vc, ks, vs,
+                                           np.ascontiguousarray(np.repeat(bt[b:b + 1], len(rows), 0)),
+                                           np.array([decs[b] + t + 1 for t in range(len(rows))], np.int32),
+                                           hq, hkv, 128, quant)
+        else:                # too many tokens for a decode row: written to the cache, no attention output
+            assert torch.isnan(out[rows].float()).all()
+            continue
+        ok, mx, bad = bf16_close(got[rows], want)
+        assert ok, "sequence %d: %d out of tolerance, max %.4g" % (b, bad, mx)
+
+
+def test_decode_tokens_argument_checks():
+    c = mixed_case([0, 0], [10, 20], CACHE_INT8, seed=1, this=[2, 2])
+    dev = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
+    for kw in (dict(decode_tokens=3), dict(decode_tokens=2, sqattn_top_k=4)):   # 3 x 4 rows > 8; not with the selector
+        with pytest.raises(ValueError):
+            fd.append_attention(dev["qkv"], dev["key_cache"], dev["value_cache"], dev["seq_lens_encoder"],
+                                dev["seq_lens_decoder"], dev["seq_lens_this_time"], dev["block_tables"],
+                                (dev["rope_cos"], dev["rope_sin"]), dev["cache_k_scale"], dev["cache_v_scale"],
+                                num_heads=32, kv_num_heads=8, max_chunk=0, cu_seqlens_q=dev["cu_seqlens_q"], **kw)
+    assert torch.equal(dev["key_cache"].cpu(), c["key_cache"])   # refused before anything was written
 
 
 def test_mixed_step_random_batches_against_the_oracle(oracle):
