@@ -40,6 +40,8 @@ class ForwardMeta:
     num_tokens: int = 0                          # filled by init_attention_metadata
     prefill_rows: Optional[int] = None           # exact count of rows with seq_lens_encoder > 0, if known (None: unknown)
     prefill_splits: int = 1                      # filled by init_attention_metadata
+    decode_tokens: int = 1                       # > 1: rows with seq_lens_encoder 0 and up to this many tokens
+                                                 # (speculative drafts) are decode rows, one decode pass for all
     extra: dict = field(default_factory=dict)
 
 
@@ -126,14 +128,16 @@ class AppendAttentionBackend:
             rope_style=self.rope_style, cache_quant_type=self.cache_quant_type, softmax_scale=self.softmax_scale,
             cu_seqlens_q=meta.cu_seqlens_q, workspace=self._workspace, out=out, qkv_bias=layer.qkv_bias,
             q_norm_weight=layer.q_norm_weight, k_norm_weight=layer.k_norm_weight, rms_norm_eps=layer.rms_norm_eps,
-            prefill_rows=meta.prefill_rows, sqattn_top_k=self.sqattn_top_k)
+            prefill_rows=meta.prefill_rows, sqattn_top_k=self.sqattn_top_k, decode_tokens=meta.decode_tokens)
 
 
 class SequenceBook:
     """Host-side bookkeeping of the sequence slots between steps: lengths, the block pool, and the
     ForwardMeta of the next step.  `schedule` takes the new tokens per slot ({slot: count}) - a count
-    above one, or any count for an empty slot, makes a prefill row - reserves blocks and returns the meta;
-    `commit` advances the lengths after the step has been enqueued.  A reservation that fails (ValueError: the
+    above one, or any count for an empty slot, makes a prefill row, unless the slot is named in `drafts`: its
+    tokens are then the draft tokens of a speculative step and the row is a decode row of several tokens -
+    reserves blocks and returns the meta; `commit` advances the lengths after the step has been enqueued (by the
+    accepted count for a slot whose drafts were partly rejected: the next step overwrites the rest).  A reservation that fails (ValueError: the
     pool is exhausted or a table row is full) leaves the slots reserved earlier in the same call with their
     blocks: finish a sequence or retry with fewer tokens."""
 
@@ -142,25 +146,32 @@ class SequenceBook:
         self.lengths = [0] * pool.max_seqs
         self._pending = None
 
-    def schedule(self, new_tokens: dict) -> ForwardMeta:
+    def schedule(self, new_tokens: dict, drafts=()) -> ForwardMeta:
         slots = self.pool.max_seqs
         enc, dec, this = [0] * slots, list(self.lengths), [0] * slots
+        decode_tokens = 1
         for s, n in new_tokens.items():
             if n <= 0:
                 continue
             self.pool.reserve(s, self.lengths[s] + n)          # all or nothing per slot; raises when the pool is full
             this[s] = n
-            if n > 1 or self.lengths[s] == 0:
+            if s in drafts and self.lengths[s] > 0:
+                decode_tokens = max(decode_tokens, n)
+            elif n > 1 or self.lengths[s] == 0:
                 enc[s] = n
         i32 = lambda v: torch.tensor(v, dtype=torch.int32).to(self.device)
         self._pending = this
         return ForwardMeta(i32(enc), i32(dec), i32(this), self.pool.block_tables_tensor(self.device),
                            max_enc_len_this_time=max(enc), num_tokens=sum(this),
-                           prefill_rows=sum(1 for n in enc if n > 0))
+                           prefill_rows=sum(1 for n in enc if n > 0), decode_tokens=decode_tokens)
 
-    def commit(self):
+    def commit(self, accepted=None):
+        """accepted: {slot: tokens of this step that stay} for speculative rows whose later drafts were rejected."""
         for s, n in enumerate(self._pending or []):
-            self.lengths[s] += n
+            keep = n if accepted is None or s not in accepted else accepted[s]
+            if not 0 <= keep <= n:
+                raise ValueError("slot %d: %d of %d tokens accepted" % (s, keep, n))
+            self.lengths[s] += keep
         self._pending = None
 
     def finish(self, slot):

@@ -33,8 +33,8 @@ def test_generation_over_steps_and_layers(oracle, quant):
         lay.append(be.allocate_layer(40, **extra) if is_dynamic(quant) else be.allocate_layer(40, ks, vs, **extra))
     cos, sin = (t.cpu() for t in be.rotary_embs)
 
-    def run_step(new_tokens):
-        meta = be.init_attention_metadata(book.schedule(new_tokens))
+    def run_step(new_tokens, drafts=(), accepted=None):
+        meta = be.init_attention_metadata(book.schedule(new_tokens, drafts))
         for l, layer in enumerate(lay):
             qkv = torch.randn((meta.num_tokens, 48 * d), generator=g).to(torch.bfloat16)
             before = dict(qkv=qkv, key_cache=layer.key_cache.cpu(), value_cache=layer.value_cache.cpu(),
@@ -48,14 +48,14 @@ def test_generation_over_steps_and_layers(oracle, quant):
             if layer.qkv_bias is not None:
                 ep = dict(qkv_bias=bits(layer.qkv_bias), q_norm_weight=np_of(layer.q_norm_weight),
                           k_norm_weight=np_of(layer.k_norm_weight), rms_norm_eps=layer.rms_norm_eps)
-            want, kc, vc = oracle_step(oracle, before, quant, **ep)
+            want, kc, vc = oracle_step(oracle, before, quant, decode_tokens=meta.decode_tokens, **ep)
             assert np.array_equal(np_of(layer.key_cache), kc) and np.array_equal(np_of(layer.value_cache), vc)
             if is_dynamic(quant):  # the scale caches follow the stored rows
                 assert np.array_equal(np_of(layer.cache_k_scale), before["scales_after"][0])
                 assert np.array_equal(np_of(layer.cache_v_scale), before["scales_after"][1])
             ok, mx, bad = bf16_close(bits(out), want)
             assert ok, "layer %d, step %r: %d out of tolerance, max %.4g" % (l, new_tokens, bad, mx)
-        book.commit()
+        book.commit(accepted)
 
     run_step({0: 150, 1: 3})                 # two prompts
     run_step({0: 1, 1: 1, 2: 200})           # both decode while a third prompt's first chunk arrives
@@ -65,4 +65,10 @@ def test_generation_over_steps_and_layers(oracle, quant):
     book.finish(1)
     run_step({0: 1, 2: 1, 3: 1, 4: 1})       # a one-token prompt in slot 4
     assert book.lengths == [154, 0, 279, 287, 1]
+    # a speculative step: slots 0 and 2 bring two draft tokens each (decode rows of two tokens), slot 3 decodes;
+    # slot 0's second draft is rejected, so its next token overwrites that position
+    run_step({0: 2, 2: 2, 3: 1}, drafts={0, 2}, accepted={0: 1})
+    assert book.lengths == [155, 0, 281, 288, 1]
+    run_step({0: 2, 2: 1, 3: 1}, drafts={0})
+    assert book.lengths == [157, 0, 282, 289, 1]
     assert pool.refcount(int(pool.block_tables[2, 0])) == 2

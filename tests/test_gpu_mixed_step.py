@@ -42,7 +42,7 @@ def mixed_case(enc, dec, quant, seed, hq=32, hkv=8, d=128, bs=64, max_pos=4096, 
                 rope_cos=cos, rope_sin=sin, T=T)
 
 
-def oracle_step(oracle, c, quant, hq=32, hkv=8, d=128, **epilogue):
+def oracle_step(oracle, c, quant, hq=32, hkv=8, d=128, decode_tokens=1, **epilogue):
     """The step composed from the oracle's pieces; returns (out bf16 bits [T, hq*d] with NaN-free rows only where
     a token exists, key cache, value cache).  For the dynamic formats the scale caches the step leaves behind are
     put into c["scales_after"]."""
@@ -54,13 +54,14 @@ def oracle_step(oracle, c, quant, hq=32, hkv=8, d=128, **epilogue):
     q, k_new, v_new = oracle.write_cache_kv(bits(c["qkv"]), kc, vc, ks, vs, np_of(c["rope_cos"]), np_of(c["rope_sin"]),
                                             bt, dec, cu, hq, hkv, d, 1, quant, want_kv_out=True, **epilogue)
     out = np.zeros((c["T"], hq * d), np.uint16)
-    drows = [b for b in range(len(enc)) if enc[b] == 0 and this[b] == 1]
+    # decode rows: every token (one; up to decode_tokens in a speculative step) attends to the cache up to itself
+    drows = [(b, t) for b in range(len(enc)) if enc[b] == 0 and 1 <= this[b] <= decode_tokens for t in range(this[b])]
     if drows:
-        qd = np.ascontiguousarray(q[[cu[b] for b in drows]])
-        od = oracle.decode_attention(qd, kc, vc, ks, vs, np.ascontiguousarray(bt[drows]),
-                                     np.ascontiguousarray(dec[drows] + 1), hq, hkv, d, quant)
-        for i, b in enumerate(drows):
-            out[cu[b]] = od[i]
+        qd = np.ascontiguousarray(q[[cu[b] + t for b, t in drows]])
+        od = oracle.decode_attention(qd, kc, vc, ks, vs, np.ascontiguousarray(bt[[b for b, _ in drows]]),
+                                     np.array([dec[b] + t + 1 for b, t in drows], np.int32), hq, hkv, d, quant)
+        for i, (b, t) in enumerate(drows):
+            out[cu[b] + t] = od[i]
     ptoks = np.array([t for b in range(len(enc)) if enc[b] > 0 for t in range(cu[b], cu[b + 1])], np.int32)
     if len(ptoks):
         op = oracle.append_attention_prefill(q, k_new, v_new, kc, vc, ks, vs, bt, dec, cu, hq, hkv, d, quant,
