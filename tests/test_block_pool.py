@@ -186,3 +186,25 @@ def test_sequence_book_builds_the_step_description():
     book.finish(3)
     book.finish(0)
     assert book.lengths[0] == 0 and pool.refcount(0) == 1 and pool.refcount(3) == 0 and pool.free_blocks == 5
+
+
+def test_sequence_book_speculative_steps():
+    """Draft slots: a slot named in `drafts` that already has tokens brings its tokens as a decode row of several
+    tokens (seq_lens_encoder 0, decode_tokens = the largest such count); an empty slot named there is still a
+    prompt.  commit(accepted) advances a slot by the tokens that were kept."""
+    from fastdeploy_amd.backend import SequenceBook
+    pool = BlockPool(num_blocks=8, block_size=16, max_seqs=4, max_blocks_per_seq=4)
+    book = SequenceBook(pool, device="cpu")
+    book.schedule({0: 20, 1: 3})
+    book.commit()
+    m = book.schedule({0: 3, 1: 2, 2: 2, 3: 1}, drafts={0, 1, 2})
+    assert m.seq_lens_encoder.tolist() == [0, 0, 2, 1]      # slot 2 is empty: its two tokens are a prompt
+    assert m.seq_lens_this_time.tolist() == [3, 2, 2, 1] and m.decode_tokens == 3
+    assert (m.prefill_rows, m.max_enc_len_this_time, m.num_tokens) == (2, 2, 8)
+    assert book.schedule({0: 1}).decode_tokens == 1         # (a schedule that is not committed changes no length)
+    m = book.schedule({0: 3, 1: 2}, drafts={0, 1})
+    book.commit(accepted={0: 1, 1: 2})
+    assert book.lengths == [21, 5, 0, 0]
+    book.schedule({0: 2}, drafts={0})
+    with pytest.raises(ValueError):
+        book.commit(accepted={0: 3})
