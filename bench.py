@@ -45,6 +45,23 @@ def time_events(fn, steps, warmup):
     return e0.elapsed_time(e1) / steps
 
 
+def time_graph(fn, steps, per_graph=10):
+    """The same average with the host taken out: `per_graph` calls captured in one HIP graph, replayed
+    steps / per_graph times.  For ops whose kernels are shorter than the Python call that launches them."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(per_graph):
+            fn()
+    n = max(steps // per_graph, 2)
+    return time_events(graph.replay, n, 2) / per_graph
+
+
 def other_workloads(args):
     """The rows of the path that are not the headline metric (configs[2], [3], [4]): one JSON line each
     with the kernel time and its roofline fraction.  Not part of the default run."""
@@ -76,7 +93,8 @@ def other_workloads(args):
         q = wr()[0]
         ms = time_events(wr, args.steps, args.warmup)
         line("configs[2] cache write (256 tokens, RoPE + int8)", ms, "hbm", 256 * (48 * 128 * 2 + 2 * 8 * 128 + 32 * 128 * 2),
-             HBM_PEAK_GBPS, "GB/s", {"note": "5.8 MB of traffic: launch-bound"})
+             HBM_PEAK_GBPS, "GB/s", {"note": "5.8 MB of traffic: bound by the Python call that launches it",
+                                     "us_from_a_hip_graph": round(time_graph(wr, args.steps) * 1e3, 2)})
         # the same kernel at prefill size: 2 sequences x 2048 new tokens behind 8192 cached ones (configs[4]'s write),
         # with the rotated K and the V handed on for the append attention - large enough to be HBM-bound
         cw = syn.write_case(num_seqs=2, max_pos=8192 + 2048, seed=1, device=dev, chunk=2048, blocks_per_seq=160)
@@ -126,7 +144,8 @@ def other_workloads(args):
                                                 c["block_tables"], c["seq_lens_decoder"], kept_blocks=kept, kept_counts=cnt,
                                                 num_heads=32, cache_quant_type="cache_fp8", workspace=ws)
         ms = time_events(sp, args.steps, args.warmup)
-        line("configs[3] sparse decode (64 of 512 blocks)", ms, "hbm", 16 * 8 * 64 * 64 * 128 * 2, HBM_PEAK_GBPS, "GB/s")
+        line("configs[3] sparse decode (64 of 512 blocks)", ms, "hbm", 16 * 8 * 64 * 64 * 128 * 2, HBM_PEAK_GBPS, "GB/s",
+             {"us_from_a_hip_graph": round(time_graph(sp, args.steps) * 1e3, 2)})
         de = lambda: fd.decode_attention(c["q"], c["key_cache"], c["value_cache"], c["cache_k_scale"], c["cache_v_scale"],
                                          c["block_tables"], c["seq_lens_decoder"], num_heads=32, cache_quant_type="cache_fp8", workspace=ws)
         ms = time_events(de, max(args.steps // 4, 5), 3)
@@ -148,7 +167,8 @@ def other_workloads(args):
                                 cache_quant_type="cache_fp8", cu_seqlens_q=cu, workspace=sws, out=sout, sqattn_top_k=64)
         ms = time_events(sparse_step, max(args.steps // 4, 5), 3)
         line("configs[3] as one call per step: cache write + selector + sparse decode", ms, "hbm",
-             16 * 32768 * 8 * 128 + 16 * 8 * 64 * 64 * 128 * 2, HBM_PEAK_GBPS, "GB/s")
+             16 * 32768 * 8 * 128 + 16 * 8 * 64 * 64 * 128 * 2, HBM_PEAK_GBPS, "GB/s",
+             {"us_from_a_hip_graph": round(time_graph(sparse_step, args.steps) * 1e3, 2)})
 
     if args.workload in ("prefill", "all"):
         # configs[4]: batch 2, 2048 new tokens on 8192 cached (int8 paged), causal
