@@ -250,7 +250,7 @@ def test_mixed_step_with_block_sparse_decode_rows(oracle, quant):
     """sqattn_top_k in the one-call step: every decode row selects its top-k blocks with its new query over the
     cache that already holds its new token, and attends to those only; prefill rows are untouched by it.  Against the
     oracle's pieces: writer, block scores + top-k, sparse decode, prefill."""
-    enc, dec = [0, 90, 0, 0, 0], [64 * 30 + 5, 700, 63, 64 * 11, 64 * 3]
+    enc, dec = [0, 90, 0, 0, 0, 0, 1], [64 * 30 + 5, 700, 63, 64 * 11, 64 * 3, 0, 0]   # + an idle slot, a 1-token prompt
     top_k = 6
     c = mixed_case(enc, dec, quant, seed=33, max_pos=4096)
     dev = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
@@ -258,7 +258,7 @@ def test_mixed_step_with_block_sparse_decode_rows(oracle, quant):
                               dev["seq_lens_decoder"], dev["seq_lens_this_time"], dev["block_tables"],
                               (dev["rope_cos"], dev["rope_sin"]), dev["cache_k_scale"], dev["cache_v_scale"],
                               num_heads=32, kv_num_heads=8, max_chunk=90, cache_quant_type=quant,
-                              cu_seqlens_q=dev["cu_seqlens_q"], prefill_rows=1, sqattn_top_k=top_k)
+                              cu_seqlens_q=dev["cu_seqlens_q"], prefill_rows=2, sqattn_top_k=top_k)
     torch.cuda.synchronize()
     # the oracle's step, with the decode rows done sparsely
     kc, vc = np_of(c["key_cache"]).copy(), np_of(c["value_cache"]).copy()
@@ -277,7 +277,7 @@ def test_mixed_step_with_block_sparse_decode_rows(oracle, quant):
     od = oracle.decode_attention(qd, kc, vc, ks, vs, btd, kvl, 32, 8, 128, quant, kept_blocks=kept, kept_counts=cnt)
     for i, b in enumerate(drows):
         want[cu[b]] = od[i]
-    ptoks = np.arange(cu[1], cu[2], dtype=np.int32)
+    ptoks = np.concatenate([np.arange(cu[1], cu[2]), np.arange(cu[6], cu[7])]).astype(np.int32)
     op = oracle.append_attention_prefill(q, k_new, v_new, kc, vc, ks, vs, bt, decs, cu, 32, 8, 128, quant, token_ids=ptoks)
     want[ptoks] = op[ptoks]
     ok, mx, bad = bf16_close(bits(out), want)
@@ -287,7 +287,7 @@ def test_mixed_step_with_block_sparse_decode_rows(oracle, quant):
                                 dev["seq_lens_decoder"], dev["seq_lens_this_time"], dev["block_tables"],
                                 (dev["rope_cos"], dev["rope_sin"]), dev["cache_k_scale"], dev["cache_v_scale"],
                                 num_heads=32, kv_num_heads=8, max_chunk=90, cache_quant_type=quant,
-                                cu_seqlens_q=dev["cu_seqlens_q"], prefill_rows=1)
+                                cu_seqlens_q=dev["cu_seqlens_q"], prefill_rows=2)
     assert not torch.equal(dense[0], out[0]) and torch.equal(dense[cu[1]:cu[2]], out[cu[1]:cu[2]])
     ok, mx, bad = bf16_close(bits(out[int(cu[4])]), bits(dense[int(cu[4])]))   # 4 blocks <= top_k: the row keeps them all
     assert ok
