@@ -199,6 +199,11 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   // the same mix of long and short workgroups and the short ones fill the end of the launch.
   const int G = a.hq / a.hkv, pairs = a.rows * a.hkv, units = a.rows * a.hq;
   const bool pack = a.pack_slot > 0;  // short chunks: the workgroup holds every query head of its KV head
+  // When a tile's global loads are issued: at the start of the matrix phase before the vector phase that stores them
+  // (one phase in flight; the long walks of a large launch are bound by the vector phase's issue time and lose 3-6 %
+  // to anything added to it), or a phase earlier, straight after the previous store (a whole tile period in flight:
+  // 10 % faster where the walks are short and few, i.e. latency-bound - the packed short-chunk mode).
+  const bool early = pack;
   int qt, b, qh;  // b: the grid row first, the sequence below; qh: the (first) query head
   if (pack) {
     qt = 0;
@@ -414,6 +419,7 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
     fetch(t0 + 1);
     commit(t0 + 1);
   }
+  if (early) fetch(t0 + lead);
   __syncthreads();
   if (grp == 1) __syncthreads();  // group 1 trails by one phase
 
@@ -439,7 +445,7 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
   for (int t = t0; t <= t1; ++t) {
     // ================= matrix phase =================
     if (t == n_pre && n_pre > 0 && t < my_tiles) load_q(false);  // the chunk's scores meet the bf16 q
-    fetch(t + lead);  // converted and written to LDS in the vector phase that follows
+    if (!early) fetch(t + lead);  // converted and written to LDS in the vector phase that follows
     // ---- O^T += V^T P^T, tile t-1, then S^T = K Q^T, tile t.  In the first product k-slot e of
     // lane group hf is key 32kb + 16ss + 8(e/4) + 4hf + e%4 (the P^T layout); lane i16 supplies
     // the row (key kbase + i16/4, channels cbase + 4(i16%4)..+3)
@@ -458,6 +464,7 @@ __global__ __launch_bounds__(64 * NW) void prefill_mfma_kernel(PrefillArgs a) {
     // ================= vector phase =================
     // staging first: its LDS writes and global loads then run under the softmax arithmetic
     commit(t + lead);
+    if (early) fetch(t + lead + 1);  // in flight for a whole tile period: this phase's arithmetic and the next matrix phase
     if (t < my_tiles) {
       if (t == n_pre && n_pre > 0) leave_prefix();
       // ---- mask + online softmax; this lane: one query, keys 32kb + (r%4) + 8(r/4) + 4hf
