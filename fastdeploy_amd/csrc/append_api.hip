@@ -111,7 +111,9 @@ extern "C" int fdattn_append_attention_ex(
   const RowMap rows{cu_seqlens_q, seq_lens_encoder};
   const size_t dws = w.select - w.decode;
   hipStream_t s = (hipStream_t)stream;
-  if (top_k > 0) {
+  if (prefill_rows >= batch) {
+    // the caller's count says that every sequence is a prefill row: no decode pass
+  } else if (top_k > 0) {
     // block-sparse decode rows: select with the new query over the cache as the writer left it, then attend to
     // the kept blocks only
     int32_t* kept = (int32_t*)(ws + w.kept);

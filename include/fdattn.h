@@ -127,6 +127,8 @@ FDATTN_API int fdattn_write_cache_kv(
  *                   query tile is shared by fdattn_prefill_auto_splits(prefill_rows, hq, max_chunk)
  *                   workgroups, each walking a part of its keys, if the workspace has room for their
  *                   partials (fdattn_append_attention_workspace_bytes_ex with that number of splits).
+ *                   A count equal to batch says that no sequence is a decode row: the decode pass is
+ *                   not launched.
  *   sqattn_top_k    (fdattn_append_attention_ex only) > 0: the decode rows of the step run block-sparse - the
  *                   selector (fdattn_sqattn_select) keeps this many blocks per (row, KV head), scored with the
  *                   row's new query against the cache that already holds its new token, and the decode

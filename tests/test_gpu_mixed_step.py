@@ -194,14 +194,17 @@ def test_mixed_step_with_key_splits_replays_from_a_hip_graph(top_k):
 
 
 def test_decode_only_and_prefill_only_steps_through_the_same_entry(oracle):
-    for enc, dec, mc in (([0, 0, 0, 0], [5, 64, 1000, 0], 0), ([64, 1, 257, 0], [0, 0, 100, 0], 257)):
+    # (the last case says that all its 3 sequences are prefill rows: the step then launches no decode pass)
+    for enc, dec, mc, rows in (([0, 0, 0, 0], [5, 64, 1000, 0], 0, None), ([64, 1, 257, 0], [0, 0, 100, 0], 257, None),
+                               ([64, 1, 257], [0, 0, 100], 257, 3)):
         c = mixed_case(enc, dec, CACHE_INT8, seed=9)
         dev = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
         ws = fd.append_attention_workspace(c["T"], len(enc), 32, 8, 128, dev["block_tables"].shape[1])
         out = fd.append_attention(dev["qkv"], dev["key_cache"], dev["value_cache"], dev["seq_lens_encoder"],
                                   dev["seq_lens_decoder"], dev["seq_lens_this_time"], dev["block_tables"],
                                   (dev["rope_cos"], dev["rope_sin"]), dev["cache_k_scale"], dev["cache_v_scale"],
-                                  num_heads=32, kv_num_heads=8, max_chunk=mc, workspace=ws)
+                                  num_heads=32, kv_num_heads=8, max_chunk=mc, workspace=ws,
+                                  cu_seqlens_q=dev["cu_seqlens_q"], prefill_rows=rows)
         torch.cuda.synchronize()
         want, kc, vc = oracle_step(oracle, c, CACHE_INT8)
         assert np.array_equal(np_of(dev["key_cache"]), kc) and np.array_equal(np_of(dev["value_cache"]), vc)
