@@ -1,6 +1,6 @@
 // Shape-agnostic decode attention over the quantised paged cache, and the split-KV
-// combine.  One wavefront per (sequence, query head, KV split): lanes own tokens for
-// q.K and channels for P.V.  This is the fall-back for shapes the MFMA kernel in
+// combine.  One wavefront per (sequence, KV head, up to 8 of its query heads, KV split): lanes own
+// tokens for q.K and channels for P.V.  This is the fall-back for shapes the MFMA kernel in
 // decode_c8.hip does not cover (any head_dim <= 256, any group size, any block size);
 // it makes no attempt to reach the HBM roofline.  The formats with one scale per stored
 // row (DYN) multiply a token's score by its K scale and its weight by its V scale.
@@ -36,21 +36,32 @@ __device__ __forceinline__ float dq(u32 byte) {
 
 constexpr int kMaxD = 256;
 
+// One wavefront per (sequence, KV head, set of up to NH (4 or 8) of its query heads, KV split): the K and V bytes it reads
+// serve all the heads of the set.  Scores: lane = token of a group of 64, its K row read in 16-byte words, one dot
+// product per head against q * k_scale * softmax_scale in LDS.  P.V: lane = four channels of one of the 64 / (d/4)
+// token rows read at a time; the rows' sums meet in LDS at the end.
 // DYN: cache scales per stored row ([num_blocks, hkv, bs]) instead of per channel.
-template <int QUANT, bool DYN>
+template <int QUANT, bool DYN, int NH>
 __global__ __launch_bounds__(64) void decode_generic_kernel(GenericDecodeArgs a) {
-  __shared__ float qs[kMaxD];
-  __shared__ float pbuf[64];
+  __shared__ __attribute__((aligned(16))) float qs[NH][kMaxD];  // q of the set's heads; at the end: their outputs
+  __shared__ float pbuf[NH][64];
   const int lane = threadIdx.x;
-  const int row = blockIdx.x, split = blockIdx.y, nsplit = gridDim.y;
-  const int b = row / a.hq, qh = row % a.hq, g = a.hq / a.hkv, h = qh / g;
+  const int split = blockIdx.y, nsplit = gridDim.y;
+  const int g = a.hq / a.hkv, sets = (g + NH - 1) / NH;
+  const int set = blockIdx.x % sets, p = blockIdx.x / sets;
+  const int b = p / a.hkv, h = p % a.hkv;
+  const int g0 = set * NH, ng = min(NH, g - g0);  // heads h*g + g0 .. + ng - 1
   const int d = a.d, bs = a.bs;
   int qrow;  // the sequence's row of q
   if (!decode_row(a.rows, b, qrow)) return;
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
 
-  for (int c = lane; c < d; c += 64)
-    qs[c] = bf16_to_f32(a.q[((size_t)qrow * a.hq + qh) * d + c]) * (DYN ? 1.0f : a.k_scale[h * d + c]) * a.sm_scale;
+  for (int i = lane; i < NH * d; i += 64) {
+    const int gg = i / d, c = i - gg * d;
+    qs[gg][c] = gg < ng ? bf16_to_f32(a.q[((size_t)qrow * a.hq + h * g + g0 + gg) * d + c]) *
+                              (DYN ? 1.0f : a.k_scale[h * d + c]) * a.sm_scale
+                        : 0.f;  // heads past the set: zero rows, so that the loops below need no test
+  }
   __syncthreads();
 
   int nblk = (kv_len + bs - 1) / bs;
@@ -63,8 +74,17 @@ __global__ __launch_bounds__(64) void decode_generic_kernel(GenericDecodeArgs a)
   const int per = (nblk + nsplit - 1) / nsplit;
   const int i0 = split * per, i1 = min(nblk, i0 + per);
 
-  float m = -INFINITY, l = 0.f;
-  float acc[kMaxD / 64] = {0.f, 0.f, 0.f, 0.f};
+  // P.V layout: lanes_per_row lanes cover a row's d channels, 4 each; rows_per_pass rows at a time
+  const int lanes_per_row = d / 4, rows_per_pass = 64 / lanes_per_row;
+  const int vslot = lane / lanes_per_row, c4 = 4 * (lane - vslot * lanes_per_row);
+  const bool vlane = vslot < rows_per_pass;
+
+  float m[NH], l[NH], acc[NH][4];
+#pragma unroll
+  for (int gg = 0; gg < NH; ++gg) {
+    m[gg] = -INFINITY, l[gg] = 0.f;
+    acc[gg][0] = acc[gg][1] = acc[gg][2] = acc[gg][3] = 0.f;
+  }
   const int32_t* table = a.block_tables + (size_t)b * a.max_blocks;
 
   for (int bi = i0; bi < i1; ++bi) {
@@ -78,49 +98,85 @@ __global__ __launch_bounds__(64) void decode_generic_kernel(GenericDecodeArgs a)
     for (int t0 = 0; t0 < bs; t0 += 64) {
       const int t = t0 + lane;
       const bool valid = t < bs && lb * bs + t < kv_len;
-      float s = -INFINITY;
-      if (valid) {
-        s = 0.f;
-        const uint8_t* kr = kp + (size_t)t * d;
-        for (int c = 0; c < d; c += 4) {
-          u32 w = *reinterpret_cast<const u32*>(kr + c);
-          s += qs[c] * dq<QUANT>(w & 0xff) + qs[c + 1] * dq<QUANT>((w >> 8) & 0xff) +
-               qs[c + 2] * dq<QUANT>((w >> 16) & 0xff) + qs[c + 3] * dq<QUANT>(w >> 24);
-        }
-        if (DYN) s *= a.k_scale[srow + t];
-      }
-      const float mb = wave_max(s);
-      if (mb == -INFINITY) continue;  // uniform: no valid token in this group
-      const float m_new = fmaxf(m, mb);
-      const float alpha = (m == -INFINITY) ? 0.f : __expf(m - m_new);
-      const float p = valid ? __expf(s - m_new) : 0.f;
-      l = l * alpha + wave_sum(p);
-      m = m_new;
-      __syncthreads();
-      pbuf[lane] = (DYN && valid) ? p * a.v_scale[srow + t] : p;  // the V row's scale rides on its weight
-      __syncthreads();
-      const int nt = min(64, bs - t0);
+      if (!__any(valid)) continue;  // no valid token in this group
+      float s[NH];
 #pragma unroll
-      for (int i = 0; i < kMaxD / 64; ++i) {
-        const int c = lane + 64 * i;
-        if (c < d) {
-          float o = acc[i] * alpha;
-          for (int tt = 0; tt < nt; ++tt) o += pbuf[tt] * dq<QUANT>(vp[(size_t)(t0 + tt) * d + c]);
-          acc[i] = o;
+      for (int gg = 0; gg < NH; ++gg) s[gg] = 0.f;
+      if (valid) {
+        const uint8_t* kr = kp + (size_t)t * d;
+        auto word = [&](u32 w, int c) {  // four channels of the row against every head's q
+          const float k0 = dq<QUANT>(w & 0xff), k1 = dq<QUANT>((w >> 8) & 0xff), k2 = dq<QUANT>((w >> 16) & 0xff),
+                      k3 = dq<QUANT>(w >> 24);
+#pragma unroll
+          for (int gg = 0; gg < NH; ++gg) {
+            const float4 qv = *reinterpret_cast<const float4*>(&qs[gg][c]);
+            s[gg] += qv.x * k0 + qv.y * k1 + qv.z * k2 + qv.w * k3;
+          }
+        };
+        int c = 0;
+        const int d16 = (d & 15) ? 0 : d;  // 16-byte words only where every row starts on one
+        for (; c < d16; c += 16) {
+          const uint4 w = *reinterpret_cast<const uint4*>(kr + c);
+          word(w.x, c), word(w.y, c + 4), word(w.z, c + 8), word(w.w, c + 12);
+        }
+        for (; c < d; c += 4) word(*reinterpret_cast<const u32*>(kr + c), c);
+      }
+      const float ksc = (DYN && valid) ? a.k_scale[srow + t] : 1.0f;
+      const float vsc = (DYN && valid) ? a.v_scale[srow + t] : 1.0f;  // the V row's scale rides on its weight
+      float alpha[NH];
+#pragma unroll
+      for (int gg = 0; gg < NH; ++gg) {
+        const float sv = valid ? s[gg] * ksc : -INFINITY;
+        const float m_new = fmaxf(m[gg], wave_max(sv));     // finite: the group has a valid token
+        alpha[gg] = (m[gg] == -INFINITY) ? 0.f : __expf(m[gg] - m_new);
+        const float pr = valid ? __expf(sv - m_new) : 0.f;
+        l[gg] = l[gg] * alpha[gg] + wave_sum(pr);
+        m[gg] = m_new;
+        pbuf[gg][lane] = pr * vsc;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int gg = 0; gg < NH; ++gg)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[gg][e] *= alpha[gg];
+      const int nt = min(64, min(bs - t0, kv_len - lb * bs - t0));  // rows past the sequence weigh 0: not read
+      if (vlane) {
+        for (int tt = vslot; tt < nt; tt += rows_per_pass) {
+          const u32 w = *reinterpret_cast<const u32*>(vp + (size_t)(t0 + tt) * d + c4);
+          const float v0 = dq<QUANT>(w & 0xff), v1 = dq<QUANT>((w >> 8) & 0xff), v2 = dq<QUANT>((w >> 16) & 0xff),
+                      v3 = dq<QUANT>(w >> 24);
+#pragma unroll
+          for (int gg = 0; gg < NH; ++gg) {
+            const float pw = pbuf[gg][tt];
+            acc[gg][0] += pw * v0, acc[gg][1] += pw * v1, acc[gg][2] += pw * v2, acc[gg][3] += pw * v3;
+          }
         }
       }
+      __syncthreads();
     }
   }
-  const size_t slot = (size_t)row * a.max_splits + split;
+  // the row slots' sums meet in LDS (q is no longer needed), one slot after the other
+  __syncthreads();
+  for (int sl = 0; sl < rows_per_pass; ++sl) {
+    if (vlane && vslot == sl) {
 #pragma unroll
-  for (int i = 0; i < kMaxD / 64; ++i) {
-    const int c = lane + 64 * i;
-    if (c < d) a.part_o[slot * d + c] = DYN ? acc[i] : acc[i] * a.v_scale[h * d + c];
+      for (int gg = 0; gg < NH; ++gg)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) qs[gg][c4 + e] = (sl == 0 ? 0.f : qs[gg][c4 + e]) + acc[gg][e];
+    }
+    __syncthreads();
   }
-  if (lane == 0) {
-    a.part_m[slot] = m;
-    a.part_l[slot] = l;
+  for (int gg = 0; gg < ng; ++gg) {
+    const size_t slot = ((size_t)b * a.hq + h * g + g0 + gg) * a.max_splits + split;
+    for (int c = lane; c < d; c += 64) a.part_o[slot * d + c] = DYN ? qs[gg][c] : qs[gg][c] * a.v_scale[h * d + c];
   }
+#pragma unroll
+  for (int gg = 0; gg < NH; ++gg)
+    if (lane == 0 && gg < ng) {
+      const size_t slot = ((size_t)b * a.hq + h * g + g0 + gg) * a.max_splits + split;
+      a.part_m[slot] = m[gg];
+      a.part_l[slot] = l[gg];
+    }
 }
 
 // out[r,:] = sum_s o_s e^(m_s - m) / sum_s l_s e^(m_s - m); one thread per channel.
@@ -174,7 +230,9 @@ int decode_generic_launch(const void* q, const void* key_cache, const void* valu
   if (workspace_bytes < need)
     return fail(FDATTN_ERR_WORKSPACE, "fdattn_decode_attention: workspace %zu B < required %zu B", workspace_bytes, need);
   const int rows = batch * hq;
-  int nsplit = 2048 / rows;
+  const int nh = hq / hkv <= 4 ? 4 : 8;  // query heads of one KV head a workgroup serves together
+  const int sets = (hq / hkv + nh - 1) / nh, wgs = batch * hkv * sets;
+  int nsplit = 4096 / wgs;
   nsplit = nsplit < 1 ? 1 : (nsplit > kGenericMaxSplits ? kGenericMaxSplits : nsplit);
   // partial layout [rows, nsplit, ...]: the combine then reads exactly the slots written
   float* part_o = (float*)workspace;
@@ -184,15 +242,17 @@ int decode_generic_launch(const void* q, const void* key_cache, const void* valu
                       k_scale, v_scale, block_tables, seq_lens_decoder, seq_lens_this_time,
                       kept_blocks, kept_counts, max_kept, part_o, part_m, part_l, rmap, batch, hq, hkv,
                       d, bs, max_blocks, num_blocks, nsplit, sm_scale};
-  const dim3 grid(rows, nsplit);
-  if (quant == FDATTN_CACHE_INT8)
-    hipLaunchKernelGGL((decode_generic_kernel<FDATTN_CACHE_INT8, false>), grid, dim3(64), 0, s, a);
-  else if (quant == FDATTN_CACHE_FP8_E4M3)
-    hipLaunchKernelGGL((decode_generic_kernel<FDATTN_CACHE_FP8_E4M3, false>), grid, dim3(64), 0, s, a);
-  else if (quant == FDATTN_CACHE_INT8_DYNAMIC)
-    hipLaunchKernelGGL((decode_generic_kernel<FDATTN_CACHE_INT8, true>), grid, dim3(64), 0, s, a);
-  else
-    hipLaunchKernelGGL((decode_generic_kernel<FDATTN_CACHE_FP8_E4M3, true>), grid, dim3(64), 0, s, a);
+  const dim3 grid(wgs, nsplit);
+#define FDATTN_GEN_LAUNCH(Q, D)                                                                     \
+  do {                                                                                              \
+    if (nh == 4) hipLaunchKernelGGL((decode_generic_kernel<Q, D, 4>), grid, dim3(64), 0, s, a);     \
+    else hipLaunchKernelGGL((decode_generic_kernel<Q, D, 8>), grid, dim3(64), 0, s, a);             \
+  } while (0)
+  if (quant == FDATTN_CACHE_INT8) FDATTN_GEN_LAUNCH(FDATTN_CACHE_INT8, false);
+  else if (quant == FDATTN_CACHE_FP8_E4M3) FDATTN_GEN_LAUNCH(FDATTN_CACHE_FP8_E4M3, false);
+  else if (quant == FDATTN_CACHE_INT8_DYNAMIC) FDATTN_GEN_LAUNCH(FDATTN_CACHE_INT8, true);
+  else FDATTN_GEN_LAUNCH(FDATTN_CACHE_FP8_E4M3, true);
+#undef FDATTN_GEN_LAUNCH
   int rc = check_launch("fdattn_decode_attention (generic)");
   if (rc) return rc;
   hipLaunchKernelGGL(splitkv_combine_kernel, dim3(rows), dim3(128), 0, s, part_o, part_m, part_l,
