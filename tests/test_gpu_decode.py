@@ -201,6 +201,45 @@ def test_decode_generic_other_shapes(oracle):
     check(got, want, "d64 g2 bs16")
 
 
+@pytest.mark.parametrize("hq,hkv,d,bs,quant", [
+    (12, 1, 128, 64, CACHE_INT8),            # 12 query heads on one KV head: two sets of heads per KV head
+    (40, 2, 96, 32, CACHE_FP8),              # 20 per KV head (sets of 8, 8, 4); 24 lanes per V row, 16 lanes idle
+    (6, 2, 256, 128, CACHE_INT8_DYNAMIC),    # a V row takes the whole wavefront; blocks of two 64-token groups
+    (5, 5, 16, 8, CACHE_FP8_DYNAMIC),        # 16 V rows per pass; blocks smaller than a token group
+    (16, 2, 20, 64, CACHE_INT8),             # head_dim not a multiple of 16: 4-byte K words
+])
+def test_decode_shape_agnostic_kernel_shapes(oracle, hq, hkv, d, bs, quant):
+    """The shape-agnostic kernel at shapes that exercise its layout arithmetic: more query heads per KV head than a
+    workgroup serves, head sizes whose V rows take 5 .. 64 lanes, blocks above and below 64 tokens; dense and sparse."""
+    lens = [0, 1, bs - 1, bs, bs + 1, 5 * bs + 3, 700]
+    case = syn.decode_case(batch=len(lens), ctx=lens, seed=77, hq=hq, hkv=hkv, d=d, bs=bs, quant=quant, row_log2=(-3, 1))
+    assert not fd.decode_uses_mfma(hq, hkv, d, bs, quant)
+    want = oracle.decode_attention(bits(case["q"]), np_of(case["key_cache"]), np_of(case["value_cache"]),
+                                   np_of(case["cache_k_scale"]), np_of(case["cache_v_scale"]),
+                                   np_of(case["block_tables"]), np_of(case["seq_lens_decoder"]), hq, hkv, d, quant)
+    check(gpu_decode(case), want, "dense")
+    rng = np.random.default_rng(5)
+    mk = 4
+    kept = np.full((len(lens), hkv, mk), -1, np.int32)
+    cnt = np.zeros((len(lens), hkv), np.int32)
+    for b, n in enumerate(lens):
+        nb = (n + bs - 1) // bs
+        for h in range(hkv):
+            k = int(rng.integers(0, min(mk, nb) + 1))
+            kept[b, h, :k] = np.sort(rng.choice(nb, k, replace=False)) if k else []
+            cnt[b, h] = k
+    dev = syn.to_device(case, "cuda")
+    out = fd.decode_attention_sparse(dev["q"], dev["key_cache"], dev["value_cache"], dev["cache_k_scale"],
+                                     dev["cache_v_scale"], dev["block_tables"], dev["seq_lens_decoder"],
+                                     kept_blocks=torch.from_numpy(kept).cuda(), kept_counts=torch.from_numpy(cnt).cuda(),
+                                     num_heads=hq, cache_quant_type=quant)
+    want = oracle.decode_attention(bits(case["q"]), np_of(case["key_cache"]), np_of(case["value_cache"]),
+                                   np_of(case["cache_k_scale"]), np_of(case["cache_v_scale"]),
+                                   np_of(case["block_tables"]), np_of(case["seq_lens_decoder"]), hq, hkv, d, quant,
+                                   kept_blocks=kept, kept_counts=cnt)
+    check(bits(out), want, "sparse")
+
+
 @pytest.mark.parametrize("impl", ["generic", "auto"])
 @pytest.mark.parametrize("quant", ALL_FORMATS)
 def test_sparse_decode(oracle, impl, quant):
