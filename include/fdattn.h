@@ -246,7 +246,7 @@ FDATTN_API int fdattn_decode_attention_sparse(
  * The shape-agnostic decode kernel behind both functions above (any head_dim <= 256
  * that is a multiple of 4, any hq/hkv, any block_size), callable directly; it is what
  * they fall back to for shapes the MFMA kernel does not cover (it covers head_dim
- * 128, hq/hkv 4, block_size 64).  kept_blocks / kept_counts may both be NULL (dense).
+ * 128, hq/hkv 1 .. 8, block_size 64).  kept_blocks / kept_counts may both be NULL (dense).
  * Same plug-in position as fdattn_decode_attention.
  */
 FDATTN_API int fdattn_decode_attention_generic(
@@ -288,7 +288,7 @@ FDATTN_API size_t fdattn_sqattn_workspace_bytes(int batch, int hkv, int max_bloc
  * top_k highest-scoring blocks per (b,h) are kept; equal scores resolve to the
  * lower block index as in TopKIndices (fastdeploy/vision/utils/utils.h:41-60).
  *   scores      f32 [batch, hkv, max_blocks_per_seq]  (optional output, may be NULL; -inf for absent blocks).
- *               For head_dim 128, hq/hkv 4, block_size 64 these are the MFMA scores the selection starts
+ *               For head_dim 128, hq/hkv 1 .. 8, block_size 64 (at most 2048 blocks per sequence) these are the MFMA scores the selection starts
  *               from (within a small relative error of the fp64 ones; blocks too close to the k-th score to
  *               call are re-scored in fp64 internally, so the kept indices are those of the fp64 scores);
  *               otherwise the fp64 scores rounded to fp32.
