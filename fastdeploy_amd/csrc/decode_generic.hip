@@ -123,22 +123,25 @@ __global__ __launch_bounds__(64) void decode_generic_kernel(GenericDecodeArgs a)
       }
       const float ksc = (DYN && valid) ? a.k_scale[srow + t] : 1.0f;
       const float vsc = (DYN && valid) ? a.v_scale[srow + t] : 1.0f;  // the V row's scale rides on its weight
-      float alpha[NH];
+      // Softmax weights against a per-head reference that is raised only when a score outgrows it by more than
+      // 2^10 (one ballot per head and group instead of a maximum over the wavefront; the weights stay below e^10);
+      // the weight sums stay per lane until the end.
 #pragma unroll
       for (int gg = 0; gg < NH; ++gg) {
         const float sv = valid ? s[gg] * ksc : -INFINITY;
-        const float m_new = fmaxf(m[gg], wave_max(sv));     // finite: the group has a valid token
-        alpha[gg] = (m[gg] == -INFINITY) ? 0.f : __expf(m[gg] - m_new);
-        const float pr = valid ? __expf(sv - m_new) : 0.f;
-        l[gg] = l[gg] * alpha[gg] + wave_sum(pr);
-        m[gg] = m_new;
+        if (__any(valid && !(sv <= m[gg] + 10.0f))) {  // also the first group (m = -inf) and NaN scores
+          const float m_new = fmaxf(m[gg], wave_max(sv));
+          const float al = (m[gg] == -INFINITY) ? 0.f : __expf(m[gg] - m_new);
+          l[gg] *= al;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[gg][e] *= al;
+          m[gg] = m_new;
+        }
+        const float pr = valid ? __expf(sv - m[gg]) : 0.f;
+        l[gg] += pr;
         pbuf[gg][lane] = pr * vsc;
       }
       __syncthreads();
-#pragma unroll
-      for (int gg = 0; gg < NH; ++gg)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc[gg][e] *= alpha[gg];
       const int nt = min(64, min(bs - t0, kv_len - lb * bs - t0));  // rows past the sequence weigh 0: not read
       if (vlane) {
         for (int tt = vslot; tt < nt; tt += rows_per_pass) {
@@ -171,12 +174,14 @@ __global__ __launch_bounds__(64) void decode_generic_kernel(GenericDecodeArgs a)
     for (int c = lane; c < d; c += 64) a.part_o[slot * d + c] = DYN ? qs[gg][c] : qs[gg][c] * a.v_scale[h * d + c];
   }
 #pragma unroll
-  for (int gg = 0; gg < NH; ++gg)
+  for (int gg = 0; gg < NH; ++gg) {
+    const float lsum = wave_sum(l[gg]);
     if (lane == 0 && gg < ng) {
       const size_t slot = ((size_t)b * a.hq + h * g + g0 + gg) * a.max_splits + split;
       a.part_m[slot] = m[gg];
-      a.part_l[slot] = l[gg];
+      a.part_l[slot] = lsum;
     }
+  }
 }
 
 // out[r,:] = sum_s o_s e^(m_s - m) / sum_s l_s e^(m_s - m); one thread per channel.
