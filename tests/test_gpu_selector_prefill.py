@@ -302,3 +302,35 @@ def test_prefill_key_splits(oracle, quant):
         assert ok, "splits %r: %d out of tolerance, max %.4g" % (splits, bad, mx)
         ok, mx, bad = bf16_close(bits(one), want)
         assert ok, "unsplit: %d out of tolerance, max %.4g" % (bad, mx)
+
+
+@pytest.mark.parametrize("hq,hkv,d,bs,quant", [
+    (12, 1, 128, 64, CACHE_INT8),            # 12 query heads on one KV head: sets of 8 and 4, one token per group
+    (6, 2, 96, 32, CACHE_FP8),               # 3 per KV head: groups of two tokens, 6 of the 8 rows in use
+    (4, 4, 256, 128, CACHE_INT8_DYNAMIC),    # 1 per KV head: groups of eight tokens; a V row takes the whole wavefront
+    (10, 2, 16, 8, CACHE_FP8_DYNAMIC),       # 5 per KV head: one token per group, 5 rows; 16 V rows per pass
+    (8, 4, 20, 16, CACHE_INT8),              # head_dim not a multiple of 16: 4-byte K words
+])
+def test_prefill_shape_agnostic_kernel_shapes(oracle, hq, hkv, d, bs, quant):
+    """The shape-agnostic prefill kernel at shapes that exercise its layout arithmetic: 1 .. 12 query heads per KV
+    head (1, 2 or 8 tokens per workgroup, row sets partly empty), chunks that are not multiples of the token group,
+    prefixes of zero, one and several 64-key groups, a prefix that ends inside a group."""
+    prefix, chunks = [0, 1, 3 * bs + 5, 200, 64], [9, 1, 70, 13, 130]
+    c = syn.decode_case(batch=len(chunks), ctx=prefix, quant=quant, seed=91, extra_blocks=20, hq=hq, hkv=hkv, d=d, bs=bs,
+                        row_log2=(-3, 1))
+    g = torch.Generator().manual_seed(92)
+    T = sum(chunks)
+    q = torch.randn((T, hq * d), generator=g).to(torch.bfloat16)
+    k = torch.randn((T, hkv * d), generator=g).to(torch.bfloat16)
+    v = torch.randn((T, hkv * d), generator=g).to(torch.bfloat16)
+    cu = torch.tensor([0] + list(np.cumsum(chunks)), dtype=torch.int32)
+    dev = syn.to_device(c, "cuda")
+    out = fd.append_attention_prefill(q.cuda(), k.cuda(), v.cuda(), dev["key_cache"], dev["value_cache"],
+                                      dev["cache_k_scale"], dev["cache_v_scale"], dev["block_tables"],
+                                      dev["seq_lens_decoder"], cu.cuda(), num_heads=hq, max_chunk=max(chunks),
+                                      cache_quant_type=quant)
+    want = oracle.append_attention_prefill(bits(q), bits(k), bits(v), np_of(c["key_cache"]), np_of(c["value_cache"]),
+                                           np_of(c["cache_k_scale"]), np_of(c["cache_v_scale"]), np_of(c["block_tables"]),
+                                           np_of(c["seq_lens_decoder"]), np_of(cu), hq, hkv, d, quant)
+    ok, mx, bad = bf16_close(bits(out), want)
+    assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
