@@ -67,6 +67,15 @@ def test_version_and_argument_errors_need_no_gpu():
     assert rc == -4
     rc = lib.fdattn_append_attention_prefill(*([None] * 11), 1, 1, 1, 32, 8, 128, 64, 1, 1, 1, 0.1, None)
     assert rc == -1
+    # the one-call step refuses what its decode rows cannot be given before it writes anything: three tokens per
+    # decode row with 4 query heads per KV head (12 rows > 8), several tokens together with the block selector,
+    # the selector at a head size its MFMA path does not cover
+    big = 1 << 40
+    for extras, hd in ((_lib.StepExtras(None, None, None, 0.0, 0, 0, 3), 128), (_lib.StepExtras(None, None, None, 0.0, 0, 4, 2), 128),
+                       (_lib.StepExtras(None, None, None, 0.0, 0, 4, 0), 64)):
+        rc = lib.fdattn_append_attention_ex(*([one] * 14), big, 4, 2, 0, 32, 8, hd, 64, 8, 16, 64, 0, 1, 0.1,
+                                            ctypes.addressof(extras), None)
+        assert rc == -2 and (b"decode_tokens" in lib.fdattn_last_error() or b"sqattn_top_k" in lib.fdattn_last_error())
     assert lib.fdattn_decode_workspace_bytes(64, 32, 8, 128, 72) >= 64 * 8 * 3 * 2080
     assert lib.fdattn_decode_uses_mfma(32, 8, 128, 64, 1) == 1 and lib.fdattn_decode_uses_mfma(32, 8, 64, 64, 1) == 0
     with pytest.raises(ValueError):

@@ -148,13 +148,14 @@ def test_mixed_step_with_key_splits_for_the_prefill_row(oracle):
     assert ok, "small workspace: %d out of tolerance, max %.4g" % (bad, mx)
 
 
-@pytest.mark.parametrize("top_k", [None, 8])
-def test_mixed_step_with_key_splits_replays_from_a_hip_graph(top_k):
+@pytest.mark.parametrize("top_k,tokens", [(None, None), (8, None), (None, 2)])
+def test_mixed_step_with_key_splits_replays_from_a_hip_graph(top_k, tokens):
     """The mixed step with key splits (writer, decode + its merge - with top_k the block selector and the sparse
     decode instead -, prefill shares, prefill merge) captured in a HIP graph: every replay, with eager work and synchronisations in between, equals the eager step on a copy of the
     state bit for bit (outputs and cache bytes)."""
     enc, dec = [0, 160, 0, 0, 0], [900, 4200, 63, 2100, 4600]
-    c = mixed_case(enc, dec, CACHE_INT8, seed=21, max_pos=8192)
+    # (tokens: three of the decode rows bring that many draft tokens - the decode kernel's several-token variant)
+    c = mixed_case(enc, dec, CACHE_INT8, seed=21, max_pos=8192, this=[tokens, 160, 1, tokens, tokens] if tokens else None)
     dev = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
     eag = {k: (v.clone() if isinstance(v, torch.Tensor) else v) for k, v in dev.items()}
     splits = fd.ops.prefill_auto_splits(1, 32, 160)
@@ -168,7 +169,7 @@ def test_mixed_step_with_key_splits_replays_from_a_hip_graph(top_k):
                                    s["seq_lens_decoder"], s["seq_lens_this_time"], s["block_tables"],
                                    (s["rope_cos"], s["rope_sin"]), s["cache_k_scale"], s["cache_v_scale"],
                                    num_heads=32, kv_num_heads=8, max_chunk=160, cu_seqlens_q=s["cu_seqlens_q"],
-                                   prefill_rows=1, workspace=ws, sqattn_top_k=top_k)
+                                   prefill_rows=1, workspace=ws, sqattn_top_k=top_k, decode_tokens=tokens)
 
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
