@@ -98,6 +98,14 @@ class AppendAttentionBackend:
         if meta.block_tables.shape[0] != slots:
             raise ValueError("block_tables has %d rows, the batch %d slots" % (meta.block_tables.shape[0], slots))
         meta.cu_seqlens_q = ops.cu_seqlens_of(this)
+        if meta.decode_tokens > 1:
+            group = self.num_heads // self.kv_num_heads
+            if (meta.decode_tokens * group > 8 or self.sqattn_top_k
+                    or not ops.decode_uses_mfma(self.num_heads, self.kv_num_heads, self.head_dim, self.block_size,
+                                                self.cache_quant_type)):
+                raise ValueError("decode rows of %d tokens need head_dim 128, block_size 64, tokens x heads per KV head "
+                                 "<= 8 (here %d) and no sqattn_top_k: schedule such rows as prefill rows instead"
+                                 % (meta.decode_tokens, meta.decode_tokens * group))
         if meta.max_enc_len_this_time is None:
             both = torch.stack([meta.cu_seqlens_q[-1], meta.seq_lens_encoder.max()]).tolist()   # one synchronisation
             meta.num_tokens, meta.max_enc_len_this_time = int(both[0]), max(int(both[1]), 0)

@@ -72,3 +72,17 @@ def test_generation_over_steps_and_layers(oracle, quant):
     run_step({0: 2, 2: 1, 3: 1}, drafts={0})
     assert book.lengths == [157, 0, 282, 289, 1]
     assert pool.refcount(int(pool.block_tables[2, 0])) == 2
+
+
+def test_backend_refuses_draft_rows_its_decode_kernel_cannot_take():
+    """8 query heads per KV head leave no room for a second token in the decode kernel's 8 rows: the metadata step
+    says so (the scheduler should send such rows as prefill rows) instead of the kernel call failing later."""
+    be = fd.AppendAttentionBackend(64, 8, 128, block_size=64, max_position=256)
+    pool = fd.BlockPool(num_blocks=8, block_size=64, max_seqs=2, max_blocks_per_seq=4)
+    book = fd.SequenceBook(pool)
+    be.init_attention_metadata(book.schedule({0: 5}))
+    book.commit()
+    with pytest.raises(ValueError, match="prefill rows"):
+        be.init_attention_metadata(book.schedule({0: 2}, drafts={0}))
+    meta = be.init_attention_metadata(book.schedule({0: 2}))     # the same tokens as a prefill row: fine
+    assert meta.decode_tokens == 1 and meta.prefill_rows == 1
