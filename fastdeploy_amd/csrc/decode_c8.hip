@@ -539,7 +539,12 @@ int c8_pick_chunk(int pairs, int max_units) {
   const int cpp = (2 * gpu_cu_count() + pairs - 1) / pairs;  // two workgroups of this kernel fit a CU
   int chunk = (max_units + cpp - 1) / cpp;
   if (chunk < kWaves) chunk = kWaves;
-  if (chunk > kMaxChunk) chunk = kMaxChunk;
+  if (chunk > kMaxChunk) {
+    // a list longer than the unit table: as few chunks as hold it, of equal size (137 units = 69 + 68, not 128 + 9:
+    // the longest chunk sets the launch's duration)
+    const int n = (max_units + kMaxChunk - 1) / kMaxChunk;
+    chunk = (max_units + n - 1) / n;
+  }
   return chunk;
 }
 
