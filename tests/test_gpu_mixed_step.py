@@ -355,40 +355,48 @@ def test_decode_tokens_argument_checks():
     assert torch.equal(dev["key_cache"].cpu(), c["key_cache"])   # refused before anything was written
 
 
-def test_mixed_step_random_batches_against_the_oracle(oracle):
-    """20 seeded random steps: 1 .. 8 slots that are prefill rows (1 .. 140 new tokens, with or without cached
-    tokens), decode rows or idle; 1 .. 8 query heads per KV head; any cache format; with and without the
-    prefill-row count.  Cache bytes (and scale caches) exact, outputs within tolerance."""
-    rng = np.random.default_rng(7)
+def random_steps(oracle, seed, iters):
+    """Seeded random steps: 1 .. 8 slots that are prefill rows (1 .. 140 new tokens, with or without cached tokens),
+    decode rows - of several draft tokens in some steps - or idle; 1 .. 8 query heads per KV head; any cache format;
+    with and without the prefill-row count.  Cache bytes (and scale caches) exact, outputs within tolerance."""
+    rng = np.random.default_rng(seed)
     formats = [CACHE_INT8, CACHE_FP8, CACHE_INT8_DYNAMIC, CACHE_FP8_DYNAMIC]
-    for it in range(20):
+    for it in range(iters):
         slots, group, hkv = int(rng.integers(1, 9)), int(rng.integers(1, 9)), int(rng.integers(1, 4))
         quant = formats[int(rng.integers(0, 4))]
-        enc, dec = [], []
+        tokens = int(rng.integers(1, 8 // group + 1)) if it % 3 == 2 else 1   # draft tokens a decode row may bring
+        enc, dec, this = [], [], []
         for _ in range(slots):
             kind = int(rng.integers(0, 4))   # prefill on nothing, prefill on a prefix, decode, idle
             enc.append(int(rng.integers(1, 141)) if kind < 2 else 0)
             dec.append(0 if kind in (0, 3) else int(rng.integers(1, 600)))
-        if not any(enc) and not any(dec):
-            dec[0] = 77
+            this.append(enc[-1] if kind < 2 else (int(rng.integers(1, tokens + 1)) if kind == 2 else 0))
+        if not any(this):
+            dec[0], this[0] = 77, 1
         hq = group * hkv
-        c = mixed_case(enc, dec, quant, seed=500 + it, hq=hq, hkv=hkv, max_pos=1024)
+        c = mixed_case(enc, dec, quant, seed=seed * 1000 + it, hq=hq, hkv=hkv, max_pos=1024, this=this)
         dev = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
         rows = sum(1 for e in enc if e > 0)
         out = fd.append_attention(dev["qkv"], dev["key_cache"], dev["value_cache"], dev["seq_lens_encoder"],
                                   dev["seq_lens_decoder"], dev["seq_lens_this_time"], dev["block_tables"],
                                   (dev["rope_cos"], dev["rope_sin"]), dev["cache_k_scale"], dev["cache_v_scale"],
                                   num_heads=hq, kv_num_heads=hkv, max_chunk=max(enc), cache_quant_type=quant,
-                                  cu_seqlens_q=dev["cu_seqlens_q"], prefill_rows=rows if it % 2 else None)
+                                  cu_seqlens_q=dev["cu_seqlens_q"], prefill_rows=rows if it % 2 else None,
+                                  decode_tokens=tokens)
         torch.cuda.synchronize()
-        what = "step %d: enc %r dec %r group %d hkv %d quant %d" % (it, enc, dec, group, hkv, quant)
-        want, kc, vc = oracle_step(oracle, c, quant, hq, hkv, 128)
+        what = "seed %d step %d: enc %r dec %r this %r group %d hkv %d quant %d tokens %d" % (
+            seed, it, enc, dec, this, group, hkv, quant, tokens)
+        want, kc, vc = oracle_step(oracle, c, quant, hq, hkv, 128, decode_tokens=tokens)
         assert np.array_equal(np_of(dev["key_cache"]), kc) and np.array_equal(np_of(dev["value_cache"]), vc), what
         if is_dynamic(quant):
             assert np.array_equal(np_of(dev["cache_k_scale"]), c["scales_after"][0]), what
             assert np.array_equal(np_of(dev["cache_v_scale"]), c["scales_after"][1]), what
         ok, mx, bad = bf16_close(bits(out), want)
         assert ok, "%s: %d out of tolerance, max %.4g" % (what, bad, mx)
+
+
+def test_mixed_step_random_batches_against_the_oracle(oracle):
+    random_steps(oracle, 7, 30)
 
 
 def test_steps_over_block_pool_tables_with_a_shared_prefix(oracle):
