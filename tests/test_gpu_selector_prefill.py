@@ -334,3 +334,60 @@ def test_prefill_shape_agnostic_kernel_shapes(oracle, hq, hkv, d, bs, quant):
                                            np_of(c["seq_lens_decoder"]), np_of(cu), hq, hkv, d, quant)
     ok, mx, bad = bf16_close(bits(out), want)
     assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
+
+
+def test_selector_random_shapes_against_the_oracle(oracle):
+    """60 seeded random cases: 1 .. 8 query heads per KV head, 1 .. 3 KV heads, the four cache formats, lengths that
+    favour zero and block boundaries, table rows wider than needed, top_k 1 .. 39: kept indices and counts exact."""
+    rng = np.random.default_rng(11)
+    for it in range(60):
+        group, hkv, quant = int(rng.integers(1, 9)), int(rng.integers(1, 4)), int(rng.integers(1, 5))
+        hq, batch = group * hkv, int(rng.integers(1, 6))
+        lens = [[0, 64 * int(rng.integers(0, 60)), int(rng.integers(1, 6000))][int(rng.integers(0, 3))] for _ in range(batch)]
+        if not any(lens):
+            lens[0] = 130
+        mb = max(lens) // 64 + 1 + int(rng.integers(0, 3))
+        top_k = int(rng.integers(1, 40))
+        c = syn.decode_case(batch=batch, ctx=lens, quant=quant, seed=3000 + it, extra_blocks=2, hq=hq, hkv=hkv,
+                            max_blocks=mb, row_log2=(-4, 2), salient=0.05)
+        what = "case %d: group %d hkv %d quant %d lens %r mb %d top_k %d" % (it, group, hkv, quant, lens, mb, top_k)
+        dev = syn.to_device(c, "cuda")
+        kept, cnt = fd.sqattn_select(dev["q"], dev["key_cache"], dev["cache_k_scale"], dev["block_tables"],
+                                     dev["seq_lens_decoder"], num_heads=hq, top_k=top_k, cache_quant_type=quant)
+        sc = oracle.sqattn_block_scores(bits(c["q"]), np_of(c["key_cache"]), np_of(c["cache_k_scale"]),
+                                        np_of(c["block_tables"]), np_of(c["seq_lens_decoder"]), hq, hkv, 128, quant)
+        wk, wc = oracle.topk_select(sc, np_of(c["seq_lens_decoder"]), 64, top_k)
+        assert np.array_equal(np_of(cnt), wc) and np.array_equal(np_of(kept), wk), what
+
+
+def test_prefill_random_shapes_against_the_oracle(oracle):
+    """40 seeded random launches of the MFMA kernel: 1 / 2 / 3 / 4 / 8 query heads per KV head, 1 .. 3 KV heads, the
+    four formats, 1 .. 4 sequences with short (packed), medium or long chunks on prefixes of zero, whole blocks or
+    anything, key splits chosen by the library or forced to 1 .. 8."""
+    rng = np.random.default_rng(12)
+    for it in range(40):
+        group, hkv, quant = [1, 2, 3, 4, 8][int(rng.integers(0, 5))], int(rng.integers(1, 4)), int(rng.integers(1, 5))
+        hq, batch, kind = group * hkv, int(rng.integers(1, 5)), int(rng.integers(0, 3))
+        hi = [max(2, 256 // group // 2), 400, 700][kind]
+        chunks = [int(rng.integers(100 if kind == 2 else 1, hi)) for _ in range(batch)]
+        prefix = [[0, 64 * int(rng.integers(0, 30)), int(rng.integers(1, 2500))][int(rng.integers(0, 3))] for _ in range(batch)]
+        c = syn.decode_case(batch=batch, ctx=prefix, quant=quant, seed=4000 + it, extra_blocks=12, hq=hq, hkv=hkv,
+                            row_log2=(-6, 0))
+        g = torch.Generator().manual_seed(4000 + it)
+        T = sum(chunks)
+        q = torch.randn((T, hq * 128), generator=g).to(torch.bfloat16)
+        k = torch.randn((T, hkv * 128), generator=g).to(torch.bfloat16)
+        v = torch.randn((T, hkv * 128), generator=g).to(torch.bfloat16)
+        cu = torch.tensor([0] + list(np.cumsum(chunks)), dtype=torch.int32)
+        ns = [None, 1, 2, 3, 5, 8][int(rng.integers(0, 6))]
+        what = "case %d: group %d hkv %d quant %d chunks %r prefix %r splits %r" % (it, group, hkv, quant, chunks, prefix, ns)
+        dev = syn.to_device(c, "cuda")
+        out = fd.append_attention_prefill(q.cuda(), k.cuda(), v.cuda(), dev["key_cache"], dev["value_cache"],
+                                          dev["cache_k_scale"], dev["cache_v_scale"], dev["block_tables"],
+                                          dev["seq_lens_decoder"], cu.cuda(), num_heads=hq, max_chunk=max(chunks),
+                                          cache_quant_type=quant, num_splits=ns)
+        want = oracle.append_attention_prefill(bits(q), bits(k), bits(v), np_of(c["key_cache"]), np_of(c["value_cache"]),
+                                               np_of(c["cache_k_scale"]), np_of(c["cache_v_scale"]), np_of(c["block_tables"]),
+                                               np_of(c["seq_lens_decoder"]), np_of(cu), hq, hkv, 128, quant)
+        ok, mx, bad = bf16_close(bits(out), want)
+        assert ok, "%s: %d out of tolerance, max %.4g" % (what, bad, mx)
