@@ -61,6 +61,23 @@ def _compile(src):
     return obj
 
 
+def highest_agpr(line):
+    """Highest accumulation register an assembly line names, -1 if none: both ends of a tuple count (`a[28:43]` reaches
+    a43 although it starts below a32), as do single registers (`a7`); whatever follows a `;` is a comment."""
+    import re
+    code, top = line.split(";")[0], -1
+    for lo, hi in re.findall(r"\ba\[(\d+):(\d+)\]", code):
+        top = max(top, int(lo), int(hi))
+    for reg in re.findall(r"\ba\[?(\d+)\b", code):
+        top = max(top, int(reg))
+    return top
+
+
+# What the hand-written register plan of prefill_v2.hip assumes of the compiler's resource report: every kernel owns
+# the whole register file of its SIMD - 256 VGPRs (the accumulation registers start right behind them) and 256 AGPRs.
+PLAN_AGPRS, PLAN_ACCUM_OFFSET = 256, 256
+
+
 def _check_register_plan():
     """prefill_v2.hip addresses the upper AGPRs by name from asm statements, behind the compiler's back; what the
     compiler itself allocates must stay in the VGPRs and the lowest AGPRs (a[0:31]; a[0:63] for the kernels of the formats
@@ -91,8 +108,25 @@ def _check_register_plan():
         elif not in_asm and not re.match(r"^\s*[;.]", line):
             if "scratch_" in line:
                 scratch[kernel] += 1
-            for reg in re.findall(r"\ba\[?(\d+)", line.split(";")[0]):
-                worst[kernel] = (max(worst[kernel][0], int(reg)), worst[kernel][1])
+            worst[kernel] = (max(worst[kernel][0], highest_agpr(line)), worst[kernel][1])
+    # the kernel descriptors of the same assembly: `.amdhsa_accum_offset` / `.amdhsa_next_free_vgpr` follow each
+    # kernel's `.amdhsa_kernel <name>` line
+    desc, cur = {}, None
+    for line in r.stdout.splitlines():
+        m = re.match(r"^\s*\.amdhsa_kernel\s+(\S+)", line)
+        if m:
+            cur = m.group(1)
+            continue
+        m = re.match(r"^\s*\.amdhsa_(accum_offset|next_free_vgpr)\s+(\d+)", line)
+        if m and cur in worst:
+            desc.setdefault(cur, {})[m.group(1)] = int(m.group(2))
+    for k in worst:
+        d = desc.get(k, {})
+        if d.get("accum_offset") != PLAN_ACCUM_OFFSET or d.get("next_free_vgpr") != PLAN_ACCUM_OFFSET + PLAN_AGPRS:
+            raise RuntimeError("register-plan check failed for %s: the kernel descriptor says accum_offset %s, "
+                               "next_free_vgpr %s; the hand-written plan needs %d and %d" %
+                               (k, d.get("accum_offset"), d.get("next_free_vgpr"), PLAN_ACCUM_OFFSET,
+                                PLAN_ACCUM_OFFSET + PLAN_AGPRS))
     if len(worst) != 4:
         raise RuntimeError("register-plan check: expected 4 prefill_v2 kernels in the assembly, found %d" % len(worst))
     for k, (hi, limit) in worst.items():

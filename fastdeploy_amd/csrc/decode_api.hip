@@ -100,15 +100,19 @@ extern "C" int fdattn_decode_attention_noalloc(
                              seq_lens_decoder, out, out, batch, hq, hkv, head_dim, block_size,
                              max_blocks_per_seq, num_blocks, cache_quant_type);
   if (rc) return rc;
-  // the least these shapes accept: a batch of very few sequences then uses the splits the scratch holds
-  const size_t need = decode_workspace_need(batch, hq, hkv, head_dim, max_blocks_per_seq, false);
+  // what the kernel that takes these shapes needs, and no more: the int8-MFMA kernel's partials (one per chunk of a
+  // block list; none at all once every list is a single chunk) or, at the other shapes, the least the split-KV kernels
+  // accept (a batch of very few sequences then uses the splits the scratch holds)
+  const bool mfma_c8 = c8_supported(hq, hkv, head_dim, block_size, cache_quant_type);
+  const size_t need = mfma_c8 ? c8_workspace_bytes(batch, hkv, max_blocks_per_seq, hq / hkv)
+                              : generic_workspace_bytes(batch, hq, head_dim, 0);
   if (need > kStaticScratchBytes)
     return fail(FDATTN_ERR_WORKSPACE, "%s: these shapes need %zu B of split-KV scratch, the library's static scratch "
                 "holds %zu B: call fdattn_decode_attention with a workspace of the caller's", fn, need, kStaticScratchBytes);
   void* ws = nullptr;
   rc = static_scratch(fn, &ws);
   if (rc) return rc;
-  if (c8_supported(hq, hkv, head_dim, block_size, cache_quant_type))
+  if (mfma_c8)
     return decode_c8_launch(q, key_cache, value_cache, cache_k_scale, cache_v_scale, block_tables,
                             seq_lens_decoder, seq_lens_this_time, nullptr, nullptr, 0, out, ws,
                             kStaticScratchBytes, batch, hq, hkv, head_dim, block_size, max_blocks_per_seq,

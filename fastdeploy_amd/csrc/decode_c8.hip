@@ -40,6 +40,7 @@
 // and the barrier sit at the end of every workgroup, where nothing hides their latency),
 // and handing chunks out through an atomic ticket counter instead of the block index.
 #include <atomic>
+#include <mutex>
 
 #include "c8_common.h"
 
@@ -559,10 +560,29 @@ constexpr int kMaxPairs = 1 << 20;
 // more chunks than 257), so the largest count over all lengths up to max_units is taken.
 size_t c8_workspace_bytes(int batch, int hkv, int max_units, int group) {
   const int pairs = batch * hkv;
-  int most = 1;
-  for (int u = 1; u <= max_units; ++u) {
-    const int chunk = c8_pick_chunk(pairs, u), n = (u + chunk - 1) / chunk;
-    if (n > most) most = n;
+  // The scan below sits on the per-step host path (every step sizes its workspace) and costs one division chain per
+  // list length - tens of microseconds at 128k-token tables - so the last few answers are kept: a serving loop
+  // asks for the same (pairs, max_units) step after step.
+  struct Memo { int pairs, max_units, cus, most; };
+  static std::mutex mu;
+  static Memo memo[8];
+  static int next = 0;
+  const int cus = gpu_cu_count();
+  int most = 0;
+  {
+    std::lock_guard<std::mutex> g(mu);
+    for (const Memo& m : memo)
+      if (m.most && m.pairs == pairs && m.max_units == max_units && m.cus == cus) most = m.most;
+  }
+  if (!most) {
+    most = 1;
+    for (int u = 1; u <= max_units; ++u) {
+      const int chunk = c8_pick_chunk(pairs, u), n = (u + chunk - 1) / chunk;
+      if (n > most) most = n;
+    }
+    std::lock_guard<std::mutex> g(mu);
+    memo[next] = Memo{pairs, max_units, cus, most};
+    next = (next + 1) % 8;
   }
   const size_t slots = (size_t)pairs * most;
   const int sets = (group + kG - 1) / kG;

@@ -241,10 +241,15 @@ FDATTN_API int fdattn_decode_attention(
  * on, held until the process ends).  It has no counterpart in the reference; it is for callers that
  * cannot allocate or size a workspace: code under HIP graph capture, tight serving loops, harnesses
  * that forbid hipMalloc.  Inputs, outputs and results are those of fdattn_decode_attention (the same
- * kernels run).  Shapes whose partials need more than the scratch holds - the smallest workspace
- * fdattn_decode_attention accepts for them (what fdattn_decode_workspace_bytes returns for a batch of
- * at least as many (sequence, KV head) pairs as the GPU has CUs) > 16 MiB, e.g. more than about 8000
- * such pairs - are refused with FDATTN_ERR_WORKSPACE and nothing is enqueued.
+ * kernels run).  Shapes whose partials need more than the scratch holds are refused with
+ * FDATTN_ERR_WORKSPACE and nothing is enqueued.  What a shape needs is what the kernel that takes it needs:
+ *   - the int8-MFMA kernel (fdattn_decode_uses_mfma() = 1): one partial of ceil(hq/hkv / 4) x 2,080 B per chunk of
+ *     a (sequence, KV head) pair's block list; lists are cut into ceil(2 x CUs / pairs) chunks (one, and then no
+ *     partial is written at all, from 512 pairs on a 256-CU GPU), more only beyond 128 blocks per chunk.  Llama-3-8B
+ *     decode at batch 64 (512 pairs, 72 blocks each) asks for 1 MiB; the limit is reached near 8,000 pairs of one
+ *     chunk each, or e.g. 512 pairs of 2,048 blocks (128k tokens) each;
+ *   - the other shapes: 16 partial rows of (head_dim + 2) floats per (sequence, query head), i.e.
+ *     batch x hq <= 2,016 at head_dim 128 (4,032 at 64; 1,016 at 256).
  * The scratch needs no clearing between calls (every partial that is read has been written by the same
  * call).  All calls on one GPU share that GPU's array: calls that overlap there - on different streams,
  * or from different threads - race; serialise them or use fdattn_decode_attention with separate

@@ -224,3 +224,17 @@ def test_pool_create_reports_bad_and_absurd_shapes():
     # a table no host could hold: an error return, nothing unwinds through the C ABI
     assert not lib.fdattn_pool_create(1, 64, 0x7fffffff, 0x7fffffff)
     assert b"out of host memory" in lib.fdattn_last_error()
+
+
+def test_register_plan_parser_reads_both_ends_of_a_register_range():
+    """The build fails when the compiler's own allocation reaches the accumulation registers that prefill_v2.hip
+    addresses by name; the check reads the device assembly, where a tuple `a[28:43]` starts below the limit of 32 and
+    ends above it."""
+    from fastdeploy_amd.build import highest_agpr
+    assert highest_agpr("\tv_accvgpr_write_b32 a[28:43], v1") == 43
+    assert highest_agpr("\tv_mfma_f32_32x32x16_f16 a[0:15], v[2:5], v[6:9], a[0:15]") == 15
+    assert highest_agpr("\tv_accvgpr_read_b32 v3, a31") == 31
+    assert highest_agpr("\tv_accvgpr_read_b32 v3, a7 ; was a[100:131]") == 7
+    assert highest_agpr("\tv_add_f32 v1, v2, v3") == -1
+    assert highest_agpr("\tds_read_b128 v[28:31], v40 offset:32") == -1
+    assert highest_agpr("\tv_accvgpr_mov_b32 a[33], a2") == 33

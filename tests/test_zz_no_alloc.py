@@ -15,13 +15,14 @@ from fastdeploy_amd import synthetic as syn
 pytestmark = pytest.mark.gpu
 
 
-def _call_pair(lib, case):
+def _call_pair(lib, case, partials=True):
     """(output of fdattn_decode_attention_noalloc, output of fdattn_decode_attention) on the same device tensors."""
     dev = syn.to_device(case, "cuda")
     batch, mb = dev["block_tables"].shape
     nb, hkv, bs, d = dev["key_cache"].shape
     hq, quant = case["hq"], case["quant"]
-    assert lib.fdattn_decode_chunks_per_sequence(batch, hkv, mb) > 1, "the case must leave partials in the scratch"
+    if partials:
+        assert lib.fdattn_decode_chunks_per_sequence(batch, hkv, mb) > 1, "the case must leave partials in the scratch"
     stream = torch.cuda.current_stream().cuda_stream
     ptrs = [dev[k].data_ptr() for k in ("q", "key_cache", "value_cache", "cache_k_scale", "cache_v_scale",
                                         "block_tables", "seq_lens_decoder")] + [None]
@@ -56,6 +57,21 @@ def test_noalloc_decode_equals_the_workspace_entry_point_twice_in_a_row(oracle, 
                                       case["hkv"], case["d"], case["quant"])
         ok, mx, bad = bf16_close(got, ref)
         assert ok, "%s call vs the oracle: %d out of tolerance, max abs %.4g" % (name, bad, mx)
+
+
+def test_noalloc_decode_takes_the_headline_shape():
+    """Batch 64 x 32 / 8 heads x head_dim 128 over 72-block tables: the int8-MFMA kernel needs 1 MiB of partials at most
+    (none in fact: every list is one chunk), well inside the scratch, whatever the other kernels would need there."""
+    lib = _lib.lib()
+    g = torch.Generator().manual_seed(3)
+    lens = torch.randint(3584, 4609, (64,), generator=g).tolist()
+    case = syn.decode_case(batch=64, ctx=lens, pool_blocks=6000, seed=2, device="cuda", max_blocks=72)
+    got, want = _call_pair(lib, case, partials=False)
+    assert np.array_equal(got, want), "headline shape: outputs of the two entry points differ"
+    # and a batch of the same sequences small enough to be cut into chunks (partials + merge), right after it
+    small = {k: (v[:5].contiguous() if k in ("q", "block_tables", "seq_lens_decoder") else v) for k, v in case.items()}
+    got, want = _call_pair(lib, small)
+    assert np.array_equal(got, want), "5 of the 64 sequences: outputs of the two entry points differ"
 
 
 def test_noalloc_decode_on_the_shape_agnostic_kernel_and_its_limit():
