@@ -195,7 +195,7 @@ def other_workloads(args):
              16 * 32768 * 8 * 128 + 16 * 8 * 64 * 64 * 128 * 2, HBM_PEAK_GBPS, "GB/s",
              {"us_from_a_hip_graph": round(time_graph(sparse_step, args.steps) * 1e3, 2)})
 
-    if args.workload in ("prefill", "all"):
+    if args.workload in ("prefill", "prefill_configs4", "all"):
         # configs[4]: batch 2, 2048 new tokens on 8192 cached (int8 paged: N(0,1) activations quantised with
         # max-abs / 127 scales, as the configuration states), causal
         c = syn.decode_case(batch=2, ctx=8192, seed=0, device=dev, extra_blocks=8)
@@ -221,14 +221,17 @@ def other_workloads(args):
                                  "frac_of_measured_gemm": round(fl / (ms * 1e-3) / 1e12 / gemm_tflops, 4)})
         # the same shape where the hand-scheduled kernel does not apply: other head sizes and block sizes (the MFMA
         # kernel for head_dim 64 / 128 / 256 at any block size), and the first chunk of two fresh prompts
+        # ("prefill_configs4" stops here: configs[4]'s launches alone, for a profiler run)
+        others = args.workload != "prefill_configs4"
         pf0 = lambda: fd.append_attention_prefill(q, k, v, c["key_cache"], c["value_cache"], c["cache_k_scale"], c["cache_v_scale"],
                                                   c["block_tables"], zeros2, cu, num_heads=32, max_chunk=2048, out=out)
         zeros2 = torch.zeros(2, dtype=torch.int32, device=dev)
-        ms = time_events(pf0, max(args.steps // 5, 20), 30)
-        line("2 x 2048 new tokens on an empty cache (the first chunk of two prompts)", ms, "mfma", 2 * syn.prefill_flops(0, 2048),
-             2500.0, "TFLOP/s")
+        if others:
+            ms = time_events(pf0, max(args.steps // 5, 20), 30)
+            line("2 x 2048 new tokens on an empty cache (the first chunk of two prompts)", ms, "mfma", 2 * syn.prefill_flops(0, 2048),
+                 2500.0, "TFLOP/s")
         del c, q, k, v, out
-        for hd, bsz in ((64, 64), (128, 16), (256, 64)):
+        for hd, bsz in ((64, 64), (128, 16), (256, 64)) if others else ():
             c2 = syn.decode_case(batch=2, ctx=8192, seed=0, device=dev, extra_blocks=8, d=hd, bs=bsz)
             q2 = torch.randn((T, 32 * hd), generator=g, device=dev).to(torch.bfloat16)
             k2 = torch.randn((T, 8 * hd), generator=g, device=dev).to(torch.bfloat16)
@@ -454,7 +457,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--pools", type=int, default=2, help="distinct cache pools rotated between steps")
-    ap.add_argument("--workload", default="decode", choices=["decode", "write_decode", "sqattn", "prefill", "mixed", "speculative", "dynamic", "shapes", "kv_wire", "all"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "write_decode", "sqattn", "prefill", "prefill_configs4", "mixed", "speculative", "dynamic", "shapes", "kv_wire", "all"],
                     help="decode = the headline metric (default); the others print one line per kernel of that row")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -494,14 +497,33 @@ def main():
         run(counter[0], impl)
         counter[0] += 1
 
+    chunks_per_pair = _lib.lib().fdattn_decode_chunks_per_sequence(B, 8, 72)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     ms_op = time_events(lambda: step("auto"), args.steps, args.warmup)
     wall = time.perf_counter() - t0
     each = time_each(lambda: step("auto"), args.steps)
-    # the dominant kernel alone (the same launches without the merge), for the roofline line
-    ms_main = time_events(lambda: step("partials"), args.steps, args.warmup)
-    ms_merge = time_events(lambda: step("merge"), args.steps, args.warmup)
+    if chunks_per_pair == 1:
+        # every (sequence, KV head) list is one chunk: the op IS one launch of decode_c8_kernel (no merge kernel), so
+        # the roofline prices the kernel with the very loop `value` comes from - the events bracket the launches and
+        # the gaps between them, i.e. an upper bound of the kernel's own duration
+        ms_main, ms_merge, kernel_timing = ms_op, 0.0, "the timed region of `value` (one kernel per step)"
+    else:
+        # the dominant kernel alone (the same launches without the merge), timed in one loop with the whole op so that
+        # both see the same clocks and cache state: step 2 i is the whole op, step 2 i + 1 the main kernel only
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2 * args.steps + 1)]
+        torch.cuda.synchronize()
+        ev[0].record()
+        for i in range(args.steps):
+            step("auto")
+            ev[2 * i + 1].record()
+            step("partials")
+            ev[2 * i + 2].record()
+        torch.cuda.synchronize()
+        ms_op2 = sum(ev[2 * i].elapsed_time(ev[2 * i + 1]) for i in range(args.steps)) / args.steps
+        ms_main = sum(ev[2 * i + 1].elapsed_time(ev[2 * i + 2]) for i in range(args.steps)) / args.steps
+        ms_main = min(ms_main, ms_op)
+        ms_merge, kernel_timing = max(ms_op2 - ms_main, 0.0), "events around alternating whole-op and main-kernel-only launches"
 
     # single launches timed one by one (event pair each): the spread behind the average
     singles = []
@@ -541,16 +563,19 @@ def main():
         "tokens_per_s_32_layers_attention_only": round(B / (32 * ms_op * 1e-3), 1),
         # chunks per (sequence, KV head): 1 = every pair is finished by the main kernel, no merge kernel is launched
         # (the merge-only call then measures an empty call: host overhead of the timing loop)
-        "chunks_per_pair": _lib.lib().fdattn_decode_chunks_per_sequence(B, 8, 72),
-        "kernel_us": {"decode_c8_kernel": round(ms_main * 1e3, 3),
-                      "merge_stage_call": round(ms_merge * 1e3, 3)},
+        "chunks_per_pair": chunks_per_pair,
+        "kernel_us": {"decode_c8_kernel": round(ms_main * 1e3, 3), "merge_kernel": round(ms_merge * 1e3, 3),
+                      "timed_by": kernel_timing},
         "roofline": {"bound": "hbm", "kernel": "decode_c8_kernel<int8,dense>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "algorithmic_bytes": alg_bytes, "traffic": int(alg_bytes * TRAFFIC_PER_ALGORITHMIC_BYTE),
                      "traffic_source": "%s: FETCH_SIZE + WRITE_SIZE per dispatch / algorithmic bytes = %.4f, applied "
                                        "to this run's algorithmic bytes" % (TRAFFIC_PROFILE, TRAFFIC_PER_ALGORITHMIC_BYTE),
                      "device_copy_gbps_same_run": round(copy_gbps, 1),
-                     "frac_of_device_copy": round(achieved / copy_gbps, 4)},
+                     "frac_of_device_copy": round(achieved / copy_gbps, 4),
+                     # the same bytes over the median of launches timed ONE BY ONE (a device sync after each): no next
+                     # launch fills the tail of this one, as a GEMM before and after it in a real layer would not
+                     "frac_isolated": round(alg_bytes / (singles[len(singles) // 2] * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)},
         "kernel_us_single_launches": {"min": round(singles[0], 2), "median": round(singles[len(singles) // 2], 2),
                                       "max": round(singles[-1], 2), "n": len(singles)},
     }

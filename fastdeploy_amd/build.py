@@ -98,7 +98,7 @@ def _check_register_plan():
             continue
         if kernel is None:
             continue
-        if "s_endpgm" in line:
+        if re.match(r"^\.Lfunc_end\d+:", line):  # (not s_endpgm: a kernel with early returns has several)
             kernel = None
             continue
         if "#ASMSTART" in line:

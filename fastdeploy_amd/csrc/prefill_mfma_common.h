@@ -39,6 +39,21 @@ __device__ __forceinline__ uint4 chunk_v_f16(uint4 v) {
   return make_uint4(hw[0], hw[1], hw[2], hw[3]);
 }
 
+// Running maximum of |x| over bf16 values, two at a time on their bit patterns (the order of non-negative floats is
+// the order of their bits; NaNs sort above everything), and the test of such a maximum against a limit
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ u32 bf16x8_absmax(uint4 v, u32 acc) {
+  const u32 vw[4] = {v.x, v.y, v.z, v.w};
+  u16x2 m = __builtin_bit_cast(u16x2, acc);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) m = __builtin_elementwise_max(m, __builtin_bit_cast(u16x2, vw[e] & 0x7fff7fffu));
+  return __builtin_bit_cast(u32, m);
+}
+__device__ __forceinline__ bool bf16_absmax_above(u32 acc, float limit) {
+  const u32 lim = __float_as_uint(limit) >> 16;  // limit: a positive value that bf16 holds exactly
+  return (acc & 0xffffu) > lim || (acc >> 16) > lim;
+}
+
 // 8 cache bytes -> 8 fp16 holding the bytes' exact values
 template <int QUANT>
 __device__ __forceinline__ uint4 cvt8(u32 w0, u32 w1) {

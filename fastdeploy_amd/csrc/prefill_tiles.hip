@@ -37,8 +37,12 @@ struct TileLay {
   // 64 B keep the rows a ds_read_b64_tr_b16 touches apart (the strides are 4 and 16 banks modulo 64 at every D)
   static constexpr int LDK = D + 8, LDV = D + 32;
   static constexpr int K_ELEMS = TK * LDK, BUF_ELEMS = TK * (LDK + LDV);
-  static constexpr size_t kBytes = 2 * (size_t)BUF_ELEMS * 2 + 2 * 3 * TK * sizeof(float);
+  static constexpr size_t kScales = 2 * (size_t)BUF_ELEMS * 2, kFlags = kScales + 2 * 3 * TK * sizeof(float);
+  static constexpr size_t kBytes = kFlags + 16;  // four ints: which staged tiles hold large V values
 };
+// Dequantised V magnitudes (the chunk's own V included) beyond which a tile's P.V product takes the softmax weights as
+// two fp16 terms (one term leaves an output element off by up to 2^-11 * sum_j p_j |v_j|): as in prefill_v2.hip.
+constexpr float kExactAbove = 6.0f;
 
 template <int QUANT, bool DYN, int D>
 __global__ __launch_bounds__(64 * waves_t<D>(), 1) void prefill_tiles_kernel(PrefillArgs a) {
@@ -71,6 +75,27 @@ __global__ __launch_bounds__(64 * waves_t<D>(), 1) void prefill_tiles_kernel(Pre
   const int g_end = wave_active ? n_pre + min(q0 + 32 * wv + 31, n_b - 1) / TK + 1 : 0;  // tiles of this wavefront
   const int32_t* const table = a.block_tables + (size_t)b * a.max_blocks;
   const float sc = a.sm_scale * 1.4426950408889634f;  // logits go to the log2 domain
+  // ---- which tiles need two-term weights.  Per-channel formats: the whole prefix of this KV head, if the largest code
+  // times its largest V scale may exceed the limit.  Formats with scale caches and the chunk's own tiles: per tile,
+  // found while the tile is staged - the threads that see a large value leave the tile's number in tile_flag[tile % 4];
+  // whatever else the word holds says no, and a stale match could only send a tile down the slower, exact path.
+  __attribute__((address_space(3))) int* const tile_flag = (__attribute__((address_space(3))) int*)((__attribute__((address_space(3))) uint8_t*)lds + L::kFlags);
+  constexpr float kCodeMax = QUANT == FDATTN_CACHE_INT8 ? 127.0f : 448.0f;
+  bool pre_exact = false;
+  if (!DYN) {
+    float m = 0.f;
+    for (int c = lane; c < D; c += 64) m = fmaxf(m, fabsf(a.v_scale[h * D + c]));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    pre_exact = !(m * kCodeMax <= kExactAbove);  // (NaN scales: the exact path)
+  }
+  auto flag_tile = [&](int t, bool large) {
+    if (__any(large) && lane == 0) tile_flag[t & 3] = t + 1;
+  };
+  auto tile_exact = [&](int t) -> bool {
+    if (t < n_pre && !DYN) return pre_exact;
+    return __builtin_amdgcn_readfirstlane(tile_flag[t & 3]) == t + 1;
+  };
 
   // ---- Q as the B operand: lane = query, channels 16 st + 8 hf .. + 7 of k-step st
   v8h qa[KT], ql[KT];  // prefix: the hi and lo fp16 terms of q x k_scale x c; chunk: qa = the bf16 q as it is
@@ -233,6 +258,7 @@ __global__ __launch_bounds__(64 * waves_t<D>(), 1) void prefill_tiles_kernel(Pre
           lds_store16(vd + row * L::LDV + ch * 16 + 8, cvt8<QUANT>(vw.z, vw.w));
         }
       }
+      if (DYN) flag_tile(t, tid >= TK && tid < 2 * TK && t * TK + (tid - TK) < p && !(fabsf(s_scale) * kCodeMax <= kExactAbove));
       if (DYN && tid < 2 * TK) {  // what the softmax needs of a key's scales, worked out once per tile
         const float sv1 = t * TK + (tid & (TK - 1)) < p ? s_scale : 1.f;  // (slots past the prefix may hold anything)
         float* const dst = lds_sc + (t & 1) * 3 * TK;
@@ -244,6 +270,7 @@ __global__ __launch_bounds__(64 * waves_t<D>(), 1) void prefill_tiles_kernel(Pre
         }
       }
     } else {
+      u32 big = 0;
 #pragma unroll
       for (int i = 0; i < 2 * NC; ++i) {
         const int idx = tid + NT * i;
@@ -251,8 +278,10 @@ __global__ __launch_bounds__(64 * waves_t<D>(), 1) void prefill_tiles_kernel(Pre
           const int row = idx / (2 * CPR), ch = idx % (2 * CPR);
           lds_store16(kd + row * L::LDK + ch * 8, sk[i]);
           lds_store16(vd + row * L::LDV + ch * 8, chunk_v_f16(sv[i]));
+          big = bf16x8_absmax(sv[i], big);
         }
       }
+      flag_tile(t, bf16_absmax_above(big, kExactAbove));
     }
   };
 
@@ -333,6 +362,7 @@ __global__ __launch_bounds__(64 * waves_t<D>(), 1) void prefill_tiles_kernel(Pre
     // tile, scores outgrowing the reference): the exact maximum, the reference raised, what the query has accumulated
     // rescaled, the weights computed again.
     u32 pw[8];
+    const bool exact = tile_exact(g);
     float esum, lsum;  // the plain sum of the lane's weights; the sum that goes to the query's weight sum
     auto weights = [&]() {
       const float cst = m_ref == -INFINITY ? 0.f : -m_ref;
@@ -378,6 +408,26 @@ __global__ __launch_bounds__(64 * waves_t<D>(), 1) void prefill_tiles_kernel(Pre
       weights();
     }
     l_run += lsum;
+    if (exact) {
+      // a tile with large V values: what the rounding to fp16 left of each weight, p - fp16(p) (exact in fp32, itself
+      // rounded to fp16: 22 bits in all), enters O += V P as a second term - 16 keys at a time, from the logits again
+      // (one more exponential per weight: cheaper in registers than keeping the fp32 weights, and the rare case)
+      const float cst = m_ref == -INFINITY ? 0.f : -m_ref;
+#pragma unroll
+      for (int ss = 0; ss < 2; ++ss) {
+        u32 w[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int r = 8 * ss + 2 * j;
+          const float e0 = __builtin_amdgcn_exp2f(x[r] + cst), e1 = __builtin_amdgcn_exp2f(x[r + 1] + cst);
+          const v2h hv = __builtin_bit_cast(v2h, pw[r >> 1]);
+          w[j] = pack_f16(e0 - (float)hv[0], e1 - (float)hv[1]);
+        }
+        const v8h pl = __builtin_bit_cast(v8h, make_uint4(w[0], w[1], w[2], w[3]));
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) o[ct] = __builtin_amdgcn_mfma_f32_32x32x16_f16(v_operand(buf, ss, ct), pl, o[ct], 0, 0, 0);
+      }
+    }
     const v8h pp[2] = {__builtin_bit_cast(v8h, make_uint4(pw[0], pw[1], pw[2], pw[3])),
                        __builtin_bit_cast(v8h, make_uint4(pw[4], pw[5], pw[6], pw[7]))};
 #pragma unroll

@@ -59,7 +59,12 @@ constexpr int kWavesPf = 4, BM = 64 * kWavesPf;  // queries per workgroup
 constexpr int kMaxSplitsV2 = 8;
 constexpr float kSumLimit = 16384.0f;  // a query's weight sum over 32 keys above which its exponent reference is raised (every weight stays inside fp16)
 constexpr size_t kLdsScales = (size_t)kSlots * BUF_ELEMS * 2, kLdsQlo = kLdsScales + (size_t)kSlots * 3 * BN * sizeof(float);
-constexpr size_t kLdsBytes = kLdsQlo + (size_t)kWavesPf * 8 * 64 * 16;
+constexpr size_t kLdsFlags = kLdsQlo + (size_t)kWavesPf * 8 * 64 * 16;  // four ints: which staged tiles hold large V values
+constexpr size_t kLdsBytes = kLdsFlags + 16;
+// Dequantised V magnitudes (the chunk's own V included) beyond which a tile's P.V product takes the softmax weights as
+// TWO fp16 terms: one term leaves an output element off by up to 2^-11 * sum_j p_j |v_j| <= 2^-11 * max|v|, which
+// passes 2e-3 only while the values a query attends to stay moderate.
+constexpr float kExactAbove = 6.0f;
 
 // Register plan.  A wavefront owns the SIMD's whole register file.  The upper AGPRs hold what only MFMAs touch and are
 // addressed BY NAME in single-instruction asm statements; the compiler is left the 256 VGPRs and a[0:31] (it parks
@@ -286,6 +291,29 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
   }
   const int32_t* table = a.block_tables + (size_t)b * a.max_blocks;
   const float sc = a.sm_scale * 1.4426950408889634f;  // logits go to the log2 domain
+  // ---- which tiles need two-term weights (see kExactAbove).  Per-channel formats: the whole prefix of this KV head, if
+  // the largest code times its largest V scale may exceed the limit (no byte is looked at).  Formats with scale caches
+  // and the chunk's own tiles: per tile, found while the tile is staged - the staging threads that see a large value
+  // leave the tile's number in tile_flag[tile % 4]; whatever else the word holds (an older tile, nothing yet) says no,
+  // and a stale match could only send a tile down the slower, exact path.
+  __attribute__((address_space(3))) int* const tile_flag = (__attribute__((address_space(3))) int*)((__attribute__((address_space(3))) uint8_t*)lds + kLdsFlags);
+  constexpr float kCodeMax = QUANT == FDATTN_CACHE_INT8 ? 127.0f : 448.0f;
+  bool pre_exact = false;
+  if (!DYN) {
+    const float2 vs2 = *reinterpret_cast<const float2*>(a.v_scale + h * HD + 2 * lane);
+    float m = fmaxf(fabsf(vs2.x), fabsf(vs2.y));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    pre_exact = !(m * kCodeMax <= kExactAbove);  // (NaN scales: the exact path)
+  }
+  auto flag_tile = [&](int t, bool large) {
+    if (__any(large) && lane == 0) tile_flag[t & 3] = t + 1;
+  };
+  auto tile_exact = [&](int t) -> bool {
+    if (t >= t1) return false;
+    if (t < n_pre && !DYN) return pre_exact;
+    return __builtin_amdgcn_readfirstlane(tile_flag[t & 3]) == t + 1;
+  };
 
   // half-tile steps of this wavefront: [g_begin, g_end); chunk halves wholly above its diagonal are not computed
   const int g_begin = 2 * t0;
@@ -421,6 +449,7 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
     lds_u16* const kd = (lds_u16*)lds + (size_t)slot * BUF_ELEMS + srow * LDK + scc;
     lds_u16* const vd = (lds_u16*)lds + (size_t)slot * BUF_ELEMS + K_ELEMS + srow * LDV + scc;
     if (t < n_pre) {
+      if (DYN) flag_tile(t, tid >= BN && tid < 2 * BN && t * BN + (tid - BN) < p && !(fabsf(stg_s) * kCodeMax <= kExactAbove));
       // rows past the cached prefix hold stale bytes (fp8 has NaN codes): zeros are staged for them
       if ((t + 1) * BN > p) {
 #pragma unroll
@@ -446,11 +475,14 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
         }
       }
     } else {
+      u32 big = 0;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         lds_store16(kd + i * 16 * LDK, stg_k[i]);
         lds_store16(vd + i * 16 * LDV, chunk_v_f16(stg_v[i]));
+        big = bf16x8_absmax(stg_v[i], big);
       }
+      flag_tile(t, bf16_absmax_above(big, kExactAbove));
     }
   };
   auto commit = [&](int t) { commit_from(t, stg_k, stg_v, stg_s); };
@@ -627,6 +659,44 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
     l_run[qb] += (DYN && pre) ? (acc.lt[0] + acc.lt[1]) + (acc.lt[2] + acc.lt[3]) : tsum;
   };
   // the whole softmax of half tile g, one query block after the other
+  // The second fp16 term of the weights of half tile g, p - fp16(p), into O += V P: for half tiles of tiles that hold
+  // large V values (tile_exact), right behind their softmax - the tile is in LDS, the scores s and the first terms pp
+  // are at hand, the query's reference is final - while the first terms follow with the next step as always.  One
+  // 16-key step of one query block at a time, from the scores again (one more exponential per weight: cheaper in
+  // registers than carrying the fp32 weights, and this is the rare case); a weight is exact in fp32 next to its first
+  // term, and the remainder is rounded to fp16: 22 bits in all.
+  auto sm_second_term = [&](int g, const v16f (&s)[2], const v8h (&pp)[2][2]) {
+    const int t = g >> 1, kb = g & 1, slot = t % kSlots;
+    const bool pre = t < n_pre;
+    const float* scales = sm_scales(g);
+    static_for<2>([&](auto QB) {
+      constexpr int qb = decltype(QB)::value;
+      const float scl = pre ? scl_pre[qb] : sc;
+      const float cst = -(m_ref[qb] == -INFINITY ? 0.f : m_ref[qb]);  // the reference the first terms were made against
+      static_for<2>([&](auto SS) {
+        constexpr int ss = decltype(SS)::value;
+        u32 w[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int r = 8 * ss + 2 * j;
+          float x0 = __builtin_fmaf(s[qb][r], scl, cst), x1 = __builtin_fmaf(s[qb][r + 1], scl, cst);
+          if (DYN && pre) {
+            x0 = __builtin_fmaf(s[qb][r], scales[8 * (r >> 2) + (r & 3)], cst) + scales[BN + 8 * (r >> 2) + (r & 3)];
+            x1 = __builtin_fmaf(s[qb][r + 1], scales[8 * ((r + 1) >> 2) + ((r + 1) & 3)], cst) + scales[BN + 8 * ((r + 1) >> 2) + ((r + 1) & 3)];
+          }
+          const float e0 = __builtin_amdgcn_exp2f(x0), e1 = __builtin_amdgcn_exp2f(x1);
+          const v2h hv = __builtin_bit_cast(v2h, __builtin_bit_cast(u4v, pp[qb][ss])[j]);
+          w[j] = pack_f16(e0 - (float)hv[0], e1 - (float)hv[1]);
+        }
+        const v8h pl = __builtin_bit_cast(v8h, make_uint4(w[0], w[1], w[2], w[3]));
+        static_for<4>([&](auto CT) {
+          constexpr int ct = decltype(CT)::value;
+          mfma_o<kAccO + 64 * qb + 16 * ct>(v_operand(slot, kb, ss, ct), pl);
+        });
+      });
+    });
+  };
+  // the whole softmax of half tile g, one query block after the other
   auto softmax = [&](int g, bool masked, v16f (&s)[2], v8h (&pp)[2][2]) {
     const bool pre = (g >> 1) < n_pre;
     mfma_settle(s);
@@ -642,6 +712,7 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
       for (int piece = 0; piece < 4; ++piece) sm_piece(pre, qb, piece, s[qb], scl, cst, scales, acc, pp[qb]);
       sm_finish(pre, qb, s[qb], scl, scales, acc, pp[qb]);
     }
+    if (tile_exact(g >> 1)) sm_second_term(g, s, pp);
   };
 
   // leaving the quantised prefix: the channels of o take their V scale (per-channel formats)
@@ -675,6 +746,7 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
   const uint8_t* st_kbp = nullptr;  // block of tile t + 3 in the caches (set by the kb 0 step, used by both)
   const uint8_t* st_vbp = nullptr;
   int st_row3 = 0;  // chunk steps: this thread's first row of tile t + 3 in the chunk
+  u32 st_vbig = 0;  // chunk steps: largest |V| this thread has staged of tile t + 2 (bf16 bit patterns, two at a time)
   auto fast_step = [&](int t, auto KB, auto CHK) {
     constexpr int kb = decltype(KB)::value;
     constexpr bool CH = decltype(CHK)::value;  // the tiles are the chunk's own keys: bf16 K against the bf16 q, one term, no scales; the softmax is masked where the wavefront's diagonal crosses the half tile
@@ -696,6 +768,7 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
       if (DYN && tid < 2 * BN) {
         const size_t srow0 = ((size_t)pb * a.hkv + h) * a.scale_rows + (a.scale_rows == 1 ? 0 : (tid & (BN - 1)));
         const float next = tid < BN ? a.k_scale[srow0] : a.v_scale[srow0];
+        flag_tile(t + 2, tid >= BN && !(fabsf(stg_s) * kCodeMax <= kExactAbove));  // (threads BN .. 2 BN - 1 hold the V scales of tile t + 2)
         if (tid < BN) {
           lds_sc[slot_st * 3 * BN + tid] = sc * stg_s;
         } else {
@@ -721,6 +794,8 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
           stg_k[i] = *reinterpret_cast<const uint4*>(k_new_seq + off);
         } else {
           lds_store16((lds_u16*)lds + (size_t)slot_st * BUF_ELEMS + K_ELEMS + (srow + 16 * i) * LDV + scc, chunk_v_f16(stg_v[i]));
+          st_vbig = bf16x8_absmax(stg_v[i], c == 4 ? 0u : st_vbig);
+          if constexpr (c == 7) flag_tile(t + 2, bf16_absmax_above(st_vbig, kExactAbove));
           stg_v[i] = *reinterpret_cast<const uint4*>(v_new_seq + off);
         }
       } else if constexpr (c < 4) {
@@ -731,6 +806,8 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
         if constexpr (half == 1) stg_v[pass] = *reinterpret_cast<const uint4*>(st_vbp + (goff + (u32)(pass * 32 * HD)));
       }
     };
+    // does half tile g + 1 (whose weights this step makes) belong to a tile with large V values?  Asked now, used at the end
+    const int flag_sm = (CH || DYN) ? tile_flag[((g + 1) >> 1) & 3] : 0;
     mfma_settle(s_sm);
     if constexpr (CH) {
       if (!unmasked(g + 1)) sm_mask(g + 1, s_sm);  // the wavefront's diagonal
@@ -858,6 +935,7 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
     va_valid = true;
     sm_finish(!CH, 0, s_sm[0], scl[0], scales, acc[0], P[0]);
     sm_finish(!CH, 1, s_sm[1], scl[1], scales, acc[1], P[1]);
+    if ((CH || DYN) ? __builtin_amdgcn_readfirstlane(flag_sm) == ((g + 1) >> 1) + 1 : pre_exact) sm_second_term(g + 1, s_sm, P);
   };
 
   // ---- prologue: two tiles into LDS, the third on its way; the first two half tiles' scores, the first softmax
@@ -893,7 +971,6 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
     // the same schedule over the chunk's own keys, for as long as this wavefront has scores to compute two half
     // tiles ahead (up to 2 t + 3; its last tile takes the plain path below)
     if (t >= n_pre && q_is_chunk && 2 * t + 3 < g_end) {
-      if (t == n_pre && t0 < n_pre) leave_prefix();
       fast_step(t, std::integral_constant<int, 0>{}, std::true_type{});
       fast_step(t, std::integral_constant<int, 1>{}, std::true_type{});
       continue;
@@ -905,9 +982,11 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
     for (int kb = 0; kb < 2; ++kb) {
       const int g = 2 * t + kb;
       if (g >= g_end) break;
-      if (g == 2 * n_pre && t0 < n_pre) leave_prefix();
       if (g + 2 < g_end && (g + 2) == 2 * n_pre && !q_is_chunk) load_q_chunk();
       pv(g, P);
+      // the prefix's last half tile is in: o leaves the quantised units here - before the softmax below, whose half
+      // tile is the chunk's first and may add its weights' second terms to o at once
+      if (g + 1 == 2 * n_pre && t0 < n_pre) leave_prefix();
       if (g + 2 < g_end) qk(g + 2, S[kb]);
       if (g + 1 < g_end) softmax(g + 1, !unmasked(g + 1), S[kb ^ 1], P);
     }
