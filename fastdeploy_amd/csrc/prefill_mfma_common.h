@@ -39,19 +39,22 @@ __device__ __forceinline__ uint4 chunk_v_f16(uint4 v) {
   return make_uint4(hw[0], hw[1], hw[2], hw[3]);
 }
 
-// Running maximum of |x| over bf16 values, two at a time on their bit patterns (the order of non-negative floats is
-// the order of their bits; NaNs sort above everything), and the test of such a maximum against a limit
-typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ u32 bf16x8_absmax(uint4 v, u32 acc) {
-  const u32 vw[4] = {v.x, v.y, v.z, v.w};
-  u16x2 m = __builtin_bit_cast(u16x2, acc);
-#pragma unroll
-  for (int e = 0; e < 4; ++e) m = __builtin_elementwise_max(m, __builtin_bit_cast(u16x2, vw[e] & 0x7fff7fffu));
-  return __builtin_bit_cast(u32, m);
+// Running maximum and minimum over fp16 values, two lanes of a register and two registers per instruction
+// (v_pk_maximum3_f16 / v_pk_minimum3_f16: 8 values cost 4 instructions), and the test of such a pair against a limit:
+// does any value lie beyond +-limit?  (NaNs propagate through both and answer yes.)
+struct F16Range { u32 mx, mn; };  // packed pairs; start from {0, 0}
+__device__ __forceinline__ void f16x8_range(uint4 h, F16Range& r) {
+  asm("v_pk_maximum3_f16 %0, %1, %2, %0" : "+v"(r.mx) : "v"(h.x), "v"(h.y));
+  asm("v_pk_maximum3_f16 %0, %1, %2, %0" : "+v"(r.mx) : "v"(h.z), "v"(h.w));
+  asm("v_pk_minimum3_f16 %0, %1, %2, %0" : "+v"(r.mn) : "v"(h.x), "v"(h.y));
+  asm("v_pk_minimum3_f16 %0, %1, %2, %0" : "+v"(r.mn) : "v"(h.z), "v"(h.w));
 }
-__device__ __forceinline__ bool bf16_absmax_above(u32 acc, float limit) {
-  const u32 lim = __float_as_uint(limit) >> 16;  // limit: a positive value that bf16 holds exactly
-  return (acc & 0xffffu) > lim || (acc >> 16) > lim;
+__device__ __forceinline__ bool f16_range_beyond(const F16Range& r, float limit) {
+  // on the bit patterns: a positive fp16 above the limit is a larger signed 16-bit integer than the limit's pattern,
+  // a negative one below -limit a larger unsigned one than -limit's pattern (positive and negative NaNs included)
+  const int pos = (int)__builtin_bit_cast(unsigned short, (_Float16)limit);
+  const u32 neg = (u32)pos | 0x8000u;
+  return (int)(short)(r.mx & 0xffffu) > pos || (int)(short)(r.mx >> 16) > pos || (r.mn & 0xffffu) > neg || (r.mn >> 16) > neg;
 }
 
 // 8 cache bytes -> 8 fp16 holding the bytes' exact values

@@ -44,8 +44,10 @@ struct TileLay {
 // two fp16 terms (one term leaves an output element off by up to 2^-11 * sum_j p_j |v_j|): as in prefill_v2.hip.
 constexpr float kExactAbove = 6.0f;
 
+// (head_dim 64 with per-channel scales fits 128 registers - two workgroups per CU, four wavefronts per SIMD - when asked
+// to: left to itself the compiler stops a few registers above, at one workgroup per CU and 1.4 times the time)
 template <int QUANT, bool DYN, int D>
-__global__ __launch_bounds__(64 * waves_t<D>(), 1) void prefill_tiles_kernel(PrefillArgs a) {
+__global__ __launch_bounds__(64 * waves_t<D>(), (D == 64 && !DYN) ? 4 : 1) void prefill_tiles_kernel(PrefillArgs a) {
   using L = TileLay<D>;
   constexpr int KT = D / 16, CT = D / 32;  // k-steps of S = K Q; 32-channel blocks of O
   constexpr int CPR = D / 16;              // 16-byte chunks per cache row
@@ -270,18 +272,19 @@ __global__ __launch_bounds__(64 * waves_t<D>(), 1) void prefill_tiles_kernel(Pre
         }
       }
     } else {
-      u32 big = 0;
+      F16Range vr = {0u, 0u};
 #pragma unroll
       for (int i = 0; i < 2 * NC; ++i) {
         const int idx = tid + NT * i;
         if (idx < 2 * NCH) {
           const int row = idx / (2 * CPR), ch = idx % (2 * CPR);
           lds_store16(kd + row * L::LDK + ch * 8, sk[i]);
-          lds_store16(vd + row * L::LDV + ch * 8, chunk_v_f16(sv[i]));
-          big = bf16x8_absmax(sv[i], big);
+          const uint4 vh = chunk_v_f16(sv[i]);
+          lds_store16(vd + row * L::LDV + ch * 8, vh);
+          f16x8_range(vh, vr);
         }
       }
-      flag_tile(t, bf16_absmax_above(big, kExactAbove));
+      flag_tile(t, f16_range_beyond(vr, kExactAbove));
     }
   };
 
@@ -362,6 +365,7 @@ __global__ __launch_bounds__(64 * waves_t<D>(), 1) void prefill_tiles_kernel(Pre
     // tile, scores outgrowing the reference): the exact maximum, the reference raised, what the query has accumulated
     // rescaled, the weights computed again.
     u32 pw[8];
+    // a tile with large V values: its weights enter O += V P as TWO fp16 terms, p = fp16(p) + fp16(p - fp16(p))
     const bool exact = tile_exact(g);
     float esum, lsum;  // the plain sum of the lane's weights; the sum that goes to the query's weight sum
     auto weights = [&]() {
@@ -408,34 +412,34 @@ __global__ __launch_bounds__(64 * waves_t<D>(), 1) void prefill_tiles_kernel(Pre
       weights();
     }
     l_run += lsum;
-    if (exact) {
-      // a tile with large V values: what the rounding to fp16 left of each weight, p - fp16(p) (exact in fp32, itself
-      // rounded to fp16: 22 bits in all), enters O += V P as a second term - 16 keys at a time, from the logits again
-      // (one more exponential per weight: cheaper in registers than keeping the fp32 weights, and the rare case)
-      const float cst = m_ref == -INFINITY ? 0.f : -m_ref;
+    // O += V P.  An exact tile runs the product twice: with the weights as rounded to fp16, then with what the rounding
+    // left - p - fp16(p), from the logits again (exact in fp32 next to the first term, itself rounded to fp16: 22 bits in
+    // all), written over the first terms.  One copy of the product's code in a loop, and no register beyond what the
+    // softmax's own peak needs: head_dim 64 has two to spare before a CU holds one workgroup instead of two.
+#pragma unroll 1
+    for (int term = 0; term < (exact ? 2 : 1); ++term) {
+      if (term == 1) {
+        const float cst = m_ref == -INFINITY ? 0.f : -m_ref;
 #pragma unroll
-      for (int ss = 0; ss < 2; ++ss) {
-        u32 w[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int r = 8 * ss + 2 * j;
+        for (int r = 0; r < 16; r += 2) {
           const float e0 = __builtin_amdgcn_exp2f(x[r] + cst), e1 = __builtin_amdgcn_exp2f(x[r + 1] + cst);
           const v2h hv = __builtin_bit_cast(v2h, pw[r >> 1]);
-          w[j] = pack_f16(e0 - (float)hv[0], e1 - (float)hv[1]);
+          pw[r >> 1] = pack_f16(e0 - (float)hv[0], e1 - (float)hv[1]);
         }
-        const v8h pl = __builtin_bit_cast(v8h, make_uint4(w[0], w[1], w[2], w[3]));
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) o[ct] = __builtin_amdgcn_mfma_f32_32x32x16_f16(v_operand(buf, ss, ct), pl, o[ct], 0, 0, 0);
       }
+      const v8h pp[2] = {__builtin_bit_cast(v8h, make_uint4(pw[0], pw[1], pw[2], pw[3])),
+                         __builtin_bit_cast(v8h, make_uint4(pw[4], pw[5], pw[6], pw[7]))};
+#pragma unroll
+      for (int ss = 0; ss < 2; ++ss)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) o[ct] = __builtin_amdgcn_mfma_f32_32x32x16_f16(v_operand(buf, ss, ct), pp[ss], o[ct], 0, 0, 0);
     }
-    const v8h pp[2] = {__builtin_bit_cast(v8h, make_uint4(pw[0], pw[1], pw[2], pw[3])),
-                       __builtin_bit_cast(v8h, make_uint4(pw[4], pw[5], pw[6], pw[7]))};
-#pragma unroll
-    for (int ss = 0; ss < 2; ++ss)
-#pragma unroll
-      for (int ct = 0; ct < CT; ++ct) o[ct] = __builtin_amdgcn_mfma_f32_32x32x16_f16(v_operand(buf, ss, ct), pp[ss], o[ct], 0, 0, 0);
   };
 
+
+  // (the flags start empty: whatever an earlier workgroup left in these words must not name one of this walk's tiles)
+  if (tid < 4) tile_flag[tid] = 0;
+  __syncthreads();
   // ---- the walk: tile g in buffer g & 1, tile g + 1 staged into the other at the start of step g, tile g + 2 in flight
   bool q_is_chunk = n_pre == 0;
   if (n_pre > 0) request_entries(0);

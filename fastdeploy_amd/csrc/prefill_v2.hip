@@ -475,14 +475,15 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
         }
       }
     } else {
-      u32 big = 0;
+      F16Range vr = {0u, 0u};
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         lds_store16(kd + i * 16 * LDK, stg_k[i]);
-        lds_store16(vd + i * 16 * LDV, chunk_v_f16(stg_v[i]));
-        big = bf16x8_absmax(stg_v[i], big);
+        const uint4 vh = chunk_v_f16(stg_v[i]);
+        lds_store16(vd + i * 16 * LDV, vh);
+        f16x8_range(vh, vr);
       }
-      flag_tile(t, bf16_absmax_above(big, kExactAbove));
+      flag_tile(t, f16_range_beyond(vr, kExactAbove));
     }
   };
   auto commit = [&](int t) { commit_from(t, stg_k, stg_v, stg_s); };
@@ -676,6 +677,7 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
       static_for<2>([&](auto SS) {
         constexpr int ss = decltype(SS)::value;
         u32 w[4];
+        const u4v first = __builtin_bit_cast(u4v, pp[qb][ss]);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const int r = 8 * ss + 2 * j;
@@ -685,7 +687,8 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
             x1 = __builtin_fmaf(s[qb][r + 1], scales[8 * ((r + 1) >> 2) + ((r + 1) & 3)], cst) + scales[BN + 8 * ((r + 1) >> 2) + ((r + 1) & 3)];
           }
           const float e0 = __builtin_amdgcn_exp2f(x0), e1 = __builtin_amdgcn_exp2f(x1);
-          const v2h hv = __builtin_bit_cast(v2h, __builtin_bit_cast(u4v, pp[qb][ss])[j]);
+          const u32 first_j = first[j];  // (a scalar copy: this compiler's bit cast of a vector ELEMENT reads element 0 whatever the index)
+          const v2h hv = __builtin_bit_cast(v2h, first_j);
           w[j] = pack_f16(e0 - (float)hv[0], e1 - (float)hv[1]);
         }
         const v8h pl = __builtin_bit_cast(v8h, make_uint4(w[0], w[1], w[2], w[3]));
@@ -746,7 +749,7 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
   const uint8_t* st_kbp = nullptr;  // block of tile t + 3 in the caches (set by the kb 0 step, used by both)
   const uint8_t* st_vbp = nullptr;
   int st_row3 = 0;  // chunk steps: this thread's first row of tile t + 3 in the chunk
-  u32 st_vbig = 0;  // chunk steps: largest |V| this thread has staged of tile t + 2 (bf16 bit patterns, two at a time)
+  F16Range st_vr = {0u, 0u};  // chunk steps: the range of the V values this thread has staged of tile t + 2
   auto fast_step = [&](int t, auto KB, auto CHK) {
     constexpr int kb = decltype(KB)::value;
     constexpr bool CH = decltype(CHK)::value;  // the tiles are the chunk's own keys: bf16 K against the bf16 q, one term, no scales; the softmax is masked where the wavefront's diagonal crosses the half tile
@@ -793,9 +796,11 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
           lds_store16((lds_u16*)lds + (size_t)slot_st * BUF_ELEMS + (srow + 16 * i) * LDK + scc, stg_k[i]);
           stg_k[i] = *reinterpret_cast<const uint4*>(k_new_seq + off);
         } else {
-          lds_store16((lds_u16*)lds + (size_t)slot_st * BUF_ELEMS + K_ELEMS + (srow + 16 * i) * LDV + scc, chunk_v_f16(stg_v[i]));
-          st_vbig = bf16x8_absmax(stg_v[i], c == 4 ? 0u : st_vbig);
-          if constexpr (c == 7) flag_tile(t + 2, bf16_absmax_above(st_vbig, kExactAbove));
+          const uint4 vh = chunk_v_f16(stg_v[i]);
+          lds_store16((lds_u16*)lds + (size_t)slot_st * BUF_ELEMS + K_ELEMS + (srow + 16 * i) * LDV + scc, vh);
+          if constexpr (c == 4) st_vr = F16Range{0u, 0u};
+          f16x8_range(vh, st_vr);
+          if constexpr (c == 7) flag_tile(t + 2, f16_range_beyond(st_vr, kExactAbove));
           stg_v[i] = *reinterpret_cast<const uint4*>(v_new_seq + off);
         }
       } else if constexpr (c < 4) {
@@ -938,6 +943,9 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
     if ((CH || DYN) ? __builtin_amdgcn_readfirstlane(flag_sm) == ((g + 1) >> 1) + 1 : pre_exact) sm_second_term(g + 1, s_sm, P);
   };
 
+  // (the flags start empty: whatever an earlier workgroup left in these words must not name one of this walk's tiles)
+  if (tid < 4) tile_flag[tid] = 0;
+  __syncthreads();
   // ---- prologue: two tiles into LDS, the third on its way; the first two half tiles' scores, the first softmax
   // Everything that depends on the sequence's lengths alone is requested before anything is waited for: the block-table
   // entries of the first three tiles, the query rows, the first tile; the conversion of q runs while they are on their
@@ -986,7 +994,8 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
       pv(g, P);
       // the prefix's last half tile is in: o leaves the quantised units here - before the softmax below, whose half
       // tile is the chunk's first and may add its weights' second terms to o at once
-      if (g + 1 == 2 * n_pre && t0 < n_pre) leave_prefix();
+      // (a share that ends with the prefix leaves it behind the loop, like every share that ends inside it)
+      if (g + 1 == 2 * n_pre && t0 < n_pre && t1 > n_pre) leave_prefix();
       if (g + 2 < g_end) qk(g + 2, S[kb]);
       if (g + 1 < g_end) softmax(g + 1, !unmasked(g + 1), S[kb ^ 1], P);
     }

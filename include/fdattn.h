@@ -423,9 +423,13 @@ FDATTN_API int fdattn_sqattn_select_exact(
  *   out   bf16 [num_tokens, hq*head_dim]
  * max_chunk bounds n_b (it sizes the launch grid).
  * Accuracy of the MFMA kernels (head_dim 64, 128, 256): scores carry 22 significant bits of
- * q * k_scale and exact cache bytes; the softmax weights enter P.V in fp16, so an output element is
- * within 2^-11 * sum_j p_j |v_j| of the fp32 result (p: the weights, v: the dequantised values) -
- * at most 2^-11 * max|v|, i.e. below 2e-3 for dequantised magnitudes up to 4 and 4e-3 up to 8.
+ * q * k_scale and exact cache bytes.  The softmax weights enter P.V in fp16: as ONE term (11 bits) for
+ * tiles of 64 (32) keys whose dequantised values stay within +-6 - an output element is then within
+ * 2^-11 * sum_j p_j |v_j| of the fp32 result (p: the normalised weights, v: the dequantised values) - and
+ * as TWO terms (22 bits) for every tile that may hold a larger value: a cached tile by its scales (largest
+ * code x the KV head's largest per-channel V scale; the row's or tile's own scale in the formats with scale
+ * caches), a tile of the chunk's own V by its values.  Either way the result is within the path's tolerance
+ * (2e-3 absolute or 1e-2 relative) of the fp32 result at any magnitude.
  * Values beyond +-65504 in the chunk's own V saturate (fp16).
  */
 FDATTN_API int fdattn_append_attention_prefill(
