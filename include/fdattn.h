@@ -428,8 +428,9 @@ FDATTN_API int fdattn_sqattn_select_exact(
  * 2^-11 * sum_j p_j |v_j| of the fp32 result (p: the normalised weights, v: the dequantised values) - and
  * as TWO terms (22 bits) for every tile that may hold a larger value: a cached tile by its scales (largest
  * code x the KV head's largest per-channel V scale; the row's or tile's own scale in the formats with scale
- * caches), a tile of the chunk's own V by its values.  Either way the result is within the path's tolerance
- * (2e-3 absolute or 1e-2 relative) of the fp32 result at any magnitude.
+ * caches), a tile of the chunk's own V by its values.  So the one-term error is at most 2^-11 * 6 = 2.9e-3 in
+ * the worst case (weights and signs aligned against the rounding), below 2e-3 whenever the weighted mean
+ * magnitude of the values a query attends to is at most 4.1, and no magnitude beyond 6 meets one-term weights.
  * Values beyond +-65504 in the chunk's own V saturate (fp16).
  */
 FDATTN_API int fdattn_append_attention_prefill(
