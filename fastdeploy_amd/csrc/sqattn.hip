@@ -646,261 +646,6 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
   if (tid == 0) a.kept_counts[p] = k;
 }
 
-// The same selection for lists of up to 64 * VPL blocks (VPL = 8: 512 blocks, 32k tokens), with no histogram and no
-// atomic: a wavefront holds ALL scores of the pair in registers (VPL per lane, block j = VPL * lane + i).  The first
-// wavefront finds the thresholds -
-//   the k-th and (k+1)-th largest approximate score, T_k and T_k+1, by a bit-by-bit search over the order-preserving
-//   integer keys (32 steps of VPL ballots), and E = the largest error bound of the list -
-// while the others put what a re-scoring would read into LDS; after one barrier every wavefront classifies its own copy.
-// Block j is surely kept if s_j - e_j > T_k+1 + E (the (k+1)-th largest upper bound is at most T_k+1 + E, so at most k
-// blocks, itself included, can reach its lower bound) and surely dropped if s_j + e_j < T_k - E; the fp32 roundings of
-// these sums are covered by 2^-22 of the largest |score| added to E.  The undecided blocks are re-scored in fp64 with the
-// rows of a block dealt to four wavefronts (16 wavefronts: four undecided blocks at a time), the exact maxima meet in
-// LDS behind a second barrier, and the first wavefront ranks them and emits.
-template <int QUANT, bool DYN, int NSET, bool MT, int VPL>
-__global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_wave_kernel(SelArgs a) {
-  constexpr int GH = kG * NSET;       // (token, head) rows the re-scoring is laid out for
-  constexpr int kSplit = 4;           // wavefronts that share the rows of one undecided block
-  constexpr int GW = GH / kSplit;     // rows per wavefront
-  constexpr int kWavesR = kResolveThreads / 64;
-  constexpr int NB = 64 * VPL;
-  __shared__ double qd[GH][kD];       // q * k_scale (DYN: q), one fp32 rounding as the score's definition says, widened
-  __shared__ double part[NB][kSplit]; // exact maxima of the undecided blocks, per row share
-  __shared__ int tbl[NB], ulist[NB], ukeep[NB];
-  __shared__ float thr[2];
-  const int p = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wv = uni(tid >> 6);
-  const int b = p / a.hkv, h = p - b * a.hkv;
-  int qrow, toks;
-  if (!sel_rows(a, b, qrow, toks)) {  // not a decode row of this step: it keeps no block
-    if (tid == 0) a.kept_counts[p] = 0;
-    return;
-  }
-  const int vg = a.group * toks;
-  const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
-  const int nblk = min((max(kv_len, 0) + kBS - 1) / kBS, a.max_blocks);
-  const int k = min(a.top_k, nblk);
-  int32_t* out = a.kept_blocks + (size_t)p * a.top_k;
-  // ---- everything the kernel may need from memory, requested in one go
-  const float* sp = a.approx + (size_t)p * a.max_blocks;
-  const float* eb = a.ebound ? a.ebound + (size_t)p * a.max_blocks : nullptr;
-  const float eps = eb ? 0.f : a.eps[p];
-  float s[VPL], e[VPL];
-#pragma unroll
-  for (int i = 0; i < VPL; ++i) {
-    const int j = VPL * lane + i;
-    s[i] = j < nblk ? sp[j] : -INFINITY;
-    e[i] = j < nblk ? (eb ? eb[j] : eps) : 0.f;
-  }
-  int tb_reg[(NB + kResolveThreads - 1) / kResolveThreads];
-#pragma unroll
-  for (int r = 0; r < (NB + kResolveThreads - 1) / kResolveThreads; ++r) {
-    const int j = tid + r * kResolveThreads;
-    tb_reg[r] = j < nblk ? a.block_tables[(size_t)b * a.max_blocks + j] : -1;
-  }
-  float q_reg[(GH * kD + kResolveThreads - 1) / kResolveThreads];
-#pragma unroll
-  for (int r = 0; r < (GH * kD + kResolveThreads - 1) / kResolveThreads; ++r) {
-    const int i = tid + r * kResolveThreads, g = i / kD, c = i % kD;
-    const int tk = g / a.group, hd = g - tk * a.group;
-    float qv = 0.f;  // rows past the pair's are zero
-    if (i < GH * kD && g < vg) {
-      qv = bf16_to_f32(a.q[((size_t)(qrow + tk) * a.hkv * a.group + h * a.group + hd) * kD + c]);
-      if (!DYN) qv = __fmul_rn(qv, a.k_scale[h * kD + c]);
-    }
-    q_reg[r] = qv;
-  }
-
-  // what the re-scoring would read goes to LDS now, while the first wavefront searches (the others have nothing else to do)
-#pragma unroll
-  for (int r = 0; r < (NB + kResolveThreads - 1) / kResolveThreads; ++r)
-    if (tid + r * kResolveThreads < NB) tbl[tid + r * kResolveThreads] = tb_reg[r];
-#pragma unroll
-  for (int r = 0; r < (GH * kD + kResolveThreads - 1) / kResolveThreads; ++r) {
-    const int i = tid + r * kResolveThreads;
-    if (i < GH * kD) qd[i / kD][i % kD] = (double)q_reg[r];
-  }
-
-  // ---- thresholds: the first wavefront alone (sixteen wavefronts searching side by side would share four SIMDs' issue
-  // ports and take four times as long); classification: every wavefront on its own copy of the scores
-  u32 km = 0, um = 0;  // bit i: block VPL * lane + i is kept / undecided
-  int nu = 0, need = 0;
-  if (k >= nblk) {
-#pragma unroll
-    for (int i = 0; i < VPL; ++i) km |= (VPL * lane + i < nblk ? 1u : 0u) << i;
-    __syncthreads();
-  } else {
-   if (wv == 0) {
-    u32 key[VPL];
-    float emax = 0.f, smax = 0.f;
-#pragma unroll
-    for (int i = 0; i < VPL; ++i) {
-      const bool in = VPL * lane + i < nblk;
-      key[i] = in ? order_key(s[i]) : 0u;  // below every key of a float
-      emax = fmaxf(emax, in ? e[i] : 0.f);
-      smax = fmaxf(smax, in ? fabsf(s[i]) : 0.f);
-    }
-    emax = wave_max(emax);
-    smax = wave_max(smax);
-    u32 tk_key = 0;  // the largest c with #{key >= c} >= k: the k-th largest key
-#pragma unroll 1
-    for (int bit = 31; bit >= 0; --bit) {
-      const u32 c = tk_key | (1u << bit);
-      int cnt = 0;
-#pragma unroll
-      for (int i = 0; i < VPL; ++i) cnt += __popcll(__ballot(key[i] >= c));
-      if (cnt >= k) tk_key = c;
-    }
-    int at_least = 0;
-    u32 below = 0;
-#pragma unroll
-    for (int i = 0; i < VPL; ++i) {
-      at_least += __popcll(__ballot(key[i] >= tk_key));
-      below = max(below, key[i] < tk_key ? key[i] : 0u);
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) below = max(below, (u32)__shfl_xor((int)below, o, 64));
-    const float t_k = key_to_float(tk_key);
-    const float t_k1 = at_least > k ? t_k : key_to_float(below);  // (k < nblk: a (k+1)-th largest exists)
-    const float slack = emax + smax * 2.384185791015625e-7f;      // E + 2^-22 max |s| (inf or NaN scores: nothing is decided)
-    if (lane == 0) thr[0] = t_k1 + slack, thr[1] = t_k - slack;
-   }
-    __syncthreads();
-    const float hi = thr[0], lo = thr[1];
-    int n_in = 0;
-#pragma unroll
-    for (int i = 0; i < VPL; ++i) {
-      const bool in = VPL * lane + i < nblk;
-      const bool sure_in = in && (s[i] - e[i] > hi);
-      const bool sure_out = in && (s[i] + e[i] < lo);
-      km |= (sure_in ? 1u : 0u) << i;
-      um |= (in && !sure_in && !sure_out ? 1u : 0u) << i;
-      n_in += __popcll(__ballot(sure_in));
-      nu += __popcll(__ballot(in && !sure_in && !sure_out));
-    }
-    need = k - n_in;
-  }
-  // this lane's undecided blocks are entries px .. of the undecided list (ascending block index)
-  int px = __popc(um);
-  {
-    int incl = px;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-      const int t = __shfl_up(incl, o, 64);
-      if (lane >= o) incl += t;
-    }
-    px = incl - px;
-  }
-  if (nu > 0) {  // (the same in every wavefront)
-    // every wavefront writes the same list (the same values to the same places) and reads back what it wrote
-    {
-      int n = 0;
-#pragma unroll
-      for (int i = 0; i < VPL; ++i)
-        if (um >> i & 1u) ulist[px + n++] = VPL * lane + i;
-    }
-    const int share = wv % kSplit, r0 = share * GW;
-    for (int u = wv / kSplit; u < nu; u += kWavesR / kSplit) {
-      const int j = ulist[u];
-      const int pb = tbl[j];
-      double best = -INFINITY;
-      if (r0 < vg && pb >= 0 && pb < a.num_blocks && j * kBS + lane < kv_len) {
-        const uint8_t* kr = a.key_cache + (((size_t)pb * a.hkv + h) * kBS + lane) * kD;
-        uint4 row[kD / 16];  // the whole row is requested before any of it is used
-#pragma unroll
-        for (int i = 0; i < kD / 16; ++i) row[i] = *reinterpret_cast<const uint4*>(kr + 16 * i);
-        const int lim = kv_len - j * kBS - lane;  // a row that sees `few` fewer keys sees this one if few < lim
-        double acc[GW];
-#pragma unroll
-        for (int g = 0; g < GW; ++g) acc[g] = 0.0;
-        // fp64, channels in ascending order; the products are exact, so fma(q, k, acc) rounds like add(acc, mul(q, k))
-        auto piece = [&](int i, const u32 (&ws)[4]) {
-#pragma unroll
-          for (int el = 0; el < 16; ++el) {
-            const double kv = dq64<QUANT>((ws[el >> 2] >> (8 * (el & 3))) & 0xff);
-#pragma unroll
-            for (int g = 0; g < GW; ++g) acc[g] = __fma_rn(qd[r0 + g][16 * i + el], kv, acc[g]);
-          }
-        };
-        if constexpr (GW == 1) {
-#pragma unroll
-          for (int i = 0; i < kD / 16; ++i) {
-            const u32 ws[4] = {row[i].x, row[i].y, row[i].z, row[i].w};
-            piece(i, ws);
-          }
-        } else {
-          // (with more rows per wavefront the loop over the eight pieces stays rolled - unrolled it does not fit the 128
-          // registers of a 16-wavefront workgroup - and picks its piece by comparisons, every register index a constant)
-#pragma unroll 1
-          for (int i = 0; i < kD / 16; ++i) {
-            u32 ws[4] = {row[0].x, row[0].y, row[0].z, row[0].w};
-#pragma unroll
-            for (int jj = 1; jj < kD / 16; ++jj) {
-              const bool pick = i == jj;
-              ws[0] = pick ? row[jj].x : ws[0];
-              ws[1] = pick ? row[jj].y : ws[1];
-              ws[2] = pick ? row[jj].z : ws[2];
-              ws[3] = pick ? row[jj].w : ws[3];
-            }
-            piece(i, ws);
-          }
-        }
-        if (DYN) {
-          const double kt = (double)a.k_scale[((size_t)pb * a.hkv + h) * a.scale_rows + (a.scale_rows == 1 ? 0 : lane)];
-#pragma unroll
-          for (int g = 0; g < GW; ++g) acc[g] = __dmul_rn(acc[g], kt);
-        }
-#pragma unroll
-        for (int g = 0; g < GW; ++g) {
-          const int few = MT ? max(toks - 1 - (r0 + g) / a.group, 0) : 0;
-          if (r0 + g < vg && few < lim) best = fmax(best, acc[g]);
-        }
-      }
-#pragma unroll
-      for (int off = 32; off > 0; off >>= 1) best = fmax(best, __shfl_xor(best, off, 64));
-      if (lane == 0) part[u][share] = best;
-    }
-    __syncthreads();
-  }
-  if (wv != 0) return;
-  if (nu > 0) {
-    // the `need` best undecided blocks: exact score descending, block index ascending
-    for (int u0 = 0; u0 < nu; u0 += 64) {
-      const int u = u0 + lane;
-      double su = -INFINITY;
-      if (u < nu) su = fmax(fmax(part[u][0], part[u][1]), fmax(part[u][2], part[u][3]));
-      int rank = 0;
-      for (int i = 0; i < nu; ++i) {
-        const double si = fmax(fmax(part[i][0], part[i][1]), fmax(part[i][2], part[i][3]));
-        rank += (si > su) || (si == su && i < u);  // (the list is in ascending block order)
-      }
-      if (u < nu) ukeep[u] = rank < need;
-    }
-    int n = 0;
-#pragma unroll
-    for (int i = 0; i < VPL; ++i)
-      if (um >> i & 1u) km |= (ukeep[px + n++] ? 1u : 0u) << i;
-  }
-  // ordered compaction of the kept blocks
-  int pk = __popc(km);
-  {
-    int incl = pk;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-      const int t = __shfl_up(incl, o, 64);
-      if (lane >= o) incl += t;
-    }
-    pk = incl - pk;
-  }
-#pragma unroll
-  for (int i = 0; i < VPL; ++i)
-    if (km >> i & 1u) {
-      if (pk < a.top_k) out[pk] = VPL * lane + i;
-      ++pk;
-    }
-  for (int j = k + lane; j < a.top_k; j += 64) out[j] = -1;
-  if (lane == 0) a.kept_counts[p] = k;
-}
-
 static bool sel_fast_supported(int hq, int hkv, int d, int bs, int max_blocks) {
   return d == kD && hkv > 0 && hq % hkv == 0 && hq / hkv <= kG * kMaxSets && bs == kBS &&
          max_blocks <= 2048;  // 28 B of LDS per block in the resolve kernel
@@ -961,14 +706,8 @@ static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_ca
 #define FDATTN_SEL_LAUNCH_N(Q, D, N)                                                                                \
   do {                                                                                                              \
     hipLaunchKernelGGL((sqattn_scores_mfma_kernel<Q, D, N>), g1, b1, 0, s, sa);                                     \
-    if (max_tokens > 1) {                                                                                           \
-      if (max_blocks_per_seq <= 512) hipLaunchKernelGGL((sqattn_resolve_wave_kernel<Q, D, N, true, 8>), g2, b2, 0, s, sa); \
-      else hipLaunchKernelGGL((sqattn_resolve_kernel<Q, D, N, true>), g2, b2, shm2, s, sa);                         \
-    } else if constexpr (N <= kMaxSets) {                                                                           \
-      if (max_blocks_per_seq <= 512) hipLaunchKernelGGL((sqattn_resolve_wave_kernel<Q, D, N, false, 8>), g2, b2, 0, s, sa); \
-      else if (max_blocks_per_seq <= 1024) hipLaunchKernelGGL((sqattn_resolve_wave_kernel<Q, D, N, false, 16>), g2, b2, 0, s, sa); \
-      else hipLaunchKernelGGL((sqattn_resolve_kernel<Q, D, N>), g2, b2, shm2, s, sa);                               \
-    }                                                                                                               \
+    if (max_tokens > 1) hipLaunchKernelGGL((sqattn_resolve_kernel<Q, D, N, true>), g2, b2, shm2, s, sa);            \
+    else if constexpr (N <= kMaxSets) hipLaunchKernelGGL((sqattn_resolve_kernel<Q, D, N>), g2, b2, shm2, s, sa);    \
   } while (0)
 #define FDATTN_SEL_LAUNCH(Q, D)                                                                                     \
   do {                                                                                                              \
