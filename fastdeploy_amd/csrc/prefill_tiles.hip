@@ -188,8 +188,9 @@ __global__ __launch_bounds__(64 * waves_t<D>(), (D == 64 && !DYN) ? 4 : 1) void 
     for (int i = 0; i < NC; ++i) ent[i] = tid + NT * i < NCH ? entry_of(t * TK + (tid + NT * i) / CPR) : -1;
     if (DYN && tid < 2 * TK) ent_s = entry_of(t * TK + (tid & (TK - 1)));
   };
-  // cache row (block, slot) of key `key` of the sequence, given its table entry (an entry that names no block: row 0
-  // of block 0 is read instead and the row is zeroed or masked later)
+  // cache row (block, slot) of key `key` of the sequence, given its table entry.  An entry inside the cached prefix must
+  // name a block; one that does not (-1, or past the pool) is read as block 0 so that no access leaves the caches - its
+  // keys then take part with block 0's contents: the prefill kernels mask by position only.
   auto cache_row = [&](int key, int pb) {
     return ((size_t)(pb >= 0 && pb < a.num_blocks ? pb : 0) * a.hkv + h) * a.bs + slot_of(key);
   };

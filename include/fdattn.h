@@ -85,6 +85,13 @@ extern "C" {
  *   then the call's rows are quantised with the tile's scale like any other.
  * A tile therefore changes only through calls that store into it, and a block shared between sequences (which
  * is always a full one) is never requantised.
+ * A tile's scale only ever GROWS, and "earlier rows" are counted by position, not by what a scheduler keeps: after a
+ * speculative step whose drafts are rejected, the rows written over them find the scale where the rejected rows put it
+ * (and the accepted rows on that grid), so the cache is a function of the calls, not of the accepted tokens - it equals
+ * what the same calls produce anywhere, not what a replay of the accepted tokens alone would.  Likewise a tile whose
+ * first call brought only zeros stays at the placeholder scale 1.0 until a row with |x| > 127 (448) arrives; rows
+ * appended to it with |x| < 0.5 quantise to 0.  A caller that needs tiles independent of rejected drafts or of leading
+ * zeros rewrites the tile from its first row (one call that stores the tile's first row sets the scale afresh).
  */
 #define FDATTN_CACHE_INT8_BLOCK 5
 #define FDATTN_CACHE_FP8_E4M3_BLOCK 6
@@ -422,6 +429,9 @@ FDATTN_API int fdattn_sqattn_select_exact(
  *   v_new bf16 [num_tokens, hkv*head_dim]   V           (v_out of the cache writer)
  *   out   bf16 [num_tokens, hq*head_dim]
  * max_chunk bounds n_b (it sizes the launch grid).
+ * block_tables: every entry that covers one of the p_b cached tokens must name a block of the pool.  An entry that
+ * does not (-1, or >= num_blocks) is read as block 0, so that no access leaves the caches, and its keys take part
+ * with block 0's contents - the prefill kernels mask by position only (the decode kernels skip such blocks).
  * Accuracy of the MFMA kernels (head_dim 64, 128, 256): scores carry 22 significant bits of
  * q * k_scale and exact cache bytes.  The softmax weights enter P.V in fp16: as ONE term (11 bits) for
  * tiles of 64 (32) keys whose dequantised values stay within +-6 - an output element is then within

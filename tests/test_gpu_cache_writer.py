@@ -212,6 +212,54 @@ def test_writer_per_block_formats_call_after_call(oracle, quant, shape):
         lens = [a + b for a, b in zip(lens, new)]
 
 
+@pytest.mark.parametrize("quant", [CACHE_INT8_BLOCK, CACHE_FP8_BLOCK])
+def test_writer_per_block_formats_after_rejected_drafts(oracle, quant):
+    """A speculative step writes three tokens per sequence, two of them large, and only the first is accepted: the next
+    step writes over the rejected rows.  A tile's scale only ever grows - it stays where the rejected rows put it, and
+    the accepted row keeps the bytes of that grid - so the cache is a function of the CALLS, not of the accepted
+    tokens: the oracle, given the same calls, must agree bit for bit after every one of them, and no scale may shrink."""
+    d, hq, hkv, bs = 128, 8, 2, 64
+    g = torch.Generator().manual_seed(17 + quant)
+    nseq, blocks = 4, 3
+    pool = nseq * blocks
+    from fastdeploy_amd.rope import rope_table
+    cos, sin = rope_table(blocks * bs, d, 10000.0, "cpu")
+    kc = torch.zeros((pool, hkv, bs, d), dtype=torch.uint8)
+    vc = torch.zeros((pool, hkv, bs, d), dtype=torch.uint8)
+    ks, vs = torch.full((pool, hkv), float("nan")), torch.full((pool, hkv), float("nan"))
+    bt = torch.randperm(pool, generator=g).to(torch.int32).view(nseq, blocks)
+    host = [np_of(t).copy() for t in (kc, vc, ks, vs)]
+    dev = [t.cuda() for t in (kc, vc, ks, vs)]
+    lens = [bs - 2, 5, 0, bs + 1]          # drafts that cross a block boundary, sit inside a tile, open the first tile
+    # (tokens per sequence, magnitude of each token of a row, tokens that stay)
+    steps = [([5, 5, 5, 5], [1.0] * 5, 5),              # some history in every tile first (sequence 2: its first rows)
+             ([3, 3, 3, 3], [1.0, 20.0, 40.0], 1),       # drafts 2 and 3 are large and rejected
+             ([3, 3, 3, 3], [0.5, 0.5, 0.5], 3),         # written over them, small: the scale stays up
+             ([1, 1, 1, 1], [0.0], 1),                   # a row of zeros
+             ([2, 2, 2, 2], [60.0, 0.1], 0)]             # everything rejected
+    for new, mags, keep in steps:
+        T = sum(new)
+        rows = torch.cat([torch.tensor(mags[:n]) for n in new])
+        qkv = (torch.randn((T, (hq + 2 * hkv) * d), generator=g) * rows[:, None]).to(torch.bfloat16)
+        this = torch.tensor(new, dtype=torch.int32)
+        cu = torch.tensor([0] + list(np.cumsum(new)), dtype=torch.int32)
+        dec = torch.tensor(lens, dtype=torch.int32)
+        before = [np_of(dev[2]).copy(), np_of(dev[3]).copy()]
+        fd.write_cache_kv(qkv.cuda(), dev[0], dev[1], dev[2], dev[3], bt.cuda(), this.cuda(), dec.cuda(), this.cuda(), cu.cuda(),
+                          (cos.cuda(), sin.cuda()), num_heads=hq, kv_num_heads=hkv, rope_style="neox", cache_quant_type=quant)
+        torch.cuda.synchronize()
+        oracle.write_cache_kv(bits(qkv), host[0], host[1], host[2], host[3], np_of(cos), np_of(sin), np_of(bt), np_of(dec),
+                              np_of(cu), hq, hkv, d, 1, quant, False)
+        what = "after the step of %r tokens x %r of which %d stay" % (new, mags, keep)
+        for i, name in ((2, "K scales"), (3, "V scales")):
+            assert np.array_equal(np_of(dev[i]).view(np.uint32), host[i].view(np.uint32)), what + ": " + name
+            was, now = before[i - 2], np_of(dev[i])
+            assert np.all((now >= was) | np.isnan(was)), what + ": a scale shrank"
+        assert np.array_equal(np_of(dev[0]), host[0]), what + ": K bytes"
+        assert np.array_equal(np_of(dev[1]), host[1]), what + ": V bytes"
+        lens = [a + keep for a in lens]
+
+
 @pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8_DYNAMIC, CACHE_INT8_BLOCK])
 def test_writer_tokens_past_the_rope_table_are_skipped_with_zeroed_rows(quant):
     """A token whose position lies outside the rotation table cannot be written: the caches (and scale caches) keep
