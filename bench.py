@@ -365,7 +365,8 @@ def other_workloads(args):
                  4096 * (48 * 128 * 2 * 2 + 2 * 8 * 128 + 2 * 64 * 4 + (2 * 8 * 4 if wname.endswith("dynamic") else 0)),
                  HBM_PEAK_GBPS, "GB/s")
             del cw
-        # a decode step's write (256 sequences, one token each) in the per-block format: token kernel + tile kernel
+        # a decode step's write (256 sequences, one token each) in the per-block format: one launch (the token kernel keeps
+        # the tiles' scales itself when a step brings no more tokens than sequences)
         cw = syn.write_case(num_seqs=256, max_pos=8192, seed=1, device=dev, blocks_per_seq=128, quant="cache_int8_block")
         rotw = (cw["rope_cos"], cw["rope_sin"])
         wr_blk = lambda: fd.write_cache_kv(cw["qkv"], cw["key_cache"], cw["value_cache"], cw["cache_k_scale"], cw["cache_v_scale"],
@@ -374,7 +375,8 @@ def other_workloads(args):
                                            cache_quant_type="cache_int8_block")
         ms = time_events(wr_blk, args.steps, args.warmup)
         line("configs[2] cache write, cache_int8_block (256 tokens; prior rows are requantised where a scale grows)", ms,
-             "hbm", 256 * (48 * 128 * 2 + 32 * 128 * 2 + 2 * 8 * 128), HBM_PEAK_GBPS, "GB/s")
+             "hbm", 256 * (48 * 128 * 2 + 32 * 128 * 2 + 2 * 8 * 128), HBM_PEAK_GBPS, "GB/s",
+             {"us_from_a_hip_graph": round(time_graph(wr_blk, args.steps) * 1e3, 2)})
         del cw
         for name in ("cache_int8_dynamic", "cache_fp8_dynamic", "cache_int8_block"):
             c = syn.decode_case(batch=2, ctx=8192, seed=0, device=dev, direct_bytes=True, extra_blocks=8, quant=name)

@@ -177,12 +177,27 @@ __device__ __forceinline__ UnitValues unit_values(const WriterArgs& a, int tok, 
 }
 
 
+// The tile that token `tok` of sequence b starts in this call.
+struct TileJob {
+  int tok;         // the call's first token of the tile
+  int r0, r1;      // positions [r0, r1) are stored into the tile by this call
+  int lb, pb;      // logical and physical block
+  int prior_rows;  // rows of earlier calls in the tile
+};
+__device__ __forceinline__ bool tile_job(const WriterArgs& a, int b, int tok, TileJob& j);
+template <int QUANT>
+__device__ __forceinline__ void write_tile_rows(const WriterArgs& a, const TileJob& j, int h, bool is_k, int head, int u,
+                                                const UnitValues& first);
+
 // One thread per unit:
 //   heads [0, hq)            Q   : rotate, round to bf16, store to q_out
 //   heads [hq, hq+hkv)       K   : rotate, (bf16 -> k_out), quantise, store to key_cache
 //   heads [hq+hkv, hq+2hkv)  V   : (copy -> v_out), quantise, store to value_cache
 // MODE 0: per-channel scales.  MODE 1: one scale per stored row, (largest magnitude of the row) / 127 or / 448, stored
 // beside the row.  MODE 2: the cache is left to write_cache_tiles_kernel (one scale per tile needs all rows of the tile).
+// MODE 3: one scale per tile, kept by this kernel itself - the threads that hold a K or V head of a token that stands
+// for a tile do the tile's whole job (write_tile_rows): for steps of at most one token per sequence, where a job is one
+// row and a second launch would cost more than the write.
 template <int QUANT, int MODE>
 __global__ __launch_bounds__(256) void write_cache_kv_kernel(WriterArgs a) {
   constexpr bool DYN = MODE == 1;
@@ -255,6 +270,11 @@ __global__ __launch_bounds__(256) void write_cache_kv_kernel(WriterArgs a) {
   }
 
   if (MODE == 2) return;
+  if constexpr (MODE == 3) {
+    TileJob j;
+    if (tile_job(a, b, tok, j)) write_tile_rows<QUANT>(a, j, h, is_k, head, u, uv);  // (the same for every thread of the workgroup)
+    return;
+  }
   const int lb = pos / a.bs, slot = pos - lb * a.bs;
   if (lb >= a.max_blocks) return;
   const int pb = a.block_tables[(size_t)b * a.max_blocks + lb];
@@ -306,13 +326,6 @@ __device__ __forceinline__ u32 requant1(u32 byte, float s_old, float s) {
 // first one this call stores into a tile - the first new token of its sequence, or one whose position is a multiple of
 // the block size - stands for the tile.
 
-// The tile that token `tok` of sequence b starts in this call.
-struct TileJob {
-  int tok;         // the call's first token of the tile
-  int r0, r1;      // positions [r0, r1) are stored into the tile by this call
-  int lb, pb;      // logical and physical block
-  int prior_rows;  // rows of earlier calls in the tile
-};
 __device__ __forceinline__ bool tile_job(const WriterArgs& a, int b, int tok, TileJob& j) {
   const int tok_first = a.cu_seqlens_q[b];
   const int tok_end = min(a.cu_seqlens_q[b + 1], a.num_tokens);
@@ -440,6 +453,59 @@ __device__ __forceinline__ void write_tile(const WriterArgs& a, const TileJob& j
   }
 }
 
+// The same job for ONE of the two tensors by the head_dim / 16 threads of the token kernel that hold the K (or V) head
+// of the token that stands for the tile - adjacent lanes of one wavefront, unit u each; `first` = the values of the job's
+// first row, which these threads have computed already.  A job of one row (every job of a decode step) costs no
+// recomputation; longer ones walk their rows one at a time.
+template <int QUANT>
+__device__ __forceinline__ void write_tile_rows(const WriterArgs& a, const TileJob& j, int h, bool is_k, int head, int u,
+                                                const UnitValues& first) {
+  const int uph = a.d / 16;
+  const size_t at = (size_t)j.pb * a.hkv + h;
+  float* const scale = is_k ? a.k_scale : a.v_scale;
+  float s_old = 0.f;  // asked for now - before anything of this tile is stored - and needed after the rows' maximum
+  if (j.prior_rows > 0) s_old = scale[at];
+  float m = 0.f;  // fmaxf drops NaNs, as the oracle's does
+  for (int r = j.r0; r < j.r1; ++r) {
+    const UnitValues x = r == j.r0 ? first : unit_values(a, j.tok + (r - j.r0), head, u, r);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) m = fmaxf(m, fmaxf(fabsf(x.g1[i]), fabsf(x.g2[i])));
+  }
+  for (int o = 1; o < uph; o <<= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  const float qmax = QUANT == FDATTN_CACHE_INT8 ? 127.0f : 448.0f;
+  const float s_now = m > 0.f ? __fdiv_rn(m, qmax) : 0.f;
+  const float sc = j.prior_rows > 0 ? (s_now > s_old ? s_now : s_old) : (s_now > 0.f ? s_now : 1.0f);
+  if (u == 0) scale[at] = sc;
+  uint8_t* const tile = (is_k ? a.key_cache : a.value_cache) + at * a.bs * a.d;
+  if (j.prior_rows > 0 && sc > s_old) {  // the scale grew: the rows of earlier calls move to the new grid
+    const int pieces = j.prior_rows * a.d / 16;
+    for (int i = u; i < pieces; i += uph) {
+      const uint4 w = *reinterpret_cast<const uint4*>(tile + (size_t)i * 16);
+      u32 ws[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        u32 o = 0;
+#pragma unroll
+        for (int by = 0; by < 4; ++by) o |= requant1<QUANT>((ws[e] >> (8 * by)) & 0xffu, s_old, sc) << (8 * by);
+        ws[e] = o;
+      }
+      *reinterpret_cast<uint4*>(tile + (size_t)i * 16) = make_uint4(ws[0], ws[1], ws[2], ws[3]);
+    }
+  }
+  for (int r = j.r0; r < j.r1; ++r) {
+    const UnitValues x = r == j.r0 ? first : unit_values(a, j.tok + (r - j.r0), head, u, r);
+    u32 q1[2] = {0, 0}, q2[2] = {0, 0};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      q1[i >> 2] |= quant1<QUANT>(x.g1[i], sc) << (8 * (i & 3));
+      q2[i >> 2] |= quant1<QUANT>(x.g2[i], sc) << (8 * (i & 3));
+    }
+    const size_t roff = (size_t)(r - j.lb * a.bs) * a.d;
+    *reinterpret_cast<uint2*>(tile + roff + x.c1) = make_uint2(q1[0], q1[1]);
+    *reinterpret_cast<uint2*>(tile + roff + x.c2) = make_uint2(q2[0], q2[1]);
+  }
+}
+
 // Steps of few tokens per sequence (decode steps, speculative steps, mixed batches): grid (kv heads, tokens), one
 // wavefront per token; the wavefront of a token that stands for a tile writes it, every other one leaves at once.
 template <int QUANT>
@@ -544,7 +610,12 @@ extern "C" int fdattn_write_cache_kv_ex(
   for (int t0 = 0; t0 < num_tokens; t0 += 65535) {
     a.tok0 = t0;
     const dim3 grid((units + 255) / 256, num_tokens - t0 < 65535 ? num_tokens - t0 : 65535);
-    if (quant_blockwise(cache_quant_type)) {
+    if (quant_blockwise(cache_quant_type) && num_tokens <= batch) {
+      // no more tokens than sequences - a decode step: one launch, the token kernel keeps the tiles itself (a tile's job
+      // is one row there; should a sequence bring several after all, its threads walk them)
+      if (quant_bytes(cache_quant_type) == FDATTN_CACHE_INT8) hipLaunchKernelGGL((write_cache_kv_kernel<FDATTN_CACHE_INT8, 3>), grid, dim3(256), 0, s, a);
+      else hipLaunchKernelGGL((write_cache_kv_kernel<FDATTN_CACHE_FP8_E4M3, 3>), grid, dim3(256), 0, s, a);
+    } else if (quant_blockwise(cache_quant_type)) {
       // Q, k_out, v_out from the token kernel; the cache and its tile scales from the tile kernel (independent of it)
       hipLaunchKernelGGL((write_cache_kv_kernel<FDATTN_CACHE_INT8, 2>), grid, dim3(256), 0, s, a);
       const bool i8 = quant_bytes(cache_quant_type) == FDATTN_CACHE_INT8;

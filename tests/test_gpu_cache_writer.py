@@ -188,7 +188,9 @@ def test_writer_per_block_formats_call_after_call(oracle, quant, shape):
     lens = [0] * nseq
     calls = [([bs + 3, 1, 0, 2 * bs, 7], 1.0, False), ([1] * nseq, 1.0, False), ([1] * nseq, 6.0, True),
              ([1, 0, 1, 1, 0], 0.2, False), ([bs - 5, 2, 3, bs, 1], 2.5, True), ([1] * nseq, 30.0, False),
-             ([3, 3, 3, 3, 3], 0.01, False)]
+             ([3, 3, 3, 3, 3], 0.01, False),
+             # no more tokens than sequences, yet rows of several tokens: the one-launch path walks them
+             ([3, 0, 0, 2, 0], 50.0, False), ([0, 2, 1, 0, 1], 0.3, True)]
     for new, mag, epilogue in calls:
         T = sum(new)
         qkv = (torch.randn((T, (hq + 2 * hkv) * d), generator=g) * mag).to(torch.bfloat16)
