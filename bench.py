@@ -30,6 +30,10 @@ HBM_PEAK_GBPS = 8000.0
 # run's algorithmic bytes.
 TRAFFIC_PROFILE = "profiles/decode_c8_kernel_configs1_b64_ctx4k.md"
 TRAFFIC_PER_ALGORITHMIC_BYTE = 1.0089
+# The same profile's kernel trace holds this script's one-by-one launches too (each follows an idle queue): the median of
+# the profiler's own begin-to-end durations of those launches, as a fraction of the HBM peak over configs[1]'s bytes.
+ISOLATED_PROFILE = TRAFFIC_PROFILE + ": decode_c8_kernel launches that follow an idle queue, profiler's durations, median 83.07 us"
+ISOLATED_FRAC_PROFILED = 0.8046
 
 
 def time_events(fn, steps, warmup):
@@ -537,6 +541,18 @@ def main():
         e1.synchronize()
         singles.append(e0.elapsed_time(e1) * 1e3)
     singles.sort()
+    # what the same event pair reads around a one-workgroup fill kernel: the part of a single launch's reading that
+    # is the two event packets and the dispatch between them, not the kernel (a profiler's begin/end stamps of a
+    # launch that follows an idle queue are the kernel's own duration in isolation)
+    tiny, floor = torch.zeros(64, dtype=torch.float32, device=dev), []
+    for _ in range(min(args.steps, 100)):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        tiny.zero_()
+        e1.record()
+        e1.synchronize()
+        floor.append(e0.elapsed_time(e1) * 1e3)
+    floor.sort()
 
     # yardstick of the same run: a plain 1 GiB device copy (reads 1 GiB, writes 1 GiB) - what the
     # memory system of this box gives a trivial kernel, beside the nominal 8 TB/s
@@ -575,11 +591,17 @@ def main():
                                        "to this run's algorithmic bytes" % (TRAFFIC_PROFILE, TRAFFIC_PER_ALGORITHMIC_BYTE),
                      "device_copy_gbps_same_run": round(copy_gbps, 1),
                      "frac_of_device_copy": round(achieved / copy_gbps, 4),
-                     # the same bytes over the median of launches timed ONE BY ONE (a device sync after each): no next
-                     # launch fills the tail of this one, as a GEMM before and after it in a real layer would not
-                     "frac_isolated": round(alg_bytes / (singles[len(singles) // 2] * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)},
+                     # the same bytes over the median of launches timed ONE BY ONE (an event pair and a device sync
+                     # each): no next launch fills the tail of this one.  The reading holds the event pair's own cost
+                     # (event_pair_around_a_fill_kernel below); ISOLATED_PROFILE has the kernel's own duration in
+                     # such launches from the profiler's stamps.
+                     "frac_isolated": round(alg_bytes / (singles[len(singles) // 2] * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                     "frac_isolated_kernel_only": ISOLATED_FRAC_PROFILED,
+                     "frac_isolated_kernel_only_source": ISOLATED_PROFILE},
         "kernel_us_single_launches": {"min": round(singles[0], 2), "median": round(singles[len(singles) // 2], 2),
-                                      "max": round(singles[-1], 2), "n": len(singles)},
+                                      "max": round(singles[-1], 2), "n": len(singles),
+                                      "event_pair_around_a_fill_kernel": {"min": round(floor[0], 2),
+                                                                          "median": round(floor[len(floor) // 2], 2)}},
     }
 
     if not args.no_cpu:

@@ -57,6 +57,60 @@ __device__ __forceinline__ bool f16_range_beyond(const F16Range& r, float limit)
   return (int)(short)(r.mx & 0xffffu) > pos || (int)(short)(r.mx >> 16) > pos || (r.mn & 0xffffu) > neg || (r.mn >> 16) > neg;
 }
 
+// Running sum of the magnitudes of fp16 values, as a packed pair (start from 0; 8 values cost 8 instructions; the
+// caller keeps the pair's sums inside fp16) and the pair's total; further down, the sum of an integer over the
+// wavefront (valid in lane 63: rotations within the rows of 16 lanes, then the rows' last lanes handed on).
+__device__ __forceinline__ void f16x8_abs_sum(uint4 h, u32& acc) {
+  const u32 w[4] = {h.x, h.y, h.z, h.w};
+  v2h a = __builtin_bit_cast(v2h, acc);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const u32 m = w[e] & 0x7fff7fffu;
+    a += __builtin_bit_cast(v2h, m);
+  }
+  acc = __builtin_bit_cast(u32, a);
+}
+// The same over cache bytes as they are: int8 codes by two instructions per four bytes (the sum of |b| is the sum of
+// absolute differences of b ^ 0x80 from 0x80, byte by byte: v_sad_u8; exact, in an integer); e4m3 codes by way of their
+// fp16 values.  acc: the integer sum (int8) or the packed pair (fp8).
+template <int QUANT>
+__device__ __forceinline__ void code_abs_sum(u32 w0, u32 w1, uint4 as_f16, u32& acc) {
+  if (QUANT == FDATTN_CACHE_INT8) {
+    acc = __builtin_amdgcn_sad_u8(w0 ^ 0x80808080u, 0x80808080u, acc);
+    acc = __builtin_amdgcn_sad_u8(w1 ^ 0x80808080u, 0x80808080u, acc);
+  } else {
+    f16x8_abs_sum(as_f16, acc);
+  }
+}
+__device__ __forceinline__ float f16_pair_total(u32 acc) {
+  const v2h a = __builtin_bit_cast(v2h, acc);
+  return (float)a[0] + (float)a[1];
+}
+// A thread's K sum and V sum of a tile (32 codes each) as one word, (K sum / unit) | (V sum / unit) << 16 with
+// unit = 32 (int8) or 64 (e4m3), rounded: a field is at most 128 (224), the sum over four wavefronts at most 2^15
+// (57344) - inside its 16 bits.  One integer reduction then serves both.
+template <int QUANT>
+__device__ __forceinline__ u32 magnitude_word(u32 k_acc, u32 v_acc) {
+  if (QUANT == FDATTN_CACHE_INT8) return ((k_acc + 16u) >> 5) | (((v_acc + 16u) >> 5) << 16);
+  const u32 k = (u32)(f16_pair_total(k_acc) * (1.0f / 64.0f) + 0.5f), v = (u32)(f16_pair_total(v_acc) * (1.0f / 64.0f) + 0.5f);
+  return k | (v << 16);
+}
+template <int QUANT>
+constexpr float magnitude_unit() { return QUANT == FDATTN_CACHE_INT8 ? 32.0f : 64.0f; }
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ u32 dpp_or_zero(u32 v) {
+  return (u32)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, 0xf, false);
+}
+__device__ __forceinline__ u32 wave_sum_lane63(u32 v) {
+  v += dpp_or_zero<0x128, 0xf>(v);  // row_ror 8, 4, 2, 1: every lane holds its row's sum
+  v += dpp_or_zero<0x124, 0xf>(v);
+  v += dpp_or_zero<0x122, 0xf>(v);
+  v += dpp_or_zero<0x121, 0xf>(v);
+  v += dpp_or_zero<0x142, 0xa>(v);  // row_bcast 15 into rows 1 and 3: rows 0 + 1, rows 2 + 3
+  v += dpp_or_zero<0x143, 0xc>(v);  // row_bcast 31 into rows 2 and 3: row 3 holds everything
+  return v;
+}
+
 // 8 cache bytes -> 8 fp16 holding the bytes' exact values
 template <int QUANT>
 __device__ __forceinline__ uint4 cvt8(u32 w0, u32 w1) {

@@ -9,11 +9,14 @@
 //
 // Numbers.  Cache bytes are staged in LDS as fp16 holding the byte's exact value (int8: the
 // integer; e4m3: the code's value); the per-channel K scale is folded into Q, which enters the
-// prefix scores as TWO fp16 terms, Q c = hi + lo (c: a power of two per query that puts the
-// row's largest element at 2^13 .. 2^14), both accumulated by the MFMA into the same fp32
+// prefix scores as up to TWO fp16 terms, Q c = hi + lo (c: a power of two per query that puts
+// the row's largest element at 2^13 .. 2^14), both accumulated by the MFMA into the same fp32
 // accumulator - 22 significant bits of q * k_scale.  One fp16 term (11 bits) leaves a relative
 // error of 2^-12 per channel in every score, which is beyond the output tolerance for caches
-// whose dequantised magnitudes reach 5 .. 8.  The formats with one scale per stored row keep
+// whose dequantised magnitudes reach 5 .. 8 and far inside it for quantised unit-scale
+// activations: the steady state computes the hi term and adds the lo term for the tiles whose
+// measured magnitudes, with the wavefront's queries, call for it (kLoAbove); the first tiles of a
+// walk and the tiles around the end of the prefix always take both.  The formats with one scale per stored row keep
 // Q unscaled - bf16 is exact in fp16, one term - and apply the row's K scale to the score and
 // its V scale to the softmax weight, both in fp32.  The chunk's own K stays bf16 and meets the
 // bf16 Q (exact inputs).  Softmax weights are fp16, round to nearest, summed as rounded; V is
@@ -60,11 +63,26 @@ constexpr int kMaxSplitsV2 = 8;
 constexpr float kSumLimit = 16384.0f;  // a query's weight sum over 32 keys above which its exponent reference is raised (every weight stays inside fp16)
 constexpr size_t kLdsScales = (size_t)kSlots * BUF_ELEMS * 2, kLdsQlo = kLdsScales + (size_t)kSlots * 3 * BN * sizeof(float);
 constexpr size_t kLdsFlags = kLdsQlo + (size_t)kWavesPf * 8 * 64 * 16;  // four ints: which staged tiles hold large V values
-constexpr size_t kLdsBytes = kLdsFlags + 16;
+constexpr size_t kLdsStats = kLdsFlags + 16;  // [4 tiles][4 wavefronts] words: what each wavefront saw of a staged prefix tile's magnitudes
+constexpr size_t kLdsSink = kLdsStats + 4 * kWavesPf * sizeof(u32);  // a word per thread: where the stores of the lanes that hold no total go
+constexpr size_t kLdsBytes = kLdsSink + BM * sizeof(float);
 // Dequantised V magnitudes (the chunk's own V included) beyond which a tile's P.V product takes the softmax weights as
 // TWO fp16 terms: one term leaves an output element off by up to 2^-11 * sum_j p_j |v_j| <= 2^-11 * max|v|, which
 // passes 2e-3 only while the values a query attends to stay moderate.
 constexpr float kExactAbove = 6.0f;
+// The second fp16 term of q * k_scale (see the head of the file) is spent per prefix tile and wavefront, where it can
+// matter.  One term rounds every q_c k_scale_c by up to 2^-12 of itself, independently per channel: the score of a key
+// is then off by a random amount of standard deviation 2^-12 / sqrt(3) * (softmax_scale * sqrt(sum_c (q_c k_scale_c
+// K_c)^2)) = 1.4e-4 * s_rms, s_rms being the size the scores themselves have, and an output element by at most about
+// half of that times the spread v_rms of the values the query mixes (two keys of weight 1/2 each: the worst shape).
+// The tile is measured while it is staged - the mean magnitude of its K codes and of its V codes, which for values
+// spread like a Gaussian is 0.8 of their root mean square (flatter distributions give more: the safe side) - and a
+// wavefront takes the second term for a tile when  s_rms * v_rms > kLoAbove  with
+//   s_rms = softmax_scale * max over its queries |q * k_scale|_2 * 1.25 * mean |K code|,
+//   v_rms = max_c v_scale_c * 1.25 * mean |V code|:
+// one term then costs an output at most 7e-5 * kLoAbove = 2.1e-4 standard deviations, a tenth of the tolerance.
+// (Quantised N(0,1) activations: s_rms * v_rms is about 1.2; measured against the oracle, single terms first fail at 13.)
+constexpr float kLoAbove = 3.0f;
 
 // Register plan.  A wavefront owns the SIMD's whole register file.  The upper AGPRs hold what only MFMAs touch and are
 // addressed BY NAME in single-instruction asm statements; the compiler is left the 256 VGPRs and a[0:31] (it parks
@@ -299,12 +317,14 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
   __attribute__((address_space(3))) int* const tile_flag = (__attribute__((address_space(3))) int*)((__attribute__((address_space(3))) uint8_t*)lds + kLdsFlags);
   constexpr float kCodeMax = QUANT == FDATTN_CACHE_INT8 ? 127.0f : 448.0f;
   bool pre_exact = false;
+  float v_scale_max = 0.f;  // per-channel formats: the largest |v_scale| of this KV head
   if (!DYN) {
     const float2 vs2 = *reinterpret_cast<const float2*>(a.v_scale + h * HD + 2 * lane);
     float m = fmaxf(fabsf(vs2.x), fabsf(vs2.y));
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
     pre_exact = !(m * kCodeMax <= kExactAbove);  // (NaN scales: the exact path)
+    v_scale_max = __any(vs2.x != vs2.x || vs2.y != vs2.y) ? NAN : m;
   }
   auto flag_tile = [&](int t, bool large) {
     if (__any(large) && lane == 0) tile_flag[t & 3] = t + 1;
@@ -314,6 +334,21 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
     if (t < n_pre && !DYN) return pre_exact;
     return __builtin_amdgcn_readfirstlane(tile_flag[t & 3]) == t + 1;
   };
+
+  // ---- which prefix tiles take the second term of q * k_scale (see kLoAbove; per-channel formats): every wavefront leaves
+  // what it staged of a tile - the sum of the K codes' magnitudes and of the V codes', as one word (magnitude_word) - in
+  // its own word of tile_stat[tile % 4]; a reader adds the four.  lo_gain: everything else of the test, per wavefront
+  // (set by q_prefix).
+  __attribute__((address_space(3))) u32* const tile_stat = (__attribute__((address_space(3))) u32*)((__attribute__((address_space(3))) uint8_t*)lds + kLdsStats);
+  const int wv_u = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // (every lane stores - lane 63 the total, the others their partial sums into a word of their own that nobody reads:
+  // a branch around the store would cut the steady state's one basic block in two)
+  const int stat_sink = (int)((kLdsSink - kLdsStats) / sizeof(u32)) + tid;
+  auto stat_put = [&](int t, u32 k_acc, u32 v_acc) {
+    const u32 total = wave_sum_lane63(magnitude_word<QUANT>(k_acc, v_acc));
+    tile_stat[lane == 63 ? (t & 3) * kWavesPf + wv_u : stat_sink] = total;
+  };
+  float lo_gain = INFINITY;  // times (sum |K code|) (sum |V code|) of a tile > 1: the tile takes the second term
 
   // half-tile steps of this wavefront: [g_begin, g_end); chunk halves wholly above its diagonal are not computed
   const int g_begin = 2 * t0;
@@ -335,7 +370,7 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
     static_for<2>([&](auto QB) {
       constexpr int qb = decltype(QB)::value;
       float x[8][8];
-      float amax = 0.f;
+      float amax = 0.f, q2 = 0.f;
 #pragma unroll
       for (int s = 0; s < 8; ++s) {
         const int c0 = 16 * s + 8 * hf;
@@ -348,10 +383,19 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
         x[s][4] = bf16lo_to_f32(w.z) * s1.x, x[s][5] = bf16hi_to_f32(w.z) * s1.y;
         x[s][6] = bf16lo_to_f32(w.w) * s1.z, x[s][7] = bf16hi_to_f32(w.w) * s1.w;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(x[s][e]));
+        for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(x[s][e])), q2 = __builtin_fmaf(x[s][e], x[s][e], q2);
       }
       float c = 1.0f, cinv = 1.0f;
       if (!DYN) {
+        // the largest |q * k_scale|_2 among the wavefront's queries (a NaN or an infinity: the second term everywhere)
+        q2 += swap32(q2);
+        float qn = q2;
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) qn = fmaxf(qn, __shfl_xor(qn, o, 64));
+        const float per_tile = 1.25f * magnitude_unit<QUANT>() / (float)(BN * HD);
+        const float gain = a.sm_scale * __builtin_sqrtf(qn) * v_scale_max * per_tile * per_tile * (1.0f / kLoAbove);
+        lo_gain = (qb == 0 || !(gain <= lo_gain)) && lo_gain == lo_gain ? gain : lo_gain;  // the larger one; a NaN stays
+
         // c = 2^(13 - floor(log2 amax)): the row's largest element lands in [2^13, 2^14)
         amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
         int e = (int)((__float_as_uint(amax) >> 23) & 0xffu) - 127;
@@ -459,13 +503,21 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
       }
       lds_u16* const pkd = (lds_u16*)lds + (size_t)slot * BUF_ELEMS + prow * LDK + pcc;
       lds_u16* const pvd = (lds_u16*)lds + (size_t)slot * BUF_ELEMS + K_ELEMS + prow * LDV + pcc;
+      u32 k_abs = 0u, v_abs = 0u;
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
-        lds_store16(pkd + i * 32 * LDK, cvt8<QUANT>(stg_k[i].x, stg_k[i].y));
-        lds_store16(pkd + i * 32 * LDK + 8, cvt8<QUANT>(stg_k[i].z, stg_k[i].w));
-        lds_store16(pvd + i * 32 * LDV, cvt8<QUANT>(stg_v[i].x, stg_v[i].y));
-        lds_store16(pvd + i * 32 * LDV + 8, cvt8<QUANT>(stg_v[i].z, stg_v[i].w));
+        const uint4 k0 = cvt8<QUANT>(stg_k[i].x, stg_k[i].y), k1 = cvt8<QUANT>(stg_k[i].z, stg_k[i].w);
+        const uint4 v0 = cvt8<QUANT>(stg_v[i].x, stg_v[i].y), v1 = cvt8<QUANT>(stg_v[i].z, stg_v[i].w);
+        lds_store16(pkd + i * 32 * LDK, k0);
+        lds_store16(pkd + i * 32 * LDK + 8, k1);
+        lds_store16(pvd + i * 32 * LDV, v0);
+        lds_store16(pvd + i * 32 * LDV + 8, v1);
+        if (!DYN) {
+          code_abs_sum<QUANT>(stg_k[i].x, stg_k[i].y, k0, k_abs), code_abs_sum<QUANT>(stg_k[i].z, stg_k[i].w, k1, k_abs);
+          code_abs_sum<QUANT>(stg_v[i].x, stg_v[i].y, v0, v_abs), code_abs_sum<QUANT>(stg_v[i].z, stg_v[i].w, v1, v_abs);
+        }
       }
+      if (!DYN) stat_put(t, k_abs, v_abs);
       if (DYN && tid < 2 * BN) {  // what the softmax needs of a row's scales, worked out once per tile
         if (tid < BN) {
           lds_sc[slot * 3 * BN + tid] = sc * stg_s;
@@ -546,6 +598,19 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
         }
       });
     }
+  };
+
+  // the second term of q * k_scale into the scores of prefix half tile g, behind their first term (per-channel formats;
+  // the steady state's steps make the first term only and call this for the tiles that need it: see kLoAbove)
+  auto qk_second_term = [&](int g, v16f (&s)[2]) {
+    const int t = g >> 1, kb = g & 1, slot = t % kSlots;
+    static_for<8>([&](auto ST) {
+      constexpr int st = decltype(ST)::value;
+      const v8h ka = k_operand(slot, kb, st);
+      const u4v ql = qlo1[64 * st];
+      mfma_s<true, kAccQlo + 4 * st>(s[0], ka);
+      mfma_s_vq(s[1], ka, ql);
+    });
   };
 
   // ---- O^T += V^T P^T of half tile g
@@ -750,6 +815,7 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
   const uint8_t* st_vbp = nullptr;
   int st_row3 = 0;  // chunk steps: this thread's first row of tile t + 3 in the chunk
   F16Range st_vr = {0u, 0u};  // chunk steps: the range of the V values this thread has staged of tile t + 2
+  u32 st_abs = 0u, st_abs_k = 0u;  // prefix steps (per-channel formats): the magnitudes of what it has staged of tile t + 2's K, then V
   auto fast_step = [&](int t, auto KB, auto CHK) {
     constexpr int kb = decltype(KB)::value;
     constexpr bool CH = decltype(CHK)::value;  // the tiles are the chunk's own keys: bf16 K against the bf16 q, one term, no scales; the softmax is masked where the wavefront's diagonal crosses the half tile
@@ -804,15 +870,30 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
           stg_v[i] = *reinterpret_cast<const uint4*>(v_new_seq + off);
         }
       } else if constexpr (c < 4) {
-        lds_store16(kd + pass * 32 * LDK + 8 * half, half ? cvt8<QUANT>(stg_k[pass].z, stg_k[pass].w) : cvt8<QUANT>(stg_k[pass].x, stg_k[pass].y));
+        const uint4 kh = half ? cvt8<QUANT>(stg_k[pass].z, stg_k[pass].w) : cvt8<QUANT>(stg_k[pass].x, stg_k[pass].y);
+        lds_store16(kd + pass * 32 * LDK + 8 * half, kh);
+        if constexpr (!DYN) {  // what this thread stages of tile t + 2's K, for the test of kLoAbove
+          if constexpr (c == 0) st_abs = 0u;
+          code_abs_sum<QUANT>(half ? stg_k[pass].z : stg_k[pass].x, half ? stg_k[pass].w : stg_k[pass].y, kh, st_abs);
+        }
         if constexpr (half == 1) stg_k[pass] = *reinterpret_cast<const uint4*>(st_kbp + (goff + (u32)(pass * 32 * HD)));
       } else {
-        lds_store16(vd + pass * 32 * LDV + 8 * half, half ? cvt8<QUANT>(stg_v[pass].z, stg_v[pass].w) : cvt8<QUANT>(stg_v[pass].x, stg_v[pass].y));
+        const uint4 vh = half ? cvt8<QUANT>(stg_v[pass].z, stg_v[pass].w) : cvt8<QUANT>(stg_v[pass].x, stg_v[pass].y);
+        lds_store16(vd + pass * 32 * LDV + 8 * half, vh);
+        if constexpr (!DYN) {
+          if constexpr (c == 4) st_abs_k = st_abs, st_abs = 0u;
+          code_abs_sum<QUANT>(half ? stg_v[pass].z : stg_v[pass].x, half ? stg_v[pass].w : stg_v[pass].y, vh, st_abs);
+        }
         if constexpr (half == 1) stg_v[pass] = *reinterpret_cast<const uint4*>(st_vbp + (goff + (u32)(pass * 32 * HD)));
+        if constexpr (!DYN && c == 7) stat_put(t + 2, st_abs_k, st_abs);
       }
     };
     // does half tile g + 1 (whose weights this step makes) belong to a tile with large V values?  Asked now, used at the end
     const int flag_sm = (CH || DYN) ? tile_flag[((g + 1) >> 1) & 3] : 0;
+    // and does half tile g + 2 (whose scores this step makes: tile t + 1) take the second term of q * k_scale?
+    u4v stat_w = {0u, 0u, 0u, 0u};
+    bool take_lo = false;
+    if constexpr (!CH && !DYN) stat_w = *(const __attribute__((address_space(3))) u4v*)(tile_stat + ((t + 1) & 3) * kWavesPf);
     mfma_settle(s_sm);
     if constexpr (CH) {
       if (!unmasked(g + 1)) sm_mask(g + 1, s_sm);  // the wavefront's diagonal
@@ -824,7 +905,7 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
     sm_begin(0, acc[0], cst[0]);
     sm_begin(1, acc[1], cst[1]);
     // ---- O += V P (g): 8 groups of two MFMAs.  The first two V operands were requested at the end of the previous
-    // fast step (va_carry); the first K operands and lo terms of the second product are requested under the last
+    // fast step (va_carry); the first K operands of the second product are requested under the last
     // groups.  Groups 4 .. 7 read P[.][1] only, so the first half of softmax(g + 1), which writes P[.][0], runs there.
     constexpr int VD = 4;  // V operands in flight ahead of the MFMA that uses them (the groups of this product are short: two MFMAs)
     v8h va[VD + 1], ka[3];
@@ -841,7 +922,8 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
       // issuing for half of its 32 cycles and leaves the other half to whatever follows it in program order.  So the
       // softmax of half tile g + 1 is cut into 16 pairs of scores x two halves and dealt out one half per MFMA: the
       // pairs of P[.][0] from group 4 of O += V P on (its MFMAs no longer read that operand), those of P[.][1] under
-      // S = K Q, three halves per k-step of four MFMAs; the staging chunks go where no softmax half is (groups 1 and 3
+      // S = K Q, three halves per k-step of two MFMAs (the hi terms of q * k_scale; a tile that needs the lo terms
+      // gets them behind the step: qk_second_term); the staging chunks go where no softmax half is (groups 1 and 3
       // of the first product, k-steps 3 and 7 of the second).  (The formats with
       // scale caches keep the coarser schedule below: their softmax reads three scales per score from LDS, which
       // comes cheaper four scores at a time.)
@@ -851,7 +933,6 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
         if constexpr (i + VD < 8) va[(i + VD) % (VD + 1)] = v_operand(slot_pv, kb, (i + VD) >> 2, (i + VD) & 3);
         if constexpr (i >= 6) {
           ka[i - 6] = k_operand(slot_qk, kb, i - 6);
-          if constexpr (!CH) ql[i - 6] = qlo1[64 * (i - 6)];
         }
         mfma_o<kAccO + 16 * (i & 3)>(va[i % (VD + 1)], P[0][i >> 2]);
         if constexpr (i >= 4) sm_pair_a(std::integral_constant<int, i - 4>{}, s_sm[0], scl[0], cst[0], c1);  // block 0, pairs 0 .. 3
@@ -862,6 +943,11 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
         if constexpr (i == 3) stage_chunk(std::integral_constant<int, 4 * kb + 1>{});
         __builtin_amdgcn_sched_barrier(0);
       });
+      if constexpr (!CH && !DYN) {  // (worked out here, long before the branch at the step's end asks for it)
+        const u32 both = (stat_w[0] + stat_w[1]) + (stat_w[2] + stat_w[3]);
+        const float risk = (float)(both & 0xffffu) * (float)(both >> 16) * lo_gain;
+        take_lo = !(__uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(risk))) <= 1.0f);
+      }
       static_for<8>([&](auto ST) {
         constexpr int st = decltype(ST)::value;
         // first pair of the k-step: block 1's pairs 0 .. 3, then block 0's pairs 4 .. 7; second pair (over two k-steps):
@@ -871,7 +957,6 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
         if (st == 0) mfma_s_first<!CH, kAccQhi>(s_new[0], kc); else mfma_s<!CH, kAccQhi + 4 * st>(s_new[0], kc);
         if constexpr (st + 2 < 8) {
           ka[(st + 2) % 3] = k_operand(slot_qk, kb, st + 2);
-          if constexpr (!CH) ql[(st + 2) % 3] = qlo1[64 * (st + 2)];
         } else {  // the next half step's first V operands: half tile g + 1
           va_carry[st - 6] = v_operand(kb == 0 ? slot_pv : slot_qk, kb ^ 1, 0, st - 6);
         }
@@ -880,11 +965,9 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
         if (st == 0) mfma_s_first<!CH, kAccQhi + 32>(s_new[1], kc); else mfma_s<!CH, kAccQhi + 32 + 4 * st>(s_new[1], kc);
         sm_pair_b(std::integral_constant<int, j1>{}, acc[qb1], c1, P[qb1]);
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (!CH && !DYN) mfma_s<true, kAccQlo + 4 * st>(s_new[0], kc);  // chunk keys: one exact bf16 term, two MFMAs per k-step
         if constexpr ((st & 1) == 0) sm_pair_a(std::integral_constant<int, j2>{}, s_sm[1], scl[1], cst[1], c2);
         else sm_pair_b(std::integral_constant<int, j2>{}, acc[1], c2, P[1]);
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (!CH && !DYN) mfma_s_vq(s_new[1], kc, ql[st % 3]);
         if constexpr (st == 3) stage_chunk(std::integral_constant<int, 4 * kb + 2>{});
         if constexpr (st == 7) stage_chunk(std::integral_constant<int, 4 * kb + 3>{});
         __builtin_amdgcn_sched_barrier(0);
@@ -941,6 +1024,9 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
     sm_finish(!CH, 0, s_sm[0], scl[0], scales, acc[0], P[0]);
     sm_finish(!CH, 1, s_sm[1], scl[1], scales, acc[1], P[1]);
     if ((CH || DYN) ? __builtin_amdgcn_readfirstlane(flag_sm) == ((g + 1) >> 1) + 1 : pre_exact) sm_second_term(g + 1, s_sm, P);
+    if constexpr (!CH && !DYN) {
+      if (take_lo) qk_second_term(g + 2, s_new);
+    }
   };
 
   // (the flags start empty: whatever an earlier workgroup left in these words must not name one of this walk's tiles)

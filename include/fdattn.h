@@ -432,8 +432,17 @@ FDATTN_API int fdattn_sqattn_select_exact(
  * block_tables: every entry that covers one of the p_b cached tokens must name a block of the pool.  An entry that
  * does not (-1, or >= num_blocks) is read as block 0, so that no access leaves the caches, and its keys take part
  * with block 0's contents - the prefill kernels mask by position only (the decode kernels skip such blocks).
- * Accuracy of the MFMA kernels (head_dim 64, 128, 256): scores carry 22 significant bits of
- * q * k_scale and exact cache bytes.  The softmax weights enter P.V in fp16: as ONE term (11 bits) for
+ * Accuracy of the MFMA kernels (head_dim 64, 128, 256): scores are made of exact cache bytes and 22 significant
+ * bits of q * k_scale (two fp16 terms).  The kernel for head_dim 128 / block_size 64 with per-channel scales spends the
+ * second term per tile of 64 cached keys and per group of 64 queries, where it can matter: one term puts a random
+ * error of standard deviation 2^-12 / sqrt(3) = 1.4e-4 times s_rms into a score (s_rms: the size the scores of the
+ * tile have, softmax_scale * |q * k_scale|_2 * the root mean square of the K codes) and at most about half of that
+ * times v_rms into an output (v_rms: that of the dequantised V values).  Both are measured as the tile is read - the
+ * mean magnitudes of its K and V codes, taken as 0.8 of their root mean square, which flatter-than-Gaussian
+ * distributions exceed (the safe side) - and the second term is taken whenever s_rms * v_rms > 3, i.e. wherever one
+ * term could cost more than 2e-4: a tenth of the tolerance.  (Quantised unit-scale activations sit near 1.2; against
+ * the CPU oracle, outputs computed with one term everywhere first leave the tolerance near 13.)
+ * The softmax weights enter P.V in fp16: as ONE term (11 bits) for
  * tiles of 64 (32) keys whose dequantised values stay within +-6 - an output element is then within
  * 2^-11 * sum_j p_j |v_j| of the fp32 result (p: the normalised weights, v: the dequantised values) - and
  * as TWO terms (22 bits) for every tile that may hold a larger value: a cached tile by its scales (largest

@@ -445,6 +445,29 @@ def test_decode_launch_shapes(oracle, quant):
         check(bits(out), oracle_decode(oracle, syn.to_device(case, "cpu")), "batch %d" % batch)
 
 
+@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8])
+@pytest.mark.parametrize("batch,hq,hkv", [(64, 32, 8), (37, 32, 16), (33, 16, 16), (64, 24, 8)])
+def test_decode_batches_of_single_chunk_lists(oracle, batch, hq, hkv, quant):
+    """Batches of at least 512 (sequence, KV head) pairs: every list is one chunk, finished by its workgroup without
+    partials.  Ragged lengths with empty sequences, equal lengths, an odd batch, lists of 1 .. 128 units (both
+    unit-table entries of a lane), 1, 2, 3 and 4 query heads per KV head."""
+    from fastdeploy_amd import _lib
+    rng = np.random.default_rng(batch * 7 + hq)
+    shapes = [("ragged", [int(x) for x in rng.integers(0, 1500, batch)], None),
+              ("equal", [777] * batch, None),
+              ("long and short", [64 * 128 - 3 if i % 5 == 0 else int(rng.integers(1, 200)) for i in range(batch)], 128)]
+    for what, lens, mb in shapes:
+        lens[3] = 0
+        mb = mb or max(lens) // 64 + 2
+        assert _lib.lib().fdattn_decode_chunks_per_sequence(batch, hkv, mb) == 1
+        case = syn.decode_case(batch=batch, ctx=lens, quant=quant, seed=batch + len(what), hq=hq, hkv=hkv, max_blocks=mb,
+                               extra_blocks=3)
+        want = oracle_decode(oracle, case)
+        got = gpu_decode(case)
+        check(got, want, "single chunks, %s" % what)
+        assert not got.reshape(batch, -1)[3].any()
+
+
 def test_decode_one_very_long_sequence(oracle):
     """One sequence of 524,288 tokens (8,192 blocks, 1 GiB of K and V): 64 chunks of 128 units per KV head and the
     merge kernel over all of them."""

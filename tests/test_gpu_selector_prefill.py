@@ -270,6 +270,41 @@ def test_prefill_constant_value_bytes(oracle, fill):
     _run_prefill_vs_oracle(oracle, c, CACHE_INT8, 300)
 
 
+def _moment_case(seed, prefix, chunk, kind, sk, sv, sq):
+    """One sequence whose cached K and V are drawn with a given shape and size - Gaussian, uniform or +-1 ("binary":
+    every code at full scale) times sk / sv - and quantised to int8 with max-abs / 127 per-channel scales; q ~ N(0, sq)."""
+    c = syn.decode_case(batch=1, ctx=prefix, quant=CACHE_INT8, seed=seed, extra_blocks=2, direct_bytes=True)
+    g = torch.Generator().manual_seed(seed)
+    shp = c["key_cache"].shape
+    draw = {"gauss": lambda: torch.randn(shp, generator=g),
+            "uniform": lambda: torch.rand(shp, generator=g) * 2 - 1,
+            "binary": lambda: torch.randint(0, 2, shp, generator=g).float() * 2 - 1}[kind]
+    k, v = draw() * sk, draw() * sv
+    ks, vs = k.abs().amax(dim=(0, 2)) / 127.0, v.abs().amax(dim=(0, 2)) / 127.0
+    c["key_cache"] = torch.clamp(torch.round(k / ks[None, :, None, :]), -127, 127).to(torch.int8).view(torch.uint8)
+    c["value_cache"] = torch.clamp(torch.round(v / vs[None, :, None, :]), -127, 127).to(torch.int8).view(torch.uint8)
+    c["cache_k_scale"], c["cache_v_scale"] = ks.contiguous().float(), vs.contiguous().float()
+    c["q_new"] = (torch.randn((chunk, 32 * 128), generator=g) * sq).to(torch.bfloat16)
+    c["k_new"] = (torch.randn((chunk, 8 * 128), generator=g) * sk).to(torch.bfloat16)
+    c["v_new"] = (torch.randn((chunk, 8 * 128), generator=g) * sv).to(torch.bfloat16)
+    c["cu_seqlens_q"] = torch.tensor([0, chunk], dtype=torch.int32)
+    return c
+
+
+@pytest.mark.parametrize("kind,sk,sv,sq", [("gauss", 1, 1, 1), ("gauss", 2, 2, 1), ("gauss", 4, 4, 1), ("gauss", 8, 8, 0.25),
+                                           ("uniform", 5, 8, 0.3), ("uniform", 5, 8, 1), ("binary", 2, 4, 0.5),
+                                           ("binary", 4, 8, 0.5)])
+def test_prefill_second_term_of_q_follows_the_tiles(oracle, kind, sk, sv, sq):
+    """The kernel for head_dim 128 / block_size 64 takes q * k_scale as one fp16 term for the tiles of the steady state
+    whose measured magnitudes (with the queries' norm) keep the rounding's effect below a tenth of the tolerance, and
+    as two terms elsewhere.  Long prefixes (the steady state) on both sides of that test - score sizes x value sizes
+    from 1 (quantised unit-scale activations: one term) to 70, distributions with every ratio of mean magnitude to
+    root mean square; computed with one term everywhere, the cases (gauss 4 4 1), (gauss 8 8 .25), (uniform 5 8 1)
+    and (binary 4 8 .5) leave the tolerance.  Every case against the oracle."""
+    c = _moment_case(3, 4096, 256, kind, sk, sv, sq)
+    _run_prefill_vs_oracle(oracle, c, CACHE_INT8, 256)
+
+
 def _config5_rows():
     """Rows of configs[4] checked against the oracle: in both sequences the first and last query of every 64-query
     wavefront (= every edge of a 64-key tile of the chunk), their neighbours, and every 7th row: 782 of 4096."""
