@@ -36,6 +36,7 @@ struct WriterArgs {
   const float* k_norm_weight;   // [d]: the same for K
   float rms_norm_eps;
   int tok0;  // first token of this launch (the grid's y dimension holds 65,535)
+  int tiles_write_rows;  // per-block formats, long chunks: k_out / v_out are the tile kernel's (the token kernel writes q_out only)
 };
 
 template <int QUANT>
@@ -184,7 +185,7 @@ struct TileJob {
   int lb, pb;      // logical and physical block
   int prior_rows;  // rows of earlier calls in the tile
 };
-__device__ __forceinline__ bool tile_job(const WriterArgs& a, int b, int tok, TileJob& j);
+__device__ __forceinline__ bool tile_job(const WriterArgs& a, const SeqRows& sr, int tok, TileJob& j);
 template <int QUANT>
 __device__ __forceinline__ void write_tile_rows(const WriterArgs& a, const TileJob& j, int h, bool is_k, int head, int u,
                                                 const UnitValues& first);
@@ -193,26 +194,45 @@ __device__ __forceinline__ void write_tile_rows(const WriterArgs& a, const TileJ
 //   heads [0, hq)            Q   : rotate, round to bf16, store to q_out
 //   heads [hq, hq+hkv)       K   : rotate, (bf16 -> k_out), quantise, store to key_cache
 //   heads [hq+hkv, hq+2hkv)  V   : (copy -> v_out), quantise, store to value_cache
+// A K or V row's unit into k_out / v_out (o: the row): V that the epilogue left unchanged goes as it was loaded.
+__device__ __forceinline__ void store_side_unit(uint16_t* o, const UnitValues& uv, bool is_v) {
+  if (is_v && !uv.changed) {
+    *reinterpret_cast<uint4*>(o + uv.c1) = uv.w1;
+    *reinterpret_cast<uint4*>(o + uv.c2) = uv.w2;
+    return;
+  }
+  u32 p1[4], p2[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    p1[i] = pack2_bf16(uv.g1[2 * i], uv.g1[2 * i + 1]);
+    p2[i] = pack2_bf16(uv.g2[2 * i], uv.g2[2 * i + 1]);
+  }
+  *reinterpret_cast<uint4*>(o + uv.c1) = make_uint4(p1[0], p1[1], p1[2], p1[3]);
+  *reinterpret_cast<uint4*>(o + uv.c2) = make_uint4(p2[0], p2[1], p2[2], p2[3]);
+}
+
 // MODE 0: per-channel scales.  MODE 1: one scale per stored row, (largest magnitude of the row) / 127 or / 448, stored
 // beside the row.  MODE 2: the cache is left to write_cache_tiles_kernel (one scale per tile needs all rows of the tile).
 // MODE 3: one scale per tile, kept by this kernel itself - the threads that hold a K or V head of a token that stands
 // for a tile do the tile's whole job (write_tile_rows): for steps of at most one token per sequence, where a job is one
-// row and a second launch would cost more than the write.
+// row and a second launch would cost more than the write.  MODE 4: q_out only - the cache, k_out and v_out are the tile
+// kernel's (long chunks: it computes every K and V row anyway); the K and V rows of skipped tokens are zeroed here.
 template <int QUANT, int MODE>
-__global__ __launch_bounds__(256) void write_cache_kv_kernel(WriterArgs a) {
+__device__ __forceinline__ void write_token_units(const WriterArgs& a, int unit_block, int tok_in_launch) {
   constexpr bool DYN = MODE == 1;
-  // grid (units of a token / 256, tokens): the token - and with it the sequence, the position and the
+  // (block of 256 units of a token, token): the token - and with it the sequence, the position and the
   // cache slot - is uniform over the workgroup and is worked out in scalar registers
   const int units_per_head = a.d / 16;
   const int heads = a.hq + 2 * a.hkv;
-  const int unit = blockIdx.x * blockDim.x + threadIdx.x;
+  const int unit = unit_block * 256 + threadIdx.x;
+  const int tok = a.tok0 + tok_in_launch;
+  BatchRows rows;  // (before any thread leaves)
+  rows.load(a.cu_seqlens_q, a.seq_lens_decoder, a.batch);
+  const SeqRows sr = rows.at(rows.seq_of(tok));
   if (unit >= heads * units_per_head) return;
   const int head = unit / units_per_head, u = unit - head * units_per_head;
-  const int tok = a.tok0 + blockIdx.y;
-
-  const int b = seq_of_token(a.cu_seqlens_q, a.batch, tok);
-  if (tok >= a.cu_seqlens_q[b + 1]) return;  // token past the last sequence
-  const int pos = a.seq_lens_decoder[b] + (tok - a.cu_seqlens_q[b]);
+  if (tok >= sr.end) return;  // token past the last sequence
+  const int pos = sr.cached + (tok - sr.first);
   // a position outside the rope table cannot be rotated: the token is skipped - nothing is written to the cache, and
   // its rows of q_out / k_out / v_out are zeros (not whatever the buffers held), so that an attention pass that still
   // counts the token reads defined values
@@ -228,12 +248,11 @@ __global__ __launch_bounds__(256) void write_cache_kv_kernel(WriterArgs a) {
     return;
   }
 
+  if (MODE == 4 && head >= a.hq) return;
   const UnitValues uv = unit_values(a, tok, head, u, pos);
   const bool is_v = head >= a.hq + a.hkv;
   const bool is_k = !is_v && head >= a.hq;
   const int c1 = uv.c1, c2 = uv.c2;
-  const uint4 w1 = uv.w1, w2 = uv.w2;
-  const bool changed = uv.changed;
   const float (&g1)[8] = uv.g1;
   const float (&g2)[8] = uv.g2;
 
@@ -242,8 +261,8 @@ __global__ __launch_bounds__(256) void write_cache_kv_kernel(WriterArgs a) {
     u32 p1[4], p2[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      p1[i] = (u32)f32_to_bf16(g1[2 * i]) | ((u32)f32_to_bf16(g1[2 * i + 1]) << 16);
-      p2[i] = (u32)f32_to_bf16(g2[2 * i]) | ((u32)f32_to_bf16(g2[2 * i + 1]) << 16);
+      p1[i] = pack2_bf16(g1[2 * i], g1[2 * i + 1]);
+      p2[i] = pack2_bf16(g2[2 * i], g2[2 * i + 1]);
     }
     *reinterpret_cast<uint4*>(o + c1) = make_uint4(p1[0], p1[1], p1[2], p1[3]);
     *reinterpret_cast<uint4*>(o + c2) = make_uint4(p2[0], p2[1], p2[2], p2[3]);
@@ -252,32 +271,17 @@ __global__ __launch_bounds__(256) void write_cache_kv_kernel(WriterArgs a) {
 
   const int h = is_k ? head - a.hq : head - a.hq - a.hkv;
   uint16_t* side = is_k ? a.k_out : a.v_out;
-  if (side != nullptr) {
-    uint16_t* o = side + ((size_t)tok * a.hkv + h) * a.d;
-    if (is_v && !changed) {
-      *reinterpret_cast<uint4*>(o + c1) = w1;
-      *reinterpret_cast<uint4*>(o + c2) = w2;
-    } else {
-      u32 p1[4], p2[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        p1[i] = (u32)f32_to_bf16(g1[2 * i]) | ((u32)f32_to_bf16(g1[2 * i + 1]) << 16);
-        p2[i] = (u32)f32_to_bf16(g2[2 * i]) | ((u32)f32_to_bf16(g2[2 * i + 1]) << 16);
-      }
-      *reinterpret_cast<uint4*>(o + c1) = make_uint4(p1[0], p1[1], p1[2], p1[3]);
-      *reinterpret_cast<uint4*>(o + c2) = make_uint4(p2[0], p2[1], p2[2], p2[3]);
-    }
-  }
+  if (side != nullptr) store_side_unit(side + ((size_t)tok * a.hkv + h) * a.d, uv, is_v);
 
-  if (MODE == 2) return;
+  if (MODE == 2 || MODE == 4) return;
   if constexpr (MODE == 3) {
     TileJob j;
-    if (tile_job(a, b, tok, j)) write_tile_rows<QUANT>(a, j, h, is_k, head, u, uv);  // (the same for every thread of the workgroup)
+    if (tile_job(a, sr, tok, j)) write_tile_rows<QUANT>(a, j, h, is_k, head, u, uv);  // (the same for every thread of the workgroup)
     return;
   }
   const int lb = pos / a.bs, slot = pos - lb * a.bs;
   if (lb >= a.max_blocks) return;
-  const int pb = a.block_tables[(size_t)b * a.max_blocks + lb];
+  const int pb = a.block_tables[(size_t)sr.b * a.max_blocks + lb];
   if (pb < 0 || pb >= a.num_blocks) return;
   uint8_t* dst = (is_k ? a.key_cache : a.value_cache) + (((size_t)pb * a.hkv + h) * a.bs + slot) * a.d;
   float s1[8], s2[8];
@@ -312,6 +316,12 @@ __global__ __launch_bounds__(256) void write_cache_kv_kernel(WriterArgs a) {
   *reinterpret_cast<uint2*>(dst + c2) = make_uint2(q2[0], q2[1]);
 }
 
+// grid (units of a token / 256, tokens)
+template <int QUANT, int MODE>
+__global__ __launch_bounds__(256) void write_cache_kv_kernel(WriterArgs a) {
+  write_token_units<QUANT, MODE>(a, blockIdx.x, blockIdx.y);
+}
+
 // One stored byte under a tile scale that grew from s_old to s: (value of the byte * s_old) / s, quantised again.
 template <int QUANT>
 __device__ __forceinline__ u32 requant1(u32 byte, float s_old, float s) {
@@ -326,11 +336,11 @@ __device__ __forceinline__ u32 requant1(u32 byte, float s_old, float s) {
 // first one this call stores into a tile - the first new token of its sequence, or one whose position is a multiple of
 // the block size - stands for the tile.
 
-__device__ __forceinline__ bool tile_job(const WriterArgs& a, int b, int tok, TileJob& j) {
-  const int tok_first = a.cu_seqlens_q[b];
-  const int tok_end = min(a.cu_seqlens_q[b + 1], a.num_tokens);
+__device__ __forceinline__ bool tile_job(const WriterArgs& a, const SeqRows& sr, int tok, TileJob& j) {
+  const int b = sr.b, tok_first = sr.first;
+  const int tok_end = min(sr.end, a.num_tokens);
   if (tok < tok_first || tok >= tok_end) return false;
-  const int p0 = a.seq_lens_decoder[b];
+  const int p0 = sr.cached;
   const int pos = p0 + (tok - tok_first);
   // tokens before position 0 or past the rope table are skipped, as by the token kernel
   const int p_first = max(p0, 0);
@@ -339,9 +349,11 @@ __device__ __forceinline__ bool tile_job(const WriterArgs& a, int b, int tok, Ti
   if (pos < p_first || pos >= p_end) return false;
   const int lb = pos / a.bs;
   if (pos != p_first && pos != lb * a.bs) return false;  // another token stands for this tile
-  if (lb >= a.max_blocks) return false;
-  const int pb = a.block_tables[(size_t)b * a.max_blocks + lb];
-  if (pb < 0 || pb >= a.num_blocks) return false;
+  int pb = lb < a.max_blocks ? a.block_tables[(size_t)b * a.max_blocks + lb] : -1;
+  if (pb < 0 || pb >= a.num_blocks) {
+    if (!a.tiles_write_rows) return false;
+    pb = -1;  // no block to store into, but the rows are still owed to k_out / v_out
+  }
   j.tok = tok;
   j.r0 = pos;
   j.r1 = min(p_end, (lb + 1) * a.bs);
@@ -351,105 +363,110 @@ __device__ __forceinline__ bool tile_job(const WriterArgs& a, int b, int tok, Ti
   return true;
 }
 
-// One tile of KV head h by NT threads (64: a wavefront on its own; 256: a workgroup, red = its reduction buffer):
-// (1) the K and V rows that the call stores into the tile, recomputed, and their largest magnitudes, (2) the tile's
-// scales - if rows of earlier calls are in the tile the scales only grow, and when one grows those rows are
-// requantised in place -, (3) the rows stored quantised (computed once more unless they fit one pass of the NT
-// threads: NT * 16 / head_dim rows).
+// The K (or the V) half of one tile of KV head h by NT threads (64: a wavefront on its own; 256: a workgroup, red = its
+// reduction buffer): (1) the rows that the call stores into the tile, recomputed, and their largest magnitude, (2) the tile's
+// scale - if rows of earlier calls are in the tile the scale only grows, and when it grows those rows are
+// requantised in place -, (3) the rows stored quantised (computed once more unless the threads hold them all: NT * 16 /
+// head_dim rows per pass, two passes' worth in a workgroup's registers).
 template <int QUANT, int NT>
-__device__ __forceinline__ void write_tile(const WriterArgs& a, const TileJob& j, int h, float (*red)[4]) {
+__device__ __forceinline__ void write_tile(const WriterArgs& a, const TileJob& j, int h, bool is_k, float (*red)[4]) {
   const int tid = threadIdx.x;
-  const size_t at = (size_t)j.pb * a.hkv + h;
-  // the old scales are asked for now - before anything of this tile is stored - and needed after the rows' maxima
-  float sk_old = 0.f, sv_old = 0.f;
-  if (j.prior_rows > 0) sk_old = a.k_scale[at], sv_old = a.v_scale[at];
+  const bool cached = j.pb >= 0;  // (false: the table names no block for these rows - they only go to k_out / v_out)
+  const size_t at = (size_t)(cached ? j.pb : 0) * a.hkv + h;
+  float* const scale = is_k ? a.k_scale : a.v_scale;
+  // the old scale is asked for now - before anything of this tile is stored - and needed after the rows' maximum
+  float s_old = 0.f;
+  if (cached && j.prior_rows > 0) s_old = scale[at];
+  // the rows as the attention kernels take them (long chunks: the token kernel leaves them to this one)
+  uint16_t* const side = is_k ? a.k_out : a.v_out;
+  auto side_row = [&](int r, const UnitValues& x) {
+    if (a.tiles_write_rows && side) store_side_unit(side + ((size_t)(j.tok + (r - j.r0)) * a.hkv + h) * a.d, x, !is_k);
+  };
 
   const int uph = a.d / 16, rows_per_pass = NT / uph;
   const int u = tid % uph, row_in_pass = tid / uph;
-  const int k_head = a.hq + h, v_head = a.hq + a.hkv + h;
+  const int head = a.hq + (is_k ? 0 : a.hkv) + h;
   const int r0 = j.r0, r1 = j.r1;
-  const bool one_pass = r1 - r0 <= rows_per_pass;
+  // a workgroup keeps two rows per thread in registers (a tile of 64 rows at head_dim 128: every row is computed once
+  // and all loads of the tile are in flight together), a wavefront one
+  constexpr int RPT = NT > 64 ? 2 : 1;
+  const bool kept = r1 - r0 <= RPT * rows_per_pass;
 
-  UnitValues k, v;  // (of the last pass; the only one if one_pass)
-  float mk = 0.f, mv = 0.f;  // fmaxf drops NaNs, as the oracle's does
-  for (int rb = r0; rb < r1; rb += rows_per_pass) {
-    const bool live = rb + row_in_pass < r1;
-    const int r = live ? rb + row_in_pass : r1 - 1;  // (idle lanes repeat the last row: the norm's butterfly needs every lane)
-    k = unit_values(a, j.tok + (r - r0), k_head, u, r);
-    v = unit_values(a, j.tok + (r - r0), v_head, u, r);
-    if (live) {
+  UnitValues x[RPT];
+  float m = 0.f;  // fmaxf drops NaNs, as the oracle's does
+  auto take = [&](const UnitValues& xx) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        mk = fmaxf(mk, fmaxf(fabsf(k.g1[i]), fabsf(k.g2[i])));
-        mv = fmaxf(mv, fmaxf(fabsf(v.g1[i]), fabsf(v.g2[i])));
-      }
+    for (int i = 0; i < 8; ++i) m = fmaxf(m, fmaxf(fabsf(xx.g1[i]), fabsf(xx.g2[i])));
+  };
+  if (kept) {
+#pragma unroll
+    for (int e = 0; e < RPT; ++e) {
+      const int rr = r0 + e * rows_per_pass + row_in_pass;
+      const int r = rr < r1 ? rr : r1 - 1;  // (idle lanes repeat the last row: the norm's butterfly needs every lane)
+      x[e] = unit_values(a, j.tok + (r - r0), head, u, r);
+      if (rr < r1) take(x[e]), side_row(rr, x[e]);
+    }
+  } else {
+    for (int rb = r0; rb < r1; rb += rows_per_pass) {
+      const bool live = rb + row_in_pass < r1;
+      const int r = live ? rb + row_in_pass : r1 - 1;
+      const UnitValues xx = unit_values(a, j.tok + (r - r0), head, u, r);
+      if (live) take(xx), side_row(r, xx);
     }
   }
-  mk = wave_max(mk);
-  mv = wave_max(mv);
+  m = wave_max(m);
   if (NT > 64) {
     __syncthreads();  // (the buffer may still be read for the workgroup's previous tile)
-    if ((tid & 63) == 0) red[0][tid >> 6] = mk, red[1][tid >> 6] = mv;
+    if ((tid & 63) == 0) red[0][tid >> 6] = m;
     __syncthreads();
-    mk = fmaxf(fmaxf(red[0][0], red[0][1]), fmaxf(red[0][2], red[0][3]));
-    mv = fmaxf(fmaxf(red[1][0], red[1][1]), fmaxf(red[1][2], red[1][3]));
+    m = fmaxf(fmaxf(red[0][0], red[0][1]), fmaxf(red[0][2], red[0][3]));
   }
   const float qmax = QUANT == FDATTN_CACHE_INT8 ? 127.0f : 448.0f;
-  const float sk_now = mk > 0.f ? __fdiv_rn(mk, qmax) : 0.f, sv_now = mv > 0.f ? __fdiv_rn(mv, qmax) : 0.f;
-  float sk, sv;
-  if (j.prior_rows > 0) {
-    sk = sk_now > sk_old ? sk_now : sk_old;
-    sv = sv_now > sv_old ? sv_now : sv_old;
-  } else {
-    sk = sk_now > 0.f ? sk_now : 1.0f;
-    sv = sv_now > 0.f ? sv_now : 1.0f;
-  }
-  if (tid == 0) a.k_scale[at] = sk, a.v_scale[at] = sv;
+  const float s_now = m > 0.f ? __fdiv_rn(m, qmax) : 0.f;
+  const float sc = j.prior_rows > 0 ? (s_now > s_old ? s_now : s_old) : (s_now > 0.f ? s_now : 1.0f);
+  if (!cached) return;  // (uniform over the workgroup; its barriers are behind it)
+  if (tid == 0) scale[at] = sc;
 
-  uint8_t* const ktile = a.key_cache + at * a.bs * a.d;
-  uint8_t* const vtile = a.value_cache + at * a.bs * a.d;
-  if (j.prior_rows > 0) {
+  uint8_t* const tile = (is_k ? a.key_cache : a.value_cache) + at * a.bs * a.d;
+  if (j.prior_rows > 0 && sc > s_old) {  // the scale grew: the rows of earlier calls move to the new grid
     const int pieces = j.prior_rows * a.d / 16;
+    for (int i = tid; i < pieces; i += NT) {
+      uint4 w = *reinterpret_cast<const uint4*>(tile + (size_t)i * 16);
+      u32 ws[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
-    for (int kv = 0; kv < 2; ++kv) {
-      const float s_old = kv ? sv_old : sk_old, s = kv ? sv : sk;
-      if (!(s > s_old)) continue;  // the scale stayed: so do the bytes
-      uint8_t* tile = kv ? vtile : ktile;
-      for (int i = tid; i < pieces; i += NT) {
-        uint4 w = *reinterpret_cast<const uint4*>(tile + (size_t)i * 16);
-        u32 ws[4] = {w.x, w.y, w.z, w.w};
+      for (int e = 0; e < 4; ++e) {
+        u32 o = 0;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          u32 o = 0;
-#pragma unroll
-          for (int by = 0; by < 4; ++by) o |= requant1<QUANT>((ws[e] >> (8 * by)) & 0xffu, s_old, s) << (8 * by);
-          ws[e] = o;
-        }
-        *reinterpret_cast<uint4*>(tile + (size_t)i * 16) = make_uint4(ws[0], ws[1], ws[2], ws[3]);
+        for (int by = 0; by < 4; ++by) o |= requant1<QUANT>((ws[e] >> (8 * by)) & 0xffu, s_old, sc) << (8 * by);
+        ws[e] = o;
       }
+      *reinterpret_cast<uint4*>(tile + (size_t)i * 16) = make_uint4(ws[0], ws[1], ws[2], ws[3]);
     }
   }
-  for (int rb = r0; rb < r1; rb += rows_per_pass) {
-    const bool live = rb + row_in_pass < r1;
-    const int r = live ? rb + row_in_pass : r1 - 1;
-    if (!one_pass) {
-      k = unit_values(a, j.tok + (r - r0), k_head, u, r);
-      v = unit_values(a, j.tok + (r - r0), v_head, u, r);
-    }
-    if (!live) continue;
-    u32 qk1[2] = {0, 0}, qk2[2] = {0, 0}, qv1[2] = {0, 0}, qv2[2] = {0, 0};
+  auto store_row = [&](int r, const UnitValues& xx) {
+    u32 q1[2] = {0, 0}, q2[2] = {0, 0};
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      qk1[i >> 2] |= quant1<QUANT>(k.g1[i], sk) << (8 * (i & 3));
-      qk2[i >> 2] |= quant1<QUANT>(k.g2[i], sk) << (8 * (i & 3));
-      qv1[i >> 2] |= quant1<QUANT>(v.g1[i], sv) << (8 * (i & 3));
-      qv2[i >> 2] |= quant1<QUANT>(v.g2[i], sv) << (8 * (i & 3));
+      q1[i >> 2] |= quant1<QUANT>(xx.g1[i], sc) << (8 * (i & 3));
+      q2[i >> 2] |= quant1<QUANT>(xx.g2[i], sc) << (8 * (i & 3));
     }
     const size_t roff = (size_t)(r - j.lb * a.bs) * a.d;
-    *reinterpret_cast<uint2*>(ktile + roff + k.c1) = make_uint2(qk1[0], qk1[1]);
-    *reinterpret_cast<uint2*>(ktile + roff + k.c2) = make_uint2(qk2[0], qk2[1]);
-    *reinterpret_cast<uint2*>(vtile + roff + v.c1) = make_uint2(qv1[0], qv1[1]);
-    *reinterpret_cast<uint2*>(vtile + roff + v.c2) = make_uint2(qv2[0], qv2[1]);
+    *reinterpret_cast<uint2*>(tile + roff + xx.c1) = make_uint2(q1[0], q1[1]);
+    *reinterpret_cast<uint2*>(tile + roff + xx.c2) = make_uint2(q2[0], q2[1]);
+  };
+  if (kept) {
+#pragma unroll
+    for (int e = 0; e < RPT; ++e) {
+      const int rr = r0 + e * rows_per_pass + row_in_pass;
+      if (rr < r1) store_row(rr, x[e]);
+    }
+  } else {
+    for (int rb = r0; rb < r1; rb += rows_per_pass) {
+      const bool live = rb + row_in_pass < r1;
+      const int r = live ? rb + row_in_pass : r1 - 1;
+      const UnitValues xx = unit_values(a, j.tok + (r - r0), head, u, r);
+      if (live) store_row(r, xx);
+    }
   }
 }
 
@@ -511,8 +528,10 @@ __device__ __forceinline__ void write_tile_rows(const WriterArgs& a, const TileJ
 template <int QUANT>
 __global__ __launch_bounds__(64) void write_cache_tiles_kernel(WriterArgs a) {
   const int h = blockIdx.x, tok = a.tok0 + blockIdx.y;
+  BatchRows rows;
+  rows.load(a.cu_seqlens_q, a.seq_lens_decoder, a.batch);
   TileJob j;
-  if (tile_job(a, seq_of_token(a.cu_seqlens_q, a.batch, tok), tok, j)) write_tile<QUANT, 64>(a, j, h, nullptr);
+  if (tile_job(a, rows.at(rows.seq_of(tok)), tok, j)) write_tile<QUANT, 64>(a, j, h, blockIdx.z == 0, nullptr);
 }
 
 // Long chunks (most tokens stand for no tile; a tile has many rows): grid (kv heads, batch + groups of 64 tokens), one
@@ -520,25 +539,34 @@ __global__ __launch_bounds__(64) void write_cache_tiles_kernel(WriterArgs a) {
 // Candidate batch + g: the tiles started at a multiple of the block size by tokens 64 g .. 64 g + 63 of the call that
 // are not the first of their sequence - walking the sequences that have tokens in that range.
 template <int QUANT>
-__global__ __launch_bounds__(256) void write_cache_tiles_chunk_kernel(WriterArgs a) {
-  __shared__ float red[2][4];
-  const int h = blockIdx.x, c = blockIdx.y;
+__device__ __forceinline__ void tile_candidate(const WriterArgs& a, int h, int c, bool is_k, float (*red)[4]) {
+  BatchRows rows;
+  rows.load(a.cu_seqlens_q, a.seq_lens_decoder, a.batch);
   TileJob j;
+  // (every thread of the workgroup stays to the end: the cross-lane reads below see whole wavefronts)
   if (c < a.batch) {
-    if (tile_job(a, c, a.cu_seqlens_q[c], j)) write_tile<QUANT, 256>(a, j, h, red);
+    const SeqRows sr = rows.at(c);
+    if (tile_job(a, sr, sr.first, j)) write_tile<QUANT, 256>(a, j, h, is_k, red);
     return;
   }
   const int t_lo = (c - a.batch) * 64, t_hi = min(t_lo + 64, a.num_tokens);
   if (t_lo >= t_hi) return;
-  for (int b = seq_of_token(a.cu_seqlens_q, a.batch, t_lo); b < a.batch && a.cu_seqlens_q[b] < t_hi; ++b) {
-    const int tok_first = a.cu_seqlens_q[b], p0 = a.seq_lens_decoder[b];
+  for (int b = rows.seq_of(t_lo); b < a.batch; ++b) {
+    const SeqRows sr = rows.at(b);
+    if (sr.first >= t_hi) break;
+    const int tok_first = sr.first, p0 = sr.cached;
     // the first token of the sequence in the range whose position is a multiple of the block size, then every bs-th
     const int t_from = max(t_lo, tok_first + 1);
     const int pos_from = p0 + (t_from - tok_first);
     const int first_aligned = (pos_from + a.bs - 1) / a.bs * a.bs;
     for (int t = t_from + (first_aligned - pos_from); t < t_hi; t += a.bs)
-      if (tile_job(a, b, t, j)) write_tile<QUANT, 256>(a, j, h, red);
+      if (tile_job(a, sr, t, j)) write_tile<QUANT, 256>(a, j, h, is_k, red);
   }
+}
+template <int QUANT>
+__global__ __launch_bounds__(256) void write_cache_tiles_chunk_kernel(WriterArgs a) {
+  __shared__ float red[1][4];
+  tile_candidate<QUANT>(a, blockIdx.x, blockIdx.y, blockIdx.z == 0, red);
 }
 
 }  // namespace fdattn
@@ -603,7 +631,7 @@ extern "C" int fdattn_write_cache_kv_ex(
                (uint8_t*)key_cache, (uint8_t*)value_cache, cache_k_scale, cache_v_scale, rope_cos,
                rope_sin, block_tables, seq_lens_decoder, cu_seqlens_q, num_tokens, batch, hq, hkv,
                head_dim, block_size, max_blocks_per_seq, num_blocks, max_pos, rope_style,
-               (const uint16_t*)ep.qkv_bias, ep.q_norm_weight, ep.k_norm_weight, ep.rms_norm_eps, 0};
+               (const uint16_t*)ep.qkv_bias, ep.q_norm_weight, ep.k_norm_weight, ep.rms_norm_eps, 0, 0};
   const int units = (hq + 2 * hkv) * (head_dim / 16);
   hipStream_t s = (hipStream_t)stream;
   // the y dimension of a grid holds 65,535 workgroups: more tokens go in slices
@@ -615,6 +643,16 @@ extern "C" int fdattn_write_cache_kv_ex(
       // is one row there; should a sequence bring several after all, its threads walk them)
       if (quant_bytes(cache_quant_type) == FDATTN_CACHE_INT8) hipLaunchKernelGGL((write_cache_kv_kernel<FDATTN_CACHE_INT8, 3>), grid, dim3(256), 0, s, a);
       else hipLaunchKernelGGL((write_cache_kv_kernel<FDATTN_CACHE_FP8_E4M3, 3>), grid, dim3(256), 0, s, a);
+    } else if (quant_blockwise(cache_quant_type) && (long long)num_tokens >= 16LL * batch && num_tokens <= 65535 &&
+               batch + (num_tokens + 63) / 64 <= 65535) {
+      // long chunks: a workgroup per candidate tile start computes the tile's K and V rows once and writes them to the
+      // cache (with the tile's scales) and to k_out / v_out; the token kernel is left the Q heads
+      a.tiles_write_rows = 1;
+      const bool i8 = quant_bytes(cache_quant_type) == FDATTN_CACHE_INT8;
+      const dim3 cgrid(hkv, batch + (num_tokens + 63) / 64, 2);  // (z: the K halves of the tiles, the V halves)
+      if (i8) hipLaunchKernelGGL((write_cache_tiles_chunk_kernel<FDATTN_CACHE_INT8>), cgrid, dim3(256), 0, s, a);
+      else hipLaunchKernelGGL((write_cache_tiles_chunk_kernel<FDATTN_CACHE_FP8_E4M3>), cgrid, dim3(256), 0, s, a);
+      hipLaunchKernelGGL((write_cache_kv_kernel<FDATTN_CACHE_INT8, 4>), grid, dim3(256), 0, s, a);
     } else if (quant_blockwise(cache_quant_type)) {
       // Q, k_out, v_out from the token kernel; the cache and its tile scales from the tile kernel (independent of it)
       hipLaunchKernelGGL((write_cache_kv_kernel<FDATTN_CACHE_INT8, 2>), grid, dim3(256), 0, s, a);
@@ -622,12 +660,12 @@ extern "C" int fdattn_write_cache_kv_ex(
       if ((long long)num_tokens >= 16LL * batch && batch + (num_tokens + 63) / 64 <= 65535) {
         // long chunks: a workgroup per candidate tile start (all in the first slice's launch: they cover every token)
         if (t0 == 0) {
-          const dim3 cgrid(hkv, batch + (num_tokens + 63) / 64);
+          const dim3 cgrid(hkv, batch + (num_tokens + 63) / 64, 2);
           if (i8) hipLaunchKernelGGL((write_cache_tiles_chunk_kernel<FDATTN_CACHE_INT8>), cgrid, dim3(256), 0, s, a);
           else hipLaunchKernelGGL((write_cache_tiles_chunk_kernel<FDATTN_CACHE_FP8_E4M3>), cgrid, dim3(256), 0, s, a);
         }
       } else {
-        const dim3 tgrid(hkv, grid.y);
+        const dim3 tgrid(hkv, grid.y, 2);
         if (i8) hipLaunchKernelGGL((write_cache_tiles_kernel<FDATTN_CACHE_INT8>), tgrid, dim3(64), 0, s, a);
         else hipLaunchKernelGGL((write_cache_tiles_kernel<FDATTN_CACHE_FP8_E4M3>), tgrid, dim3(64), 0, s, a);
       }

@@ -55,6 +55,42 @@ __device__ __forceinline__ int seq_of_token(const int32_t* cu, int batch, int to
   return lo;
 }
 
+// The batch's row bounds and cached lengths, held by a wavefront: lane l keeps sequence l's cu_seqlens_q[l],
+// cu_seqlens_q[l + 1] and seq_lens_decoder[l] - three independent loads, one round trip to memory for everything a
+// kernel needs to place a token, where a search through cu_seqlens_q followed by the sequence's entries is a chain of
+// dependent ones (a microsecond each, and short-lived workgroups consist of little else).  Batches of more than 64
+// sequences fall back to those loads.
+// EVERY lane of the wavefront must be active in load(), seq_of() and at(): they read across lanes, and what a lane
+// that has left a kernel early holds in its registers is undefined (the compiler moves and copies values under the
+// mask of the lanes still active).  Take a sequence's SeqRows out first, branch afterwards.
+struct SeqRows { int b, first, end, cached; };  // sequence b: its rows [first, end) of the call, its cached tokens
+struct BatchRows {
+  const int32_t* cu;
+  const int32_t* dec;
+  int batch;
+  int c0, c1, d;  // lane l: sequence l
+  __device__ __forceinline__ void load(const int32_t* cu_seqlens_q, const int32_t* seq_lens_decoder, int n) {
+    cu = cu_seqlens_q, dec = seq_lens_decoder, batch = n;
+    const int lane = threadIdx.x & 63;
+    const bool in = n <= 64 && lane < n;
+    c0 = in ? cu[lane] : 0x7fffffff;
+    c1 = in ? cu[lane + 1] : 0x7fffffff;
+    d = in ? dec[lane] : 0;
+  }
+  __device__ __forceinline__ SeqRows at(int b) const {
+    if (batch <= 64) return SeqRows{b, __builtin_amdgcn_readlane(c0, b), __builtin_amdgcn_readlane(c1, b), __builtin_amdgcn_readlane(d, b)};
+    return SeqRows{b, cu[b], cu[b + 1], dec[b]};
+  }
+  // the sequence of token tok, as seq_of_token gives it (tok: uniform over the wavefront)
+  __device__ __forceinline__ int seq_of(int tok) const {
+    if (batch > 64) return seq_of_token(cu, batch, tok);
+    const unsigned long long holds = __ballot(c0 <= tok && tok < c1);
+    if (holds) return __ffsll((long long)holds) - 1;
+    const unsigned long long before = __ballot(c0 <= tok);  // no sequence holds it: the last one that starts at or before it
+    return before ? 63 - __clzll((long long)before) : 0;
+  }
+};
+
 // cache_quant_type -> how the bytes are encoded / where the scales live
 __host__ __device__ constexpr int quant_bytes(int q) {
   return q == FDATTN_CACHE_INT8_DYNAMIC || q == FDATTN_CACHE_INT8_BLOCK
@@ -90,6 +126,15 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
   if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
   u += 0x7fffu + ((u >> 16) & 1u);
   return (uint16_t)(u >> 16);
+}
+
+// two at once, by the hardware's conversion (v_cvt_pk_bf16_f32): the same bits as f32_to_bf16 for every one of the
+// 2^32 inputs - NaNs and subnormals included (checked exhaustively on the GPU) - at a sixth of the instructions
+__device__ __forceinline__ u32 pack2_bf16(float lo, float hi) {
+  typedef float f2v __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf2v __attribute__((ext_vector_type(2)));
+  const f2v x = {lo, hi};
+  return __builtin_bit_cast(u32, __builtin_convertvector(x, bf2v));
 }
 
 // fp8 e4m3fn (OCP): 1-4-3, bias 7, max 448, no infinities.
