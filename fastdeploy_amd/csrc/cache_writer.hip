@@ -52,6 +52,24 @@ __device__ __forceinline__ u32 quant1(float x, float s) {
   }
 }
 
+// The same byte as quant1(x, s) when many values share the scale: x * (1 / s) with the hardware's reciprocal (rs, taken
+// once) is within a few units in the last place of the correctly rounded x / s, so the two can only round to different
+// integers next to a tie - there, and for anything that is not a number, the division decides.  int8 only (the e4m3
+// grid is not uniform: fp8 takes quant1).
+template <int QUANT>
+__device__ __forceinline__ u32 quant1_shared(float x, float s, float rs) {
+  if (QUANT != FDATTN_CACHE_INT8) return quant1<QUANT>(x, s);
+  float q = __fmul_rn(x, rs);
+  float t = __builtin_rintf(q);
+  if (!(fabsf(q - t) <= 0.499f)) {
+    q = __fdiv_rn(x, s);
+    if (q != q) return 0u;
+    t = __builtin_rintf(q);
+  }
+  t = fminf(fmaxf(t, -127.0f), 127.0f);
+  return (u32)(int)t & 0xffu;
+}
+
 // The values of one unit - 8 rotation pairs (16 channels) of one head of one token - after the projection's
 // epilogue and the rotation, in channel order: g1 = channels c1 .. c1+7, g2 = channels c2 .. c2+7.
 // The RMS norm's sum runs over the d/16 adjacent lanes that hold the head's units: every one of them must be here.
@@ -307,10 +325,19 @@ __device__ __forceinline__ void write_token_units(const WriterArgs& a, int unit_
     for (int i = 0; i < 8; ++i) { s1[i] = t1[i]; s2[i] = t2[i]; }
   }
   u32 q1[2] = {0, 0}, q2[2] = {0, 0};
+  if (DYN) {  // one scale for the row
+    const float rs = __builtin_amdgcn_rcpf(s1[0]);
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    q1[i >> 2] |= quant1<QUANT>(g1[i], s1[i]) << (8 * (i & 3));
-    q2[i >> 2] |= quant1<QUANT>(g2[i], s2[i]) << (8 * (i & 3));
+    for (int i = 0; i < 8; ++i) {
+      q1[i >> 2] |= quant1_shared<QUANT>(g1[i], s1[0], rs) << (8 * (i & 3));
+      q2[i >> 2] |= quant1_shared<QUANT>(g2[i], s1[0], rs) << (8 * (i & 3));
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      q1[i >> 2] |= quant1<QUANT>(g1[i], s1[i]) << (8 * (i & 3));
+      q2[i >> 2] |= quant1<QUANT>(g2[i], s2[i]) << (8 * (i & 3));
+    }
   }
   *reinterpret_cast<uint2*>(dst + c1) = make_uint2(q1[0], q1[1]);
   *reinterpret_cast<uint2*>(dst + c2) = make_uint2(q2[0], q2[1]);
@@ -443,12 +470,13 @@ __device__ __forceinline__ void write_tile(const WriterArgs& a, const TileJob& j
       *reinterpret_cast<uint4*>(tile + (size_t)i * 16) = make_uint4(ws[0], ws[1], ws[2], ws[3]);
     }
   }
+  const float rsc = __builtin_amdgcn_rcpf(sc);
   auto store_row = [&](int r, const UnitValues& xx) {
     u32 q1[2] = {0, 0}, q2[2] = {0, 0};
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      q1[i >> 2] |= quant1<QUANT>(xx.g1[i], sc) << (8 * (i & 3));
-      q2[i >> 2] |= quant1<QUANT>(xx.g2[i], sc) << (8 * (i & 3));
+      q1[i >> 2] |= quant1_shared<QUANT>(xx.g1[i], sc, rsc) << (8 * (i & 3));
+      q2[i >> 2] |= quant1_shared<QUANT>(xx.g2[i], sc, rsc) << (8 * (i & 3));
     }
     const size_t roff = (size_t)(r - j.lb * a.bs) * a.d;
     *reinterpret_cast<uint2*>(tile + roff + xx.c1) = make_uint2(q1[0], q1[1]);
@@ -509,13 +537,14 @@ __device__ __forceinline__ void write_tile_rows(const WriterArgs& a, const TileJ
       *reinterpret_cast<uint4*>(tile + (size_t)i * 16) = make_uint4(ws[0], ws[1], ws[2], ws[3]);
     }
   }
+  const float rsc = __builtin_amdgcn_rcpf(sc);
   for (int r = j.r0; r < j.r1; ++r) {
     const UnitValues x = r == j.r0 ? first : unit_values(a, j.tok + (r - j.r0), head, u, r);
     u32 q1[2] = {0, 0}, q2[2] = {0, 0};
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      q1[i >> 2] |= quant1<QUANT>(x.g1[i], sc) << (8 * (i & 3));
-      q2[i >> 2] |= quant1<QUANT>(x.g2[i], sc) << (8 * (i & 3));
+      q1[i >> 2] |= quant1_shared<QUANT>(x.g1[i], sc, rsc) << (8 * (i & 3));
+      q2[i >> 2] |= quant1_shared<QUANT>(x.g2[i], sc, rsc) << (8 * (i & 3));
     }
     const size_t roff = (size_t)(r - j.lb * a.bs) * a.d;
     *reinterpret_cast<uint2*>(tile + roff + x.c1) = make_uint2(q1[0], q1[1]);
@@ -567,6 +596,21 @@ template <int QUANT>
 __global__ __launch_bounds__(256) void write_cache_tiles_chunk_kernel(WriterArgs a) {
   __shared__ float red[1][4];
   tile_candidate<QUANT>(a, blockIdx.x, blockIdx.y, blockIdx.z == 0, red);
+}
+
+// Long chunks in one launch: the first kv_heads x candidates x 2 workgroups are write_cache_tiles_chunk_kernel's (they
+// run longest - a chain of loads, a reduction, stores - and start first), the others the token kernel's, which here
+// writes q_out only; neither reads what the other writes.
+template <int QUANT>
+__global__ __launch_bounds__(256) void write_cache_chunk_kernel(WriterArgs a, int candidates, int unit_blocks) {
+  __shared__ float red[1][4];
+  const int tiles = 2 * a.hkv * candidates;
+  if ((int)blockIdx.x < tiles) {
+    const int i = blockIdx.x >> 1;
+    tile_candidate<QUANT>(a, i % a.hkv, i / a.hkv, (blockIdx.x & 1) == 0, red);
+  } else {
+    write_token_units<QUANT, 4>(a, (blockIdx.x - tiles) % unit_blocks, (blockIdx.x - tiles) / unit_blocks);
+  }
 }
 
 }  // namespace fdattn
@@ -644,15 +688,17 @@ extern "C" int fdattn_write_cache_kv_ex(
       if (quant_bytes(cache_quant_type) == FDATTN_CACHE_INT8) hipLaunchKernelGGL((write_cache_kv_kernel<FDATTN_CACHE_INT8, 3>), grid, dim3(256), 0, s, a);
       else hipLaunchKernelGGL((write_cache_kv_kernel<FDATTN_CACHE_FP8_E4M3, 3>), grid, dim3(256), 0, s, a);
     } else if (quant_blockwise(cache_quant_type) && (long long)num_tokens >= 16LL * batch && num_tokens <= 65535 &&
-               batch + (num_tokens + 63) / 64 <= 65535) {
+               2LL * hkv * (batch + (num_tokens + 63) / 64) + (long long)grid.x * num_tokens <= 0x7fffffffLL) {
       // long chunks: a workgroup per candidate tile start computes the tile's K and V rows once and writes them to the
       // cache (with the tile's scales) and to k_out / v_out; the token kernel is left the Q heads
       a.tiles_write_rows = 1;
       const bool i8 = quant_bytes(cache_quant_type) == FDATTN_CACHE_INT8;
-      const dim3 cgrid(hkv, batch + (num_tokens + 63) / 64, 2);  // (z: the K halves of the tiles, the V halves)
-      if (i8) hipLaunchKernelGGL((write_cache_tiles_chunk_kernel<FDATTN_CACHE_INT8>), cgrid, dim3(256), 0, s, a);
-      else hipLaunchKernelGGL((write_cache_tiles_chunk_kernel<FDATTN_CACHE_FP8_E4M3>), cgrid, dim3(256), 0, s, a);
-      hipLaunchKernelGGL((write_cache_kv_kernel<FDATTN_CACHE_INT8, 4>), grid, dim3(256), 0, s, a);
+      const int candidates = batch + (num_tokens + 63) / 64;
+      // (only the Q heads' unit blocks of a token do anything in the token part - plus the K and V rows of skipped
+      // tokens, which is why all of them are launched)
+      const dim3 mgrid((unsigned)(2 * hkv * candidates + (int)grid.x * num_tokens));
+      if (i8) hipLaunchKernelGGL((write_cache_chunk_kernel<FDATTN_CACHE_INT8>), mgrid, dim3(256), 0, s, a, candidates, (int)grid.x);
+      else hipLaunchKernelGGL((write_cache_chunk_kernel<FDATTN_CACHE_FP8_E4M3>), mgrid, dim3(256), 0, s, a, candidates, (int)grid.x);
     } else if (quant_blockwise(cache_quant_type)) {
       // Q, k_out, v_out from the token kernel; the cache and its tile scales from the tile kernel (independent of it)
       hipLaunchKernelGGL((write_cache_kv_kernel<FDATTN_CACHE_INT8, 2>), grid, dim3(256), 0, s, a);

@@ -48,6 +48,25 @@ def test_writer_bit_exact_small(oracle, quant, style):
         _run_both(oracle, syn.write_case(num_seqs=19, max_pos=1000, quant=quant, seed=seed, rope_style=style))
 
 
+@pytest.mark.parametrize("quant", [CACHE_INT8_DYNAMIC, CACHE_INT8_BLOCK])
+@pytest.mark.parametrize("chunk", [1, 40])
+def test_writer_shared_scales_at_exact_ties(oracle, quant, chunk):
+    """The formats whose rows share a scale quantise with the scale's reciprocal and fall back to the division next to
+    a tie: V rows made of half-integers k + 1/2 (every one a tie under the scale 1 = 127 / 127, which the row's or
+    tile's largest element, 127, sets; under the scale 1/2 every other one), without rotation so that K meets the same
+    values.  Bytes and scales as the oracle's, bit for bit - rint's ties-to-even included."""
+    case = syn.write_case(num_seqs=7, max_pos=300, quant=quant, seed=11, chunk=chunk)
+    T, hq, hkv, d = case["qkv"].shape[0], case["hq"], case["hkv"], case["d"]
+    g = torch.Generator().manual_seed(5)
+    half = torch.randint(-126, 126, (T, (hq + 2 * hkv) * d), generator=g).float() + 0.5   # exact in bf16: 8 bits
+    half[:, 0::d] = 127.0                                                                # every head's row: maximum 127
+    rows = torch.arange(T) % 2 == 1
+    half[rows] = half[rows] * 0.5                                                        # odd tokens: scale 1/2 (rows) / mixed tiles
+    case["qkv"] = half.to(torch.bfloat16)
+    assert torch.equal(case["qkv"].float(), half)
+    _run_both(oracle, case, rope=False)
+
+
 def test_writer_config3_shape_bit_exact(oracle):
     """256 new tokens, positions U{0..8191}, theta 500000, int8, block_size 64."""
     for seed in range(2):
