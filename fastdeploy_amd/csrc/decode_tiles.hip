@@ -51,12 +51,16 @@ struct DecLay {
 template <int D>
 constexpr int waves_per_simd() { return D <= 64 ? 4 : (D <= 128 ? 3 : 2); }
 
-// FAST: the block size is 32 or a power-of-two multiple, so a tile lies inside one block - one table entry, the same
-// for every lane, and constant per-lane offsets.  MT: decode rows may bring several tokens (the one-token launches carry
+// TB: the cache blocks a tile of 32 keys is made of when the block size says so - 1: the block size is 32 or a
+// power-of-two multiple, the tile lies inside one block; 2: the block size is 16, the tile is two whole blocks - each
+// with one table entry, the same for every lane, and constant per-lane offsets (FAST); 0: any other block size, every
+// row through its own table entry.  MT: decode rows may bring several tokens (the one-token launches carry
 // none of that bookkeeping)
-template <int QUANT, bool DYN, int D, bool FAST, bool MT>
+template <int QUANT, bool DYN, int D, int TB, bool MT>
 __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_tiles_kernel(GenericDecodeArgs a) {
   using L = DecLay<D>;
+  constexpr bool FAST = TB > 0;
+  constexpr int RPB = FAST ? 32 / TB : 32;  // FAST: rows of a tile per block
   constexpr int KT = D / 32, DB = D / 16, NC = D / 32;  // k-steps of S = K Q (32 channels each); 16-channel blocks of O; 16-byte chunks per lane and tensor of a tile
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -117,9 +121,10 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
   u32 okq = 0u;     // bit n: row crow + RPI n of the tile in registers is a key; bit 31: the key whose scale the lane carries is one;
                     // bit 30: one of the lane's keys lies past the row's first token (rows of several tokens mask by column there)
   constexpr u32 kLate = 1u << 30;
-  int posq[FAST || !MT ? 1 : NC];  // MT: the positions of the lane's rows of the tile in registers (FAST: of the tile's first row)
+  constexpr int NP = !MT ? 1 : (FAST ? TB : NC);
+  int posq[NP];  // MT: the positions of the lane's rows of the tile in registers (FAST: of the first row of each of the tile's blocks)
 #pragma unroll
-  for (int n = 0; n < (FAST || !MT ? 1 : NC); ++n) posq[n] = 0;
+  for (int n = 0; n < NP; ++n) posq[n] = 0;
   // the logical block of key r of tile t (-1: none), its physical block (-1: none)
   auto logical = [&](int t, int r) {
     const int x = 32 * t + r;
@@ -136,7 +141,7 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
     pos = ok ? lb * a.bs + off : 0x7fffffff;
     return ok;
   };
-  constexpr int NB = FAST ? 1 : NC;
+  constexpr int NB = FAST ? TB : NC;
   int lb1[NB], pb1[NB], lb2[NB];  // the blocks of this lane's rows of the next tile to request (FAST: of the tile); the logical ones of the tile after
   int lbs1 = -1, pbs1 = -1, lbs2 = -1;  // DYN, not FAST: the same for the key whose scale the lane carries
   const u32 lane_off = (u32)crow * D + 16 * cch;  // FAST: this lane's chunk of the first RPI rows of a tile
@@ -144,28 +149,46 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
   auto request = [&](int t) {
     u32 ok = 0;
     if constexpr (FAST) {
-      const int lb = __builtin_amdgcn_readfirstlane(lb1[0]), pb = __builtin_amdgcn_readfirstlane(pb1[0]);
-      const int off0 = (32 * t) & (a.bs - 1);
-      const bool blk = pb >= 0 && pb < a.num_blocks;
-      const long long left = (long long)kv_len - ((long long)lb * a.bs + off0);  // keys from the tile's first row to the sequence's end
-      // (a tile that is none reads block 0; rows past the sequence's end lie in the tile's block: zeroed and masked later)
-      const size_t row0 = blk ? ((size_t)pb * a.hkv + h) * a.bs + off0 : 0;
-      const uint8_t* const kp = a.key_cache + row0 * D + lane_off;
-      const uint8_t* const vp = a.value_cache + row0 * D + lane_off;
+      static_assert(RPI <= RPB, "a load instruction's rows must lie inside one block");
+      const uint8_t* kp[TB];
+      const uint8_t* vp[TB];
+      long long left[TB];  // keys from the block's first row of the tile to the sequence's end
+      bool blk[TB];
+      size_t row0[TB], tile_id[TB];  // the tile's first row of block e in the caches; (block, KV head)
+#pragma unroll
+      for (int e = 0; e < TB; ++e) {
+        const int lb = __builtin_amdgcn_readfirstlane(lb1[e]), pb = __builtin_amdgcn_readfirstlane(pb1[e]);
+        const int off0 = TB == 1 ? (32 * t) & (a.bs - 1) : 0;
+        blk[e] = pb >= 0 && pb < a.num_blocks;
+        left[e] = (long long)kv_len - ((long long)lb * a.bs + off0);
+        // (a block that is none reads block 0; rows past the sequence's end lie in the tile's block: zeroed and masked later)
+        tile_id[e] = blk[e] ? (size_t)pb * a.hkv + h : 0;
+        row0[e] = blk[e] ? tile_id[e] * a.bs + off0 : 0;
+        kp[e] = a.key_cache + row0[e] * D + lane_off;
+        vp[e] = a.value_cache + row0[e] * D + lane_off;
+        if constexpr (MT) {
+          posq[e] = blk[e] ? lb * a.bs + off0 : 0x7fffffff;
+          if (blk[e] && left[e] > 0 && (long long)posq[e] + min(left[e], (long long)RPB) - 1 > p0) ok |= kLate;
+        }
+      }
 #pragma unroll
       for (int n = 0; n < NC; ++n) {
-        kq[n] = nt_load16(kp + n * RPI * D);
-        vq[n] = nt_load16(vp + n * RPI * D);
-        ok |= blk && crow + RPI * n < left ? 1u << n : 0u;
-      }
-      if constexpr (MT) {
-        posq[0] = blk ? lb * a.bs + off0 : 0x7fffffff;
-        if (blk && left > 0 && (long long)posq[0] + min(left, 32LL) - 1 > p0) ok |= kLate;
+        const int e = (RPI * n) / RPB, in_block = RPI * n - RPB * e;  // (constants once unrolled)
+        kq[n] = nt_load16(kp[e] + in_block * D);
+        vq[n] = nt_load16(vp[e] + in_block * D);
+        ok |= blk[e] && crow + in_block < left[e] ? 1u << n : 0u;
       }
       if (DYN) {
-        const bool oks = blk && j32 < left;
+        const int e = TB == 1 ? 0 : j32 / RPB, in_block = j32 - RPB * e;
+        bool blk_e = blk[0];
+        long long left_e = left[0];
+        size_t row0_e = row0[0], tile_e = tile_id[0];
+#pragma unroll
+        for (int x = 1; x < TB; ++x)
+          if (e == x) blk_e = blk[x], left_e = left[x], row0_e = row0[x], tile_e = tile_id[x];
+        const bool oks = blk_e && in_block < left_e;
         ok |= oks ? 1u << 31 : 0u;
-        const size_t srow = a.scale_rows == 1 ? (blk ? (size_t)pb * a.hkv + h : 0) : row0 + j32;
+        const size_t srow = a.scale_rows == 1 ? tile_e : row0_e + in_block;
         ssc = hf ? a.v_scale[srow] : a.k_scale[srow];
       }
       return ok;
@@ -196,7 +219,7 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
   // moves the block pipeline on by one tile: t is the tile whose logical blocks are requested now
   auto advance = [&](int t) {
 #pragma unroll
-    for (int n = 0; n < NB; ++n) lb1[n] = lb2[n], pb1[n] = physical(lb1[n]), lb2[n] = logical(t, FAST ? 0 : crow + RPI * n);
+    for (int n = 0; n < NB; ++n) lb1[n] = lb2[n], pb1[n] = physical(lb1[n]), lb2[n] = logical(t, FAST ? RPB * n : crow + RPI * n);
     if (DYN && !FAST) lbs1 = lbs2, pbs1 = physical(lbs1), lbs2 = logical(t, j32);
   };
 
@@ -205,7 +228,7 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
   int t = wv;
 #pragma unroll
   for (int n = 0; n < NB; ++n) {
-    lb1[n] = logical(t, FAST ? 0 : crow + RPI * n), lb2[n] = logical(t + kWavesDt, FAST ? 0 : crow + RPI * n);
+    lb1[n] = logical(t, FAST ? RPB * n : crow + RPI * n), lb2[n] = logical(t + kWavesDt, FAST ? RPB * n : crow + RPI * n);
     pb1[n] = physical(lb1[n]);
   }
   if (DYN && !FAST) lbs1 = logical(t, j32), lbs2 = logical(t + kWavesDt, j32), pbs1 = physical(lbs1);
@@ -339,7 +362,11 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
     if (by_column && cch == 0) {  // the keys' positions, for the columns to compare with their own
       int* const wpos = reinterpret_cast<int*>(wsc + 96);
 #pragma unroll
-      for (int n = 0; n < NC; ++n) wpos[crow + RPI * n] = FAST ? (posq[0] == 0x7fffffff ? posq[0] : posq[0] + crow + RPI * n) : posq[FAST || !MT ? 0 : n];
+      for (int n = 0; n < NC; ++n) {
+        const int e = FAST ? (RPI * n) / RPB : 0, in_block = crow + RPI * n - RPB * e;
+        const int first = posq[MT && FAST ? e : 0];
+        wpos[crow + RPI * n] = FAST ? (first == 0x7fffffff ? first : first + in_block) : posq[FAST || !MT ? 0 : n];
+      }
     }
     if (more) okq = request(tn);
     // (the wavefront's LDS instructions execute in order: what its lanes stored above is there for the reads below)
@@ -507,7 +534,7 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
   }
 }
 
-template <int QUANT, bool DYN, int D, bool FAST, bool MT>
+template <int QUANT, bool DYN, int D, int TB, bool MT>
 hipError_t launch_dt_f(const GenericDecodeArgs& a, hipStream_t s) {
   using L = DecLay<D>;
   // the dynamic LDS limit is a per-device property of the kernel: raise it once on each device
@@ -516,22 +543,23 @@ hipError_t launch_dt_f(const GenericDecodeArgs& a, hipStream_t s) {
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
   if (dev >= 64 || !(raised.load(std::memory_order_relaxed) >> dev & 1ull)) {
-    e = hipFuncSetAttribute((const void*)decode_tiles_kernel<QUANT, DYN, D, FAST, MT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)L::bytes(16));
+    e = hipFuncSetAttribute((const void*)decode_tiles_kernel<QUANT, DYN, D, TB, MT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)L::bytes(16));
     if (e != hipSuccess) return e;
     if (dev < 64) raised.fetch_or(1ull << dev, std::memory_order_relaxed);
   }
   const int sets = (a.hq / a.hkv + 15) / 16;
   const dim3 grid((unsigned)a.batch * a.hkv * sets, a.max_splits), block(64 * kWavesDt);
   const int columns = a.max_tokens * (a.hq / a.hkv) < 16 ? a.max_tokens * (a.hq / a.hkv) : 16;
-  hipLaunchKernelGGL((decode_tiles_kernel<QUANT, DYN, D, FAST, MT>), grid, block, L::bytes(columns), s, a);
+  hipLaunchKernelGGL((decode_tiles_kernel<QUANT, DYN, D, TB, MT>), grid, block, L::bytes(columns), s, a);
   return hipSuccess;
 }
 
 template <int QUANT, bool DYN, int D>
 hipError_t launch_dt(const GenericDecodeArgs& a, hipStream_t s) {
-  const bool fast = a.bs >= 32 && (a.bs & (a.bs - 1)) == 0;
-  if (a.max_tokens > 1) return fast ? launch_dt_f<QUANT, DYN, D, true, true>(a, s) : launch_dt_f<QUANT, DYN, D, false, true>(a, s);
-  return fast ? launch_dt_f<QUANT, DYN, D, true, false>(a, s) : launch_dt_f<QUANT, DYN, D, false, false>(a, s);
+  const int tb = a.bs >= 32 && (a.bs & (a.bs - 1)) == 0 ? 1 : (a.bs == 16 ? 2 : 0);
+  if (a.max_tokens > 1)
+    return tb == 1 ? launch_dt_f<QUANT, DYN, D, 1, true>(a, s) : (tb == 2 ? launch_dt_f<QUANT, DYN, D, 2, true>(a, s) : launch_dt_f<QUANT, DYN, D, 0, true>(a, s));
+  return tb == 1 ? launch_dt_f<QUANT, DYN, D, 1, false>(a, s) : (tb == 2 ? launch_dt_f<QUANT, DYN, D, 2, false>(a, s) : launch_dt_f<QUANT, DYN, D, 0, false>(a, s));
 }
 
 template <int D>
