@@ -19,6 +19,7 @@ SIGNATURES = {
     "fdattn_decode_attention_noalloc": (_i, [_vp] * 9 + [_i] * 8 + [_f, _vp]),
     "fdattn_decode_uses_mfma": (_i, [_i] * 5),
     "fdattn_decode_chunks_per_sequence": (_i, [_i] * 3),
+    "fdattn_sqattn_path": (_i, [_i] * 5),
     "fdattn_decode_attention_stages": (_i, [_vp] * 10 + [_sz] + [_i] * 8 + [_f, _i, _vp]),
     "fdattn_decode_attention_generic": (_i, [_vp] * 10 + [_i] + [_vp] * 2 + [_sz] + [_i] * 8 + [_f, _vp]),
     "fdattn_decode_attention_tiles": (_i, [_vp] * 10 + [_i] + [_vp] * 2 + [_sz] + [_i] * 8 + [_f, _vp]),

@@ -56,9 +56,24 @@ constexpr int waves_per_simd() { return D <= 64 ? 4 : (D <= 128 ? 3 : 2); }
 // with one table entry, the same for every lane, and constant per-lane offsets (FAST); 0: any other block size, every
 // row through its own table entry.  MT: decode rows may bring several tokens (the one-token launches carry
 // none of that bookkeeping)
-template <int QUANT, bool DYN, int D, int TB, bool MT>
+// a float as an int that orders the same way (for an integer atomic maximum); the smallest int stands for "nothing yet"
+__device__ __forceinline__ int score_key(float f) {
+  const int u = __float_as_int(f);
+  return u >= 0 ? u : u ^ 0x7fffffff;
+}
+__device__ __forceinline__ float key_score(int k) {
+  if (k == (int)0x80000000) return -INFINITY;
+  return __int_as_float(k >= 0 ? k : k ^ 0x7fffffff);
+}
+
+// SCORES: the kernel as the block selector's scoring pass - K only: per block of the split the largest score over its
+// keys and the KV head's query heads (plain q . k, no softmax scale), kept in LDS while the wavefronts walk and written
+// to a.sel_approx at the end, with a bound on its distance to the score summed in fp64 (a.sel_eps per pair; a.sel_ebound
+// per block for the formats with scale caches).
+template <int QUANT, bool DYN, int D, int TB, bool MT, bool SCORES = false>
 __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_tiles_kernel(GenericDecodeArgs a) {
   using L = DecLay<D>;
+  static_assert(!(SCORES && MT), "the scoring pass takes rows of one token");
   constexpr bool FAST = TB > 0;
   constexpr int RPB = FAST ? 32 / TB : 32;  // FAST: rows of a tile per block
   constexpr int KT = D / 32, DB = D / 16, NC = D / 32;  // k-steps of S = K Q (32 channels each); 16-channel blocks of O; 16-byte chunks per lane and tensor of a tile
@@ -85,11 +100,15 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
   const bool live = c16 < toks * G;
   const int p0 = kv_len - toks;     // keys before the row's first token
   const int lim = p0 + tok + 1;     // this column sees keys [0, lim)
-  const float sc = a.sm_scale * 1.4426950408889634f;  // logits go to the log2 domain
+  const float sc = SCORES ? 1.0f : a.sm_scale * 1.4426950408889634f;  // logits go to the log2 domain (the scoring pass: plain scores)
   typedef __attribute__((address_space(3))) uint8_t lds_u8;
   lds_u8* const kt = (lds_u8*)lds + (size_t)wv * L::kWaveBytes;  // this wavefront's K tile, then its V tile, then its scales
   lds_u8* const vt = kt + L::T_BYTES;
   float* const wsc = reinterpret_cast<float*>(lds + (size_t)wv * (L::kWaveBytes / 2) + L::T_BYTES);
+  // the scoring pass: per block of the split its largest score (as an ordered int) and its largest K scale (bits of a
+  // non-negative float), behind everything the decode pass keeps in LDS
+  int* const sel_bmax = reinterpret_cast<int*>(reinterpret_cast<uint8_t*>(lds) + L::bytes(16));
+  unsigned* const sel_smax = reinterpret_cast<unsigned*>(sel_bmax + a.sel_blocks_per_split);
 
   // ---- the split's keys: units [i0, i1) of the sequence's blocks (or of its list of kept blocks), bs keys each;
   // key x of the split sits in unit i0 + x / bs at slot x % bs, and tile t holds keys 32 t .. 32 t + 31
@@ -175,7 +194,7 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
       for (int n = 0; n < NC; ++n) {
         const int e = (RPI * n) / RPB, in_block = RPI * n - RPB * e;  // (constants once unrolled)
         kq[n] = nt_load16(kp[e] + in_block * D);
-        vq[n] = nt_load16(vp[e] + in_block * D);
+        if constexpr (!SCORES) vq[n] = nt_load16(vp[e] + in_block * D);
         ok |= blk[e] && crow + in_block < left[e] ? 1u << n : 0u;
       }
       if (DYN) {
@@ -189,7 +208,7 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
         const bool oks = blk_e && in_block < left_e;
         ok |= oks ? 1u << 31 : 0u;
         const size_t srow = a.scale_rows == 1 ? tile_e : row0_e + in_block;
-        ssc = hf ? a.v_scale[srow] : a.k_scale[srow];
+        ssc = hf && !SCORES ? a.v_scale[srow] : a.k_scale[srow];
       }
       return ok;
     }
@@ -204,7 +223,7 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
         if constexpr (!FAST) posq[n] = pos;
       }
       kq[n] = nt_load16(a.key_cache + (size_t)row * D + 16 * cch);
-      vq[n] = nt_load16(a.value_cache + (size_t)row * D + 16 * cch);
+      if constexpr (!SCORES) vq[n] = nt_load16(a.value_cache + (size_t)row * D + 16 * cch);
     }
     if (DYN) {
       u32 row;
@@ -212,7 +231,7 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
       const bool oks = cache_row(t, j32, lbs1, pbs1, row, pos);
       ok |= oks ? 1u << 31 : 0u;
       const size_t srow = a.scale_rows == 1 ? (oks ? (size_t)pbs1 * a.hkv + h : 0) : row;  // one scale per (block, head) tile, or per stored row
-      ssc = hf ? a.v_scale[srow] : a.k_scale[srow];
+      ssc = hf && !SCORES ? a.v_scale[srow] : a.k_scale[srow];
     }
     return ok;
   };
@@ -248,6 +267,7 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
   const int q_step = live ? 4 * QC : 0;  // slots from one (k-step, term) to the next
   auto q_operand = [&](int st, int term) { return __builtin_bit_cast(v8h, q_lane[(QT * st + term) * q_step]); };
   float scl = sc;      // log2-logit per unit of the accumulator
+  float sel_bound = 0.f;  // the scoring pass: how far a score of this pair may lie from the fp64 score (DYN: per unit of K scale)
   {
     const uint16_t* const qr = a.q + ((size_t)(qrow + (live ? tok : 0)) * a.hq + hq0 + (live ? head : 0)) * D;
     // the row times its K scales: once for its largest element, once more (every fourth k-step) for the operands
@@ -281,6 +301,57 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
       cinv = __uint_as_float((u32)(127 - e) << 23);
     }
     scl = sc * cinv;
+    if constexpr (SCORES) {
+      // sum_c |q_c k_scale_c| of the lane's column: what every error term below is proportional to
+      // (read through a pointer of its own that the compiler cannot see through: merged with the loads of the operand
+      // loop below - which picks its k-step by the wavefront's number - this loop's values came out wrong in one
+      // element of the upper k-steps, for the formats with scale caches)
+      float asum = 0.f, amx = 0.f;
+      const uint16_t* qr_own = qr;
+      const float* ks_own = a.k_scale;
+      asm volatile("" : "+v"(qr_own), "+v"(ks_own));
+#pragma unroll
+      for (int st = 0; st < KT; ++st) {
+        const int c0 = 64 * (st >> 1) + 16 * g4 + 8 * (st & 1);
+        const uint4 w = live ? *reinterpret_cast<const uint4*>(qr_own + c0) : make_uint4(0u, 0u, 0u, 0u);
+        const u32 ws[4] = {w.x, w.y, w.z, w.w};
+        float ksc[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};
+        if (!DYN) {
+          const float4 s0 = *reinterpret_cast<const float4*>(ks_own + h * D + c0), s1 = *reinterpret_cast<const float4*>(ks_own + h * D + c0 + 4);
+          ksc[0] = s0.x, ksc[1] = s0.y, ksc[2] = s0.z, ksc[3] = s0.w, ksc[4] = s1.x, ksc[5] = s1.y, ksc[6] = s1.z, ksc[7] = s1.w;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float x0 = fabsf(bf16lo_to_f32(ws[e]) * ksc[2 * e]), x1 = fabsf(bf16hi_to_f32(ws[e]) * ksc[2 * e + 1]);
+          asum += x0 + x1;
+          amx = fmaxf(amx, fmaxf(x0, x1));
+        }
+      }
+      asum += __shfl_xor(asum, 16, 64);
+      asum += swap32(asum);
+      amx = fmaxf(amx, __shfl_xor(amx, 16, 64));
+      amx = fmaxf(amx, swap32(amx));
+      constexpr float kCodeTop = QUANT == FDATTN_CACHE_INT8 ? 127.0f : 448.0f;
+      constexpr float u22 = 2.384185791015625e-07f, u25 = 2.9802322387695312e-08f;  // 2^-22, 2^-25
+      float bound;
+      if (DYN) {
+        // q as it is (bf16 in fp16: exact above fp16's subnormals, 2^-25 at most below; beyond fp16's range the
+        // operand saturates: then nothing is known), D products accumulated in fp32 by the matrix unit (taken at four
+        // times the textbook bound: its internal order and rounding are not documented), then one fp32 product with
+        // the key's scale - everything per unit of that scale
+        bound = kCodeTop * (asum * ((float)(D + 8) * u22 + 0.5f * u22) * 1.01f + (float)D * u25);
+        if (!(amx <= 65000.0f)) bound = INFINITY;
+      } else {
+        // q * k_scale * c as hi + lo: off by 2^-22 of itself, or 2^-25 where lo is subnormal; 2 D products accumulated
+        // in fp32 (four times the textbook bound again); the scaling by 1 / c is exact
+        bound = kCodeTop * (asum * (float)(2 * D + 9) * u22 * 1.01f + (float)D * u25 * cinv);
+      }
+      bound = live ? bound : 0.f;
+#pragma unroll
+      for (int o = 1; o < 16; o <<= 1) bound = fmaxf(bound, __shfl_xor(bound, o, 64));
+      sel_bound = bound;  // (the same in every lane of every wavefront; a NaN q leaves a NaN: every block then undecided)
+      for (int j = tid; j < a.sel_blocks_per_split; j += 64 * kWavesDt) sel_bmax[j] = (int)0x80000000, sel_smax[j] = 0u;
+    }
     for (int st = wv; st < KT; st += kWavesDt) {
       float x[8];
       scaled(st, x);
@@ -328,7 +399,7 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
   };
   auto v_operand = [&](int db) {
     const v2i r = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i*)(v_lane + 16 * db));
-    return __builtin_bit_cast(v8h, cvt8<QUANT>((u32)r.x, (u32)r.y));
+    return __builtin_bit_cast(v8h, cvt8_for_mfma<QUANT>((u32)r.x, (u32)r.y));
   };
 
   // one tile: its bytes into LDS (and, `more`, tile tn's requested), S = K Q, softmax, O += V P
@@ -339,18 +410,30 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
     if (!all_ok) {  // keys that are none count as rows of zeros: stale bytes may be fp8 NaN codes
 #pragma unroll
       for (int n = 0; n < NC; ++n)
-        if (!(okq >> n & 1u)) kq[n] = make_uint4(0u, 0u, 0u, 0u), vq[n] = make_uint4(0u, 0u, 0u, 0u);
+        if (!(okq >> n & 1u)) {
+          kq[n] = make_uint4(0u, 0u, 0u, 0u);
+          if constexpr (!SCORES) vq[n] = make_uint4(0u, 0u, 0u, 0u);
+        }
     }
 #pragma unroll
     for (int n = 0; n < NC; ++n) {
-      const u4v kw = {kq[n].x, kq[n].y, kq[n].z, kq[n].w}, vw = {vq[n].x, vq[n].y, vq[n].z, vq[n].w};
+      const u4v kw = {kq[n].x, kq[n].y, kq[n].z, kq[n].w};
       *reinterpret_cast<__attribute__((address_space(3))) u4v*>(kt + (crow + RPI * n) * L::RS + 16 * cch) = kw;
-      *reinterpret_cast<__attribute__((address_space(3))) u4v*>(vt + (crow + RPI * n) * L::RS + 16 * cch) = vw;
+      if constexpr (!SCORES) {
+        const u4v vw = {vq[n].x, vq[n].y, vq[n].z, vq[n].w};
+        *reinterpret_cast<__attribute__((address_space(3))) u4v*>(vt + (crow + RPI * n) * L::RS + 16 * cch) = vw;
+      }
     }
     if (DYN) {  // what the softmax needs of a key's scales, worked out once per tile
       const bool oks = okq >> 31 != 0;
       if (hf == 0) {
         wsc[j32] = oks ? sc * ssc : 0.f;
+        // the scoring pass: the block's largest K scale, for its error bound
+        if constexpr (SCORES) {
+          if (oks) atomicMax(sel_smax + block_of(32 * t + j32), __float_as_uint(fabsf(ssc)));
+        }
+      } else if constexpr (SCORES) {
+        wsc[32 + j32] = oks ? 0.f : -INFINITY;  // (the mask only)
       } else {
         wsc[32 + j32] = oks ? __builtin_amdgcn_logf(ssc) : -INFINITY;  // log2
         wsc[64 + j32] = oks ? __builtin_amdgcn_rcpf(ssc) : 0.f;
@@ -392,8 +475,8 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
           const uint4 wa = kw[cur][0], wb = kw[cur][1];
-          const v8h ka = __builtin_bit_cast(v8h, u ? cvt8<QUANT>(wa.z, wa.w) : cvt8<QUANT>(wa.x, wa.y));
-          const v8h kb = __builtin_bit_cast(v8h, u ? cvt8<QUANT>(wb.z, wb.w) : cvt8<QUANT>(wb.x, wb.y));
+          const v8h ka = __builtin_bit_cast(v8h, u ? cvt8_for_mfma<QUANT>(wa.z, wa.w) : cvt8_for_mfma<QUANT>(wa.x, wa.y));
+          const v8h kb = __builtin_bit_cast(v8h, u ? cvt8_for_mfma<QUANT>(wb.z, wb.w) : cvt8_for_mfma<QUANT>(wb.x, wb.y));
 #pragma unroll
           for (int term = 0; term < QT; ++term) {
             sa = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qo[cur][QT * u + term], sa, 0, 0, 0);
@@ -435,6 +518,44 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
         x[4 * half] = p4.x < lim ? x[4 * half] : -INFINITY, x[4 * half + 1] = p4.y < lim ? x[4 * half + 1] : -INFINITY;
         x[4 * half + 2] = p4.z < lim ? x[4 * half + 2] : -INFINITY, x[4 * half + 3] = p4.w < lim ? x[4 * half + 3] : -INFINITY;
       }
+    }
+    if constexpr (SCORES) {
+      // the largest score of every block the tile touches, over its keys and the live columns, into the split's LDS array
+      if (!live) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = -INFINITY;
+      }
+      auto over_columns = [&](float v) {  // the 16 lanes of a quarter hold the 16 columns
+        v = fmaxf(v, dpp_or_zero<0x128, 0xf>(v));
+        v = fmaxf(v, dpp_or_zero<0x124, 0xf>(v));
+        v = fmaxf(v, dpp_or_zero<0x122, 0xf>(v));
+        return fmaxf(v, dpp_or_zero<0x121, 0xf>(v));
+      };
+      if constexpr (TB >= 1) {  // each half of the tile (16 keys) lies inside one block
+        float ma = fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), mb = fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7]));
+        if (TB == 1) ma = fmaxf(ma, mb);
+        ma = over_columns(ma);
+        ma = fmaxf(ma, __shfl_xor(ma, 16, 64));
+        ma = fmaxf(ma, swap32(ma));
+        if (TB == 2) {
+          mb = over_columns(mb);
+          mb = fmaxf(mb, __shfl_xor(mb, 16, 64));
+          mb = fmaxf(mb, swap32(mb));
+        }
+        if (lane == 0) {
+          atomicMax(sel_bmax + block_of(32 * t), score_key(ma));
+          if (TB == 2 && 32 * t + 16 < n_x) atomicMax(sel_bmax + block_of(32 * t + 16), score_key(mb));  // (an odd number of blocks: the last tile holds one)
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float v = over_columns(x[i]);
+          const int key = i < 4 ? 4 * g4 + i : 16 + 4 * g4 + (i - 4);
+          if (c16 == 0 && 32 * t + key < n_x) atomicMax(sel_bmax + block_of(32 * t + key), score_key(v));
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+      return;
     }
     // the reference is raised when a score outgrows it by 2^13, which keeps every weight inside fp16
     float mt = -INFINITY;
@@ -480,6 +601,25 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
     advance(t + 3 * kWavesDt);
   }
 
+  if constexpr (SCORES) {
+    __syncthreads();
+    const size_t row = (size_t)pair * a.max_blocks;
+    for (int j = tid; j < i1 - i0; j += 64 * kWavesDt) {
+      const float v = key_score(sel_bmax[j]);
+      a.sel_approx[row + i0 + j] = v;
+      if (a.sel_scores_out) a.sel_scores_out[row + i0 + j] = v;
+      if (DYN) a.sel_ebound[row + i0 + j] = sel_bound * __uint_as_float(sel_smax[j]);
+    }
+    if (split == 0) {  // the blocks past the sequence's end score nothing
+      for (int j = nblk + tid; j < a.max_blocks; j += 64 * kWavesDt) {
+        a.sel_approx[row + j] = -INFINITY;
+        if (a.sel_scores_out) a.sel_scores_out[row + j] = -INFINITY;
+        if (DYN) a.sel_ebound[row + j] = 0.f;
+      }
+      if (tid == 0) a.sel_eps[pair] = DYN ? 0.f : sel_bound;
+    }
+    return;
+  }
   // ---- the four wavefronts meet: a common reference per column, o and l summed in LDS (over the tiles)
   float l_tot = l_run + __shfl_xor(l_run, 16, 64);
   l_tot += swap32(l_tot);
@@ -554,6 +694,39 @@ hipError_t launch_dt_f(const GenericDecodeArgs& a, hipStream_t s) {
   return hipSuccess;
 }
 
+template <int QUANT, bool DYN, int D, int TB>
+hipError_t launch_scores_f(const GenericDecodeArgs& a, hipStream_t s) {
+  using L = DecLay<D>;
+  const size_t shm = L::bytes(16) + (size_t)a.sel_blocks_per_split * 2 * sizeof(int);
+  static std::atomic<unsigned long long> raised{0};  // (as in launch_dt_f)
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev >= 64 || !(raised.load(std::memory_order_relaxed) >> dev & 1ull)) {
+    e = hipFuncSetAttribute((const void*)decode_tiles_kernel<QUANT, DYN, D, TB, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)(L::bytes(16) + (size_t)kSelTilesMaxBlocksPerSplit * 2 * sizeof(int)));
+    if (e != hipSuccess) return e;
+    if (dev < 64) raised.fetch_or(1ull << dev, std::memory_order_relaxed);
+  }
+  const dim3 grid((unsigned)a.batch * a.hkv, a.max_splits), block(64 * kWavesDt);
+  hipLaunchKernelGGL((decode_tiles_kernel<QUANT, DYN, D, TB, false, true>), grid, block, shm, s, a);
+  return hipSuccess;
+}
+
+template <int QUANT, bool DYN, int D>
+hipError_t launch_scores(const GenericDecodeArgs& a, hipStream_t s) {
+  const int tb = a.bs >= 32 && (a.bs & (a.bs - 1)) == 0 ? 1 : (a.bs == 16 ? 2 : 0);
+  return tb == 1 ? launch_scores_f<QUANT, DYN, D, 1>(a, s) : (tb == 2 ? launch_scores_f<QUANT, DYN, D, 2>(a, s) : launch_scores_f<QUANT, DYN, D, 0>(a, s));
+}
+
+template <int D>
+hipError_t launch_scores_d(const GenericDecodeArgs& a, int quant, hipStream_t s) {
+  if (quant == FDATTN_CACHE_INT8) return launch_scores<FDATTN_CACHE_INT8, false, D>(a, s);
+  if (quant == FDATTN_CACHE_FP8_E4M3) return launch_scores<FDATTN_CACHE_FP8_E4M3, false, D>(a, s);
+  if (quant_bytes(quant) == FDATTN_CACHE_INT8) return launch_scores<FDATTN_CACHE_INT8, true, D>(a, s);
+  return launch_scores<FDATTN_CACHE_FP8_E4M3, true, D>(a, s);
+}
+
 template <int QUANT, bool DYN, int D>
 hipError_t launch_dt(const GenericDecodeArgs& a, hipStream_t s) {
   const int tb = a.bs >= 32 && (a.bs & (a.bs - 1)) == 0 ? 1 : (a.bs == 16 ? 2 : 0);
@@ -592,6 +765,12 @@ int decode_tiles_splits(int pairs, int d, int max_keys, int most) {
   if (fill > max_keys / 256) fill = max_keys / 256;
   if (n < fill) n = fill;
   return n < 1 ? 1 : (n > most ? most : n);
+}
+
+hipError_t sqattn_scores_tiles_launch(const GenericDecodeArgs& a, int quant, hipStream_t s) {
+  if (a.d == 64) return launch_scores_d<64>(a, quant, s);
+  if (a.d == 128) return launch_scores_d<128>(a, quant, s);
+  return launch_scores_d<256>(a, quant, s);
 }
 
 hipError_t decode_tiles_launch(const GenericDecodeArgs& a, int quant, hipStream_t s) {

@@ -101,6 +101,10 @@ template <int CTRL, int ROW_MASK>
 __device__ __forceinline__ u32 dpp_or_zero(u32 v) {
   return (u32)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, 0xf, false);
 }
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_or_zero(float v) {  // (the bits travel; a float must not be converted on its way into the integer version)
+  return __uint_as_float(dpp_or_zero<CTRL, ROW_MASK>(__float_as_uint(v)));
+}
 __device__ __forceinline__ u32 wave_sum_lane63(u32 v) {
   v += dpp_or_zero<0x128, 0xf>(v);  // row_ror 8, 4, 2, 1: every lane holds its row's sum
   v += dpp_or_zero<0x124, 0xf>(v);
@@ -137,6 +141,27 @@ __device__ __forceinline__ uint4 cvt8(u32 w0, u32 w1) {
   const v2h a = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((int)w0, 1.0f, false), b = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((int)w0, 1.0f, true);
   const v2h c = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((int)w1, 1.0f, false), d = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((int)w1, 1.0f, true);
   return make_uint4(__builtin_bit_cast(u32, a), __builtin_bit_cast(u32, b), __builtin_bit_cast(u32, c), __builtin_bit_cast(u32, d));
+}
+
+// The same conversion in instructions the compiler can see (five per four int8 bytes instead of four): for results
+// that go straight into an MFMA.  The sub-dword writes above sit inside asm statements, which the compiler counts as one
+// instruction each when it spaces a register's last write from the MFMA that reads it - and the register written
+// by a statement's LAST instruction then reaches the MFMA one wait state too early (seen as one wrong element of
+// eight in the scoring pass of the block selector).  b ^ 0x80 behind the exponent byte 0x64 is the fp16 number
+// 1024 + 128 + b; a packed subtraction of 1152 leaves b.
+template <int QUANT>
+__device__ __forceinline__ uint4 cvt8_for_mfma(u32 w0, u32 w1) {
+  if (QUANT != FDATTN_CACHE_INT8) return cvt8<QUANT>(w0, w1);
+  const v2h off = {(_Float16)1152.0f, (_Float16)1152.0f};
+  u32 o[4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const u32 x = (i ? w1 : w0) ^ 0x80808080u;
+    const u32 lo = __builtin_amdgcn_perm(0x64646464u, x, 0x04010400u), hi = __builtin_amdgcn_perm(0x64646464u, x, 0x04030402u);
+    o[2 * i] = __builtin_bit_cast(u32, __builtin_bit_cast(v2h, lo) - off);
+    o[2 * i + 1] = __builtin_bit_cast(u32, __builtin_bit_cast(v2h, hi) - off);
+  }
+  return make_uint4(o[0], o[1], o[2], o[3]);
 }
 
 // Workgroup barrier that orders LDS traffic only: __syncthreads() also waits for every global load in flight

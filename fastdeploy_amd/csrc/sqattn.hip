@@ -19,6 +19,7 @@
 //    beat it whatever the errors are) or undecided; only the undecided blocks - those
 //    within 2*eps of the k-th score, a handful - are re-scored in fp64 and ranked exactly.
 #include "c8_common.h"
+#include "decode_generic.h"
 #include "launch.h"
 
 namespace fdattn {
@@ -180,6 +181,7 @@ struct SelArgs {
   // row v is token v / group, head v % group - token t of T scores the keys it attends to (T - 1 - t fewer than the
   // last token) and a block's score is the maximum over all the row's tokens and heads: one list per (row, KV head)
   int max_tokens;
+  int bs;  // block size (64 on the int8 / fp8-MFMA scoring kernel; any on the fp16-MFMA one)
 };
 
 // this step's q rows of sequence b: false if it is not a decode row; toks = its tokens (1 outside such steps)
@@ -479,7 +481,9 @@ __device__ void radix_select2_desc(const float* v, const float* e, int n, int r0
 // One workgroup per (sequence, KV head): classify, re-score the undecided blocks in fp64, emit.
 // MT: rows of several tokens (SelArgs::max_tokens > 1): the rows of the re-scoring are (token, head) pairs with their
 // own visible lengths, taken four at a time (sixteen fp64 accumulators would not fit beside the row).
-template <int QUANT, bool DYN, int NSET, bool MT = false>
+// DD: head_dim (128 behind the int8 / fp8-MFMA scoring kernel; 64, 128 or 256 behind the fp16-MFMA one); the block size is
+// a.bs.
+template <int QUANT, bool DYN, int NSET, bool MT = false, int DD = kD>
 __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs a) {
   constexpr int GH = kG * NSET;  // query heads the re-scoring loop is unrolled for (those past the group are skipped)
   extern __shared__ double smd[];                  // exact scores of undecided blocks [max_blocks]
@@ -488,7 +492,7 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
   int* state = reinterpret_cast<int*>(se + a.max_blocks);         // 0 dropped, 1 kept, 2 undecided
   int* ulist = state + a.max_blocks;                              // undecided block ids
   int* tbl = ulist + a.max_blocks;                                // this sequence's block table row
-  __shared__ float qs[GH][kD];
+  __shared__ float qs[GH][DD];
   __shared__ int few[GH];  // row g is token g / group, which sees toks - 1 - token fewer keys than the row's last token
   __shared__ int n_in, n_unc, wave_tot[kResolveThreads / 64], running;
   __shared__ __attribute__((aligned(16))) int hist[4 * 512];
@@ -513,15 +517,15 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
     se[j] = eb ? eb[j] : eps;
     tbl[j] = a.block_tables[(size_t)b * a.max_blocks + j];
   }
-  for (int i = tid; i < GH * kD; i += kResolveThreads) {
-    const int g = i / kD, c = i % kD;
+  for (int i = tid; i < GH * DD; i += kResolveThreads) {
+    const int g = i / DD, c = i % DD;
     const int tk = g / a.group, hd = g - tk * a.group;
     // rows past the pair's are zero: the re-scoring loop runs over all GH rows without a test, the maximum skips them
-    const float qv = g < vg ? bf16_to_f32(a.q[((size_t)(qrow + tk) * a.hkv * a.group + h * a.group + hd) * kD + c]) : 0.f;
-    qs[g][c] = DYN ? qv : __fmul_rn(qv, a.k_scale[h * kD + c]);
+    const float qv = g < vg ? bf16_to_f32(a.q[((size_t)(qrow + tk) * a.hkv * a.group + h * a.group + hd) * DD + c]) : 0.f;
+    qs[g][c] = DYN ? qv : __fmul_rn(qv, a.k_scale[h * DD + c]);
   }
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
-  const int nblk = min((max(kv_len, 0) + kBS - 1) / kBS, a.max_blocks);
+  const int nblk = min((max(kv_len, 0) + a.bs - 1) / a.bs, a.max_blocks);
   const int k = min(a.top_k, nblk);
   int32_t* out = a.kept_blocks + (size_t)p * a.top_k;
   if (tid == 0) { n_in = 0; n_unc = 0; running = 0; }
@@ -554,17 +558,25 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
         const int j = ulist[u];
         const int pb = tbl[j];
         double best = -INFINITY;
-        if (pb >= 0 && pb < a.num_blocks && j * kBS + lane < kv_len) {
-          const uint8_t* kr = a.key_cache + (((size_t)pb * a.hkv + h) * kBS + lane) * kD;
+        // (blocks of more than 64 tokens: 64 at a time)
+        for (int tok = lane; tok - lane < a.bs; tok += 64)
+        if (pb >= 0 && pb < a.num_blocks && tok < a.bs && j * a.bs + tok < kv_len) {
+          const uint8_t* kr = a.key_cache + (((size_t)pb * a.hkv + h) * a.bs + tok) * DD;
           // the whole row is requested before any of it is used (eight 16-byte loads in flight: one round trip to
           // memory instead of eight in a row - this loop is most of the kernel's time when a block is undecided); the
           // loop over the eight pieces stays rolled (unrolled it would not fit the registers) and picks its piece by
           // comparisons, every register index a constant
-          uint4 row[kD / 16];
+          // (head_dim 256: the row in two halves of eight pieces, requested per pass - sixteen would not fit beside the
+          // accumulators at 16 wavefronts per workgroup)
+          constexpr int RP = DD / 16 > 8 ? 8 : DD / 16, RG = DD / 16 / RP;  // pieces per group, groups per row
+          uint4 row[RP];
+          auto load_group = [&](int hg) {
 #pragma unroll
-          for (int i = 0; i < kD / 16; ++i) row[i] = *reinterpret_cast<const uint4*>(kr + 16 * i);
+            for (int i = 0; i < RP; ++i) row[i] = *reinterpret_cast<const uint4*>(kr + 16 * (RP * hg + i));
+          };
+          if (RG == 1) load_group(0);
           constexpr int GP = MT ? 4 : GH;  // rows per pass
-          const int lim = kv_len - j * kBS - lane;  // a row that sees `few` fewer keys sees this one if few < lim
+          const int lim = kv_len - j * a.bs - tok;  // a row that sees `few` fewer keys sees this one if few < lim
 #pragma unroll 1
           for (int g0 = 0; g0 < GH; g0 += GP) {
             double acc[GP];
@@ -572,26 +584,30 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
             for (int g = 0; g < GP; ++g) acc[g] = 0.0;
             // the products are exact in fp64, so fma(q, k, acc) rounds exactly like add(acc, mul(q, k))
 #pragma unroll 1
-            for (int i = 0; i < kD / 16; ++i) {
-              const int c = 16 * i;
-              u32 ws[4] = {row[0].x, row[0].y, row[0].z, row[0].w};
+            for (int hg = 0; hg < RG; ++hg) {
+              if (RG > 1) load_group(hg);
+#pragma unroll 1
+              for (int i = 0; i < RP; ++i) {
+                const int c = 16 * (RP * hg + i);
+                u32 ws[4] = {row[0].x, row[0].y, row[0].z, row[0].w};
 #pragma unroll
-              for (int j = 1; j < kD / 16; ++j) {
-                const bool pick = i == j;
-                ws[0] = pick ? row[j].x : ws[0];
-                ws[1] = pick ? row[j].y : ws[1];
-                ws[2] = pick ? row[j].z : ws[2];
-                ws[3] = pick ? row[j].w : ws[3];
-              }
+                for (int j = 1; j < RP; ++j) {
+                  const bool pick = i == j;
+                  ws[0] = pick ? row[j].x : ws[0];
+                  ws[1] = pick ? row[j].y : ws[1];
+                  ws[2] = pick ? row[j].z : ws[2];
+                  ws[3] = pick ? row[j].w : ws[3];
+                }
 #pragma unroll
-              for (int e = 0; e < 16; ++e) {
-                const double kv = dq64<QUANT>((ws[e >> 2] >> (8 * (e & 3))) & 0xff);
+                for (int e = 0; e < 16; ++e) {
+                  const double kv = dq64<QUANT>((ws[e >> 2] >> (8 * (e & 3))) & 0xff);
 #pragma unroll
-                for (int g = 0; g < GP; ++g) acc[g] = __fma_rn((double)qs[g0 + g][c + e], kv, acc[g]);
+                  for (int g = 0; g < GP; ++g) acc[g] = __fma_rn((double)qs[g0 + g][c + e], kv, acc[g]);
+                }
               }
             }
             if (DYN) {
-              const double kt = (double)a.k_scale[((size_t)pb * a.hkv + h) * a.scale_rows + (a.scale_rows == 1 ? 0 : lane)];
+              const double kt = (double)a.k_scale[((size_t)pb * a.hkv + h) * a.scale_rows + (a.scale_rows == 1 ? 0 : tok)];
 #pragma unroll
               for (int g = 0; g < GP; ++g) acc[g] = __dmul_rn(acc[g], kt);
             }
@@ -646,6 +662,12 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
   if (tid == 0) a.kept_counts[p] = k;
 }
 
+// the shapes of the fp16-MFMA scoring pass (decode_tiles.hip): head_dim 64 / 128 / 256, any block size up to 256, up to 8
+// query heads per KV head, rows of one token
+static bool sel_tiles_supported(int hq, int hkv, int d, int bs, int max_blocks) {
+  return (d == 64 || d == 128 || d == 256) && hkv > 0 && hq % hkv == 0 && hq / hkv <= kG * kMaxSets && bs >= 1 && bs <= 256 &&
+         max_blocks <= 2048;
+}
 static bool sel_fast_supported(int hq, int hkv, int d, int bs, int max_blocks) {
   return d == kD && hkv > 0 && hq % hkv == 0 && hq / hkv <= kG * kMaxSets && bs == kBS &&
          max_blocks <= 2048;  // 28 B of LDS per block in the resolve kernel
@@ -699,7 +721,7 @@ static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_ca
                seq_lens_this_time, approx, eps, cache_quant_type == FDATTN_CACHE_INT8 ? nullptr : ebound, scores,
                kept_blocks, kept_counts, batch, hkv,
                max_blocks_per_seq, num_blocks, chunk, cpp, top_k, hq / hkv, rows, scale_rows(cache_quant_type, kBS),
-               max_tokens};
+               max_tokens, kBS};
     const size_t shm2 = (size_t)max_blocks_per_seq * (sizeof(double) + 2 * sizeof(float) + 3 * sizeof(int));
     const dim3 g1(pairs * cpp), g2(pairs), b1(256), b2(kResolveThreads);
     const int sets = (hq / hkv * max_tokens + kG - 1) / kG;  // sets of four MFMA rows: (token, head) pairs
@@ -726,6 +748,52 @@ static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_ca
   }
   if (max_tokens > 1)
     return fail(FDATTN_ERR_SHAPE, "fdattn_sqattn_select: rows of several tokens need the MFMA selector's shapes");
+  if (allow_fast && sel_tiles_supported(hq, hkv, head_dim, block_size, max_blocks_per_seq)) {
+    // head_dim 64 / 128 / 256 at any block size: scores and bounds from the fp16-MFMA decode kernel's K half, then the
+    // same classification and fp64 re-scoring of the undecided blocks
+    const int pairs = batch * hkv;
+    float* approx = (float*)workspace;
+    float* ebound = approx + (size_t)pairs * max_blocks_per_seq;
+    float* eps = ebound + (size_t)pairs * max_blocks_per_seq;
+    const bool dyn = quant_dynamic(cache_quant_type);
+    long long max_keys = (long long)max_blocks_per_seq * block_size;
+    if (max_keys > 0x7fffffffLL) max_keys = 0x7fffffffLL;
+    int splits = decode_tiles_splits(pairs, head_dim, (int)max_keys, 64);
+    if (splits > max_blocks_per_seq) splits = max_blocks_per_seq;
+    const int per = (max_blocks_per_seq + splits - 1) / splits;  // <= 2048: the resolve kernel's limit on max_blocks
+    GenericDecodeArgs ga{};
+    ga.q = (const uint16_t*)q, ga.key_cache = (const uint8_t*)key_cache, ga.k_scale = cache_k_scale;
+    ga.block_tables = block_tables, ga.seq_lens_decoder = seq_lens_decoder, ga.seq_lens_this_time = seq_lens_this_time;
+    ga.rows = rows, ga.batch = batch, ga.hq = hq, ga.hkv = hkv, ga.d = head_dim, ga.bs = block_size;
+    ga.max_blocks = max_blocks_per_seq, ga.num_blocks = num_blocks, ga.max_splits = splits, ga.sm_scale = 1.0f;
+    ga.scale_rows = scale_rows(cache_quant_type, block_size), ga.max_tokens = 1;
+    ga.sel_approx = approx, ga.sel_ebound = dyn ? ebound : nullptr, ga.sel_eps = eps, ga.sel_scores_out = scores;
+    ga.sel_blocks_per_split = per;
+    const hipError_t e = sqattn_scores_tiles_launch(ga, cache_quant_type, s);
+    if (e != hipSuccess) return fail((int)e, "fdattn_sqattn_select (fp16-mfma scores): %s", hipGetErrorString(e));
+    int rc = check_launch("fdattn_sqattn_select (fp16-mfma scores)");
+    if (rc) return rc;
+    SelArgs sa{(const uint16_t*)q, (const uint8_t*)key_cache, cache_k_scale, block_tables, seq_lens_decoder,
+               seq_lens_this_time, approx, eps, dyn ? ebound : nullptr, nullptr, kept_blocks, kept_counts, batch, hkv,
+               max_blocks_per_seq, num_blocks, 0, 0, top_k, hq / hkv, rows, scale_rows(cache_quant_type, block_size), 1,
+               block_size};
+    const size_t shm2 = (size_t)max_blocks_per_seq * (sizeof(double) + 2 * sizeof(float) + 3 * sizeof(int));
+    const dim3 g2(pairs), b2(kResolveThreads);
+#define FDATTN_RES_LAUNCH(Q, DY, DD) hipLaunchKernelGGL((sqattn_resolve_kernel<Q, DY, 2, false, DD>), g2, b2, shm2, s, sa)
+#define FDATTN_RES_LAUNCH_D(Q, DY)                                     \
+  do {                                                                 \
+    if (head_dim == 64) FDATTN_RES_LAUNCH(Q, DY, 64);                  \
+    else if (head_dim == 128) FDATTN_RES_LAUNCH(Q, DY, 128);           \
+    else FDATTN_RES_LAUNCH(Q, DY, 256);                                \
+  } while (0)
+    if (cache_quant_type == FDATTN_CACHE_INT8) FDATTN_RES_LAUNCH_D(FDATTN_CACHE_INT8, false);
+    else if (cache_quant_type == FDATTN_CACHE_FP8_E4M3) FDATTN_RES_LAUNCH_D(FDATTN_CACHE_FP8_E4M3, false);
+    else if (quant_bytes(cache_quant_type) == FDATTN_CACHE_INT8) FDATTN_RES_LAUNCH_D(FDATTN_CACHE_INT8, true);
+    else FDATTN_RES_LAUNCH_D(FDATTN_CACHE_FP8_E4M3, true);
+#undef FDATTN_RES_LAUNCH_D
+#undef FDATTN_RES_LAUNCH
+    return check_launch("fdattn_sqattn_select (resolve)");
+  }
   ScoreArgs a{(const uint16_t*)q, (const uint8_t*)key_cache, cache_k_scale, block_tables, seq_lens_decoder,
               seq_lens_this_time, (double*)workspace, scores, batch, hq, hkv, head_dim, block_size,
               max_blocks_per_seq, num_blocks, scale_rows(cache_quant_type, block_size), rows};
@@ -756,6 +824,11 @@ extern "C" int fdattn_sqattn_select(const void* q, const void* key_cache, const 
   return sqattn_select_impl(true, q, key_cache, cache_k_scale, block_tables, seq_lens_decoder, seq_lens_this_time,
                             scores, kept_blocks, kept_counts, workspace, workspace_bytes, batch, hq, hkv, head_dim,
                             block_size, max_blocks_per_seq, num_blocks, top_k, cache_quant_type, stream);
+}
+
+extern "C" int fdattn_sqattn_path(int hq, int hkv, int head_dim, int block_size, int max_blocks_per_seq) {
+  if (sel_fast_supported(hq, hkv, head_dim, block_size, max_blocks_per_seq)) return 1;
+  return sel_tiles_supported(hq, hkv, head_dim, block_size, max_blocks_per_seq) ? 2 : 0;
 }
 
 extern "C" int fdattn_sqattn_select_exact(const void* q, const void* key_cache, const float* cache_k_scale,

@@ -93,6 +93,41 @@ def test_selector_other_group_sizes(oracle, group, quant):
             assert np.array_equal(np_of(kept), okept) and np.array_equal(np_of(cnt), ocnt), (k, impl)
 
 
+@pytest.mark.parametrize("quant", ALL_FORMATS)
+@pytest.mark.parametrize("hq,hkv,d,bs", [(8, 4, 64, 16), (8, 2, 64, 64), (16, 4, 128, 32), (32, 8, 128, 16), (8, 8, 128, 128),
+                                         (8, 4, 256, 64), (4, 2, 256, 8), (6, 2, 128, 24), (8, 1, 64, 48), (14, 2, 128, 256)])
+def test_selector_other_shapes_on_the_mfma_path(oracle, hq, hkv, d, bs, quant):
+    """head_dim 64 / 128 / 256 at block sizes 8 .. 256 (two that are no powers of two): block scores and bounds from the
+    fp16-MFMA decode kernel's K half, classification, fp64 re-scoring of the undecided blocks.  Kept indices bit for bit
+    as the oracle's and as the all-fp64 path's - ragged lengths with partial last blocks, planted ties (identical
+    pages: the lower index wins) - and the MFMA scores close to the fp64 ones, -inf in the same places."""
+    from fastdeploy_amd import _lib
+    assert _lib.lib().fdattn_sqattn_path(hq, hkv, d, bs, 2048) == (1 if (d, bs) == (128, 64) else 2)
+    nb = 40
+    lens = [bs * nb, bs * 17 + max(bs // 3, 1), max(bs // 2, 1), bs * 29 - 1]
+    case = syn.decode_case(batch=len(lens), ctx=lens, quant=quant, seed=d + bs + hq, salient=0.1, hq=hq, hkv=hkv, d=d, bs=bs,
+                           max_blocks=nb + 1)
+    bt = case["block_tables"]
+    for j in (6, 11):
+        case["key_cache"][int(bt[0, j])] = case["key_cache"][int(bt[0, 2])]
+        if is_dynamic(quant):
+            case["cache_k_scale"][int(bt[0, j])] = case["cache_k_scale"][int(bt[0, 2])]
+    dev = syn.to_device(case, "cuda")
+    for k in (1, 7, 16):
+        s, okept, ocnt = oracle_select(oracle, case, k)
+        for impl in ("auto", "exact"):
+            kept, cnt, sc = fd.sqattn_select(dev["q"], dev["key_cache"], dev["cache_k_scale"], dev["block_tables"],
+                                             dev["seq_lens_decoder"], num_heads=hq, top_k=k, cache_quant_type=quant, impl=impl,
+                                             return_scores=True)
+            assert np.array_equal(np_of(cnt), ocnt), (k, impl)
+            assert np.array_equal(np_of(kept), okept), (k, impl)
+            if impl == "auto":
+                got = np_of(sc).astype(np.float64)
+                fin = np.isfinite(s)
+                assert np.array_equal(np.isfinite(got), fin)
+                assert np.abs(got[fin] - s[fin]).max() <= 1e-3 * np.abs(s[fin]).max()
+
+
 def test_selector_longest_sequences_of_the_fast_path_and_beyond(oracle):
     """2048 blocks per sequence (131,072 tokens) is the most the fast path's resolve kernel holds in LDS; one block
     more goes to the all-fp64 path.  Both against the oracle."""
