@@ -415,6 +415,19 @@ def other_workloads(args):
                  t["auto"], "hbm", syn.decode_algorithmic_bytes(lens, 64, d=hd, bs=bsz), HBM_PEAK_GBPS, "GB/s",
                  {"us_on_the_vector_alu_kernel": round(t["generic"] * 1e3, 2)})
             del c, ws, out
+        # configs[3]'s selector (batch 16, 32k tokens, fp8, top-64) at two of these shapes: scores and bounds from the
+        # fp16-MFMA kernel's K half, with the all-fp64 selector beside it
+        for hd, bsz in ((128, 16), (64, 64)):
+            mb = 32768 // bsz
+            c = syn.decode_case(batch=16, ctx=32768, quant=2, seed=0, device=dev, d=hd, bs=bsz, max_blocks=mb, direct_bytes=True)
+            t = {}
+            for impl in ("auto", "exact"):
+                sel = lambda: fd.sqattn_select(c["q"], c["key_cache"], c["cache_k_scale"], c["block_tables"], c["seq_lens_decoder"],
+                                               num_heads=32, top_k=64 * 64 // bsz, cache_quant_type=2, impl=impl)
+                t[impl] = time_events(sel, max(args.steps // 4, 10), 5)
+            line("configs[3]'s selector at head_dim %d, block_size %d, top-%d of %d blocks (scores on the fp16 MFMAs)" % (hd, bsz, 64 * 64 // bsz, mb),
+                 t["auto"], "hbm", 16 * 32768 * 8 * hd, HBM_PEAK_GBPS, "GB/s", {"us_all_fp64": round(t["exact"] * 1e3, 2)})
+            del c
         # a speculative step at one of these shapes: the 64 sequences with 4 new tokens each as decode rows of four
         # tokens, head_dim 256 (16 (token, head) columns per KV head), one call: cache write + one decode pass
         from fastdeploy_amd.rope import rope_table
