@@ -75,6 +75,7 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
   using L = DecLay<D>;
   static_assert(!(SCORES && MT), "the scoring pass takes rows of one token");
   constexpr bool FAST = TB > 0;
+  constexpr bool TWO_AHEAD = SCORES && FAST;  // the scoring pass keeps two K tiles in flight per wavefront (see the walk)
   constexpr int RPB = FAST ? 32 / TB : 32;  // FAST: rows of a tile per block
   constexpr int KT = D / 32, DB = D / 16, NC = D / 32;  // k-steps of S = K Q (32 channels each); 16-channel blocks of O; 16-byte chunks per lane and tensor of a tile
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
@@ -149,9 +150,15 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
     const int x = 32 * t + r;
     if (x >= n_x) return -1;
     const int u = i0 + block_of(x);
+    if constexpr (SCORES) return u;  // (the scoring pass walks the sequence's own blocks)
     return list ? list[u] : u;
   };
   auto physical = [&](int lb) { return lb >= 0 && lb < a.max_blocks ? table[lb] : -1; };
+  // the entry of lb clamped into the table, without a branch around the load: the compiler then counts the loads in
+  // flight across it instead of waiting for all of them (the scoring pass keeps another tile's bytes in flight over
+  // this load)
+  // and whether lb is a block at all is asked when the entry is used (request): a test here would wait for the load
+  auto physical_always = [&](int lb) { return table[min(max(lb, 0), max(a.max_blocks, 1) - 1)]; };
   // cache row of key r of tile t given its blocks (false: none; row 0 of the cache is read instead, zeroed and masked later)
   auto cache_row = [&](int t, int r, int lb, int pb, u32& row, int& pos) {
     const int off = slot_of(32 * t + r);
@@ -164,8 +171,8 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
   int lb1[NB], pb1[NB], lb2[NB];  // the blocks of this lane's rows of the next tile to request (FAST: of the tile); the logical ones of the tile after
   int lbs1 = -1, pbs1 = -1, lbs2 = -1;  // DYN, not FAST: the same for the key whose scale the lane carries
   const u32 lane_off = (u32)crow * D + 16 * cch;  // FAST: this lane's chunk of the first RPI rows of a tile
-  // requests tile t's chunks given its rows' blocks (lb1 / pb1); returns the keys-that-are bits
-  auto request = [&](int t) {
+  // requests tile t's chunks into kd (and vq) given its rows' blocks lbr / pbr; returns the keys-that-are bits
+  auto request = [&](int t, uint4 (&kd)[NC], float& sd, const int (&lbr)[NB], const int (&pbr)[NB]) {
     u32 ok = 0;
     if constexpr (FAST) {
       static_assert(RPI <= RPB, "a load instruction's rows must lie inside one block");
@@ -176,9 +183,9 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
       size_t row0[TB], tile_id[TB];  // the tile's first row of block e in the caches; (block, KV head)
 #pragma unroll
       for (int e = 0; e < TB; ++e) {
-        const int lb = __builtin_amdgcn_readfirstlane(lb1[e]), pb = __builtin_amdgcn_readfirstlane(pb1[e]);
+        const int lb = __builtin_amdgcn_readfirstlane(lbr[e]), pb = __builtin_amdgcn_readfirstlane(pbr[e]);
         const int off0 = TB == 1 ? (32 * t) & (a.bs - 1) : 0;
-        blk[e] = pb >= 0 && pb < a.num_blocks;
+        blk[e] = pb >= 0 && pb < a.num_blocks && (!TWO_AHEAD || (lb >= 0 && lb < a.max_blocks));
         left[e] = (long long)kv_len - ((long long)lb * a.bs + off0);
         // (a block that is none reads block 0; rows past the sequence's end lie in the tile's block: zeroed and masked later)
         tile_id[e] = blk[e] ? (size_t)pb * a.hkv + h : 0;
@@ -193,7 +200,7 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
 #pragma unroll
       for (int n = 0; n < NC; ++n) {
         const int e = (RPI * n) / RPB, in_block = RPI * n - RPB * e;  // (constants once unrolled)
-        kq[n] = nt_load16(kp[e] + in_block * D);
+        kd[n] = nt_load16(kp[e] + in_block * D);
         if constexpr (!SCORES) vq[n] = nt_load16(vp[e] + in_block * D);
         ok |= blk[e] && crow + in_block < left[e] ? 1u << n : 0u;
       }
@@ -208,7 +215,7 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
         const bool oks = blk_e && in_block < left_e;
         ok |= oks ? 1u << 31 : 0u;
         const size_t srow = a.scale_rows == 1 ? tile_e : row0_e + in_block;
-        ssc = hf && !SCORES ? a.v_scale[srow] : a.k_scale[srow];
+        sd = hf && !SCORES ? a.v_scale[srow] : a.k_scale[srow];
       }
       return ok;
     }
@@ -216,13 +223,13 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
     for (int n = 0; n < NC; ++n) {
       u32 row;
       int pos;
-      const bool okn = cache_row(t, crow + RPI * n, lb1[n], pb1[n], row, pos);
+      const bool okn = cache_row(t, crow + RPI * n, lbr[n], pbr[n], row, pos);
       ok |= okn ? 1u << n : 0u;
       if constexpr (MT) {
         ok |= okn && pos > p0 ? kLate : 0u;
         if constexpr (!FAST) posq[n] = pos;
       }
-      kq[n] = nt_load16(a.key_cache + (size_t)row * D + 16 * cch);
+      kd[n] = nt_load16(a.key_cache + (size_t)row * D + 16 * cch);
       if constexpr (!SCORES) vq[n] = nt_load16(a.value_cache + (size_t)row * D + 16 * cch);
     }
     if (DYN) {
@@ -231,7 +238,7 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
       const bool oks = cache_row(t, j32, lbs1, pbs1, row, pos);
       ok |= oks ? 1u << 31 : 0u;
       const size_t srow = a.scale_rows == 1 ? (oks ? (size_t)pbs1 * a.hkv + h : 0) : row;  // one scale per (block, head) tile, or per stored row
-      ssc = hf && !SCORES ? a.v_scale[srow] : a.k_scale[srow];
+      sd = hf && !SCORES ? a.v_scale[srow] : a.k_scale[srow];
     }
     return ok;
   };
@@ -251,8 +258,23 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
     pb1[n] = physical(lb1[n]);
   }
   if (DYN && !FAST) lbs1 = logical(t, j32), lbs2 = logical(t + kWavesDt, j32), pbs1 = physical(lbs1);
-  if (t < n_t) okq = request(t);
+  if (t < n_t) okq = request(t, kq, ssc, lb1, pb1);
   advance(t + 2 * kWavesDt);
+  // The scoring pass has no V tile: the registers that would hold it take the wavefront's NEXT K tile, so that two
+  // tiles' bytes are in flight per wavefront as in the decode pass (fewer bytes in flight do not fill the memory
+  // pipeline).  Each of the two sets of registers has its own table entries (lb1 / pb1 and lbY / pbY), fetched a whole
+  // tile period before the request that uses them: a wait for such an entry then never waits for the other set's bytes.
+  int lbY[NB], pbY[NB];
+  u32 okq2 = 0u;
+  float ssc2 = 1.f;
+  if constexpr (TWO_AHEAD) {
+    okq2 = request(t + kWavesDt, vq, ssc2, lb1, pb1);
+#pragma unroll
+    for (int n = 0; n < NB; ++n) {
+      lb1[n] = lb2[n], pb1[n] = physical_always(lb1[n]);
+      lbY[n] = logical(t + 3 * kWavesDt, RPB * n), pbY[n] = physical_always(lbY[n]);
+    }
+  }
 
   // ---- Q as the B operand of S^T = K Q^T (v_mfma_f32_16x16x32_f16): lane = (column c16 = query head of the KV head,
   // quarter g4); k-step st holds, for quarter g4, channels 64 (st / 2) + 16 g4 + 8 (st % 2) .. + 7 - the order in
@@ -403,7 +425,7 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
   };
 
   // one tile: its bytes into LDS (and, `more`, tile tn's requested), S = K Q, softmax, O += V P
-  auto compute = [&](int tn, bool more) {
+  auto compute = [&](int t, int tn, bool more, uint4 (&kq)[NC], u32& okq, float& ssc, const int (&lbr)[NB], const int (&pbr)[NB]) {
     const u32 want = (NC >= 32 ? 0xffffffffu : (1u << NC) - 1u) | (DYN ? 1u << 31 : 0u);
     const bool all_ok = __all((okq & ~kLate) == want) != 0;  // (uniform) most tiles: every key is one
     const bool by_column = MT && toks > 1 && __any((okq & kLate) != 0u);  // (uniform) keys that some of the row's tokens do not see
@@ -451,7 +473,17 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
         wpos[crow + RPI * n] = FAST ? (first == 0x7fffffff ? first : first + in_block) : posq[FAST || !MT ? 0 : n];
       }
     }
-    if (more) okq = request(tn);
+    if constexpr (TWO_AHEAD) {
+      // The loop issues and takes the same loads in every iteration, whatever is left of the split: where two paths
+      // with different loads in flight meet, the compiler's count of them keeps the smaller one, and every wait behind
+      // the meeting point waits for too much - the other tile's bytes included.
+      int lbu[NB], pbu[NB];
+#pragma unroll
+      for (int n = 0; n < NB; ++n) lbu[n] = __builtin_amdgcn_readfirstlane(lbr[n]), pbu[n] = __builtin_amdgcn_readfirstlane(pbr[n]);
+      okq = request(tn, kq, ssc, lbu, pbu);  // (past the split's last tile: rows of block 0 that count as no keys)
+    } else {
+      if (more) okq = request(tn, kq, ssc, lbr, pbr);
+    }
     // (the wavefront's LDS instructions execute in order: what its lanes stored above is there for the reads below)
     __builtin_amdgcn_wave_barrier();
     // S^T = K Q^T for the two score tiles: two accumulators, so that an MFMA does not wait for the one before it, and
@@ -542,7 +574,7 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
           mb = fmaxf(mb, __shfl_xor(mb, 16, 64));
           mb = fmaxf(mb, swap32(mb));
         }
-        if (lane == 0) {
+        if (lane == 0 && 32 * t < n_x) {  // (the walk may compute one tile past the split's end)
           atomicMax(sel_bmax + block_of(32 * t), score_key(ma));
           if (TB == 2 && 32 * t + 16 < n_x) atomicMax(sel_bmax + block_of(32 * t + 16), score_key(mb));  // (an odd number of blocks: the last tile holds one)
         }
@@ -596,9 +628,20 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
   // ---- the walk: tile t computed; the bytes of the wavefront's next tile in flight (requested as soon as the
   // registers that receive them have been stored), the table entries of the tile after it and the list entries of the
   // one after that as well
-  for (; t < n_t; t += kWavesDt) {
-    compute(t + kWavesDt, t + kWavesDt < n_t);
-    advance(t + 3 * kWavesDt);
+  if constexpr (TWO_AHEAD) {
+    for (; t < n_t; t += 2 * kWavesDt) {
+      compute(t, t + 2 * kWavesDt, true, kq, okq, ssc, lb1, pb1);
+#pragma unroll
+      for (int n = 0; n < NB; ++n) lb1[n] = logical(t + 4 * kWavesDt, RPB * n), pb1[n] = physical_always(lb1[n]);
+      compute(t + kWavesDt, t + 3 * kWavesDt, true, vq, okq2, ssc2, lbY, pbY);  // (a tile past the end: no keys, no scores)
+#pragma unroll
+      for (int n = 0; n < NB; ++n) lbY[n] = logical(t + 5 * kWavesDt, RPB * n), pbY[n] = physical_always(lbY[n]);
+    }
+  } else {
+    for (; t < n_t; t += kWavesDt) {
+      compute(t, t + kWavesDt, t + kWavesDt < n_t, kq, okq, ssc, lb1, pb1);
+      advance(t + 3 * kWavesDt);
+    }
   }
 
   if constexpr (SCORES) {

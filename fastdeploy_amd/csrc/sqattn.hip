@@ -46,6 +46,17 @@ __device__ __forceinline__ double dq64(u32 byte) {
   if (QUANT == FDATTN_CACHE_INT8) return (double)(int)(int8_t)byte;
   return (double)e4m3_to_f32(byte);
 }
+// byte e (0 .. 3) of word w as a double.  e4m3: the code's exponent and mantissa bits land on the top of a double's
+// (a double of exponent field E: (1 + m / 8) 2^(E - 1023), or m / 8 2^-1022 for E = 0) and one exact product with
+// 2^1016 puts the value where it belongs, (1 + m / 8) 2^(E - 7) or m / 8 2^-6 - the same value as e4m3_to_f32's
+template <int QUANT>
+__device__ __forceinline__ double dq64_of_word(u32 w, int e) {
+  if (QUANT == FDATTN_CACHE_INT8) return (double)((int)(w << (24 - 8 * e)) >> 24);
+  const int sh = 17 - 8 * e;
+  const u32 mag = (sh >= 0 ? w << sh : w >> -sh) & 0x00fe0000u;
+  const u32 sgn = (w << (24 - 8 * e)) & 0x80000000u;
+  return __dmul_rn(__hiloint2double((int)(mag | sgn), 0), 0x1p1016);
+}
 
 // grid (max_blocks, hkv, batch), one wavefront: lane = token of the block
 template <int QUANT, bool DYN>
@@ -492,7 +503,7 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
   int* state = reinterpret_cast<int*>(se + a.max_blocks);         // 0 dropped, 1 kept, 2 undecided
   int* ulist = state + a.max_blocks;                              // undecided block ids
   int* tbl = ulist + a.max_blocks;                                // this sequence's block table row
-  __shared__ float qs[GH][DD];
+  __shared__ __attribute__((aligned(16))) double qs[DD][GH];  // q * k_scale as the re-scoring takes it: a channel's rows side by side
   __shared__ int few[GH];  // row g is token g / group, which sees toks - 1 - token fewer keys than the row's last token
   __shared__ int n_in, n_unc, wave_tot[kResolveThreads / 64], running;
   __shared__ __attribute__((aligned(16))) int hist[4 * 512];
@@ -522,7 +533,7 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
     const int tk = g / a.group, hd = g - tk * a.group;
     // rows past the pair's are zero: the re-scoring loop runs over all GH rows without a test, the maximum skips them
     const float qv = g < vg ? bf16_to_f32(a.q[((size_t)(qrow + tk) * a.hkv * a.group + h * a.group + hd) * DD + c]) : 0.f;
-    qs[g][c] = DYN ? qv : __fmul_rn(qv, a.k_scale[h * DD + c]);
+    qs[c][g] = (double)(DYN ? qv : __fmul_rn(qv, a.k_scale[h * DD + c]));
   }
   const int kv_len = a.seq_lens_decoder[b] + (a.seq_lens_this_time ? a.seq_lens_this_time[b] : 0);
   const int nblk = min((max(kv_len, 0) + a.bs - 1) / a.bs, a.max_blocks);
@@ -553,13 +564,19 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
     const int nu = n_unc, need = k - n_in;
     if (nu > 0) {
 
-      // exact score of each undecided block: fp64, channels in ascending order, lane = token
-      for (int u = wv; u < nu; u += kResolveThreads / 64) {
-        const int j = ulist[u];
-        const int pb = tbl[j];
+      // exact score of each undecided block: fp64, channels in ascending order, lane = token; blocks of 32 tokens or
+      // fewer (a power of two) sit side by side in a wavefront, 64 / bs of them
+      const bool side_by_side = a.bs <= 32 && (a.bs & (a.bs - 1)) == 0;
+      const int span = side_by_side ? a.bs : 64, per_wave = 64 / span;
+      const int sub = side_by_side ? lane >> (__ffs(a.bs) - 1) : 0, tok0 = lane - sub * span;
+      for (int u0 = wv * per_wave; u0 < nu; u0 += (kResolveThreads / 64) * per_wave) {
+        const int u = u0 + sub;
+        const bool have = u < nu;
+        const int j = have ? ulist[u] : 0;
+        const int pb = have ? tbl[j] : -1;
         double best = -INFINITY;
         // (blocks of more than 64 tokens: 64 at a time)
-        for (int tok = lane; tok - lane < a.bs; tok += 64)
+        for (int tok = tok0; tok - tok0 < a.bs; tok += 64)
         if (pb >= 0 && pb < a.num_blocks && tok < a.bs && j * a.bs + tok < kv_len) {
           const uint8_t* kr = a.key_cache + (((size_t)pb * a.hkv + h) * a.bs + tok) * DD;
           // the whole row is requested before any of it is used (eight 16-byte loads in flight: one round trip to
@@ -575,7 +592,7 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
             for (int i = 0; i < RP; ++i) row[i] = *reinterpret_cast<const uint4*>(kr + 16 * (RP * hg + i));
           };
           if (RG == 1) load_group(0);
-          constexpr int GP = MT ? 4 : GH;  // rows per pass
+          constexpr int GP = 4;  // rows per pass (eight accumulators would not fit beside the row at 16 wavefronts per workgroup)
           const int lim = kv_len - j * a.bs - tok;  // a row that sees `few` fewer keys sees this one if few < lim
 #pragma unroll 1
           for (int g0 = 0; g0 < GH; g0 += GP) {
@@ -600,9 +617,14 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
                 }
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                  const double kv = dq64<QUANT>((ws[e >> 2] >> (8 * (e & 3))) & 0xff);
+                  const double kv = dq64_of_word<QUANT>(ws[e >> 2], e & 3);
+                  const double2* const qrow2 = reinterpret_cast<const double2*>(&qs[c + e][g0]);  // (the same address in every lane)
 #pragma unroll
-                  for (int g = 0; g < GP; ++g) acc[g] = __fma_rn((double)qs[g0 + g][c + e], kv, acc[g]);
+                  for (int g = 0; g < GP; g += 2) {
+                    const double2 qq = qrow2[g >> 1];
+                    acc[g] = __fma_rn(qq.x, kv, acc[g]);
+                    acc[g + 1] = __fma_rn(qq.y, kv, acc[g + 1]);
+                  }
                 }
               }
             }
@@ -618,8 +640,9 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
           }
         }
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1) best = fmax(best, __shfl_xor(best, off, 64));
-        if (lane == 0) smd[u] = best;
+        for (int off = 32; off > 0; off >>= 1)
+          if (off < span) best = fmax(best, __shfl_xor(best, off, 64));
+        if (tok0 == 0 && have) smd[u] = best;
       }
       __syncthreads();
       // the `need` best undecided blocks: exact score descending, block index ascending
@@ -779,7 +802,11 @@ static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_ca
                block_size};
     const size_t shm2 = (size_t)max_blocks_per_seq * (sizeof(double) + 2 * sizeof(float) + 3 * sizeof(int));
     const dim3 g2(pairs), b2(kResolveThreads);
-#define FDATTN_RES_LAUNCH(Q, DY, DD) hipLaunchKernelGGL((sqattn_resolve_kernel<Q, DY, 2, false, DD>), g2, b2, shm2, s, sa)
+#define FDATTN_RES_LAUNCH(Q, DY, DD)                                                                      \
+  do {                                                                                                   \
+    if (hq / hkv <= kG) hipLaunchKernelGGL((sqattn_resolve_kernel<Q, DY, 1, false, DD>), g2, b2, shm2, s, sa); \
+    else hipLaunchKernelGGL((sqattn_resolve_kernel<Q, DY, 2, false, DD>), g2, b2, shm2, s, sa);          \
+  } while (0)
 #define FDATTN_RES_LAUNCH_D(Q, DY)                                     \
   do {                                                                 \
     if (head_dim == 64) FDATTN_RES_LAUNCH(Q, DY, 64);                  \
