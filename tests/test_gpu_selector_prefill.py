@@ -165,6 +165,36 @@ def test_selector_config4_shape_indices_bit_exact(oracle, quant):
     assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
 
 
+@pytest.mark.parametrize("d,bs,batch,quant", [(64, 64, 16, CACHE_FP8), (128, 16, 8, CACHE_FP8), (256, 64, 4, CACHE_FP8_DYNAMIC),
+                                              (128, 32, 4, CACHE_INT8_BLOCK)])
+def test_selector_full_size_at_the_other_shapes(oracle, d, bs, batch, quant):
+    """configs[3]'s sequences (32768 tokens, 32 query / 8 KV heads, an eighth of the blocks kept, 5 % salient blocks) at
+    head_dim 64 / 128 / 256 and block sizes 16 / 32 / 64: the fp16-MFMA scoring pass at its full launch shape (several
+    key splits per pair, 512 .. 2048 blocks per sequence), indices bit for bit as the oracle's; then the decode over
+    the kept blocks against the oracle's."""
+    from fastdeploy_amd import _lib
+    mb = 32768 // bs
+    top_k = mb // 8
+    assert _lib.lib().fdattn_sqattn_path(32, 8, d, bs, mb) == 2
+    case = syn.decode_case(batch=batch, ctx=32768, quant=quant, seed=1, device="cuda", salient=0.05, row_log2=(-6, 0), d=d, bs=bs,
+                           max_blocks=mb)
+    kept, cnt = fd.sqattn_select(case["q"], case["key_cache"], case["cache_k_scale"], case["block_tables"],
+                                 case["seq_lens_decoder"], num_heads=32, top_k=top_k, cache_quant_type=quant)
+    torch.cuda.synchronize()
+    cpu = syn.to_device(case, "cpu")
+    _, okept, ocnt = oracle_select(oracle, cpu, top_k)
+    assert np.array_equal(np_of(cnt), ocnt)
+    assert np.array_equal(np_of(kept), okept)
+    out = fd.decode_attention_sparse(case["q"], case["key_cache"], case["value_cache"], case["cache_k_scale"],
+                                     case["cache_v_scale"], case["block_tables"], case["seq_lens_decoder"],
+                                     kept_blocks=kept, kept_counts=cnt, num_heads=32, cache_quant_type=quant)
+    want = oracle.decode_attention(bits(cpu["q"]), np_of(cpu["key_cache"]), np_of(cpu["value_cache"]),
+                                   np_of(cpu["cache_k_scale"]), np_of(cpu["cache_v_scale"]), np_of(cpu["block_tables"]),
+                                   np_of(cpu["seq_lens_decoder"]), 32, 8, d, quant, kept_blocks=okept, kept_counts=ocnt)
+    ok, mx, bad = bf16_close(bits(out), want)
+    assert ok, "%d out of tolerance, max %.4g" % (bad, mx)
+
+
 def _prefill_case(seed, prefix, chunks, quant=CACHE_INT8):
     batch = len(chunks)
     # the dynamic formats: the stored rows differ in scale by up to 2^6 and reach twice unit scale (dequantised
