@@ -353,6 +353,36 @@ def test_sparse_decode(oracle, impl, quant):
     check(bits(out), oracle_decode(oracle, case, kept_blocks=kept, kept_counts=cnt), "sparse")
 
 
+@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8_DYNAMIC])
+def test_per_token_block_lists_for_the_tokens_of_one_sequence(oracle, quant):
+    """Block lists per draft TOKEN of a speculative step (the one-call step keeps one list per row): the selector and
+    the sparse decode take every token as a row of its own whose table row repeats the sequence's - rows may name the
+    same blocks, as sequences with a shared prefix do - and whose length ends at that token.  Four tokens per
+    sequence, the last of them across a block boundary; lists and outputs against the oracle's on the same rows."""
+    T, top_k = 4, 6
+    # (dynamic format: the largest rows at unit scale, where the absolute part of the output tolerance applies)
+    base = syn.decode_case(batch=3, ctx=[64 * 30 + 2, 64 * 17, 900], quant=quant, seed=21, salient=0.1, row_log2=(-6, 0))
+    lens = np_of(base["seq_lens_decoder"])
+    rows = [(b, int(lens[b]) - T + t + 1) for b in range(3) for t in range(T)]
+    g = torch.Generator().manual_seed(5)
+    case = dict(base)
+    case["q"] = torch.randn((len(rows), 32 * 128), generator=g).to(torch.bfloat16)
+    case["block_tables"] = base["block_tables"][[b for b, _ in rows]].contiguous()
+    case["seq_lens_decoder"] = torch.tensor([n for _, n in rows], dtype=torch.int32)
+    dev = syn.to_device(case, "cuda")
+    kept, cnt = fd.sqattn_select(dev["q"], dev["key_cache"], dev["cache_k_scale"], dev["block_tables"],
+                                 dev["seq_lens_decoder"], num_heads=32, top_k=top_k, cache_quant_type=quant)
+    s = oracle.sqattn_block_scores(bits(case["q"]), np_of(case["key_cache"]), np_of(case["cache_k_scale"]),
+                                   np_of(case["block_tables"]), np_of(case["seq_lens_decoder"]), 32, 8, 128, quant)
+    okept, ocnt = oracle.topk_select(s, np_of(case["seq_lens_decoder"]), 64, top_k)
+    assert np.array_equal(np_of(cnt), ocnt) and np.array_equal(np_of(kept), okept)
+    assert any(not np.array_equal(okept[i], okept[i + 1]) for i in range(T - 1))   # the tokens' lists do differ
+    out = fd.decode_attention_sparse(dev["q"], dev["key_cache"], dev["value_cache"], dev["cache_k_scale"],
+                                     dev["cache_v_scale"], dev["block_tables"], dev["seq_lens_decoder"],
+                                     kept_blocks=kept, kept_counts=cnt, num_heads=32, cache_quant_type=quant)
+    check(bits(out), oracle_decode(oracle, case, kept_blocks=okept, kept_counts=ocnt), "per-token lists")
+
+
 def test_splitkv_combine_entry_point(oracle):
     g = torch.Generator().manual_seed(0)
     po = torch.randn((37, 9, 128), generator=g)
