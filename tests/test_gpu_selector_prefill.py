@@ -128,6 +128,23 @@ def test_selector_other_shapes_on_the_mfma_path(oracle, hq, hkv, d, bs, quant):
                 assert np.abs(got[fin] - s[fin]).max() <= 1e-3 * np.abs(s[fin]).max()
 
 
+@pytest.mark.parametrize("quant", ALL_FORMATS)
+@pytest.mark.parametrize("hq,hkv,d,bs", [(8, 2, 64, 64), (32, 8, 128, 16), (8, 4, 256, 32), (4, 4, 128, 8), (16, 2, 64, 128)])
+def test_selector_other_shapes_empty_and_tiny_sequences(oracle, hq, hkv, d, bs, quant):
+    """The fp16-MFMA scoring pass on sequences of 0, 1, one block, one block and a token, and a few blocks, with top_k
+    below, at and beyond the number of blocks (a wavefront's walk then starts past its split's end, or ends one tile
+    past it): indices as the oracle's, on the MFMA path and on the all-fp64 one."""
+    lens = [0, 1, bs, bs + 1, 5 * bs - 1, 7 * bs]
+    case = syn.decode_case(batch=len(lens), ctx=lens, quant=quant, seed=3, hq=hq, hkv=hkv, d=d, bs=bs, max_blocks=9, extra_blocks=2)
+    dev = syn.to_device(case, "cuda")
+    for k in (1, 3, 100):
+        _, okept, ocnt = oracle_select(oracle, case, k)
+        for impl in ("auto", "exact"):
+            kept, cnt = fd.sqattn_select(dev["q"], dev["key_cache"], dev["cache_k_scale"], dev["block_tables"],
+                                         dev["seq_lens_decoder"], num_heads=hq, top_k=k, cache_quant_type=quant, impl=impl)
+            assert np.array_equal(np_of(cnt), ocnt) and np.array_equal(np_of(kept), okept), (k, impl)
+
+
 def test_selector_longest_sequences_of_the_fast_path_and_beyond(oracle):
     """2048 blocks per sequence (131,072 tokens) is the most the fast path's resolve kernel holds in LDS; one block
     more goes to the all-fp64 path.  Both against the oracle."""
