@@ -20,6 +20,10 @@
 //    within 2*eps of the k-th score, a handful - are re-scored in fp64 and ranked exactly.
 #include "c8_common.h"
 #include "decode_generic.h"
+#include <mutex>
+#include <set>
+#include <utility>
+
 #include "launch.h"
 
 namespace fdattn {
@@ -687,9 +691,27 @@ __global__ __launch_bounds__(kResolveThreads) void sqattn_resolve_kernel(SelArgs
 
 // the shapes of the fp16-MFMA scoring pass (decode_tiles.hip): head_dim 64 / 128 / 256, any block size up to 256, up to 8
 // query heads per KV head, rows of one token
+constexpr size_t kResolveLdsPerBlock = sizeof(double) + 2 * sizeof(float) + 3 * sizeof(int);  // the resolve kernel's dynamic LDS
+// A launch with more dynamic LDS than every kernel may have by default (64 KiB): the limit is a per-device property of
+// the kernel, raised once per device to `most`.
+static hipError_t allow_lds(const void* kernel, size_t bytes, size_t most) {
+  if (bytes <= 64 * 1024) return hipSuccess;
+  static std::mutex mu;
+  static std::set<std::pair<const void*, int>> raised;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  std::lock_guard<std::mutex> lock(mu);
+  if (raised.count({kernel, dev})) return hipSuccess;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)most);
+  if (e == hipSuccess) raised.insert({kernel, dev});
+  return e;
+}
+// (4096 blocks per sequence: 28 B of LDS per block in the resolve kernel, 112 KiB of the CU's 160)
+constexpr int kSelTilesMaxBlocks = 4096;
 static bool sel_tiles_supported(int hq, int hkv, int d, int bs, int max_blocks) {
   return (d == 64 || d == 128 || d == 256) && hkv > 0 && hq % hkv == 0 && hq / hkv <= kG * kMaxSets && bs >= 1 && bs <= 256 &&
-         max_blocks <= 2048;
+         max_blocks <= kSelTilesMaxBlocks;
 }
 static bool sel_fast_supported(int hq, int hkv, int d, int bs, int max_blocks) {
   return d == kD && hkv > 0 && hq % hkv == 0 && hq / hkv <= kG * kMaxSets && bs == kBS &&
@@ -782,8 +804,11 @@ static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_ca
     long long max_keys = (long long)max_blocks_per_seq * block_size;
     if (max_keys > 0x7fffffffLL) max_keys = 0x7fffffffLL;
     int splits = decode_tiles_splits(pairs, head_dim, (int)max_keys, 64);
+    // (a split's blocks have their maxima in the scoring workgroup's LDS: at most kSelTilesMaxBlocksPerSplit of them)
+    const int least = (max_blocks_per_seq + kSelTilesMaxBlocksPerSplit - 1) / kSelTilesMaxBlocksPerSplit;
+    if (splits < least) splits = least;
     if (splits > max_blocks_per_seq) splits = max_blocks_per_seq;
-    const int per = (max_blocks_per_seq + splits - 1) / splits;  // <= 2048: the resolve kernel's limit on max_blocks
+    const int per = (max_blocks_per_seq + splits - 1) / splits;
     GenericDecodeArgs ga{};
     ga.q = (const uint16_t*)q, ga.key_cache = (const uint8_t*)key_cache, ga.k_scale = cache_k_scale;
     ga.block_tables = block_tables, ga.seq_lens_decoder = seq_lens_decoder, ga.seq_lens_this_time = seq_lens_this_time;
@@ -800,12 +825,19 @@ static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_ca
                seq_lens_this_time, approx, eps, dyn ? ebound : nullptr, nullptr, kept_blocks, kept_counts, batch, hkv,
                max_blocks_per_seq, num_blocks, 0, 0, top_k, hq / hkv, rows, scale_rows(cache_quant_type, block_size), 1,
                block_size};
-    const size_t shm2 = (size_t)max_blocks_per_seq * (sizeof(double) + 2 * sizeof(float) + 3 * sizeof(int));
+    const size_t shm2 = (size_t)max_blocks_per_seq * kResolveLdsPerBlock;
     const dim3 g2(pairs), b2(kResolveThreads);
+#define FDATTN_RES_LAUNCH_N(Q, DY, N, DD)                                                                 \
+  do {                                                                                                   \
+    const hipError_t er = allow_lds((const void*)sqattn_resolve_kernel<Q, DY, N, false, DD>, shm2,        \
+                                    (size_t)kSelTilesMaxBlocks * kResolveLdsPerBlock);                    \
+    if (er != hipSuccess) return fail((int)er, "fdattn_sqattn_select (resolve): %s", hipGetErrorString(er)); \
+    hipLaunchKernelGGL((sqattn_resolve_kernel<Q, DY, N, false, DD>), g2, b2, shm2, s, sa);               \
+  } while (0)
 #define FDATTN_RES_LAUNCH(Q, DY, DD)                                                                      \
   do {                                                                                                   \
-    if (hq / hkv <= kG) hipLaunchKernelGGL((sqattn_resolve_kernel<Q, DY, 1, false, DD>), g2, b2, shm2, s, sa); \
-    else hipLaunchKernelGGL((sqattn_resolve_kernel<Q, DY, 2, false, DD>), g2, b2, shm2, s, sa);          \
+    if (hq / hkv <= kG) FDATTN_RES_LAUNCH_N(Q, DY, 1, DD);                                               \
+    else FDATTN_RES_LAUNCH_N(Q, DY, 2, DD);                                                              \
   } while (0)
 #define FDATTN_RES_LAUNCH_D(Q, DY)                                     \
   do {                                                                 \
@@ -819,6 +851,7 @@ static int sqattn_select_impl(bool allow_fast, const void* q, const void* key_ca
     else FDATTN_RES_LAUNCH_D(FDATTN_CACHE_FP8_E4M3, true);
 #undef FDATTN_RES_LAUNCH_D
 #undef FDATTN_RES_LAUNCH
+#undef FDATTN_RES_LAUNCH_N
     return check_launch("fdattn_sqattn_select (resolve)");
   }
   ScoreArgs a{(const uint16_t*)q, (const uint8_t*)key_cache, cache_k_scale, block_tables, seq_lens_decoder,

@@ -386,11 +386,12 @@ FDATTN_API size_t fdattn_sqattn_workspace_bytes(int batch, int hkv, int max_bloc
  * top_k highest-scoring blocks per (b,h) are kept; equal scores resolve to the
  * lower block index as in TopKIndices (fastdeploy/vision/utils/utils.h:41-60).
  *   scores      f32 [batch, hkv, max_blocks_per_seq]  (optional output, may be NULL; -inf for absent blocks).
- *               For head_dim 64, 128 or 256, hq/hkv 1 .. 8, block sizes up to 256 and at most 2048 blocks per sequence
+ *               For head_dim 64, 128 or 256, hq/hkv 1 .. 8, block sizes up to 256 and at most 4096 blocks per sequence
  *               these are the MFMA scores the selection starts from (within a small relative error of the fp64
  *               ones; blocks too close to the k-th score to call are re-scored in fp64 internally, so the kept
- *               indices are those of the fp64 scores): at head_dim 128 / block_size 64 computed on the int8 / fp8
- *               MFMAs straight from the cache bytes, elsewhere on the fp16 MFMAs (fdattn_sqattn_path says which);
+ *               indices are those of the fp64 scores): at head_dim 128 / block_size 64 with at most 2048 blocks per
+ *               sequence computed on the int8 / fp8 MFMAs straight from the cache bytes, elsewhere on the fp16 MFMAs
+ *               (fdattn_sqattn_path says which);
  *               otherwise the fp64 scores rounded to fp32.
  *   kept_blocks i32 [batch, hkv, top_k]  ascending logical block indices, -1 padded
  *   kept_counts i32 [batch, hkv]         min(top_k, ceil(kv_len / block_size))
@@ -407,8 +408,9 @@ FDATTN_API int fdattn_sqattn_select(
 
 /*
  * Which scoring pass fdattn_sqattn_select runs for a shape: 1 = the int8 / fp8 MFMAs on the cache bytes as they are
- * (head_dim 128, block_size 64), 2 = the fp16 MFMAs (head_dim 64 / 128 / 256, any block size up to 256), 0 = every
- * block in fp64 on the vector ALU (everything else).  The kept indices are the same on all three.
+ * (head_dim 128, block_size 64, at most 2048 blocks per sequence), 2 = the fp16 MFMAs (head_dim 64 / 128 / 256, any
+ * block size up to 256, at most 4096 blocks per sequence), 0 = every block in fp64 on the vector ALU (everything
+ * else).  The kept indices are the same on all three.
  */
 FDATTN_API int fdattn_sqattn_path(int hq, int hkv, int head_dim, int block_size, int max_blocks_per_seq);
 

@@ -145,10 +145,29 @@ def test_selector_other_shapes_empty_and_tiny_sequences(oracle, hq, hkv, d, bs, 
             assert np.array_equal(np_of(cnt), ocnt) and np.array_equal(np_of(kept), okept), (k, impl)
 
 
+@pytest.mark.parametrize("quant", [CACHE_FP8, CACHE_INT8_DYNAMIC])
+def test_selector_4096_blocks_of_16_tokens(oracle, quant):
+    """65,536 tokens at block_size 16: the most blocks the fp16-MFMA selector takes (two splits of 2048 blocks at least:
+    a scoring workgroup keeps a split's maxima in LDS), with a shorter sequence beside it."""
+    from fastdeploy_amd import _lib
+    assert _lib.lib().fdattn_sqattn_path(32, 8, 128, 16, 4096) == 2
+    case = syn.decode_case(batch=2, ctx=[16 * 4096, 16 * 3000 + 5], quant=quant, seed=6, device="cuda", salient=0.05, d=128, bs=16,
+                           max_blocks=4096, row_log2=(-6, 0))
+    for k in (1, 300):
+        kept, cnt = fd.sqattn_select(case["q"], case["key_cache"], case["cache_k_scale"], case["block_tables"],
+                                     case["seq_lens_decoder"], num_heads=32, top_k=k, cache_quant_type=quant)
+        torch.cuda.synchronize()
+        _, okept, ocnt = oracle_select(oracle, syn.to_device(case, "cpu"), k)
+        assert np.array_equal(np_of(cnt), ocnt) and np.array_equal(np_of(kept), okept), k
+
+
 def test_selector_longest_sequences_of_the_fast_path_and_beyond(oracle):
-    """2048 blocks per sequence (131,072 tokens) is the most the fast path's resolve kernel holds in LDS; one block
-    more goes to the all-fp64 path.  Both against the oracle."""
-    for ctx in (64 * 2048, 64 * 2049 + 5):
+    """2048 blocks per sequence (131,072 tokens) is the most the int8 / fp8-MFMA scoring pass takes; one block more goes
+    to the fp16-MFMA pass, whose resolve kernel holds 4096 blocks in LDS (262,144 tokens: the selector's limit, also
+    on the all-fp64 path).  All against the oracle."""
+    from fastdeploy_amd import _lib
+    assert [_lib.lib().fdattn_sqattn_path(32, 8, 128, 64, n) for n in (2048, 2049, 4096)] == [1, 2, 2]
+    for ctx in (64 * 2048, 64 * 2049 + 5, 64 * 4096):
         case = syn.decode_case(batch=1, ctx=ctx, quant=CACHE_INT8, seed=4, device="cuda", direct_bytes=True)
         kept, cnt = fd.sqattn_select(case["q"], case["key_cache"], case["cache_k_scale"], case["block_tables"],
                                      case["seq_lens_decoder"], num_heads=32, top_k=100, cache_quant_type=CACHE_INT8)
