@@ -816,6 +816,7 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
   int st_row3 = 0;  // chunk steps: this thread's first row of tile t + 3 in the chunk
   F16Range st_vr = {0u, 0u};  // chunk steps: the range of the V values this thread has staged of tile t + 2
   u32 st_abs = 0u, st_abs_k = 0u;  // prefix steps (per-channel formats): the magnitudes of what it has staged of tile t + 2's K, then V
+  bool take_lo = false;            // prefix steps (per-channel formats): does tile t + 1 take the second term of q * k_scale?
   auto fast_step = [&](int t, auto KB, auto CHK) {
     constexpr int kb = decltype(KB)::value;
     constexpr bool CH = decltype(CHK)::value;  // the tiles are the chunk's own keys: bf16 K against the bf16 q, one term, no scales; the softmax is masked where the wavefront's diagonal crosses the half tile
@@ -891,9 +892,9 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
     // does half tile g + 1 (whose weights this step makes) belong to a tile with large V values?  Asked now, used at the end
     const int flag_sm = (CH || DYN) ? tile_flag[((g + 1) >> 1) & 3] : 0;
     // and does half tile g + 2 (whose scores this step makes: tile t + 1) take the second term of q * k_scale?
+    // (both half tiles of tile t + 1 get the same answer: worked out in the step of the first, kept for the second)
     u4v stat_w = {0u, 0u, 0u, 0u};
-    bool take_lo = false;
-    if constexpr (!CH && !DYN) stat_w = *(const __attribute__((address_space(3))) u4v*)(tile_stat + ((t + 1) & 3) * kWavesPf);
+    if constexpr (!CH && !DYN && kb == 0) stat_w = *(const __attribute__((address_space(3))) u4v*)(tile_stat + ((t + 1) & 3) * kWavesPf);
     mfma_settle(s_sm);
     if constexpr (CH) {
       if (!unmasked(g + 1)) sm_mask(g + 1, s_sm);  // the wavefront's diagonal
@@ -943,7 +944,7 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
         if constexpr (i == 3) stage_chunk(std::integral_constant<int, 4 * kb + 1>{});
         __builtin_amdgcn_sched_barrier(0);
       });
-      if constexpr (!CH && !DYN) {  // (worked out here, long before the branch at the step's end asks for it)
+      if constexpr (!CH && !DYN && kb == 0) {  // (worked out here, long before the branch at the step's end asks for it)
         const u32 both = (stat_w[0] + stat_w[1]) + (stat_w[2] + stat_w[3]);
         const float risk = (float)(both & 0xffffu) * (float)(both >> 16) * lo_gain;
         take_lo = !(__uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(risk))) <= 1.0f);
