@@ -679,8 +679,13 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
   auto sm_pair_b = [&](auto J, SmAcc& acc, const SmCarry& c, v8h (&pp)[2]) {
     constexpr int j = decltype(J)::value;
     const float w1 = __builtin_amdgcn_exp2f(c.t1);
-    acc.ls[(2 * j) & 3] += c.w0;
-    acc.ls[(2 * j + 1) & 3] += w1;
+    if constexpr (j < 2) {  // (the four partial sums start with their first weights, not with a zero and an add)
+      acc.ls[(2 * j) & 3] = c.w0;
+      acc.ls[(2 * j + 1) & 3] = w1;
+    } else {
+      acc.ls[(2 * j) & 3] += c.w0;
+      acc.ls[(2 * j + 1) & 3] += w1;
+    }
     u4v words = __builtin_bit_cast(u4v, pp[j >> 2]);
     words[j & 3] = pack_f16(c.w0, w1);
     pp[j >> 2] = __builtin_bit_cast(v8h, words);
