@@ -145,17 +145,18 @@ def test_selector_other_shapes_empty_and_tiny_sequences(oracle, hq, hkv, d, bs, 
             assert np.array_equal(np_of(cnt), ocnt) and np.array_equal(np_of(kept), okept), (k, impl)
 
 
-@pytest.mark.parametrize("quant", [CACHE_FP8, CACHE_INT8_DYNAMIC])
-def test_selector_4096_blocks_of_16_tokens(oracle, quant):
+@pytest.mark.parametrize("quant,hq,hkv,d", [(CACHE_FP8, 32, 8, 128), (CACHE_INT8_DYNAMIC, 32, 8, 128), (CACHE_INT8, 8, 1, 256)])
+def test_selector_4096_blocks_of_16_tokens(oracle, quant, hq, hkv, d):
     """65,536 tokens at block_size 16: the most blocks the fp16-MFMA selector takes (two splits of 2048 blocks at least:
-    a scoring workgroup keeps a split's maxima in LDS), with a shorter sequence beside it."""
+    a scoring workgroup keeps a split's maxima in LDS), with a shorter sequence beside it; at head_dim 256 with eight
+    query heads per KV head the resolve kernel's LDS is at its largest."""
     from fastdeploy_amd import _lib
-    assert _lib.lib().fdattn_sqattn_path(32, 8, 128, 16, 4096) == 2
-    case = syn.decode_case(batch=2, ctx=[16 * 4096, 16 * 3000 + 5], quant=quant, seed=6, device="cuda", salient=0.05, d=128, bs=16,
-                           max_blocks=4096, row_log2=(-6, 0))
+    assert _lib.lib().fdattn_sqattn_path(hq, hkv, d, 16, 4096) == 2
+    case = syn.decode_case(batch=2, ctx=[16 * 4096, 16 * 3000 + 5], quant=quant, seed=6, device="cuda", salient=0.05, hq=hq, hkv=hkv,
+                           d=d, bs=16, max_blocks=4096, row_log2=(-6, 0))
     for k in (1, 300):
         kept, cnt = fd.sqattn_select(case["q"], case["key_cache"], case["cache_k_scale"], case["block_tables"],
-                                     case["seq_lens_decoder"], num_heads=32, top_k=k, cache_quant_type=quant)
+                                     case["seq_lens_decoder"], num_heads=hq, top_k=k, cache_quant_type=quant)
         torch.cuda.synchronize()
         _, okept, ocnt = oracle_select(oracle, syn.to_device(case, "cpu"), k)
         assert np.array_equal(np_of(cnt), ocnt) and np.array_equal(np_of(kept), okept), k
