@@ -664,7 +664,8 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
     acc.w[wi + 1] = pack_f16(e4[2], e4[3]);
     // the weight sum takes the weights before their rounding to fp16 (relative difference < 2^-12 per weight, random in
     // sign): plain adds - a dot-product instruction between MFMAs of the same wavefront stalls it for ~10 cycles
-    acc.ls[0] += e4[0], acc.ls[1] += e4[1], acc.ls[2] += e4[2], acc.ls[3] += e4[3];
+    if (piece == 0) acc.ls[0] = e4[0], acc.ls[1] = e4[1], acc.ls[2] = e4[2], acc.ls[3] = e4[3];  // (a constant where it is called: no add to a zero)
+    else acc.ls[0] += e4[0], acc.ls[1] += e4[1], acc.ls[2] += e4[2], acc.ls[3] += e4[3];
     if (piece & 1) pp[piece >> 1] = __builtin_bit_cast(v8h, make_uint4(acc.w[0], acc.w[1], acc.w[2], acc.w[3]));
   };
   // The same in units of two scores, split in two halves that fit behind one MFMA each (per-channel formats, whole
