@@ -32,8 +32,8 @@ TRAFFIC_PROFILE = "profiles/decode_c8_kernel_configs1_b64_ctx4k.md"
 TRAFFIC_PER_ALGORITHMIC_BYTE = 1.0089
 # The same profile's kernel trace holds this script's one-by-one launches too (each follows an idle queue): the median of
 # the profiler's own begin-to-end durations of those launches, as a fraction of the HBM peak over configs[1]'s bytes.
-ISOLATED_PROFILE = TRAFFIC_PROFILE + ": decode_c8_kernel launches that follow an idle queue, profiler's durations, median 83.27 us"
-ISOLATED_FRAC_PROFILED = 0.8026
+ISOLATED_PROFILE = TRAFFIC_PROFILE + ": decode_c8_kernel launches that follow an idle queue, profiler's durations, median 83.19 us"
+ISOLATED_FRAC_PROFILED = 0.8034
 
 
 def time_events(fn, steps, warmup):
