@@ -823,12 +823,14 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
   F16Range st_vr = {0u, 0u};  // chunk steps: the range of the V values this thread has staged of tile t + 2
   u32 st_abs = 0u, st_abs_k = 0u;  // prefix steps (per-channel formats): the magnitudes of what it has staged of tile t + 2's K, then V
   bool take_lo = false;            // prefix steps (per-channel formats): does tile t + 1 take the second term of q * k_scale?
+  // the LDS slots of tiles t, t + 1, t + 2 of the walk's loop, rotated as it goes (a division per step otherwise)
+  int slot_now = t0 % kSlots, slot_1 = (t0 + 1) % kSlots, slot_2 = (t0 + 2) % kSlots;
   auto fast_step = [&](int t, auto KB, auto CHK) {
     constexpr int kb = decltype(KB)::value;
     constexpr bool CH = decltype(CHK)::value;  // the tiles are the chunk's own keys: bf16 K against the bf16 q, one term, no scales; the softmax is masked where the wavefront's diagonal crosses the half tile
     constexpr bool PAIRS = !DYN || CH;
     const int g = 2 * t + kb;
-    const int slot_pv = t % kSlots, slot_qk = (t + 1) % kSlots, slot_st = (t + 2) % kSlots;
+    const int slot_pv = slot_now, slot_qk = slot_1, slot_st = slot_2;  // t % kSlots, (t + 1) % kSlots, (t + 2) % kSlots: kept by the walk
     v16f (&s_new)[2] = S[kb];
     v16f (&s_sm)[2] = S[kb ^ 1];
     lds_u16* const kd = (lds_u16*)lds + (size_t)slot_st * BUF_ELEMS + prow * LDK + pcc;
@@ -1062,7 +1064,7 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
   if (g_begin + 1 < g_end) qk(g_begin + 1, S[1]);
   if (g_begin < g_end) softmax(g_begin, !unmasked(g_begin), S[0], P);
 
-  for (int t = t0; t < t1; ++t) {
+  for (int t = t0; t < t1; ++t, slot_now = slot_1, slot_1 = slot_2, slot_2 = slot_2 == kSlots - 1 ? 0 : slot_2 + 1) {
     lds_barrier();  // tile t + 1 is in LDS; nobody reads tile t - 1 any more
     if (t + 3 < n_pre && t + 3 < t1 && 2 * t + 3 < g_end) {  // tiles t .. t + 3 are whole prefix tiles of this walk
       fast_step(t, std::integral_constant<int, 0>{}, std::false_type{});
