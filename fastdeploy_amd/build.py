@@ -91,7 +91,7 @@ def _check_register_plan():
         raise RuntimeError("hipcc -S failed on prefill_v2.hip:\n" + r.stderr)
     kernel, in_asm, worst, scratch = None, False, {}, {}
     for line in r.stdout.splitlines():
-        m = re.match(r"^(_ZN6fdattn17prefill_v2_kernelILi\d+ELb([01])EEEvNS_11PrefillArgsE):", line)
+        m = re.match(r"^(_ZN6fdattn17prefill_v2_kernelILi\d+ELb([01])ELb[01]EEEvNS_11PrefillArgsE):", line)
         if m:
             kernel, dyn = m.group(1), m.group(2) == "1"
             worst[kernel], scratch[kernel] = (-1, 64 if dyn else 32), 0
@@ -127,8 +127,8 @@ def _check_register_plan():
                                "next_free_vgpr %s; the hand-written plan needs %d and %d" %
                                (k, d.get("accum_offset"), d.get("next_free_vgpr"), PLAN_ACCUM_OFFSET,
                                 PLAN_ACCUM_OFFSET + PLAN_AGPRS))
-    if len(worst) != 4:
-        raise RuntimeError("register-plan check: expected 4 prefill_v2 kernels in the assembly, found %d" % len(worst))
+    if len(worst) != 6:
+        raise RuntimeError("register-plan check: expected 6 prefill_v2 kernels in the assembly, found %d" % len(worst))
     for k, (hi, limit) in worst.items():
         if hi >= limit or scratch[k]:
             raise RuntimeError("register-plan check failed for %s: the compiler allocated a%d (limit a%d), %d scratch "

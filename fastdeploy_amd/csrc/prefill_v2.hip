@@ -201,8 +201,10 @@ __device__ __forceinline__ int launch_splits_v2(const PrefillArgs& a, int& count
 
 }  // namespace
 
-template <int QUANT, bool DYN>
+// BLKF (with DYN): the scale caches hold one scale per (block, KV head) tile (PrefillArgs::scale_rows == 1)
+template <int QUANT, bool DYN, bool BLKF>
 __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1, 1))) void prefill_v2_kernel(PrefillArgs a) {
+  static_assert(DYN || !BLKF, "per-tile scales are scale caches");
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];  // [kSlots][K tile | V tile], then (DYN) [kSlots][3][64]: per key sc * K scale, log2(V scale), 1 / V scale
   float* const lds_sc = reinterpret_cast<float*>(lds + (size_t)kSlots * BUF_ELEMS);
   // this lane's Q lo operands of query block 1: k-step st at + 64 st
@@ -699,7 +701,9 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
   // the optimistic weights are in pp; if some query's sum over the 32 keys says that its reference was too low (or it had
   // none yet): exact maximum, raise the reference of the queries that asked for it, rescale what they have
   // accumulated, compute the weights again.  Rare: the first half tile, and scores outgrowing the reference.
-  auto sm_finish = [&](bool pre, int qb, const v16f& s, float scl, const float* scales, SmAcc& acc, v8h (&pp)[2]) {
+  // PER_TILE (per-block formats on the schedule in pairs): tile_iv = 1 / the tile's V scale - the pairs summed the
+  // weights as they are stored, V scale included, and the weight sum takes them without it
+  auto sm_finish = [&](bool pre, int qb, const v16f& s, float scl, const float* scales, SmAcc& acc, v8h (&pp)[2], auto PER_TILE, float tile_iv) {
     float tsum = (acc.ls[0] + acc.ls[1]) + (acc.ls[2] + acc.ls[3]);
     const float qsum = tsum + swap32(tsum);
     const bool redo = !(qsum <= kSumLimit) || m_ref[qb] == -INFINITY;  // also true for inf / NaN sums
@@ -727,8 +731,11 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
 #pragma unroll
       for (int piece = 0; piece < 4; ++piece) sm_piece(pre, qb, piece, s, scl, cst, scales, acc, pp);
       tsum = (acc.ls[0] + acc.ls[1]) + (acc.ls[2] + acc.ls[3]);
+      // (this pass summed the weights without their V scales itself: in the form the statement below takes)
+      if constexpr (decltype(PER_TILE)::value) tsum = ((acc.lt[0] + acc.lt[1]) + (acc.lt[2] + acc.lt[3])) / tile_iv;
     }
-    l_run[qb] += (DYN && pre) ? (acc.lt[0] + acc.lt[1]) + (acc.lt[2] + acc.lt[3]) : tsum;
+    if constexpr (decltype(PER_TILE)::value) l_run[qb] = __builtin_fmaf(tsum, tile_iv, l_run[qb]);
+    else l_run[qb] += (DYN && pre) ? (acc.lt[0] + acc.lt[1]) + (acc.lt[2] + acc.lt[3]) : tsum;
   };
   // the whole softmax of half tile g, one query block after the other
   // The second fp16 term of the weights of half tile g, p - fp16(p), into O += V P: for half tiles of tiles that hold
@@ -784,7 +791,7 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
       sm_begin(qb, acc, cst);
 #pragma unroll
       for (int piece = 0; piece < 4; ++piece) sm_piece(pre, qb, piece, s[qb], scl, cst, scales, acc, pp[qb]);
-      sm_finish(pre, qb, s[qb], scl, scales, acc, pp[qb]);
+      sm_finish(pre, qb, s[qb], scl, scales, acc, pp[qb], std::false_type{}, 0.f);
     }
     if (tile_exact(g >> 1)) sm_second_term(g, s, pp);
   };
@@ -825,10 +832,14 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
   bool take_lo = false;            // prefix steps (per-channel formats): does tile t + 1 take the second term of q * k_scale?
   // the LDS slots of tiles t, t + 1, t + 2 of the walk's loop, rotated as it goes (a division per step otherwise)
   int slot_now = t0 % kSlots, slot_1 = (t0 + 1) % kSlots, slot_2 = (t0 + 2) % kSlots;
-  auto fast_step = [&](int t, auto KB, auto CHK) {
+  auto fast_step = [&](int t, auto KB, auto CHK, auto BLKC) {
     constexpr int kb = decltype(KB)::value;
     constexpr bool CH = decltype(CHK)::value;  // the tiles are the chunk's own keys: bf16 K against the bf16 q, one term, no scales; the softmax is masked where the wavefront's diagonal crosses the half tile
-    constexpr bool PAIRS = !DYN || CH;
+    // prefix tiles of a per-block format: one K scale and one V scale per tile, so the softmax needs no per-key scales -
+    // the K scale is the step's score scale, the V scale's logarithm joins the exponent reference, and the weight sum
+    // takes the tile's sum times 1 / V scale: the schedule in pairs of the per-channel formats, with no second terms
+    constexpr bool BLK = DYN && !CH && decltype(BLKC)::value;
+    constexpr bool PAIRS = !DYN || CH || BLK;
     const int g = 2 * t + kb;
     const int slot_pv = slot_now, slot_qk = slot_1, slot_st = slot_2;  // t % kSlots, (t + 1) % kSlots, (t + 2) % kSlots: kept by the walk
     v16f (&s_new)[2] = S[kb];
@@ -907,12 +918,21 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
     if constexpr (CH) {
       if (!unmasked(g + 1)) sm_mask(g + 1, s_sm);  // the wavefront's diagonal
     }
-    const float* scales = sm_scales(g + 1);
-    const float scl[2] = {CH ? sc : scl_pre[0], CH ? sc : scl_pre[1]};
+    // (sm_scales(g + 1), from the slots the walk keeps: half tile g + 1 is the second half of tile t or the first of t + 1)
+    const float* scales = lds_sc + (kb == 0 ? slot_pv : slot_qk) * 3 * BN + HB * (kb ^ 1) + 4 * hf;
+    float scl[2] = {CH ? sc : scl_pre[0], CH ? sc : scl_pre[1]};
     SmAcc acc[2];
     float cst[2];
     sm_begin(0, acc[0], cst[0]);
     sm_begin(1, acc[1], cst[1]);
+    float tile_iv = 0.f;
+    if constexpr (BLK) {  // the scales of half tile g + 1's tile, as its keys' entries hold them (all 64 the same)
+      const float* const sct = lds_sc + (kb == 0 ? slot_pv : slot_qk) * 3 * BN;
+      scl[0] = scl[1] = sct[0];
+      const float lv = sct[BN];
+      cst[0] += lv, cst[1] += lv;
+      tile_iv = sct[2 * BN];
+    }
     // ---- O += V P (g): 8 groups of two MFMAs.  The first two V operands were requested at the end of the previous
     // fast step (va_carry); the first K operands of the second product are requested under the last
     // groups.  Groups 4 .. 7 read P[.][1] only, so the first half of softmax(g + 1), which writes P[.][0], runs there.
@@ -1030,8 +1050,8 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
       });
     }
     va_valid = true;
-    sm_finish(!CH, 0, s_sm[0], scl[0], scales, acc[0], P[0]);
-    sm_finish(!CH, 1, s_sm[1], scl[1], scales, acc[1], P[1]);
+    sm_finish(!CH, 0, s_sm[0], scl[0], scales, acc[0], P[0], std::bool_constant<BLK>{}, tile_iv);
+    sm_finish(!CH, 1, s_sm[1], scl[1], scales, acc[1], P[1], std::bool_constant<BLK>{}, tile_iv);
     if ((CH || DYN) ? __builtin_amdgcn_readfirstlane(flag_sm) == ((g + 1) >> 1) + 1 : pre_exact) sm_second_term(g + 1, s_sm, P);
     if constexpr (!CH && !DYN) {
       if (take_lo) qk_second_term(g + 2, s_new);
@@ -1067,15 +1087,15 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
   for (int t = t0; t < t1; ++t, slot_now = slot_1, slot_1 = slot_2, slot_2 = slot_2 == kSlots - 1 ? 0 : slot_2 + 1) {
     lds_barrier();  // tile t + 1 is in LDS; nobody reads tile t - 1 any more
     if (t + 3 < n_pre && t + 3 < t1 && 2 * t + 3 < g_end) {  // tiles t .. t + 3 are whole prefix tiles of this walk
-      fast_step(t, std::integral_constant<int, 0>{}, std::false_type{});
-      fast_step(t, std::integral_constant<int, 1>{}, std::false_type{});
+      fast_step(t, std::integral_constant<int, 0>{}, std::false_type{}, std::bool_constant<BLKF>{});
+      fast_step(t, std::integral_constant<int, 1>{}, std::false_type{}, std::bool_constant<BLKF>{});
       continue;
     }
     // the same schedule over the chunk's own keys, for as long as this wavefront has scores to compute two half
     // tiles ahead (up to 2 t + 3; its last tile takes the plain path below)
     if (t >= n_pre && q_is_chunk && 2 * t + 3 < g_end) {
-      fast_step(t, std::integral_constant<int, 0>{}, std::true_type{});
-      fast_step(t, std::integral_constant<int, 1>{}, std::true_type{});
+      fast_step(t, std::integral_constant<int, 0>{}, std::true_type{}, std::false_type{});
+      fast_step(t, std::integral_constant<int, 1>{}, std::true_type{}, std::false_type{});
       continue;
     }
     va_valid = false;
@@ -1229,7 +1249,7 @@ bool prefill_mfma_supported(int hq, int hkv, int d, int bs, int quant) {
 
 namespace {
 
-template <int QUANT, bool DYN>
+template <int QUANT, bool DYN, bool BLKF = false>
 hipError_t launch_v2(const PrefillArgs& a, int max_chunk, hipStream_t s) {
   PrefillArgs args = a;
   args.q_tiles = a.pack_slot > 0 ? 1 : (max_chunk + BM - 1) / BM;
@@ -1241,11 +1261,11 @@ hipError_t launch_v2(const PrefillArgs& a, int max_chunk, hipStream_t s) {
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
   if (dev >= 64 || !(raised.load(std::memory_order_relaxed) >> dev & 1ull)) {
-    e = hipFuncSetAttribute((const void*)prefill_v2_kernel<QUANT, DYN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
+    e = hipFuncSetAttribute((const void*)prefill_v2_kernel<QUANT, DYN, BLKF>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
     if (e != hipSuccess) return e;
     if (dev < 64) raised.fetch_or(1ull << dev, std::memory_order_relaxed);
   }
-  hipLaunchKernelGGL((prefill_v2_kernel<QUANT, DYN>), grid, block, kLdsBytes, s, args);
+  hipLaunchKernelGGL((prefill_v2_kernel<QUANT, DYN, BLKF>), grid, block, kLdsBytes, s, args);
   return hipSuccess;
 }
 
@@ -1292,8 +1312,10 @@ int prefill_mfma_launch(const PrefillArgs& a_in, int max_chunk, int quant, hipSt
   hipError_t e;
   if (quant == FDATTN_CACHE_INT8) e = launch_v2<FDATTN_CACHE_INT8, false>(a, max_chunk, s);
   else if (quant == FDATTN_CACHE_FP8_E4M3) e = launch_v2<FDATTN_CACHE_FP8_E4M3, false>(a, max_chunk, s);
-  else if (quant_bytes(quant) == FDATTN_CACHE_INT8) e = launch_v2<FDATTN_CACHE_INT8, true>(a, max_chunk, s);
-  else e = launch_v2<FDATTN_CACHE_FP8_E4M3, true>(a, max_chunk, s);
+  else if (quant_bytes(quant) == FDATTN_CACHE_INT8)
+    e = a.scale_rows == 1 ? launch_v2<FDATTN_CACHE_INT8, true, true>(a, max_chunk, s) : launch_v2<FDATTN_CACHE_INT8, true>(a, max_chunk, s);
+  else
+    e = a.scale_rows == 1 ? launch_v2<FDATTN_CACHE_FP8_E4M3, true, true>(a, max_chunk, s) : launch_v2<FDATTN_CACHE_FP8_E4M3, true>(a, max_chunk, s);
   if (e != hipSuccess) return fail((int)e, "fdattn_append_attention_prefill: %s", hipGetErrorString(e));
   int rc = check_launch("fdattn_append_attention_prefill (mfma)");
   if (rc || a.n_splits <= 1) return rc;
