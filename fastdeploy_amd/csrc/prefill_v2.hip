@@ -644,13 +644,22 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
   };
   // weights of 4 scores (elements 4 piece .. + 3 of query block qb): half of one P operand, partial sums into ls / lt
   struct SmAcc { float ls[4], lt[4]; u32 w[4]; };
+  struct SmScales { float4 tk, lv, iv; };
   auto sm_piece = [&](bool pre, int qb, int piece, const v16f& s, float scl, float cst, const float* scales, SmAcc& acc,
-                      v8h (&pp)[2]) {
+                      v8h (&pp)[2], SmScales* kept = nullptr) {
     float e4[4];
     if (DYN && pre) {
-      const float4 tk = *reinterpret_cast<const float4*>(scales + 8 * piece);
-      const float4 lv = *reinterpret_cast<const float4*>(scales + BN + 8 * piece);
-      const float4 iv = *reinterpret_cast<const float4*>(scales + 2 * BN + 8 * piece);
+      // (the two query blocks have the same keys: where a caller deals with a piece of block 0 and then the same piece
+      // of block 1, the second call takes the scales the first one read - `kept` - instead of reading them again)
+      float4 tk, lv, iv;
+      if (kept && qb == 1) {
+        tk = kept->tk, lv = kept->lv, iv = kept->iv;
+      } else {
+        tk = *reinterpret_cast<const float4*>(scales + 8 * piece);
+        lv = *reinterpret_cast<const float4*>(scales + BN + 8 * piece);
+        iv = *reinterpret_cast<const float4*>(scales + 2 * BN + 8 * piece);
+        if (kept) kept->tk = tk, kept->lv = lv, kept->iv = iv;
+      }
       const float tks[4] = {tk.x, tk.y, tk.z, tk.w}, lvs[4] = {lv.x, lv.y, lv.z, lv.w}, ivs[4] = {iv.x, iv.y, iv.z, iv.w};
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -1002,6 +1011,7 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
         __builtin_amdgcn_sched_barrier(0);
       });
     } else {
+      SmScales piece_scales;  // a piece's scales, read for query block 0 and kept for block 1
     static_for<8>([&](auto I) {
         constexpr int i = decltype(I)::value;
         if constexpr (i + VD < 8) va[(i + VD) % (VD + 1)] = v_operand(slot_pv, kb, (i + VD) >> 2, (i + VD) & 3);
@@ -1015,7 +1025,7 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
         if constexpr (i == 3) stage_chunk(std::integral_constant<int, 4 * kb + 1>{});
         if constexpr (i >= 4) {
           constexpr int qb = i & 1, piece = (i - 4) >> 1;
-          sm_piece(true, qb, piece, s_sm[qb], scl_pre[qb], cst[qb], scales, acc[qb], P[qb]);
+          sm_piece(true, qb, piece, s_sm[qb], scl_pre[qb], cst[qb], scales, acc[qb], P[qb], &piece_scales);
         }
         __builtin_amdgcn_sched_barrier(0);
       });
@@ -1042,7 +1052,7 @@ __global__ __launch_bounds__(64 * kWavesPf) __attribute__((amdgpu_waves_per_eu(1
         }
         if constexpr (st < 4) {
           constexpr int qb = st & 1, piece = 2 + (st >> 1);
-          sm_piece(true, qb, piece, s_sm[qb], scl_pre[qb], cst[qb], scales, acc[qb], P[qb]);
+          sm_piece(true, qb, piece, s_sm[qb], scl_pre[qb], cst[qb], scales, acc[qb], P[qb], &piece_scales);
         }
         if constexpr (st == 4) stage_chunk(std::integral_constant<int, 4 * kb + 2>{});
         if constexpr (st == 6) stage_chunk(std::integral_constant<int, 4 * kb + 3>{});
