@@ -455,10 +455,32 @@ __device__ void radix_select2_desc(const float* v, const float* e, int n, int r0
   for (int pass = 0; pass < 4; ++pass) {
     const int shift = 24 - 8 * pass;
     int* hp = hist + 512 * pass;
-    for (int j = tid; j < n; j += kResolveThreads) {
-      const unsigned k0 = order_key(v[j] - e[j]), k1 = order_key(v[j] + e[j]);
-      if ((k0 & mask) == prefix[0]) atomicAdd(&hp[(k0 >> shift) & 255u], 1);
-      if ((k1 & mask) == prefix[1]) atomicAdd(&hp[256 + ((k1 >> shift) & 255u)], 1);
+    if (pass == 0) {
+      // The first digit is the sign and the top of the exponent: scores of one pair share it, and 64 lanes adding to
+      // one LDS word take their turns.  A wavefront adds once per distinct digit instead (one or two rounds).
+      for (int j0 = 0; j0 < n; j0 += kResolveThreads) {  // (every lane of a wavefront stays in the loop: ballots)
+        const int j = j0 + tid;
+        const bool in = j < n;
+        const unsigned k0 = in ? order_key(v[j] - e[j]) : 0u, k1 = in ? order_key(v[j] + e[j]) : 0u;
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+          const unsigned bin = ((w ? k1 : k0) >> shift) & 255u;
+          unsigned long long todo = __ballot(in);
+          while (todo) {
+            const int leader = __ffsll((long long)todo) - 1;
+            const unsigned b = (unsigned)__shfl((int)bin, leader, 64);
+            const unsigned long long same = __ballot(in && bin == b);
+            if (lane == leader) atomicAdd(&hp[256 * w + b], (int)__popcll(same));
+            todo &= ~same;
+          }
+        }
+      }
+    } else {
+      for (int j = tid; j < n; j += kResolveThreads) {
+        const unsigned k0 = order_key(v[j] - e[j]), k1 = order_key(v[j] + e[j]);
+        if ((k0 & mask) == prefix[0]) atomicAdd(&hp[(k0 >> shift) & 255u], 1);
+        if ((k1 & mask) == prefix[1]) atomicAdd(&hp[256 + ((k1 >> shift) & 255u)], 1);
+      }
     }
     __syncthreads();
     if (wv < 2) {
