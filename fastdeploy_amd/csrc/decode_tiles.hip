@@ -450,9 +450,19 @@ __global__ __launch_bounds__(64 * kWavesDt, waves_per_simd<D>()) void decode_til
       const bool oks = okq >> 31 != 0;
       if (hf == 0) {
         wsc[j32] = oks ? sc * ssc : 0.f;
-        // the scoring pass: the block's largest K scale, for its error bound
+        // the scoring pass: the block's largest K scale, for its error bound (a tile inside one or two blocks: the 16
+        // lanes of a row agree on the block, so the row's maximum goes there once - 32 lanes on one LDS word take turns)
         if constexpr (SCORES) {
-          if (oks) atomicMax(sel_smax + block_of(32 * t + j32), __float_as_uint(fabsf(ssc)));
+          u32 big = oks ? __float_as_uint(fabsf(ssc)) : 0u;
+          if constexpr (TB >= 1) {
+            big = max(big, dpp_or_zero<0x128, 0xf>(big));
+            big = max(big, dpp_or_zero<0x124, 0xf>(big));
+            big = max(big, dpp_or_zero<0x122, 0xf>(big));
+            big = max(big, dpp_or_zero<0x121, 0xf>(big));
+            if ((j32 & 15) == 0 && big != 0u) atomicMax(sel_smax + block_of(32 * t + j32), big);
+          } else {
+            if (oks) atomicMax(sel_smax + block_of(32 * t + j32), big);
+          }
         }
       } else if constexpr (SCORES) {
         wsc[32 + j32] = oks ? 0.f : -INFINITY;  // (the mask only)
