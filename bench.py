@@ -304,6 +304,18 @@ def other_workloads(args):
         ms = time_events(lambda: spec(twos, max_chunk=2), args.steps, 30)
         line("the same step as prefill rows of two tokens (write + packed append attention)", ms, "hbm", nbytes,
              HBM_PEAK_GBPS, "GB/s")
+        # the rows of two tokens block-sparse (16 of their ~64 blocks kept): one list per row, scored by both tokens in
+        # one pass over K, then a list per token (selector and sparse decode over tokens as rows: K is streamed per token)
+        sparse_bytes = sum(lens) * 8 * 128 + 64 * 8 * 16 * 64 * 128 * 2
+        for per_token in (False, True):
+            swsx = fd.append_attention_workspace(128, 128 if per_token else 64, 32, 8, 128, 72, dev)
+            ms = time_events(lambda: fd.append_attention(qkv, c["key_cache"], c["value_cache"], zeros, cached, twos,
+                                                         c["block_tables"], rot, c["cache_k_scale"], c["cache_v_scale"],
+                                                         num_heads=32, kv_num_heads=8, cu_seqlens_q=cu, workspace=swsx,
+                                                         out=sout, max_chunk=0, decode_tokens=2, sqattn_top_k=16,
+                                                         sqattn_per_token=per_token), args.steps, args.warmup)
+            line("speculative step, 64 x 2 tokens on ctx ~4k, block-sparse (16 blocks kept per KV head): %s"
+                 % ("a list per token" if per_token else "one list per row"), ms, "hbm", sparse_bytes, HBM_PEAK_GBPS, "GB/s")
         # the same sequences with 4 tokens each (16 (token, head) pairs per KV head: the step hands such rows to the
         # fp16-MFMA decode kernel, whose 16 columns they fill)
         qkv4 = torch.randn((256, 48 * 128), generator=g, device=dev).to(torch.bfloat16)

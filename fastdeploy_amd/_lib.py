@@ -60,7 +60,7 @@ SIGNATURES = {
 class StepExtras(ctypes.Structure):
     """fdattn_step_extras of include/fdattn.h"""
     _fields_ = [("qkv_bias", _vp), ("q_norm_weight", _vp), ("k_norm_weight", _vp), ("rms_norm_eps", _f),
-                ("prefill_rows", _i), ("sqattn_top_k", _i), ("decode_tokens", _i)]
+                ("prefill_rows", _i), ("sqattn_top_k", _i), ("decode_tokens", _i), ("sqattn_per_token", _i)]
 
 
 _lib = None

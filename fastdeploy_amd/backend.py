@@ -50,7 +50,7 @@ class ForwardMeta:
 class AppendAttentionBackend:
     def __init__(self, num_heads, kv_num_heads, head_dim, *, block_size=64, max_position=8192, rope_theta=10000.0,
                  rope_style="neox", cache_quant_type="cache_int8", softmax_scale=None, device="cuda",
-                 sqattn_top_k=None):
+                 sqattn_top_k=None, sqattn_per_token=False):
         from .rope import rope_table
         if num_heads % kv_num_heads:
             raise ValueError("num_heads %d is not a multiple of kv_num_heads %d" % (num_heads, kv_num_heads))
@@ -58,6 +58,8 @@ class AppendAttentionBackend:
         self.block_size, self.rope_style, self.cache_quant_type = block_size, rope_style, cache_quant_type
         self.softmax_scale = softmax_scale
         self.sqattn_top_k = sqattn_top_k   # > 0: decode rows attend to their top-k blocks only (block-sparse)
+        # block-sparse decode rows of several tokens: one list per row (False) or one per token (True)
+        self.sqattn_per_token = bool(sqattn_per_token)
         self.device = device
         self.rotary_embs = rope_table(max_position, head_dim, rope_theta, device)
         self._workspace = None
@@ -105,7 +107,8 @@ class AppendAttentionBackend:
             raise ValueError("a sequence reaches %d tokens in this step, the rotation table holds %d positions "
                              "(max_position)" % (meta.max_len_after, self.rotary_embs[0].shape[0]))
         meta.cu_seqlens_q = ops.cu_seqlens_of(this)
-        if meta.decode_tokens > 1:
+        per_token = self.sqattn_per_token and (self.sqattn_top_k or 0) > 0 and meta.decode_tokens > 1
+        if meta.decode_tokens > 1 and not per_token:
             group = self.num_heads // self.kv_num_heads
             if meta.decode_tokens * group > 16 or self.head_dim not in (64, 128, 256):
                 raise ValueError("decode rows of %d tokens need head_dim 64, 128 or 256 and tokens x heads per KV head "
@@ -121,7 +124,8 @@ class AppendAttentionBackend:
         if meta.prefill_rows and meta.max_enc_len_this_time > 0:
             meta.prefill_splits = ops.prefill_auto_splits(meta.prefill_rows, self.num_heads, meta.max_enc_len_this_time,
                                                            self.kv_num_heads)
-        need = ops.append_attention_workspace_bytes(meta.num_tokens, slots, self.num_heads, self.kv_num_heads,
+        need = ops.append_attention_workspace_bytes(meta.num_tokens, slots * meta.decode_tokens if per_token else slots,
+                                                    self.num_heads, self.kv_num_heads,
                                                     self.head_dim, meta.block_tables.shape[1], meta.prefill_splits)
         if self._workspace is None or self._workspace.numel() < need:
             self._workspace = torch.empty(need, dtype=torch.uint8, device=self.device)
@@ -141,7 +145,8 @@ class AppendAttentionBackend:
             rope_style=self.rope_style, cache_quant_type=self.cache_quant_type, softmax_scale=self.softmax_scale,
             cu_seqlens_q=meta.cu_seqlens_q, workspace=self._workspace, out=out, qkv_bias=layer.qkv_bias,
             q_norm_weight=layer.q_norm_weight, k_norm_weight=layer.k_norm_weight, rms_norm_eps=layer.rms_norm_eps,
-            prefill_rows=meta.prefill_rows, sqattn_top_k=self.sqattn_top_k, decode_tokens=meta.decode_tokens)
+            prefill_rows=meta.prefill_rows, sqattn_top_k=self.sqattn_top_k, decode_tokens=meta.decode_tokens,
+            sqattn_per_token=self.sqattn_per_token)
 
 
 class SequenceBook:

@@ -10,8 +10,35 @@ namespace fdattn {
 static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 
 struct StepWorkspace {
-  size_t q_rot, k_new, v_new, decode, select, kept, split, total;  // byte offsets of the parts, and the sum
+  size_t q_rot, k_new, v_new, decode, select, kept, split, view, total;  // byte offsets of the parts, and the sum
 };
+
+// The arrays of the token-as-row view of a step (fdattn_step_extras.sqattn_per_token): per view row a table row, then
+// cu_seqlens_q (rows + 1), seq_lens_encoder, seq_lens_decoder and seq_lens_this_time of the view.
+static size_t view_bytes(int rows, int max_blocks) { return ((size_t)rows * ((size_t)max_blocks + 4) + 1) * sizeof(int32_t); }
+
+// Every token of a decode row as a row of its own: view row r = sequence r / T, token r % T.  Its table row repeats the
+// sequence's, its cached length ends in front of that token and it brings one token, so the kernels behind see the
+// step's decode tokens as so many decode rows of one token - which is what "every token selects its own blocks" means.
+// Rows of tokens that a sequence does not have, and the rows of sequences that are no decode rows of this step, carry
+// seq_lens_encoder 1: the decode-side kernels pass them over.
+__global__ __launch_bounds__(256) void rows_per_token_kernel(const int32_t* cu, const int32_t* enc, const int32_t* dec,
+                                                             const int32_t* tables, int batch, int T, int max_blocks,
+                                                             int32_t* tables_v, int32_t* cu_v, int32_t* enc_v,
+                                                             int32_t* dec_v, int32_t* this_v) {
+  const int r = blockIdx.x, b = r / T, j = r - b * T;
+  const int c0 = cu[b], n = cu[b + 1] - c0;
+  const bool valid = enc[b] == 0 && j < n && n <= T;
+  if (threadIdx.x == 0) {
+    cu_v[r] = c0 + min(j, n);
+    if (r == 0) cu_v[batch * T] = cu[batch];
+    enc_v[r] = valid ? 0 : 1;
+    dec_v[r] = dec[b] + j;
+    this_v[r] = 1;
+  }
+  for (int i = threadIdx.x; i < max_blocks; i += 256)
+    tables_v[(size_t)r * max_blocks + i] = valid ? tables[(size_t)b * max_blocks + i] : -1;
+}
 
 static StepWorkspace step_workspace(int num_tokens, int batch, int hq, int hkv, int d, int max_blocks, int prefill_splits) {
   StepWorkspace w;
@@ -29,7 +56,8 @@ static StepWorkspace step_workspace(int num_tokens, int batch, int hq, int hkv, 
   w.select = w.decode + align256(dec);
   w.kept = w.select + align256(fdattn_sqattn_workspace_bytes(batch, hkv, max_blocks));
   w.split = w.kept + align256((size_t)batch * hkv * ((size_t)max_blocks + 1) * sizeof(int32_t));
-  w.total = w.split + align256(prefill_split_workspace_bytes(num_tokens, hq, prefill_splits));
+  w.view = w.split + align256(prefill_split_workspace_bytes(num_tokens, hq, prefill_splits));
+  w.total = w.view + align256(view_bytes(batch, max_blocks));
   return w;
 }
 
@@ -82,28 +110,34 @@ extern "C" int fdattn_append_attention_ex(
   // laid out for the most)
   const int prefill_rows = extras && extras->prefill_rows > 0 ? extras->prefill_rows : 0;
   int splits = max_chunk > 0 ? prefill_auto_splits(prefill_rows > 0 ? prefill_rows : 1, hq, max_chunk, hkv) : 1;
-  StepWorkspace w = step_workspace(num_tokens, batch, hq, hkv, head_dim, max_blocks_per_seq, splits);
-  while (splits > 1 && workspace_bytes < w.total)  // a workspace sized for fewer splits: use as many as it holds
-    w = step_workspace(num_tokens, batch, hq, hkv, head_dim, max_blocks_per_seq, --splits);
-  if (workspace_bytes < w.total)
-    return fail(FDATTN_ERR_WORKSPACE, "fdattn_append_attention: workspace %zu B < required %zu B", workspace_bytes,
-                w.total);
-  // what the decode rows ask for, checked before anything is written
   const int top_k = extras && extras->sqattn_top_k > 0 ? (extras->sqattn_top_k < max_blocks_per_seq ? extras->sqattn_top_k : max_blocks_per_seq) : 0;
   const int decode_tokens = extras && extras->decode_tokens > 1 ? extras->decode_tokens : 1;
+  // every token of a decode row with a block list of its own: the decode side of the step runs over the token-as-row
+  // view, whose batch is what the workspace must be sized for
+  const bool per_token = top_k > 0 && decode_tokens > 1 && extras->sqattn_per_token != 0;
+  if (per_token && (long long)batch * decode_tokens > 0x7fffffffLL / 64)
+    return fail(FDATTN_ERR_SHAPE, "fdattn_append_attention: batch %d x decode_tokens %d is too large", batch, decode_tokens);
+  const int dbatch = per_token ? batch * decode_tokens : batch;
+  StepWorkspace w = step_workspace(num_tokens, dbatch, hq, hkv, head_dim, max_blocks_per_seq, splits);
+  while (splits > 1 && workspace_bytes < w.total)  // a workspace sized for fewer splits: use as many as it holds
+    w = step_workspace(num_tokens, dbatch, hq, hkv, head_dim, max_blocks_per_seq, --splits);
+  if (workspace_bytes < w.total)
+    return fail(FDATTN_ERR_WORKSPACE, "fdattn_append_attention: workspace %zu B < required %zu B%s", workspace_bytes,
+                w.total, per_token ? " (sqattn_per_token: size it for batch x decode_tokens sequences)" : "");
+  // what the decode rows ask for, checked before anything is written
   const bool c8 = c8_supported(hq, hkv, head_dim, block_size, cache_quant_type);
-  if (decode_tokens > 1 && ((!c8 && !decode_tiles_supported(hq, hkv, head_dim)) || hq % hkv != 0 ||
-                            decode_tokens * (hq / hkv) > 16))
+  if (decode_tokens > 1 && !per_token && ((!c8 && !decode_tiles_supported(hq, hkv, head_dim)) || hq % hkv != 0 ||
+                                          decode_tokens * (hq / hkv) > 16))
     return fail(FDATTN_ERR_SHAPE, "fdattn_append_attention: decode_tokens %d needs head_dim 64, 128 or 256 and "
                 "decode_tokens x query heads per KV head <= 16", decode_tokens);
   // block-sparse decode rows: the MFMA selector and the int8-MFMA kernel at their shapes; elsewhere the exact (fp64)
   // selector and the kernels of the other shapes, for rows of one token
   const bool sel_fast = c8 && sqattn_fast_supported(hq, hkv, head_dim, block_size, max_blocks_per_seq);
-  if (top_k > 0 && !sel_fast && (decode_tokens > 1 || hq % hkv != 0 || hq / hkv > 8 || head_dim > 256 || head_dim % 4 != 0 ||
+  if (top_k > 0 && !sel_fast && ((decode_tokens > 1 && !per_token) || hq % hkv != 0 || hq / hkv > 8 || head_dim > 256 || head_dim % 4 != 0 ||
                                  max_blocks_per_seq > 4096))
     return fail(FDATTN_ERR_SHAPE, "fdattn_append_attention: sqattn_top_k needs at most 8 query heads per KV head, head_dim "
-                "<= 256 and at most 4096 blocks per sequence (with decode_tokens: head_dim 128, block_size 64, at most 2048 "
-                "blocks)");
+                "<= 256 and at most 4096 blocks per sequence (with decode_tokens and one list per row: head_dim 128, "
+                "block_size 64, at most 2048 blocks)");
   char* ws = (char*)workspace;
   void* q_rot = ws + w.q_rot;
   const bool any_prefill = max_chunk > 0;  // the caller's word: 0 = no sequence has seq_lens_encoder > 0
@@ -121,6 +155,34 @@ extern "C" int fdattn_append_attention_ex(
   hipStream_t s = (hipStream_t)stream;
   if (prefill_rows >= batch) {
     // the caller's count says that every sequence is a prefill row: no decode pass
+  } else if (per_token) {
+    // block-sparse decode rows of several tokens, every token with its own list: selector and sparse decode over the
+    // token-as-row view (rows of one token; the kernels and their shapes are those of the case below)
+    int32_t* tables_v = (int32_t*)(ws + w.view);
+    int32_t* cu_v = tables_v + (size_t)dbatch * max_blocks_per_seq;
+    int32_t* enc_v = cu_v + dbatch + 1;
+    int32_t* dec_v = enc_v + dbatch;
+    int32_t* this_v = dec_v + dbatch;
+    hipLaunchKernelGGL(rows_per_token_kernel, dim3((unsigned)dbatch), dim3(256), 0, s, cu_seqlens_q, seq_lens_encoder,
+                       seq_lens_decoder, block_tables, batch, decode_tokens, max_blocks_per_seq, tables_v, cu_v, enc_v,
+                       dec_v, this_v);
+    rc = check_launch("fdattn_append_attention (token-as-row view)");
+    if (rc) return rc;
+    const RowMap vrows{cu_v, enc_v};
+    int32_t* kept = (int32_t*)(ws + w.kept);
+    int32_t* counts = kept + (size_t)dbatch * hkv * top_k;
+    rc = sqattn_select_launch(q_rot, key_cache, cache_k_scale, tables_v, dec_v, this_v, kept, counts, ws + w.select,
+                              w.kept - w.select, dbatch, hq, hkv, head_dim, block_size, max_blocks_per_seq, num_blocks,
+                              top_k, cache_quant_type, s, vrows, 1);
+    if (rc) return rc;
+    if (sel_fast)
+      rc = decode_c8_launch(q_rot, key_cache, value_cache, cache_k_scale, cache_v_scale, tables_v, dec_v, this_v, kept,
+                            counts, top_k, out, ws + w.decode, dws, dbatch, hq, hkv, head_dim, block_size,
+                            max_blocks_per_seq, num_blocks, cache_quant_type, softmax_scale, s, 3, vrows, 1);
+    else
+      rc = decode_generic_launch(q_rot, key_cache, value_cache, cache_k_scale, cache_v_scale, tables_v, dec_v, this_v,
+                                 kept, counts, top_k, out, ws + w.decode, dws, dbatch, hq, hkv, head_dim, block_size,
+                                 max_blocks_per_seq, num_blocks, cache_quant_type, softmax_scale, s, vrows);
   } else if (top_k > 0) {
     // block-sparse decode rows: select with the new query over the cache as the writer left it, then attend to
     // the kept blocks only (a row of several tokens: one list, scored by all of them)

@@ -120,7 +120,7 @@ def _scales(cache_k_scale, cache_v_scale, hkv, d, quant=CACHE_INT8, nb=0, bs=0):
 
 
 def _extras(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, width, d, prefill_rows=0, sqattn_top_k=0,
-            decode_tokens=0):
+            decode_tokens=0, sqattn_per_token=False):
     """fdattn_step_extras for the optional projection epilogue / prefill splits / block-sparse decode rows / decode
     rows of several tokens, or None"""
     if (qkv_bias is None and q_norm_weight is None and k_norm_weight is None and prefill_rows <= 0
@@ -135,7 +135,7 @@ def _extras(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, width, d, pref
         if t is not None and t.numel() != d:
             raise ValueError("%s has %d entries, head_dim is %d" % (name, t.numel(), d))
     return _lib.StepExtras(pb or None, pq or None, pk or None, float(rms_norm_eps), int(prefill_rows), int(sqattn_top_k),
-                           int(decode_tokens))
+                           int(decode_tokens), 1 if sqattn_per_token else 0)
 
 
 def prefill_auto_splits(rows, num_heads, max_chunk, kv_num_heads=None):
@@ -462,7 +462,7 @@ def append_attention(qkv, key_cache, value_cache, seq_lens_encoder, seq_lens_dec
                      max_chunk, rope_style="neox", cache_quant_type="cache_int8", softmax_scale=None,
                      cu_seqlens_q=None, workspace=None, out=None, qkv_bias=None, q_norm_weight=None,
                      k_norm_weight=None, rms_norm_eps=1e-6, prefill_rows=None, sqattn_top_k=None,
-                     decode_tokens=None):
+                     decode_tokens=None, sqattn_per_token=False):
     """One attention step of a layer over a mixed batch (one call into the library):
     every new token is rotated and written to the cache, decode rows (one token,
     seq_lens_encoder == 0) attend to the cache, prefill rows (seq_lens_encoder > 0)
@@ -482,6 +482,9 @@ def append_attention(qkv, key_cache, value_cache, seq_lens_encoder, seq_lens_dec
     token t attends to the cached tokens and the new ones up to itself, all read from the cache, in one decode pass
     (head_dim 64 / 128 / 256, decode_tokens x heads per KV head <= 16).  With sqattn_top_k such a row keeps one
     list of blocks per KV head, scored by all its tokens (the maximum over tokens and heads).
+    sqattn_per_token: with sqattn_top_k and decode_tokens, every token of a decode row keeps a list of its own, scored
+    with its own query over the keys it attends to (the step then runs its decode side over batch x decode_tokens
+    rows of one token; a workspace passed in must be sized for that many sequences).
     Returns bf16 [num_tokens, num_heads*head_dim]."""
     nb, hkv, bs, d = _cache_dims(key_cache, value_cache)
     if hkv != kv_num_heads:
@@ -527,12 +530,14 @@ def append_attention(qkv, key_cache, value_cache, seq_lens_encoder, seq_lens_dec
         raise ValueError("out holds %d values, the step writes num_tokens*num_heads*head_dim = %d"
                          % (out.numel(), T * num_heads * d))
     splits = prefill_auto_splits(prefill_rows or 1, num_heads, max_chunk, hkv) if max_chunk > 0 else 1
-    need = _lib.lib().fdattn_append_attention_workspace_bytes_ex(T, batch, num_heads, hkv, d, mb, splits)
+    per_token = bool(sqattn_per_token) and (sqattn_top_k or 0) > 0 and (decode_tokens or 0) > 1
+    need = _lib.lib().fdattn_append_attention_workspace_bytes_ex(T, batch * decode_tokens if per_token else batch,
+                                                                 num_heads, hkv, d, mb, splits)
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=qkv.device)
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(d)
     ep = _extras(qkv_bias, q_norm_weight, k_norm_weight, rms_norm_eps, qkv.shape[1], d, prefill_rows or 0,
-                 sqattn_top_k or 0, decode_tokens or 0)
+                 sqattn_top_k or 0, decode_tokens or 0, per_token)
     rc = _lib.lib().fdattn_append_attention_ex(
         p_qkv, p_kc, p_vc, p_ks, p_vs, p_cos, p_sin, p_bt, p_enc, p_dec, p_this, p_cu,
         _chk(out, "out", torch.bfloat16), workspace.data_ptr(), workspace.numel() * workspace.element_size(),

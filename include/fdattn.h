@@ -186,6 +186,14 @@ FDATTN_API int fdattn_write_cache_kv(
  *                   tokens (each over the keys it attends to) and query heads, min(top_k, blocks of the row) are
  *                   kept, and token t attends to the kept blocks' keys up to itself.  0 / 1: such
  *                   rows get no attention output (they are prefill rows if seq_lens_encoder says so).
+ *   sqattn_per_token (fdattn_append_attention_ex only; with sqattn_top_k > 0 and decode_tokens > 1) != 0: every
+ *                   token of a decode row keeps a list of its own - min(top_k, the blocks it sees) blocks per KV
+ *                   head, scored with its own query over the seq_lens_decoder[b] + t + 1 keys it attends to - and
+ *                   attends to those: the step treats the row's tokens as so many decode rows of one token (a
+ *                   small kernel lays that view out in the workspace), so every shape of sqattn_top_k is served
+ *                   and decode_tokens is bounded by the workspace alone.  The decode side then runs over batch x
+ *                   decode_tokens rows: size the workspace with that number as `batch`
+ *                   (fdattn_append_attention_workspace_bytes[_ex]); the selector streams the keys once per token.
  */
 typedef struct fdattn_step_extras {
   const void* qkv_bias;
@@ -195,6 +203,7 @@ typedef struct fdattn_step_extras {
   int prefill_rows;
   int sqattn_top_k;
   int decode_tokens;
+  int sqattn_per_token;
 } fdattn_step_extras;
 
 /* fdattn_write_cache_kv with the extras (host pointer, read during the call; NULL = none). */

@@ -76,6 +76,13 @@ def test_version_and_argument_errors_need_no_gpu():
         rc = lib.fdattn_append_attention_ex(*([one] * 14), big, 4, 2, 0, 32, 8, hd, 64, 8, 16, 64, 0, 1, 0.1,
                                             ctypes.addressof(extras), None)
         assert rc == -2 and (b"decode_tokens" in lib.fdattn_last_error() or b"sqattn_top_k" in lib.fdattn_last_error())
+    # a list per token: the decode side runs over batch x decode_tokens rows, and the workspace is sized for those
+    per_token = _lib.StepExtras(None, None, None, 0.0, 0, 4, 3, 1)
+    fits_the_batch = lib.fdattn_append_attention_workspace_bytes_ex(4, 2, 32, 8, 128, 8, 1)
+    assert lib.fdattn_append_attention_workspace_bytes_ex(4, 6, 32, 8, 128, 8, 1) > fits_the_batch
+    rc = lib.fdattn_append_attention_ex(*([one] * 14), fits_the_batch, 4, 2, 0, 32, 8, 128, 64, 8, 16, 64, 0, 1, 0.1,
+                                        ctypes.addressof(per_token), None)
+    assert rc == -4 and b"sqattn_per_token" in lib.fdattn_last_error()
     assert lib.fdattn_decode_workspace_bytes(64, 32, 8, 128, 72) >= 64 * 8 * 3 * 2080
     # at least 16 partial rows (head_dim + 2 floats) per output row at any shape; a batch of fewer (sequence, KV head)
     # pairs than the GPU has CUs gets room for the up to 64 key splits that put a workgroup on each of them

@@ -86,3 +86,36 @@ def test_backend_refuses_draft_rows_its_decode_kernel_cannot_take():
         be.init_attention_metadata(book.schedule({0: 3}, drafts={0}))
     meta = be.init_attention_metadata(book.schedule({0: 3}))     # the same tokens as a prefill row: fine
     assert meta.decode_tokens == 1 and meta.prefill_rows == 1
+
+
+def test_backend_with_a_block_list_per_draft_token(oracle):
+    """sqattn_per_token on the backend: the same 3 draft tokens at 8 query heads per KV head that the one-list step
+    refuses are decode rows here, every token with its own top-k blocks (the decode side runs over tokens as rows, so
+    the rows-per-KV-head limit of the kernels for rows of several tokens does not apply); each step against the oracle."""
+    hq, hkv, d, bs, top_k = 64, 8, 128, 64, 3
+    g = torch.Generator().manual_seed(77)
+    be = fd.AppendAttentionBackend(hq, hkv, d, block_size=bs, max_position=1024, rope_theta=500000.0, sqattn_top_k=top_k,
+                                   sqattn_per_token=True)
+    pool = fd.BlockPool(num_blocks=24, block_size=bs, max_seqs=3, max_blocks_per_seq=8)
+    book = fd.SequenceBook(pool)
+    ks = (torch.rand((hkv, d), generator=g) * 2 + 2.0) / 127.0
+    vs = (torch.rand((hkv, d), generator=g) * 2 + 2.0) / 127.0
+    layer = be.allocate_layer(24, ks, vs)
+    cos, sin = (t.cpu() for t in be.rotary_embs)
+    for new_tokens, drafts in (({0: 380, 1: 200}, ()), ({0: 3, 1: 1}, {0}), ({0: 2, 1: 3, 2: 9}, {0, 1})):
+        meta = be.init_attention_metadata(book.schedule(new_tokens, drafts))
+        qkv = torch.randn((meta.num_tokens, (hq + 2 * hkv) * d), generator=g).to(torch.bfloat16)
+        before = dict(qkv=qkv, key_cache=layer.key_cache.cpu(), value_cache=layer.value_cache.cpu(),
+                      cache_k_scale=layer.cache_k_scale.cpu(), cache_v_scale=layer.cache_v_scale.cpu(),
+                      block_tables=meta.block_tables.cpu(), seq_lens_encoder=meta.seq_lens_encoder.cpu(),
+                      seq_lens_decoder=meta.seq_lens_decoder.cpu(), seq_lens_this_time=meta.seq_lens_this_time.cpu(),
+                      cu_seqlens_q=meta.cu_seqlens_q.cpu(), rope_cos=cos, rope_sin=sin, T=meta.num_tokens)
+        out = be.forward_mixed(qkv.cuda(), layer, meta)
+        torch.cuda.synchronize()
+        want, kc, vc = oracle_step(oracle, before, CACHE_INT8, hq=hq, hkv=hkv, decode_tokens=meta.decode_tokens,
+                                   top_k=top_k, per_token=True)
+        assert np.array_equal(np_of(layer.key_cache), kc) and np.array_equal(np_of(layer.value_cache), vc)
+        ok, mx, bad = bf16_close(bits(out), want)
+        assert ok, "step %r: %d out of tolerance, max %.4g" % (new_tokens, bad, mx)
+        book.commit()
+    assert book.lengths == [385, 204, 9]

@@ -7,7 +7,7 @@ import torch
 import fastdeploy_amd as fd
 from conftest import bf16_close, bits, np_of
 from fastdeploy_amd.ops import (CACHE_FP8, CACHE_FP8_BLOCK, CACHE_FP8_DYNAMIC, CACHE_INT8, CACHE_INT8_BLOCK,
-                                CACHE_INT8_DYNAMIC, byte_format, cu_seqlens_of, is_dynamic, scale_cache_shape,
+                                CACHE_INT8_DYNAMIC, append_attention_workspace_bytes, byte_format, cu_seqlens_of, is_dynamic, scale_cache_shape,
                                 seq_lens_this_time_of)
 from fastdeploy_amd.rope import rope_table
 
@@ -44,11 +44,12 @@ def mixed_case(enc, dec, quant, seed, hq=32, hkv=8, d=128, bs=64, max_pos=4096, 
                 rope_cos=cos, rope_sin=sin, T=T)
 
 
-def oracle_step(oracle, c, quant, hq=32, hkv=8, d=128, decode_tokens=1, top_k=0, **epilogue):
+def oracle_step(oracle, c, quant, hq=32, hkv=8, d=128, decode_tokens=1, top_k=0, per_token=False, **epilogue):
     """The step composed from the oracle's pieces; returns (out bf16 bits [T, hq*d] with NaN-free rows only where
     a token exists, key cache, value cache).  For the dynamic formats the scale caches the step leaves behind are
     put into c["scales_after"].  top_k > 0: the decode rows are block-sparse - a row keeps one list per KV head, a
-    block's score being the maximum over the row's tokens (each at its own length) and query heads."""
+    block's score being the maximum over the row's tokens (each at its own length) and query heads - or, per_token, every
+    token keeps its own list, scored by itself alone."""
     kc, vc = np_of(c["key_cache"]).copy(), np_of(c["value_cache"]).copy()
     ks, vs = np_of(c["cache_k_scale"]).copy(), np_of(c["cache_v_scale"]).copy()
     c["scales_after"] = (ks, vs)
@@ -70,7 +71,9 @@ def oracle_step(oracle, c, quant, hq=32, hkv=8, d=128, decode_tokens=1, top_k=0,
                 sc[i, :, (kvl[i] + 63) // 64:] = -np.inf   # blocks past a token's length are not scored by it
             kept = np.zeros((len(drows), hkv, top_k), np.int32)
             cnt = np.zeros((len(drows), hkv), np.int32)
-            for b in sorted(set(b for b, _ in drows)):
+            if per_token:
+                kept, cnt = oracle.topk_select(sc, kvl, 64, top_k)
+            for b in sorted(set(b for b, _ in drows)) if not per_token else ():
                 idx = [i for i, (bb, _) in enumerate(drows) if bb == b]
                 kb, cb = oracle.topk_select(sc[idx].max(axis=0, keepdims=True), kvl[idx[-1]:idx[-1] + 1], 64, top_k)
                 kept[idx], cnt[idx] = kb, cb
@@ -170,13 +173,15 @@ def test_mixed_step_with_key_splits_for_the_prefill_row(oracle):
     assert ok, "small workspace: %d out of tolerance, max %.4g" % (bad, mx)
 
 
-@pytest.mark.parametrize("top_k,tokens,rows", [(None, None, 1), (8, None, 1), (None, 2, 1), (8, 3, 1), (None, None, None),
-                                               (8, 2, None)])
-def test_mixed_step_with_key_splits_replays_from_a_hip_graph(top_k, tokens, rows):
+@pytest.mark.parametrize("top_k,tokens,rows,per_token", [(None, None, 1, False), (8, None, 1, False), (None, 2, 1, False),
+                                                         (8, 3, 1, False), (None, None, None, False), (8, 2, None, False),
+                                                         (8, 3, 1, True)])
+def test_mixed_step_with_key_splits_replays_from_a_hip_graph(top_k, tokens, rows, per_token):
     """The mixed step with key splits (writer, decode + its merge - with top_k the block selector and the sparse
     decode instead -, prefill shares, prefill merge) captured in a HIP graph: every replay, with eager work and synchronisations in between, equals the eager step on a copy of the
     state bit for bit (outputs and cache bytes).  rows None: without the host's count of prefill rows (the prefill
-    kernel counts them)."""
+    kernel counts them).  per_token: a block list per draft token (the token-as-row view is laid out by a kernel of
+    the step, inside the graph)."""
     enc, dec = [0, 160, 0, 0, 0], [900, 4200, 63, 2100, 4600]
     # (tokens: three of the decode rows bring that many draft tokens - the decode kernel's several-token variant)
     c = mixed_case(enc, dec, CACHE_INT8, seed=21, max_pos=8192, this=[tokens, 160, 1, tokens, tokens] if tokens else None)
@@ -185,15 +190,17 @@ def test_mixed_step_with_key_splits_replays_from_a_hip_graph(top_k, tokens, rows
     splits = fd.ops.prefill_auto_splits(1, 32, 160)
     assert splits > 1
     mb = dev["block_tables"].shape[1]
-    ws_g = fd.append_attention_workspace(c["T"], 5, 32, 8, 128, mb, prefill_splits=splits)
-    ws_e = fd.append_attention_workspace(c["T"], 5, 32, 8, 128, mb, prefill_splits=splits)
+    seqs = 5 * tokens if per_token else 5   # (a list per token: the decode side runs over batch x decode_tokens rows)
+    ws_g = fd.append_attention_workspace(c["T"], seqs, 32, 8, 128, mb, prefill_splits=splits)
+    ws_e = fd.append_attention_workspace(c["T"], seqs, 32, 8, 128, mb, prefill_splits=splits)
 
     def step(s, ws):
         return fd.append_attention(s["qkv"], s["key_cache"], s["value_cache"], s["seq_lens_encoder"],
                                    s["seq_lens_decoder"], s["seq_lens_this_time"], s["block_tables"],
                                    (s["rope_cos"], s["rope_sin"]), s["cache_k_scale"], s["cache_v_scale"],
                                    num_heads=32, kv_num_heads=8, max_chunk=160, cu_seqlens_q=s["cu_seqlens_q"],
-                                   prefill_rows=rows, workspace=ws, sqattn_top_k=top_k, decode_tokens=tokens)
+                                   prefill_rows=rows, workspace=ws, sqattn_top_k=top_k, decode_tokens=tokens,
+                                   sqattn_per_token=per_token)
 
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -444,6 +451,79 @@ def test_mixed_step_with_block_sparse_decode_rows_of_several_tokens(oracle, quan
                                            kept_counts=np.ascontiguousarray(np.repeat(cnt, n, 0)))
         ok, mx, bad = bf16_close(got[rows], want)
         assert ok, "sequence %d: %d out of tolerance, max %.4g" % (b, bad, mx)
+
+
+@pytest.mark.parametrize("quant,hq,hkv,tokens,d,bs", [
+    (CACHE_FP8, 32, 8, 4, 128, 64),            # the int8 / fp8-MFMA selector and sparse decode kernel
+    (CACHE_INT8_DYNAMIC, 16, 8, 3, 128, 64),
+    (CACHE_INT8, 32, 8, 6, 128, 64),           # 24 (token, head) pairs per KV head: more than one list per row allows
+    (CACHE_FP8_BLOCK, 8, 2, 3, 64, 16),        # the fp16-MFMA scoring pass and decode kernel
+    (CACHE_INT8, 16, 4, 2, 256, 32),
+    (CACHE_FP8, 6, 2, 3, 96, 32),              # the exact selector and the vector-ALU decode kernel
+])
+def test_mixed_step_with_a_block_list_per_token(oracle, quant, hq, hkv, tokens, d, bs):
+    """sqattn_top_k, decode_tokens and sqattn_per_token together: every token of a decode row of several tokens keeps
+    its OWN list - scored with its own query over the keys it attends to - and attends to it.  Against the oracle's
+    pieces per token: block scores at that token's length, top-k (indices must agree exactly, or the outputs would
+    not), one sparse decode.  Rows whose new tokens straddle a block boundary, a row on an empty cache, rows of fewer
+    tokens, rows with no more blocks than are kept, an idle slot, a prefill row; and the lists of a row's tokens do
+    differ, so the result is not the one-list step's."""
+    T, top_k = tokens, 5
+    enc = [0, 50, 0, 0, 0, 0, 0, 0, 0]
+    dec = [bs * 20 + 7, 300, bs * 9 - 1, 0, bs * 31 - T + 1, bs * 3, bs * 12 + 30 % bs, bs * 15, 77]
+    this = [T, 50, T, T, T, T, max(T - 1, 1), 1, 0]
+    c = mixed_case(enc, dec, quant, seed=170 + T, hq=hq, hkv=hkv, d=d, bs=bs, max_pos=4096, this=this)
+    dev = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
+    kw = dict(num_heads=hq, kv_num_heads=hkv, max_chunk=50, cache_quant_type=quant, cu_seqlens_q=dev["cu_seqlens_q"],
+              prefill_rows=1, sqattn_top_k=top_k, decode_tokens=T)
+    args = lambda: (dev["qkv"], dev["key_cache"], dev["value_cache"], dev["seq_lens_encoder"], dev["seq_lens_decoder"],
+                    dev["seq_lens_this_time"], dev["block_tables"], (dev["rope_cos"], dev["rope_sin"]),
+                    dev["cache_k_scale"], dev["cache_v_scale"])
+    out = fd.append_attention(*args(), sqattn_per_token=True, **kw)
+    torch.cuda.synchronize()
+    kc, vc = np_of(c["key_cache"]).copy(), np_of(c["value_cache"]).copy()
+    ks, vs = np_of(c["cache_k_scale"]).copy(), np_of(c["cache_v_scale"]).copy()
+    bt, cu, decs = np_of(c["block_tables"]), np_of(c["cu_seqlens_q"]), np_of(c["seq_lens_decoder"])
+    q, k_new, v_new = oracle.write_cache_kv(bits(c["qkv"]), kc, vc, ks, vs, np_of(c["rope_cos"]), np_of(c["rope_sin"]),
+                                            bt, decs, cu, hq, hkv, d, 1, quant, want_kv_out=True)
+    assert np.array_equal(np_of(dev["key_cache"]), kc) and np.array_equal(np_of(dev["value_cache"]), vc)
+    got = bits(out)
+    lists_differ = False
+    for b in range(len(enc)):
+        rows = list(range(cu[b], cu[b + 1]))
+        if not rows:
+            continue
+        if enc[b] > 0:
+            want = oracle.append_attention_prefill(q, k_new, v_new, kc, vc, ks, vs, bt, decs, cu, hq, hkv, d, quant,
+                                                   token_ids=np.array(rows, np.int32))[rows]
+        else:
+            n = len(rows)
+            qd = np.ascontiguousarray(q[rows])
+            btd = np.ascontiguousarray(np.repeat(bt[b:b + 1], n, 0))
+            kvl = np.array([decs[b] + t + 1 for t in range(n)], np.int32)
+            sc = oracle.sqattn_block_scores(qd, kc, ks, btd, kvl, hq, hkv, d, quant)   # [n, hkv, max_blocks]
+            kept, cnt = oracle.topk_select(sc, kvl, bs, top_k)
+            lists_differ |= any(not np.array_equal(kept[t], kept[t + 1]) for t in range(n - 1))
+            want = oracle.decode_attention(qd, kc, vc, ks, vs, btd, kvl, hq, hkv, d, quant, kept_blocks=kept, kept_counts=cnt)
+        ok, mx, bad = bf16_close(got[rows], want)
+        assert ok, "sequence %d: %d out of tolerance, max %.4g" % (b, bad, mx)
+    assert lists_differ
+    # a workspace of the caller's, sized for batch x decode_tokens sequences, full of garbage, used twice
+    ws = torch.full((append_attention_workspace_bytes(c["T"], len(enc) * T, hq, hkv, d, bt.shape[1], 1),), 0xAB,
+                    dtype=torch.uint8, device="cuda")
+    for _ in range(2):
+        dev2 = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
+        again = fd.append_attention(dev2["qkv"], dev2["key_cache"], dev2["value_cache"], dev2["seq_lens_encoder"],
+                                    dev2["seq_lens_decoder"], dev2["seq_lens_this_time"], dev2["block_tables"],
+                                    (dev2["rope_cos"], dev2["rope_sin"]), dev2["cache_k_scale"], dev2["cache_v_scale"],
+                                    sqattn_per_token=True, workspace=ws, **kw)
+        live = [t for b in range(len(enc)) for t in range(cu[b], cu[b + 1])]
+        assert torch.equal(again[live], out[live])
+    # one sized for the batch alone is refused before anything is written
+    small = torch.empty(append_attention_workspace_bytes(c["T"], len(enc), hq, hkv, d, bt.shape[1], 1), dtype=torch.uint8,
+                        device="cuda")
+    with pytest.raises(ValueError, match="sqattn_per_token"):
+        fd.append_attention(*args(), sqattn_per_token=True, workspace=small, **kw)
 
 
 @pytest.mark.parametrize("quant,hq,hkv,tokens", [(CACHE_INT8, 32, 8, 2), (CACHE_FP8, 32, 8, 2), (CACHE_INT8_DYNAMIC, 32, 8, 2),
