@@ -700,7 +700,8 @@ def test_mixed_step_counts_its_prefill_rows(oracle, enc, dec, hq, hkv, quant):
 
 def random_steps(oracle, seed, iters):
     """Seeded random steps: 1 .. 8 slots that are prefill rows (1 .. 140 new tokens, with or without cached tokens),
-    decode rows - of several draft tokens in some steps, block-sparse (top 1 .. 6 blocks) in some - or idle; 1 .. 8
+    decode rows - of several draft tokens in some steps, block-sparse (top 1 .. 6 blocks) in some, with one block list
+    per row or per token where both meet - or idle; 1 .. 8
     query heads per KV head; any cache format; with and without the prefill-row count.  Cache bytes (and scale
     caches) exact, outputs within tolerance."""
     rng = np.random.default_rng(seed)
@@ -710,6 +711,7 @@ def random_steps(oracle, seed, iters):
         quant = formats[int(rng.integers(0, len(formats)))]
         tokens = int(rng.integers(1, 16 // group + 1)) if it % 3 == 2 else 1   # draft tokens a decode row may bring
         top_k = int(rng.integers(1, 7)) if it % 4 == 1 else 0                   # block-sparse decode rows
+        per_token = it % 24 == 5   # (of the steps with both, every other one keeps a block list per token)
         enc, dec, this = [], [], []
         for _ in range(slots):
             kind = int(rng.integers(0, 4))   # prefill on nothing, prefill on a prefix, decode, idle
@@ -727,11 +729,12 @@ def random_steps(oracle, seed, iters):
                                   (dev["rope_cos"], dev["rope_sin"]), dev["cache_k_scale"], dev["cache_v_scale"],
                                   num_heads=hq, kv_num_heads=hkv, max_chunk=max(enc), cache_quant_type=quant,
                                   cu_seqlens_q=dev["cu_seqlens_q"], prefill_rows=rows if it % 2 else None,
-                                  decode_tokens=tokens, sqattn_top_k=top_k)
+                                  decode_tokens=tokens, sqattn_top_k=top_k, sqattn_per_token=per_token)
         torch.cuda.synchronize()
-        what = "seed %d step %d: enc %r dec %r this %r group %d hkv %d quant %d tokens %d top_k %d" % (
-            seed, it, enc, dec, this, group, hkv, quant, tokens, top_k)
-        want, kc, vc = oracle_step(oracle, c, quant, hq, hkv, 128, decode_tokens=tokens, top_k=top_k)
+        what = "seed %d step %d: enc %r dec %r this %r group %d hkv %d quant %d tokens %d top_k %d per token %d" % (
+            seed, it, enc, dec, this, group, hkv, quant, tokens, top_k, per_token)
+        want, kc, vc = oracle_step(oracle, c, quant, hq, hkv, 128, decode_tokens=tokens, top_k=top_k,
+                                   per_token=per_token and tokens > 1 and top_k > 0)
         assert np.array_equal(np_of(dev["key_cache"]), kc) and np.array_equal(np_of(dev["value_cache"]), vc), what
         if is_dynamic(quant):
             assert np.array_equal(np_of(dev["cache_k_scale"]), c["scales_after"][0]), what
