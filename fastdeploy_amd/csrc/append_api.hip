@@ -115,8 +115,9 @@ extern "C" int fdattn_append_attention_ex(
   // every token of a decode row with a block list of its own: the decode side of the step runs over the token-as-row
   // view, whose batch is what the workspace must be sized for
   const bool per_token = top_k > 0 && decode_tokens > 1 && extras->sqattn_per_token != 0;
-  if (per_token && (long long)batch * decode_tokens > 0x7fffffffLL / 64)
-    return fail(FDATTN_ERR_SHAPE, "fdattn_append_attention: batch %d x decode_tokens %d is too large", batch, decode_tokens);
+  if (per_token && (long long)batch * decode_tokens * hkv > (1LL << 20))  // (the decode launchers' limit on (row, KV head) pairs)
+    return fail(FDATTN_ERR_SHAPE, "fdattn_append_attention: sqattn_per_token: batch %d x decode_tokens %d x %d KV heads "
+                "exceeds %d rows", batch, decode_tokens, hkv, 1 << 20);
   const int dbatch = per_token ? batch * decode_tokens : batch;
   StepWorkspace w = step_workspace(num_tokens, dbatch, hq, hkv, head_dim, max_blocks_per_seq, splits);
   while (splits > 1 && workspace_bytes < w.total)  // a workspace sized for fewer splits: use as many as it holds
