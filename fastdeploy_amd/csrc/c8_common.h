@@ -13,6 +13,7 @@ constexpr int kSlotFloats = kG * kD;       // partial o of one row set
 constexpr int kMaxSets = 2;                // row sets a decode wavefront carries: up to 8 query heads per KV head
 constexpr int kMaxSetsSpec = 4;            // decode rows of several tokens: up to 16 (token, head) rows
 constexpr int kMaxChunk = 128;        // units per chunk: two unit-table entries per lane
+constexpr int kMaxChunkDecode = 256;  // the decode kernel with one or two row sets: four entries per lane
 
 __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
 

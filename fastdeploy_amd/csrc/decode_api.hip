@@ -129,7 +129,7 @@ extern "C" int fdattn_decode_uses_mfma(int hq, int hkv, int head_dim, int block_
 
 extern "C" int fdattn_decode_chunks_per_sequence(int batch, int hkv, int max_blocks_per_seq) {
   if (batch <= 0 || hkv <= 0 || max_blocks_per_seq <= 0) return 0;
-  const int chunk = c8_pick_chunk(batch * hkv, max_blocks_per_seq);
+  const int chunk = c8_pick_chunk(batch * hkv, max_blocks_per_seq, 256);  // (rows of one token: the wide unit table)
   return (max_blocks_per_seq + chunk - 1) / chunk;
 }
 

@@ -6,7 +6,8 @@
 // chunks of `chunk` units; one workgroup of 4 wavefronts takes one chunk (grid = chunks
 // per pair x pairs, workgroups past the end of a list do nothing).  The chunk length is
 // picked so that the launch fills the GPU's workgroup slots once (c8_pick_chunk): as
-// few, as long workgroups as that allows, up to 128 units each.  Pair and chunk follow
+// few, as long workgroups as that allows, up to 256 units each (128 where rows of several
+// tokens need three or four row sets).  Pair and chunk follow
 // from the block index, the physical blocks from one coalesced read of the block table.
 //
 // Inside a workgroup every wavefront is autonomous: it takes units wave, wave+4, ... of
@@ -110,9 +111,13 @@ __global__ __launch_bounds__(kWaves * 64, NSET > 2 ? 1 : 2) void decode_c8_kerne
   // loads of the sequence's length below instead of behind them - under load every dependent
   // round trip to memory at the start of a workgroup costs microseconds in which its LDS slots
   // carry nothing.
-  int lb[2] = {-1, -1}, pb_raw[2] = {-1, -1};
+  // (kEnt entries per lane: four hold chunks of up to 256 units; the kernels with three or four row sets, which have no
+  // registers to spare, keep two)
+  constexpr int kEnt = NSET <= 2 ? 4 : 2;
+  int lb[kEnt], pb_raw[kEnt];
 #pragma unroll
-  for (int e = 0; e < 2; ++e) {
+  for (int e = 0; e < kEnt; ++e) {
+    lb[e] = -1, pb_raw[e] = -1;
     const int u = lane + 64 * e;
     if (u < a.chunk) {
       int l = first + u;
@@ -152,22 +157,31 @@ __global__ __launch_bounds__(kWaves * 64, NSET > 2 ? 1 : 2) void decode_c8_kerne
   const int n16 = lane & 15, g4 = lane >> 4;
 
   // lane j describes units first + j and first + j + 64 (physical block, valid tokens)
-  int my_pb[2] = {0, 0}, my_valid[2] = {0, 0};
+  int my_pb[kEnt], my_valid[kEnt];
   {
     // the table loads are consumed here on every path: nothing of the table build stays in
     // flight when the streaming loop starts
-    asm volatile("" ::"v"(lb[0]), "v"(pb_raw[0]), "v"(lb[1]), "v"(pb_raw[1]));
 #pragma unroll
-    for (int e = 0; e < 2; ++e)
+    for (int e = 0; e < kEnt; ++e) asm volatile("" ::"v"(lb[e]), "v"(pb_raw[e]));
+#pragma unroll
+    for (int e = 0; e < kEnt; ++e) {
+      my_pb[e] = 0, my_valid[e] = 0;
       if (lane + 64 * e < cnt && pb_raw[e] >= 0 && pb_raw[e] < a.num_blocks) {
         my_pb[e] = pb_raw[e];
         // SPEC: not cut at the block's size, so that an earlier token's smaller count can be taken from it
         my_valid[e] = min(max(kv_len - lb[e] * kBS, 0), SPEC ? kBS + 4 * kMaxSetsSpec : kBS);
       }
+    }
   }
   // entry of unit j (uniform)
-  auto unit_pb = [&](int j) { return j < 64 ? __builtin_amdgcn_readlane(my_pb[0], j) : __builtin_amdgcn_readlane(my_pb[1], j - 64); };
-  auto unit_valid = [&](int j) { return j < 64 ? __builtin_amdgcn_readlane(my_valid[0], j) : __builtin_amdgcn_readlane(my_valid[1], j - 64); };
+  auto entry = [&](const int (&v)[kEnt], int j) {
+    if (j < 64) return __builtin_amdgcn_readlane(v[0], j);
+    if (kEnt == 2 || j < 128) return __builtin_amdgcn_readlane(v[1], j - 64);
+    if (j < 192) return __builtin_amdgcn_readlane(v[kEnt > 2 ? 2 : 0], j - 128);
+    return __builtin_amdgcn_readlane(v[kEnt > 2 ? 3 : 0], j - 192);
+  };
+  auto unit_pb = [&](int j) { return entry(my_pb, j); };
+  auto unit_valid = [&](int j) { return entry(my_valid, j); };
 
   const size_t tile_stride = (size_t)kBS * kD;  // bytes of one (block, head) tile
   const uint8_t* const kbase = a.key_cache + (size_t)h * tile_stride;
@@ -540,18 +554,21 @@ int gpu_cu_count() {
   return cus;
 }
 
-int c8_pick_chunk(int pairs, int max_units) {
+int c8_pick_chunk(int pairs, int max_units, int most) {
   const int cpp = (2 * gpu_cu_count() + pairs - 1) / pairs;  // two workgroups of this kernel fit a CU
   int chunk = (max_units + cpp - 1) / cpp;
   if (chunk < kWaves) chunk = kWaves;
-  if (chunk > kMaxChunk) {
-    // a list longer than the unit table: as few chunks as hold it, of equal size (137 units = 69 + 68, not 128 + 9:
+  if (chunk > most) {
+    // a list longer than the unit table: as few chunks as hold it, of equal size (273 units = 137 + 136, not 256 + 17:
     // the longest chunk sets the launch's duration)
-    const int n = (max_units + kMaxChunk - 1) / kMaxChunk;
+    const int n = (max_units + most - 1) / most;
     chunk = (max_units + n - 1) / n;
   }
   return chunk;
 }
+
+// the decode kernel's unit table by its row sets (ceil(rows per KV head / 4))
+static int decode_table_units(int sets) { return sets <= 2 ? kMaxChunkDecode : kMaxChunk; }
 
 constexpr int kMaxPairs = 1 << 20;
 
@@ -577,7 +594,7 @@ size_t c8_workspace_bytes(int batch, int hkv, int max_units, int group) {
   if (!most) {
     most = 1;
     for (int u = 1; u <= max_units; ++u) {
-      const int chunk = c8_pick_chunk(pairs, u), n = (u + chunk - 1) / chunk;
+      const int chunk = c8_pick_chunk(pairs, u, kMaxChunk), n = (u + chunk - 1) / chunk;  // (the smaller table: never fewer chunks)
       if (n > most) most = n;
     }
     std::lock_guard<std::mutex> g(mu);
@@ -630,7 +647,7 @@ int decode_c8_launch(const void* q, const void* key_cache, const void* value_cac
     return fail(FDATTN_ERR_SHAPE, "fdattn_decode_attention: decode rows of up to %d tokens need a step's row map and "
                 "tokens x query heads per KV head <= %d (here %d)", max_tokens, kG * kMaxSetsSpec, vgmax);
   const int max_units = sparse ? (max_kept < max_blocks ? max_kept : max_blocks) : max_blocks;
-  const int chunk = c8_pick_chunk(pairs, max_units);
+  const int chunk = c8_pick_chunk(pairs, max_units, decode_table_units(sets));
   const int cpp = ((max_units + chunk - 1) / chunk);
   if (pairs > kMaxPairs)
     return fail(FDATTN_ERR_SHAPE, "fdattn_decode_attention: batch*kv_heads = %d exceeds %d", pairs, kMaxPairs);

@@ -20,8 +20,9 @@ constexpr int kDecodeAuto = 0, kDecodeVectorAlu = 1, kDecodeTiles = 2;
 // compute units of the current device (256 on MI355X; that value if the query fails)
 int gpu_cu_count();
 // units (cache blocks) per workgroup for `pairs` block lists of at most max_units blocks: as few chunks per
-// list as fill the GPU's workgroup slots once, at most kMaxChunk units each
-int c8_pick_chunk(int pairs, int max_units);
+// list as fill the GPU's workgroup slots once, at most `most` units each (the kernel's unit table: 128, or the 256 of
+// the decode kernel with one or two row sets)
+int c8_pick_chunk(int pairs, int max_units, int most = 128);
 size_t c8_workspace_bytes(int batch, int hkv, int max_units, int group = 4);
 bool c8_supported(int hq, int hkv, int d, int bs, int quant);
 // stages: 1 = the split-KV kernel, 2 = the merge of its partials, 3 = both

@@ -261,7 +261,7 @@ FDATTN_API int fdattn_decode_attention(
  * FDATTN_ERR_WORKSPACE and nothing is enqueued.  What a shape needs is what the kernel that takes it needs:
  *   - the int8-MFMA kernel (fdattn_decode_uses_mfma() = 1): one partial of ceil(hq/hkv / 4) x 2,080 B per chunk of
  *     a (sequence, KV head) pair's block list; lists are cut into ceil(2 x CUs / pairs) chunks (one, and then no
- *     partial is written at all, from 512 pairs on a 256-CU GPU), more only beyond 128 blocks per chunk.  Llama-3-8B
+ *     partial is written at all, from 512 pairs on a 256-CU GPU), more only beyond 256 blocks per chunk.  Llama-3-8B
  *     decode at batch 64 (512 pairs, 72 blocks each) asks for 1 MiB; the limit is reached near 8,000 pairs of one
  *     chunk each, or e.g. 512 pairs of 2,048 blocks (128k tokens) each;
  *   - the other shapes: 16 partial rows of (head_dim + 2) floats per (sequence, query head), i.e.

@@ -420,6 +420,28 @@ def test_workspace_is_reusable_across_calls_and_shapes(oracle):
             check(got, oracle_decode(oracle, case), "reuse rep %d" % rep)
 
 
+@pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_FP8_DYNAMIC])
+def test_decode_lists_of_up_to_256_blocks_in_one_chunk(oracle, quant):
+    """64 sequences (512 (sequence, KV head) pairs: one chunk per list) of 8.2k to 16.4k tokens: lists of 129 .. 256
+    blocks, the third and fourth entries per lane of the int8-MFMA kernel's unit table, go through one workgroup each
+    with no partial and no merge launch; 257 blocks make two chunks.  The tables draw from a pool of 3,000 blocks, so
+    sequences share blocks (as after a fork); against the oracle."""
+    from fastdeploy_amd import _lib
+    assert _lib.lib().fdattn_decode_chunks_per_sequence(64, 8, 256) == 1
+    assert _lib.lib().fdattn_decode_chunks_per_sequence(64, 8, 257) == 2
+    g = torch.Generator().manual_seed(11)
+    base = syn.decode_case(batch=64, ctx=64, pool_blocks=3000, seed=3, quant=quant, direct_bytes=True, max_blocks=257)
+    lens = torch.randint(64 * 128 + 1, 64 * 256 + 1, (64,), generator=g)
+    lens[0], lens[1], lens[2] = 64 * 256, 64 * 128 + 1, 64 * 192 + 1   # the table's last entry, its 129th, its 193rd
+    case = dict(base)
+    case["seq_lens_decoder"] = lens.to(torch.int32)
+    case["block_tables"] = torch.randint(0, 3000, (64, 257), generator=g).to(torch.int32)
+    for mb in (256, 257):
+        c = dict(case)
+        c["block_tables"] = case["block_tables"][:, :mb].contiguous()
+        check(gpu_decode(c), oracle_decode(oracle, c), "tables of %d entries" % mb)
+
+
 @pytest.mark.parametrize("quant", [CACHE_INT8, CACHE_INT8_DYNAMIC])
 def test_decode_config2_full_size(oracle, quant):
     """batch 64, ctx U[3584, 4608], int8 KV (per-channel scales, and one scale per stored row), block tables a random permutation over a 6000-block pool:
